@@ -1,0 +1,114 @@
+"""In-tree build of the native libraries (gfx950 only).
+
+    libbt_hip.so               HIP kernels + C ABI          (hipcc, include/bt_hip.h)
+    libbytetransformer.so      host C++ BertTransformer API (g++,   include/bytetransformer/, bt_encoder.h)
+    libths_bytetransformer.so  PyTorch operator             (g++ against the installed PyTorch-ROCm)
+
+Run `python -m bytetransformer_amd.build [kernels|host|th_op|all]`.  Outputs
+land in bytetransformer_amd/lib/.
+"""
+import os
+import subprocess
+import sys
+import time
+
+PKG = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(PKG)
+CSRC = os.path.join(PKG, "csrc")
+LIB = os.path.join(PKG, "lib")
+INC = os.path.join(ROOT, "include")
+ROCM = os.environ.get("ROCM_PATH", "/opt/rocm")
+HIPCC = os.path.join(ROCM, "bin", "hipcc")
+
+KERNEL_SOURCES = ["padding.hip", "layernorm.hip", "gemm.hip", "attention.hip"]
+HOST_SOURCES = ["attention.cc", "bert_transformer.cc", "c_api.cc"]
+TH_OP_SOURCES = ["ths_op_f.cc", "ths_op.cc"]
+
+# Packed-fp32 VALU ops are switched off for every device compile.
+HIP_FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
+             "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+             "-Wno-unused-command-line-argument"]
+HOST_FLAGS = ["-O2", "-std=c++17", "-fPIC", "-D__HIP_PLATFORM_AMD__", "-Wall"]
+
+
+def _run(cmd):
+    t0 = time.time()
+    proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    out = "\n".join(l for l in proc.stdout.splitlines()
+                    if "packed-fp32-ops" not in l and "is not a recognized feature" not in l)
+    if proc.returncode != 0:
+        raise RuntimeError("build step failed:\n  %s\n%s" % (" ".join(cmd), out))
+    if out.strip():
+        print(out)
+    print("[build] %.1fs  %s" % (time.time() - t0, os.path.basename(cmd[cmd.index("-o") + 1])))
+
+
+def _parallel(cmds, jobs=4):
+    from concurrent.futures import ThreadPoolExecutor
+    with ThreadPoolExecutor(max_workers=jobs) as ex:
+        list(ex.map(_run, cmds))
+
+
+def build_kernels():
+    os.makedirs(LIB, exist_ok=True)
+    obj_dir = os.path.join(PKG, "_build")
+    os.makedirs(obj_dir, exist_ok=True)
+    objs, cmds = [], []
+    for src in KERNEL_SOURCES:
+        obj = os.path.join(obj_dir, src.replace(".hip", ".o"))
+        objs.append(obj)
+        cmds.append([HIPCC] + HIP_FLAGS + ["-I", INC, "-I", os.path.join(CSRC, "kernels"), "-c",
+                                           os.path.join(CSRC, "kernels", src), "-o", obj])
+    _parallel(cmds)
+    out = os.path.join(LIB, "libbt_hip.so")
+    _run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC"] + objs + ["-o", out])
+    return out
+
+
+def build_host():
+    os.makedirs(LIB, exist_ok=True)
+    out = os.path.join(LIB, "libbytetransformer.so")
+    srcs = [os.path.join(CSRC, "host", s) for s in HOST_SOURCES]
+    _run(["g++"] + HOST_FLAGS + ["-shared", "-I", INC, "-I", os.path.join(ROCM, "include")] + srcs +
+         ["-L", LIB, "-lbt_hip", "-Wl,-rpath,$ORIGIN", "-o", out])
+    return out
+
+
+def build_th_op():
+    import torch
+    from torch.utils import cpp_extension
+    os.makedirs(LIB, exist_ok=True)
+    out = os.path.join(LIB, "libths_bytetransformer.so")
+    inc = []
+    for p in cpp_extension.include_paths():
+        inc += ["-isystem", p]
+    torch_lib = os.path.join(os.path.dirname(torch.__file__), "lib")
+    abi = int(torch._C._GLIBCXX_USE_CXX11_ABI)
+    obj_dir = os.path.join(PKG, "_build")
+    os.makedirs(obj_dir, exist_ok=True)
+    objs, cmds = [], []
+    for s in TH_OP_SOURCES:
+        path = os.path.join(CSRC, "th_op", s)
+        if not os.path.exists(path):
+            continue
+        obj = os.path.join(obj_dir, "th_" + s.replace(".cc", ".o"))
+        objs.append(obj)
+        cmds.append(["g++"] + HOST_FLAGS + ["-DUSE_ROCM", "-D_GLIBCXX_USE_CXX11_ABI=%d" % abi,
+                                            "-Wno-unused-variable", "-Wno-deprecated-declarations",
+                                            "-I", INC, "-I", os.path.join(CSRC, "th_op"),
+                                            "-isystem", os.path.join(ROCM, "include")] + inc +
+                    ["-c", path, "-o", obj])
+    _parallel(cmds)
+    _run(["g++", "-shared", "-fPIC"] + objs +
+         ["-L", LIB, "-lbytetransformer", "-lbt_hip", "-L", torch_lib, "-lc10", "-lc10_hip",
+          "-ltorch_cpu", "-ltorch_hip", "-ltorch", "-Wl,-rpath,$ORIGIN", "-o", out])
+    return out
+
+
+def build_all():
+    return [build_kernels(), build_host(), build_th_op()]
+
+
+if __name__ == "__main__":
+    what = sys.argv[1] if len(sys.argv) > 1 else "all"
+    {"kernels": build_kernels, "host": build_host, "th_op": build_th_op, "all": build_all}[what]()

@@ -1,0 +1,40 @@
+// Attention<OpType>::infer - picks one of the two fused MHA kernels.
+// Dispatch role of the reference's attention.h:124-139 and of the path
+// selection in bert_transformer.h:132-185, reduced to what exists on gfx950:
+// an LDS-resident short-sequence kernel and a streaming grouped kernel.
+#include "bytetransformer/attention.h"
+
+#include <cmath>
+
+namespace bytetransformer {
+
+template <OperationType OpType>
+void Attention<OpType>::infer(AttentionInferParam infer_param) {
+  if (OpType != OperationType::HALF)
+    throw std::runtime_error("[BT][ERROR] Attention: only OperationType::HALF is implemented");
+  if (infer_param.attention_bias != nullptr)
+    throw std::runtime_error("[BT][ERROR] Attention: attention_bias is not supported");
+  if (infer_param.et_param.batch_idx == nullptr)
+    throw std::runtime_error("[BT][ERROR] Attention: et_param.batch_idx must be set");
+  if (infer_param.batch_size > max_batch_size_ || infer_param.seq_len > max_seq_len_)
+    throw std::runtime_error("[BT][ERROR] Attention: batch_size/seq_len exceed the constructed maximum");
+
+  const int rows_cap = infer_param.batch_size * infer_param.seq_len;
+  const float scale = 1.0f / std::sqrt((float)size_per_head_) / param_.tao;
+  const int padded_rows = is_remove_padding_ ? 0 : 1;
+  if (uses_short_kernel(infer_param.seq_len))
+    check_bt_error(bt_attention_short(infer_param.qkv, infer_param.attention_output,
+                                      infer_param.et_param.batch_idx, infer_param.batch_size,
+                                      infer_param.seq_len, rows_cap, head_num_, size_per_head_,
+                                      scale, padded_rows, infer_param.stream));
+  else
+    check_bt_error(bt_attention_grouped(infer_param.qkv, infer_param.attention_output,
+                                        infer_param.et_param.batch_idx, infer_param.batch_size,
+                                        infer_param.seq_len, rows_cap, head_num_, size_per_head_,
+                                        scale, padded_rows, infer_param.stream));
+}
+
+template class Attention<OperationType::FP32>;
+template class Attention<OperationType::HALF>;
+
+}  // namespace bytetransformer

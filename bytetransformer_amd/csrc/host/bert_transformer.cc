@@ -1,0 +1,122 @@
+// BertTransformer<OpType>::bert_infer - host orchestration of one encoder
+// layer over the C ABI.  Same operation order, residual choices and buffer
+// reuse as the reference's bytetransformer/src/bert_transformer.cu:28-130; what
+// differs is that nothing here waits for the device: the valid-token count
+// stays in batch_idx[batch_size] and every kernel bounds itself with it.
+#include "bytetransformer/bert_transformer.h"
+
+namespace bytetransformer {
+
+template <OperationType OpType>
+void BertTransformer<OpType>::bert_infer(BertTransformerInferParam infer_param) {
+  if (OpType != OperationType::HALF)
+    throw std::runtime_error(
+        "[BT][ERROR] BertTransformer: only OperationType::HALF is implemented");
+  if (inner_buf_size_ == 0) cal_bufsize();
+
+  const DataType_ *from_tensor = infer_param.input_tensor;
+  const DataType_ *atten_mask = infer_param.atten_mask;
+  DataType_ *transformer_out = infer_param.transformer_output;
+  const int batch_size = infer_param.batch_size;
+  const int seq_len = infer_param.seq_len;
+  hipStream_t stream = infer_param.stream;
+
+  if (!from_tensor || !atten_mask || !transformer_out || !infer_param.buf)
+    throw std::runtime_error("[BT][ERROR] BertTransformer: null input/mask/output/buf pointer");
+  if (batch_size <= 0 || seq_len <= 0 || batch_size > max_batch_size_ || seq_len > max_seq_len_)
+    throw std::runtime_error(
+        "[BT][ERROR] BertTransformer: batch_size/seq_len outside the constructed maximum");
+  if (infer_param.attention_bias != nullptr)
+    throw std::runtime_error("[BT][ERROR] BertTransformer: attention_bias is not supported");
+  if (from_tensor == transformer_out && is_remove_padding_)
+    throw std::runtime_error(
+        "[BT][ERROR] BertTransformer: transformer_output must not alias input_tensor");
+
+  const int hidden = head_num_ * size_per_head_;
+  const int inter = hidden * param_.intermediate_size;
+  const int rows = batch_size * seq_len;
+  const size_t tensor = (size_t)rows * hidden;
+
+  // carve the scratch with the maxima, exactly as cal_bufsize() laid it out
+  const unsigned long long max_rows = (unsigned long long)max_batch_size_ * max_seq_len_;
+  const unsigned long long max_tensor = max_rows * hidden;
+  uint8_t *base = (uint8_t *)infer_param.buf;
+  DataType_ *inner_buf = (DataType_ *)base;
+  DataType_ *qkv_buf = inner_buf;
+  DataType_ *attr_out_buf = inner_buf + 3 * tensor;
+  DataType_ *attr_matmul_buf = inner_buf + 4 * tensor;
+  DataType_ *inter_matmul_buf = inner_buf + 5 * tensor;
+  unsigned long long off =
+      align_up((5 + param_.intermediate_size) * max_tensor * sizeof(DataType_), 256);
+  ET_Param et_param;
+  et_param.word_idx = (int *)(base + off);
+  et_param.batch_idx = et_param.word_idx + max_rows;
+  et_param.valid_word_num = rows;
+  off += align_up(max_rows * 2 * sizeof(int) + 2 * sizeof(int), 256);
+  DataType_ *wt_qkv = (DataType_ *)(base + off);
+  DataType_ *wt_proj = wt_qkv + (size_t)3 * hidden * hidden;
+  DataType_ *wt_inter = wt_proj + (size_t)hidden * hidden;
+  DataType_ *wt_out = wt_inter + (size_t)hidden * inter;
+
+  // lengths from the mask (needed on both paths: keys past len_b are excluded)
+  check_bt_error(bt_build_offsets(atten_mask, Traits_::dtype, batch_size, seq_len,
+                                  et_param.batch_idx, et_param.word_idx, nullptr, stream));
+  const int *valid_rows = nullptr;
+  DataType_ *restore_target = nullptr;
+  if (is_remove_padding_) {
+    // packed x lives in the caller's output buffer until the final restore
+    check_bt_error(bt_compress(from_tensor, transformer_out, et_param.batch_idx,
+                               et_param.word_idx, batch_size, seq_len, hidden, stream));
+    from_tensor = transformer_out;
+    restore_target = transformer_out;
+    transformer_out = inner_buf;  // FFN2 output reuses the dead qkv region
+    valid_rows = et_param.batch_idx + batch_size;
+  }
+
+  // k-contiguous weight pre-pack
+  check_bt_error(bt_transpose_weight(param_.attr_kernel_QKV, wt_qkv, hidden, 3 * hidden, stream));
+  check_bt_error(bt_transpose_weight(param_.attr_output_kernel, wt_proj, hidden, hidden, stream));
+  check_bt_error(bt_transpose_weight(param_.inter_kernel, wt_inter, hidden, inter, stream));
+  check_bt_error(bt_transpose_weight(param_.output_kernel, wt_out, inter, hidden, stream));
+
+  check_bt_error(bt_gemm_qkv_bias_split(from_tensor, wt_qkv, param_.attention_param.attr_bias_QKV,
+                                        qkv_buf, valid_rows, rows, head_num_, size_per_head_,
+                                        stream));
+
+  struct AttentionInferParam<DataType_> attention_infer_param {
+    qkv_buf, atten_mask, attr_out_buf, base + inner_buf_size_, batch_size, seq_len,
+        infer_param.cublas_handle, stream, et_param
+  };
+  attention_infer_param.attention_bias = infer_param.attention_bias;
+  attention_layer_->infer(attention_infer_param);
+
+  check_bt_error(
+      bt_gemm(attr_out_buf, wt_proj, attr_matmul_buf, valid_rows, rows, hidden, hidden, stream));
+
+  check_bt_error(bt_add_bias_residual_layernorm(
+      attr_matmul_buf, from_tensor, param_.attr_output_bias, param_.attr_output_layernorm_gamma,
+      param_.attr_output_layernorm_beta, use_fp32_ ? 1 : 0, valid_rows, rows, hidden,
+      layernorm_eps, stream));
+
+  check_bt_error(bt_gemm_bias_gelu(attr_matmul_buf, wt_inter, param_.inter_bias, inter_matmul_buf,
+                                   valid_rows, rows, inter, hidden, stream));
+
+  check_bt_error(
+      bt_gemm(inter_matmul_buf, wt_out, transformer_out, valid_rows, rows, hidden, inter, stream));
+
+  if (is_remove_padding_)
+    check_bt_error(bt_add_bias_residual_layernorm_restore(
+        transformer_out, attr_matmul_buf, param_.output_bias, param_.output_layernorm_gamma,
+        param_.output_layernorm_beta, use_fp32_ ? 1 : 0, restore_target, et_param.batch_idx,
+        batch_size, seq_len, hidden, layernorm_eps, stream));
+  else
+    check_bt_error(bt_add_bias_residual_layernorm(
+        transformer_out, attr_matmul_buf, param_.output_bias, param_.output_layernorm_gamma,
+        param_.output_layernorm_beta, use_fp32_ ? 1 : 0, nullptr, rows, hidden, layernorm_eps,
+        stream));
+}
+
+template class BertTransformer<OperationType::FP32>;
+template class BertTransformer<OperationType::HALF>;
+
+}  // namespace bytetransformer

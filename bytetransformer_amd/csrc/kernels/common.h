@@ -1,0 +1,73 @@
+// Shared device helpers for the gfx950 kernels: vector types, wave64
+// reductions, error plumbing for the C ABI.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <hip/hip_fp16.h>
+
+#include <cstdarg>
+#include <cstdio>
+
+#include "bt_hip.h"
+
+namespace bt {
+
+constexpr int kWave = 64;
+
+typedef _Float16 half_t;
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+typedef float float4_t __attribute__((ext_vector_type(4)));
+typedef float float16_t __attribute__((ext_vector_type(16)));
+typedef unsigned int uint4_t __attribute__((ext_vector_type(4)));
+typedef unsigned int uint2_t __attribute__((ext_vector_type(2)));
+
+// ---- error plumbing -------------------------------------------------------
+void set_error(const char *fmt, ...);
+int hip_fail(hipError_t e, const char *what);
+
+#define BT_REQUIRE(cond, code, ...) \
+  do {                              \
+    if (!(cond)) {                  \
+      ::bt::set_error(__VA_ARGS__); \
+      return (code);                \
+    }                               \
+  } while (0)
+
+#define BT_CHECK_LAUNCH(what)                     \
+  do {                                            \
+    hipError_t e__ = hipGetLastError();           \
+    if (e__ != hipSuccess)                        \
+      return ::bt::hip_fail(e__, what);           \
+  } while (0)
+
+// ---- tuning options (bt_set_option) ----------------------------------------
+int option_gemm_tile();      // -1 = heuristic, else index into the tile table
+int option_attention_qb();   // -1 = heuristic, 1 or 2 = query blocks per wave
+
+inline hipStream_t as_stream(void *s) { return reinterpret_cast<hipStream_t>(s); }
+
+// ---- wave64 reductions ----------------------------------------------------
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+  return v;
+}
+
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+  return v;
+}
+
+// Inclusive prefix sum across the 64 lanes of a wave.
+__device__ __forceinline__ int wave_inclusive_scan(int v, int lane) {
+#pragma unroll
+  for (int o = 1; o < 64; o <<= 1) {
+    int t = __shfl_up(v, o, 64);
+    if (lane >= o) v += t;
+  }
+  return v;
+}
+
+}  // namespace bt

@@ -1,0 +1,179 @@
+// add-bias + residual + LayerNorm, packed in place and packed -> padded with
+// zero fill.  Memory-bound: one wave64 per row, 16-byte lanes, the row lives in
+// registers between the two statistics passes, reductions are wave shuffles
+// (no LDS, no block barrier).
+//
+// Numerics follow bytetransformer/include/layernorm.h:114-159,273-296,334-373:
+// x = (out + residual) + bias with both adds rounded to fp16, mean and biased
+// variance in fp32 (two-pass), y = (x - mean) * rsqrt(var + eps) * gamma + beta.
+#include "common.h"
+
+namespace bt {
+
+constexpr int kLnRowsPerBlock = 4;
+
+template <int NC, bool RESTORE, bool GB32>
+__global__ __launch_bounds__(kLnRowsPerBlock *kWave) void layernorm_kernel(
+    const half8_t *src, const half8_t *__restrict__ residual,
+    const half8_t *__restrict__ bias, const void *__restrict__ gamma,
+    const void *__restrict__ beta, half8_t *dst, const int *__restrict__ idx,
+    int B, int S, int rows_cap, int chunks, float inv_n, float eps) {
+  const int r = blockIdx.x * kLnRowsPerBlock + (threadIdx.x >> 6);
+  const int lane = threadIdx.x & 63;
+  if (r >= rows_cap) return;
+
+  size_t src_row, dst_row = r;
+  if (RESTORE) {
+    // r walks the padded [B, S] grid; idx = batch_idx
+    const int b = r / S, s = r - b * S;
+    const int start = idx[b], len = idx[b + 1] - start;
+    if (s >= len) {
+      const half8_t z = {0, 0, 0, 0, 0, 0, 0, 0};
+      for (int c = lane; c < chunks; c += kWave) dst[dst_row * chunks + c] = z;
+      return;
+    }
+    src_row = (size_t)start + s;
+  } else {
+    // idx = pointer to the live-row count (or null: all rows live)
+    const int M = idx ? *idx : rows_cap;
+    if (r >= M) return;
+    src_row = r;
+  }
+
+  const half8_t *a = src + src_row * chunks;
+  const half8_t *b = residual + src_row * chunks;
+  float v[NC][8];
+  float sum = 0.f;
+#pragma unroll
+  for (int i = 0; i < NC; ++i) {
+    const int c = lane + i * kWave;
+    if (c < chunks) {
+      half8_t x = (a[c] + b[c]) + bias[c];  // two fp16-rounded adds
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        v[i][j] = (float)x[j];
+        sum += v[i][j];
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) v[i][j] = 0.f;
+    }
+  }
+  const float mean = wave_sum(sum) * inv_n;
+  float sq = 0.f;
+#pragma unroll
+  for (int i = 0; i < NC; ++i) {
+    const int c = lane + i * kWave;
+    if (c < chunks) {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        v[i][j] -= mean;
+        sq += v[i][j] * v[i][j];
+      }
+    }
+  }
+  const float rstd = rsqrtf(wave_sum(sq) * inv_n + eps);
+
+  half8_t *o = dst + dst_row * chunks;
+#pragma unroll
+  for (int i = 0; i < NC; ++i) {
+    const int c = lane + i * kWave;
+    if (c < chunks) {
+      float g[8], bt_[8];
+      if (GB32) {
+        const float4_t *gp = (const float4_t *)gamma + 2 * c;
+        const float4_t *bp = (const float4_t *)beta + 2 * c;
+        float4_t g0 = gp[0], g1 = gp[1], b0 = bp[0], b1 = bp[1];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          g[j] = g0[j];
+          g[4 + j] = g1[j];
+          bt_[j] = b0[j];
+          bt_[4 + j] = b1[j];
+        }
+      } else {
+        half8_t gh = ((const half8_t *)gamma)[c], bh = ((const half8_t *)beta)[c];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          g[j] = (float)gh[j];
+          bt_[j] = (float)bh[j];
+        }
+      }
+      half8_t y;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) y[j] = (half_t)(v[i][j] * rstd * g[j] + bt_[j]);
+      o[c] = y;
+    }
+  }
+}
+
+template <bool RESTORE>
+static int launch_ln(const void *src, const void *residual, const void *bias, const void *gamma,
+                     const void *beta, int gb32, void *dst, const int *idx, int B, int S,
+                     int rows_cap, int H, float eps, hipStream_t s, const char *who) {
+  BT_REQUIRE(H > 0 && H % 8 == 0, BT_ERR_UNSUPPORTED, "%s: hidden_dim %d must be a multiple of 8",
+             who, H);
+  const int chunks = H / 8;
+  const int nc = (chunks + kWave - 1) / kWave;
+  BT_REQUIRE(nc <= 8, BT_ERR_UNSUPPORTED, "%s: hidden_dim %d exceeds 4096", who, H);
+  if (rows_cap == 0) return BT_OK;
+  const int grid = (rows_cap + kLnRowsPerBlock - 1) / kLnRowsPerBlock;
+  const float inv_n = 1.0f / (float)H;
+#define BT_LN_LAUNCH(NC_, GB_)                                                                  \
+  layernorm_kernel<NC_, RESTORE, GB_><<<grid, kLnRowsPerBlock * kWave, 0, s>>>(                 \
+      (const half8_t *)src, (const half8_t *)residual, (const half8_t *)bias, gamma, beta,      \
+      (half8_t *)dst, idx, B, S, rows_cap, chunks, inv_n, eps)
+#define BT_LN_NC(NC_)              \
+  do {                             \
+    if (gb32)                      \
+      BT_LN_LAUNCH(NC_, true);     \
+    else                           \
+      BT_LN_LAUNCH(NC_, false);    \
+  } while (0)
+  if (nc <= 1)
+    BT_LN_NC(1);
+  else if (nc <= 2)
+    BT_LN_NC(2);
+  else if (nc <= 4)
+    BT_LN_NC(4);
+  else
+    BT_LN_NC(8);
+#undef BT_LN_NC
+#undef BT_LN_LAUNCH
+  BT_CHECK_LAUNCH(who);
+  return BT_OK;
+}
+
+}  // namespace bt
+
+using namespace bt;
+
+extern "C" int bt_add_bias_residual_layernorm(void *out, const void *residual, const void *bias,
+                                              const void *gamma, const void *beta,
+                                              int gamma_beta_fp32, const int *valid_rows,
+                                              int rows_cap, int hidden_dim, float eps,
+                                              void *stream) {
+  BT_REQUIRE(out && residual && bias && gamma && beta, BT_ERR_INVALID_ARGUMENT,
+             "bt_add_bias_residual_layernorm: null pointer argument");
+  BT_REQUIRE(rows_cap >= 0, BT_ERR_INVALID_ARGUMENT,
+             "bt_add_bias_residual_layernorm: negative rows_cap");
+  return launch_ln<false>(out, residual, bias, gamma, beta, gamma_beta_fp32, out, valid_rows, 0,
+                          1, rows_cap, hidden_dim, eps, as_stream(stream),
+                          "bt_add_bias_residual_layernorm");
+}
+
+extern "C" int bt_add_bias_residual_layernorm_restore(
+    const void *out, const void *residual, const void *bias, const void *gamma, const void *beta,
+    int gamma_beta_fp32, void *out_padded, const int *batch_idx, int batch_size, int seq_len,
+    int hidden_dim, float eps, void *stream) {
+  BT_REQUIRE(out && residual && bias && gamma && beta && out_padded && batch_idx,
+             BT_ERR_INVALID_ARGUMENT,
+             "bt_add_bias_residual_layernorm_restore: null pointer argument");
+  BT_REQUIRE(batch_size > 0 && seq_len > 0, BT_ERR_INVALID_ARGUMENT,
+             "bt_add_bias_residual_layernorm_restore: sizes must be positive");
+  BT_REQUIRE((long long)batch_size * seq_len < (1ll << 31), BT_ERR_UNSUPPORTED,
+             "bt_add_bias_residual_layernorm_restore: too many rows");
+  return launch_ln<true>(out, residual, bias, gamma, beta, gamma_beta_fp32, out_padded, batch_idx,
+                         batch_size, seq_len, batch_size * seq_len, hidden_dim, eps,
+                         as_stream(stream), "bt_add_bias_residual_layernorm_restore");
+}

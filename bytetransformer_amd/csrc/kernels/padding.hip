@@ -1,0 +1,182 @@
+// Padding removal: mask prefix sum -> packed-token offsets, and the gather of
+// valid rows into the packed layout.  Integer outputs are bit-exact with the
+// reference's parallel_prefix (bytetransformer/include/remove_padding.h:36-86).
+#include "common.h"
+
+#include <atomic>
+#include <cstring>
+#include <string>
+
+namespace bt {
+
+// ---- error plumbing shared by every translation unit ------------------------
+static thread_local std::string g_last_error;
+
+void set_error(const char *fmt, ...) {
+  char buf[512];
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(buf, sizeof(buf), fmt, ap);
+  va_end(ap);
+  g_last_error = buf;
+}
+
+int hip_fail(hipError_t e, const char *what) {
+  set_error("[BT][ERROR] HIP runtime error: %s (%s)", hipGetErrorString(e), what);
+  return BT_ERR_HIP;
+}
+
+// ---- tuning options ---------------------------------------------------------
+static std::atomic<int> g_gemm_tile{-1};
+static std::atomic<int> g_attention_qb{-1};
+int option_gemm_tile() { return g_gemm_tile.load(std::memory_order_relaxed); }
+int option_attention_qb() { return g_attention_qb.load(std::memory_order_relaxed); }
+
+// ---- offsets ----------------------------------------------------------------
+constexpr int kOffsetThreads = 1024;
+constexpr int kOffsetWaves = kOffsetThreads / kWave;
+
+// Every block recomputes all B lengths (B*S mask elements, a few KB) and the
+// exclusive scan, then writes word_idx for the sequences it owns; block 0 also
+// writes batch_idx.  No inter-block communication, so the grid can be as wide
+// as the batch.
+template <typename T>
+__global__ __launch_bounds__(kOffsetThreads) void build_offsets_kernel(
+    const T *__restrict__ mask, int *__restrict__ batch_idx, int *__restrict__ word_idx, int B,
+    int S) {
+  extern __shared__ int smem[];
+  int *s_len = smem;          // [B]
+  int *s_off = smem + B;      // [B + 1]
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+
+  // one wave per sequence: count row-0 mask elements >= 0.5 with a 64-wide ballot
+  for (int b = wave; b < B; b += kOffsetWaves) {
+    const T *row = mask + (size_t)b * S * S;
+    int count = 0;
+    for (int i0 = 0; i0 < S; i0 += kWave) {
+      int i = i0 + lane;
+      bool on = (i < S) && ((float)row[i] >= 0.5f);
+      count += __popcll(__ballot(on));
+    }
+    if (lane == 0) s_len[b] = count;
+  }
+  __syncthreads();
+
+  // wave 0: exclusive scan of the lengths in chunks of 64
+  if (wave == 0) {
+    int carry = 0;
+    for (int i0 = 0; i0 < B; i0 += kWave) {
+      int i = i0 + lane;
+      int len = i < B ? s_len[i] : 0;
+      int incl = wave_inclusive_scan(len, lane);
+      if (i < B) s_off[i] = carry + incl - len;
+      carry += __shfl(incl, 63, 64);
+    }
+    if (lane == 0) s_off[B] = carry;
+  }
+  __syncthreads();
+
+  if (blockIdx.x == 0)
+    for (int i = tid; i <= B; i += kOffsetThreads) batch_idx[i] = s_off[i];
+
+  for (int b = blockIdx.x; b < B; b += gridDim.x) {
+    const int off = s_off[b], len = s_len[b];
+    for (int i = tid; i < len; i += kOffsetThreads) word_idx[off + i] = b * S + i;
+  }
+}
+
+// ---- compress ---------------------------------------------------------------
+// One wave per packed row, 16-byte lanes.  M is read from batch_idx[B]; rows
+// past it retire immediately, so the grid is sized for B*S without a host sync.
+constexpr int kRowsPerBlock = 4;
+
+__global__ __launch_bounds__(kRowsPerBlock *kWave) void compress_kernel(
+    const uint4_t *__restrict__ from, uint4_t *__restrict__ to, const int *__restrict__ batch_idx,
+    const int *__restrict__ word_idx, int B, int chunks /* H/8 */) {
+  const int t = blockIdx.x * kRowsPerBlock + (threadIdx.x >> 6);
+  const int M = batch_idx[B];
+  if (t >= M) return;
+  const int lane = threadIdx.x & 63;
+  const size_t src = (size_t)word_idx[t] * chunks;
+  const size_t dst = (size_t)t * chunks;
+  for (int c = lane; c < chunks; c += kWave) to[dst + c] = from[src + c];
+}
+
+}  // namespace bt
+
+using namespace bt;
+
+extern "C" int bt_version(void) { return 1; }
+
+extern "C" const char *bt_last_error_string(void) { return g_last_error.c_str(); }
+
+extern "C" int bt_set_option(const char *name, int value) {
+  BT_REQUIRE(name, BT_ERR_INVALID_ARGUMENT, "bt_set_option: null name");
+  if (!strcmp(name, "gemm_tile")) {
+    BT_REQUIRE(value >= -1 && value <= 2, BT_ERR_INVALID_ARGUMENT,
+               "bt_set_option: gemm_tile=%d outside [-1, 2]", value);
+    g_gemm_tile.store(value);
+  } else if (!strcmp(name, "attention_qb")) {
+    BT_REQUIRE(value == -1 || value == 1 || value == 2, BT_ERR_INVALID_ARGUMENT,
+               "bt_set_option: attention_qb=%d must be -1, 1 or 2", value);
+    g_attention_qb.store(value);
+  } else {
+    set_error("bt_set_option: unknown option '%s'", name);
+    return BT_ERR_INVALID_ARGUMENT;
+  }
+  return BT_OK;
+}
+
+extern "C" int bt_build_offsets(const void *atten_mask, int mask_dtype, int batch_size,
+                                int seq_len, int *batch_idx, int *word_idx,
+                                int *valid_word_num_host, void *stream) {
+  BT_REQUIRE(atten_mask && batch_idx && word_idx, BT_ERR_INVALID_ARGUMENT,
+             "bt_build_offsets: null pointer argument");
+  BT_REQUIRE(batch_size > 0 && seq_len > 0, BT_ERR_INVALID_ARGUMENT,
+             "bt_build_offsets: batch_size=%d seq_len=%d must be positive", batch_size, seq_len);
+  BT_REQUIRE(mask_dtype == BT_F16 || mask_dtype == BT_F32, BT_ERR_INVALID_ARGUMENT,
+             "bt_build_offsets: unknown mask dtype %d", mask_dtype);
+  BT_REQUIRE((long long)batch_size * seq_len < (1ll << 31), BT_ERR_UNSUPPORTED,
+             "bt_build_offsets: batch_size*seq_len overflows int32");
+  const size_t smem = (2 * (size_t)batch_size + 1) * sizeof(int);
+  BT_REQUIRE(smem <= 64 * 1024, BT_ERR_UNSUPPORTED,
+             "bt_build_offsets: batch_size %d too large (limit 8191)", batch_size);
+  hipStream_t s = as_stream(stream);
+  const int grid = batch_size < 64 ? batch_size : 64;
+  if (mask_dtype == BT_F16)
+    build_offsets_kernel<half_t><<<grid, kOffsetThreads, smem, s>>>(
+        (const half_t *)atten_mask, batch_idx, word_idx, batch_size, seq_len);
+  else
+    build_offsets_kernel<float><<<grid, kOffsetThreads, smem, s>>>(
+        (const float *)atten_mask, batch_idx, word_idx, batch_size, seq_len);
+  BT_CHECK_LAUNCH("build_offsets_kernel");
+  if (valid_word_num_host) {
+    hipError_t e = hipMemcpyAsync(valid_word_num_host, batch_idx + batch_size, sizeof(int),
+                                  hipMemcpyDeviceToHost, s);
+    if (e != hipSuccess) return hip_fail(e, "copy of valid_word_num");
+    e = hipStreamSynchronize(s);
+    if (e != hipSuccess) return hip_fail(e, "stream synchronize for valid_word_num");
+  }
+  return BT_OK;
+}
+
+extern "C" int bt_compress(const void *from_tensor, void *to_tensor, const int *batch_idx,
+                           const int *word_idx, int batch_size, int seq_len, int hidden_dim,
+                           void *stream) {
+  BT_REQUIRE(from_tensor && to_tensor && batch_idx && word_idx, BT_ERR_INVALID_ARGUMENT,
+             "bt_compress: null pointer argument");
+  BT_REQUIRE(batch_size > 0 && seq_len > 0 && hidden_dim > 0, BT_ERR_INVALID_ARGUMENT,
+             "bt_compress: sizes must be positive");
+  BT_REQUIRE(hidden_dim % 8 == 0, BT_ERR_UNSUPPORTED,
+             "bt_compress: hidden_dim %d must be a multiple of 8", hidden_dim);
+  const long long rows = (long long)batch_size * seq_len;
+  BT_REQUIRE(rows < (1ll << 31), BT_ERR_UNSUPPORTED, "bt_compress: too many rows");
+  const int grid = (int)((rows + kRowsPerBlock - 1) / kRowsPerBlock);
+  compress_kernel<<<grid, kRowsPerBlock * kWave, 0, as_stream(stream)>>>(
+      (const uint4_t *)from_tensor, (uint4_t *)to_tensor, batch_idx, word_idx, batch_size,
+      hidden_dim / 8);
+  BT_CHECK_LAUNCH("compress_kernel");
+  return BT_OK;
+}

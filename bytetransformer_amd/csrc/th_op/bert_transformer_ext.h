@@ -1,0 +1,112 @@
+// BTEncoder<T>: binds twelve weight tensors to a BertTransformerParam and runs
+// one layer on the caller's current HIP stream.  Role of the reference's
+// bytetransformer/th_op/bert_transformer_ext.h:30-117.
+#pragma once
+#include "bytetransformer/bert_transformer.h"
+#include "util.h"
+
+namespace bytetransformer {
+namespace torch_ext {
+using torch::Tensor;
+
+template <typename T>
+struct THTraits;
+template <>
+struct THTraits<float> {
+  static const OperationType OpType = OperationType::FP32;
+};
+template <>
+struct THTraits<__half> {
+  static const OperationType OpType = OperationType::HALF;
+};
+
+class IBTEncoder {
+ public:
+  virtual ~IBTEncoder() {}
+  virtual void forward(int batch_size, int seq_len, Tensor &input, Tensor &attr_mask,
+                       Tensor &output, bool is_remove_padding, bool use_fused_attention,
+                       const ModelType model_type = ModelType::Bert,
+                       const Tensor attention_bias = Tensor()) = 0;
+};
+
+template <typename T>
+class BTEncoder : public IBTEncoder {
+  static const OperationType kOp = THTraits<T>::OpType;
+
+ public:
+  BTEncoder(int head_num, int head_size, const std::vector<Tensor> &w)
+      : head_num_(head_num), head_size_(head_size), weights_(w) {
+    TORCH_CHECK(w.size() == 12, "expected 12 weight tensors");
+    param_.attr_kernel_QKV = get_ptr<T>(weights_[0]);
+    param_.attention_param.attr_bias_QKV = get_ptr<T>(weights_[1]);
+    param_.attr_output_kernel = get_ptr<T>(weights_[2]);
+    param_.attr_output_bias = get_ptr<T>(weights_[3]);
+    param_.attr_output_layernorm_gamma = get_ptr<void>(weights_[4]);
+    param_.attr_output_layernorm_beta = get_ptr<void>(weights_[5]);
+    param_.inter_kernel = get_ptr<T>(weights_[6]);
+    param_.inter_bias = get_ptr<T>(weights_[7]);
+    param_.output_kernel = get_ptr<T>(weights_[8]);
+    param_.output_bias = get_ptr<T>(weights_[9]);
+    param_.output_layernorm_gamma = get_ptr<void>(weights_[10]);
+    param_.output_layernorm_beta = get_ptr<void>(weights_[11]);
+    // fp32 gamma/beta next to fp16 weights, detected from the last LayerNorm
+    // gamma like the reference does (bert_transformer_ext.h:60-63)
+    use_fp32_ = kOp == OperationType::HALF && weights_[10].scalar_type() == at::ScalarType::Float;
+    // FFN width from the weight itself (the reference leaves it at 4)
+    const int64_t hidden = (int64_t)head_num * head_size;
+    if (weights_[6].dim() == 2 && hidden > 0 && weights_[6].size(1) % hidden == 0)
+      param_.intermediate_size = (int)(weights_[6].size(1) / hidden);
+  }
+
+  void forward(int batch_size, int seq_len, Tensor &input, Tensor &attr_mask, Tensor &output,
+               bool is_remove_padding = true, bool use_fused_attention = true,
+               const ModelType model_type = ModelType::Bert,
+               const Tensor attention_bias = Tensor()) override {
+    CHECK_SEQ_LEN(seq_len);
+    TORCH_CHECK(!attention_bias.defined(), "attention_bias is not supported");
+    c10::DeviceGuard device_guard(input.device());
+
+    BertTransformer<kOp> encoder(batch_size, head_num_, head_size_, seq_len, use_fused_attention,
+                                 is_remove_padding, use_fp32_, model_type);
+    encoder.initialize(param_);
+    const unsigned long long buf_size = encoder.cal_bufsize();
+    auto buf_tensor = torch::empty({(int64_t)buf_size},
+                                   torch::dtype(torch::kInt8).device(input.device()));
+    hipStream_t stream = c10::hip::getCurrentHIPStream(input.device().index()).stream();
+    struct BertTransformerInferParam<T> infer_param {
+      get_ptr<T>(input), get_ptr<T>(attr_mask), get_ptr<T>(output), get_ptr<void>(buf_tensor),
+          batch_size, seq_len, nullptr, stream
+    };
+    encoder.infer(infer_param);
+  }
+
+ private:
+  const int head_num_, head_size_;
+  bool use_fp32_ = false;
+  std::vector<Tensor> weights_;
+  BertTransformerParam<kOp> param_;
+};
+
+inline void check_layer_shapes(int64_t head_num, int64_t head_size, const std::vector<Tensor> &w) {
+  const int64_t H = head_num * head_size;
+  TORCH_CHECK(head_num > 0 && head_size > 0, "head_num and head_size must be positive");
+  TORCH_CHECK(w[0].dim() == 2 && w[0].size(0) == H && w[0].size(1) == 3 * H,
+              "qkv_kernel must be [hidden_dim, 3 * hidden_dim]");
+  TORCH_CHECK(w[1].numel() == 3 * H, "qkv_bias must have 3 * hidden_dim elements");
+  TORCH_CHECK(w[2].dim() == 2 && w[2].size(0) == H && w[2].size(1) == H,
+              "attr_output_kernel must be [hidden_dim, hidden_dim]");
+  TORCH_CHECK(w[6].dim() == 2 && w[6].size(0) == H && w[6].size(1) % H == 0,
+              "inter_kernel must be [hidden_dim, k * hidden_dim]");
+  const int64_t F = w[6].size(1);
+  TORCH_CHECK(w[7].numel() == F, "inter_bias must match inter_kernel");
+  TORCH_CHECK(w[8].dim() == 2 && w[8].size(0) == F && w[8].size(1) == H,
+              "output_kernel must be [k * hidden_dim, hidden_dim]");
+  for (int i : {3, 4, 5, 9, 10, 11})
+    TORCH_CHECK(w[i].numel() == H, "bias / gamma / beta tensors must have hidden_dim elements");
+  TORCH_CHECK(w[4].scalar_type() == w[5].scalar_type() &&
+                  w[4].scalar_type() == w[10].scalar_type() &&
+                  w[4].scalar_type() == w[11].scalar_type(),
+              "LayerNorm gamma / beta must share one dtype");
+}
+}  // namespace torch_ext
+}  // namespace bytetransformer

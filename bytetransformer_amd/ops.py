@@ -1,0 +1,145 @@
+"""Tensor-level wrappers over the C ABI: each function takes torch tensors that
+already live on the GPU, passes their addresses and the current stream to one
+bt_* entry point and raises on a non-zero status.  Used by the tests and the
+benchmark; no arithmetic happens in Python."""
+import ctypes
+
+import torch
+
+from ._lib import kernel_lib
+
+BT_F32, BT_F16 = 0, 1
+
+
+class BtError(RuntimeError):
+    pass
+
+
+def _check(rc):
+    if rc != 0:
+        raise BtError("bt status %d: %s" % (rc, kernel_lib().bt_last_error_string().decode()))
+
+
+def _ptr(t):
+    if t is None:
+        return None
+    if not t.is_cuda:
+        raise BtError("tensor must live on the GPU")
+    if not t.is_contiguous():
+        raise BtError("tensor must be contiguous")
+    return ctypes.c_void_p(t.data_ptr())
+
+
+def _stream():
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _dtype_code(t):
+    if t.dtype == torch.float16:
+        return BT_F16
+    if t.dtype == torch.float32:
+        return BT_F32
+    raise BtError("unsupported dtype %s" % t.dtype)
+
+
+def set_option(name, value):
+    _check(kernel_lib().bt_set_option(name.encode(), int(value)))
+
+
+def build_offsets(mask, want_count=False):
+    """mask [B,S,S] -> (batch_idx int32[B+1], word_idx int32[B*S], M or None)."""
+    B, S = mask.shape[0], mask.shape[1]
+    batch_idx = torch.empty(B + 1, dtype=torch.int32, device=mask.device)
+    word_idx = torch.empty(B * S, dtype=torch.int32, device=mask.device)
+    cnt = ctypes.c_int(-1)
+    _check(kernel_lib().bt_build_offsets(_ptr(mask), _dtype_code(mask), B, S, _ptr(batch_idx),
+                                         _ptr(word_idx),
+                                         ctypes.byref(cnt) if want_count else None, _stream()))
+    return batch_idx, word_idx, (cnt.value if want_count else None)
+
+
+def compress(x, batch_idx, word_idx, out=None):
+    B, S, H = x.shape
+    if out is None:
+        out = torch.zeros(B * S, H, dtype=x.dtype, device=x.device)
+    _check(kernel_lib().bt_compress(_ptr(x), _ptr(out), _ptr(batch_idx), _ptr(word_idx), B, S, H,
+                                    _stream()))
+    return out
+
+
+def transpose_weight(w):
+    K, N = w.shape
+    wt = torch.empty(N, K, dtype=w.dtype, device=w.device)
+    _check(kernel_lib().bt_transpose_weight(_ptr(w), _ptr(wt), K, N, _stream()))
+    return wt
+
+
+def gemm(a, wt, valid_rows=None, out=None):
+    rows, K = a.shape
+    N = wt.shape[0]
+    if out is None:
+        out = torch.zeros(rows, N, dtype=a.dtype, device=a.device)
+    _check(kernel_lib().bt_gemm(_ptr(a), _ptr(wt), _ptr(out), _ptr(valid_rows), rows, N, K,
+                                _stream()))
+    return out
+
+
+def gemm_bias_gelu(a, wt, bias, valid_rows=None, out=None):
+    rows, K = a.shape
+    N = wt.shape[0]
+    if out is None:
+        out = torch.zeros(rows, N, dtype=a.dtype, device=a.device)
+    _check(kernel_lib().bt_gemm_bias_gelu(_ptr(a), _ptr(wt), _ptr(bias), _ptr(out),
+                                          _ptr(valid_rows), rows, N, K, _stream()))
+    return out
+
+
+def gemm_qkv_bias_split(a, wt_qkv, bias_qkv, head_num, size_per_head=64, valid_rows=None,
+                        out=None):
+    rows = a.shape[0]
+    if out is None:
+        out = torch.zeros(3, head_num, rows, size_per_head, dtype=a.dtype, device=a.device)
+    _check(kernel_lib().bt_gemm_qkv_bias_split(_ptr(a), _ptr(wt_qkv), _ptr(bias_qkv), _ptr(out),
+                                               _ptr(valid_rows), rows, head_num, size_per_head,
+                                               _stream()))
+    return out
+
+
+def _attention(fn, qkv_heads, batch_idx, batch_size, seq_len, scale, padded_rows, out):
+    _, head_num, rows_cap, d = qkv_heads.shape
+    if out is None:
+        out = torch.zeros(rows_cap, head_num * d, dtype=qkv_heads.dtype, device=qkv_heads.device)
+    _check(fn(_ptr(qkv_heads), _ptr(out), _ptr(batch_idx), batch_size, seq_len, rows_cap,
+              head_num, d, float(scale), int(padded_rows), _stream()))
+    return out
+
+
+def attention_short(qkv_heads, batch_idx, batch_size, seq_len, scale, padded_rows=False, out=None):
+    return _attention(kernel_lib().bt_attention_short, qkv_heads, batch_idx, batch_size, seq_len,
+                      scale, padded_rows, out)
+
+
+def attention_grouped(qkv_heads, batch_idx, batch_size, seq_len, scale, padded_rows=False,
+                      out=None):
+    return _attention(kernel_lib().bt_attention_grouped, qkv_heads, batch_idx, batch_size,
+                      seq_len, scale, padded_rows, out)
+
+
+def add_bias_residual_layernorm(out, residual, bias, gamma, beta, eps=1e-6, valid_rows=None):
+    rows, H = out.shape
+    _check(kernel_lib().bt_add_bias_residual_layernorm(
+        _ptr(out), _ptr(residual), _ptr(bias), _ptr(gamma), _ptr(beta),
+        int(gamma.dtype == torch.float32), _ptr(valid_rows), rows, H, float(eps), _stream()))
+    return out
+
+
+def add_bias_residual_layernorm_restore(out, residual, bias, gamma, beta, batch_idx, batch_size,
+                                        seq_len, eps=1e-6, out_padded=None):
+    H = out.shape[-1]
+    if out_padded is None:
+        out_padded = torch.empty(batch_size, seq_len, H, dtype=out.dtype, device=out.device)
+    _check(kernel_lib().bt_add_bias_residual_layernorm_restore(
+        _ptr(out), _ptr(residual), _ptr(bias), _ptr(gamma), _ptr(beta),
+        int(gamma.dtype == torch.float32), _ptr(out_padded), _ptr(batch_idx), batch_size, seq_len,
+        H, float(eps), _stream()))
+    return out_padded

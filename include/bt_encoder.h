@@ -1,0 +1,65 @@
+/*
+ * bt_encoder.h - C entry points of the host library (libbytetransformer.so)
+ * for callers that cannot instantiate the C++ BertTransformer<OpType> class
+ * template (ctypes, cgo, JNI ...).  One call = one encoder layer, exactly what
+ * BertTransformer::infer does (reference: bytetransformer/include/
+ * bert_transformer.h:98-224, bytetransformer/src/bert_transformer.cu:28-130).
+ *
+ * Pointers are device pointers unless stated; `stream` is a hipStream_t passed
+ * as void*.  Returns 0 or a bt_status code; the message of a failure is
+ * available from bt_encoder_last_error().  Never allocates device memory.
+ */
+#ifndef BT_ENCODER_H_
+#define BT_ENCODER_H_
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* The twelve per-layer tensors, in the order of the PyTorch operator's
+ * arguments (reference: bytetransformer/th_op/ths_op_f.cc:28-34). */
+typedef struct bt_layer_weights {
+  const void *qkv_kernel;                  /* [H, 3H]  */
+  const void *qkv_bias;                    /* [3H]     */
+  const void *attr_output_kernel;          /* [H, H]   */
+  const void *attr_output_bias;            /* [H]      */
+  const void *attr_output_layernorm_gamma; /* [H] dtype or fp32 (gamma_beta_fp32) */
+  const void *attr_output_layernorm_beta;
+  const void *inter_kernel;                /* [H, mult*H] */
+  const void *inter_bias;                  /* [mult*H]    */
+  const void *output_kernel;               /* [mult*H, H] */
+  const void *output_bias;                 /* [H]         */
+  const void *output_layernorm_gamma;
+  const void *output_layernorm_beta;
+} bt_layer_weights;
+
+typedef struct bt_encoder_config {
+  int dtype;               /* BT_F16 (BT_F32 is rejected: not implemented) */
+  int max_batch_size;
+  int max_seq_len;
+  int head_num;
+  int size_per_head;
+  int intermediate_size;   /* FFN width as a multiple of hidden_dim; reference default 4 */
+  int use_fused_attention; /* reference default 1 */
+  int is_remove_padding;   /* reference default 1; forced off when max_batch_size <= 2 */
+  int gamma_beta_fp32;     /* LayerNorm gamma/beta are float even when dtype is fp16 */
+  float tao;               /* softmax temperature, reference default 1 */
+  float layernorm_eps;     /* reference kernels: 1e-6 */
+} bt_encoder_config;
+
+/* Bytes of scratch `buf` that bt_encoder_layer_forward needs (cal_bufsize()). */
+unsigned long long bt_encoder_bufsize(const bt_encoder_config *cfg);
+
+/* One encoder layer: padded input [B,S,H] + mask [B,S,S] -> padded output
+ * [B,S,H] (rows past each sequence's length are zero on the remove-padding
+ * path).  `output` must not alias `input`. */
+int bt_encoder_layer_forward(const bt_encoder_config *cfg, const bt_layer_weights *weights,
+                             const void *input, const void *atten_mask, void *output, void *buf,
+                             int batch_size, int seq_len, void *stream);
+
+const char *bt_encoder_last_error(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* BT_ENCODER_H_ */

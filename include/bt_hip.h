@@ -1,0 +1,171 @@
+/*
+ * bt_hip.h - C ABI of the gfx950 kernel library (libbt_hip.so) behind the
+ * padding-free BERT encoder-layer forward.
+ *
+ * Conventions for every entry point:
+ *   - plain C types only; `stream` is a hipStream_t passed as void* (NULL = the
+ *     null stream); all work is enqueued asynchronously on it;
+ *   - returns BT_OK (0) or a BT_ERR_* code, never throws, never allocates
+ *     device memory; the caller owns every buffer, scratch included;
+ *   - after a non-zero return bt_last_error_string() describes the failure
+ *     (thread-local);
+ *   - activations and weights are fp16 (IEEE binary16) unless a dtype argument
+ *     says otherwise; "packed" means the M valid token rows of the batch laid
+ *     out back to back in (batch, position) order;
+ *   - `valid_rows` arguments point at ONE int in device memory holding the
+ *     number of live rows M (normally batch_idx + batch_size); kernels size
+ *     their grids for `rows_cap` rows and retire rows >= M on the device, so
+ *     the host never waits for M.  NULL means all rows_cap rows are live.
+ *
+ * Each declaration cites the reference interface it replaces (paths relative
+ * to the ByteTransformer tree).
+ */
+#ifndef BT_HIP_H_
+#define BT_HIP_H_
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum bt_status {
+  BT_OK = 0,
+  BT_ERR_INVALID_ARGUMENT = 1,
+  BT_ERR_UNSUPPORTED = 2,
+  BT_ERR_HIP = 3
+};
+
+enum bt_dtype { BT_F32 = 0, BT_F16 = 1 };
+
+/* ABI revision of the loaded library. */
+int bt_version(void);
+
+/* Text of the last error raised on the calling thread ("" if none). */
+const char *bt_last_error_string(void);
+
+/*
+ * Tuning knob for experiments and tests; no counterpart in the reference.
+ *   "gemm_tile"     -1 heuristic | 0: 256x256 | 1: 256x128 | 2: 128x128 workgroup tile
+ *   "attention_qb"  -1 heuristic | 1 | 2: 16-query blocks per wave in the grouped kernel
+ * Process-wide; results do not depend on it beyond fp32 summation order.
+ */
+int bt_set_option(const char *name, int value);
+
+/*
+ * Mask prefix sum.  Replaces build_sequence_length_padding_offset_kernelLauncher
+ * and parallel_prefix (bytetransformer/include/remove_padding.h:36-101).
+ *   atten_mask  [batch_size, seq_len, seq_len], dtype mask_dtype (BT_F16/BT_F32);
+ *               only row 0 of each batch is read; an element counts when >= 0.5
+ *   batch_idx   int[batch_size + 1]  exclusive prefix sum of the lengths, total last
+ *   word_idx    int[batch_size * seq_len]; first M entries = b*seq_len + i, i < len_b
+ *   valid_word_num_host  NULL, or a host int that receives M; passing it makes
+ *               the call wait for the stream (the reference always does)
+ */
+int bt_build_offsets(const void *atten_mask, int mask_dtype, int batch_size, int seq_len,
+                     int *batch_idx, int *word_idx, int *valid_word_num_host, void *stream);
+
+/*
+ * Gather valid rows: to_tensor[t, :] = from_tensor[word_idx[t], :], t < M.
+ * Replaces compressBertInput_kernelLauncher (remove_padding.h:104-121).
+ * hidden_dim % 8 == 0.  M is read on the device from batch_idx[batch_size].
+ */
+int bt_compress(const void *from_tensor, void *to_tensor, const int *batch_idx,
+                const int *word_idx, int batch_size, int seq_len, int hidden_dim, void *stream);
+
+/*
+ * Weight pre-pack: wt[n, k] = w[k, n].  The reference hands cuBLAS the
+ * [in, out] row-major weight directly (gemm.cu:27-39); the MFMA kernels here
+ * want both operands contiguous along k, so the host transposes each weight
+ * once per infer() into scratch.  k % 8 == 0, n % 8 == 0.
+ */
+int bt_transpose_weight(const void *w, void *wt, int k, int n, void *stream);
+
+/*
+ * c[rows, n] = a[rows, k] . w[k, n], fp16 in/out, fp32 accumulate on MFMA.
+ * Replaces dense_layer_kernel_launcher (bytetransformer/src/gemm.cu:32-39) at
+ * its attention-output-projection and FFN2 call sites
+ * (bert_transformer.cu:102-104,115-117).  `wt` is the [n, k] pre-packed weight.
+ * k % 64 == 0, n % 8 == 0.
+ */
+int bt_gemm(const void *a, const void *wt, void *c, const int *valid_rows, int rows_cap, int n,
+            int k, void *stream);
+
+/*
+ * c = gelu_tanh(a . w + bias).  Replaces gemm_bias_gelu
+ * (bytetransformer/src/gemm_bias_act.cu:76-148; tanh constants
+ * gemm_bias_act.h:80-87).
+ */
+int bt_gemm_bias_gelu(const void *a, const void *wt, const void *bias, void *c,
+                      const int *valid_rows, int rows_cap, int n, int k, void *stream);
+
+/*
+ * QKV projection with the bias add and the head split fused into the store:
+ *   qkv_heads[which][g][t][0:d] = (a . w_qkv + bias)[t, which*H + g*d : +d]
+ * with which in {Q, K, V}, H = head_num*size_per_head, layout
+ * [3][head_num][rows_cap][size_per_head].  Replaces the bias-free QKV
+ * dense_layer_kernel_launcher call (bert_transformer.cu:85-87) plus
+ * add_QKV_bias_padding (attention_nofused_utils.cu:143-184) / the in-kernel
+ * bias add of attention_fused.cu:318-325.  size_per_head must be 64.
+ */
+int bt_gemm_qkv_bias_split(const void *a, const void *wt_qkv, const void *bias_qkv,
+                           void *qkv_heads, const int *valid_rows, int rows_cap, int head_num,
+                           int size_per_head, void *stream);
+
+/*
+ * Fused multi-head attention over the head-major Q/K/V written by
+ * bt_gemm_qkv_bias_split; output is token-major [rows, H] with head g at
+ * columns [g*d, g*d+d).  Per sequence b and head g:
+ *   P = exp(scale*Q.K^T - rowmax) / (rowsum + 1e-6),  O = fp16(P) . V
+ * keys >= len_b are excluded by index, len_b = batch_idx[b+1] - batch_idx[b].
+ *   padded_rows == 0: sequence b owns packed rows [batch_idx[b], batch_idx[b+1])
+ *   padded_rows != 0: sequence b owns rows [b*seq_len, (b+1)*seq_len), all
+ *                     seq_len query rows are computed against the len_b keys
+ *
+ * bt_attention_short keeps the whole logits row of a query tile in registers
+ * (exact two-pass softmax, seq_len <= 512).  Replaces wmma_attention[_rm]_kernel
+ * and wmma_attention_long[_rm]_kernel with their dispatch tables
+ * (attention_fused.cu:168-491, attention_fused_long.cu:30-488).
+ *
+ * bt_attention_grouped streams K/V tiles with an online softmax over a
+ * variable-length work list, any seq_len.  Replaces
+ * CutlassAttention::infer_impl (cutlass_attention.cu:150-210): the grouped
+ * GEMM0 + partial softmax, softmax_reduction_kernel and grouped GEMM1, without
+ * the logits round trip through HBM.
+ */
+int bt_attention_short(const void *qkv_heads, void *attention_output, const int *batch_idx,
+                       int batch_size, int seq_len, int rows_cap, int head_num,
+                       int size_per_head, float scale, int padded_rows, void *stream);
+
+int bt_attention_grouped(const void *qkv_heads, void *attention_output, const int *batch_idx,
+                         int batch_size, int seq_len, int rows_cap, int head_num,
+                         int size_per_head, float scale, int padded_rows, void *stream);
+
+/*
+ * out = LayerNorm((out + residual) + bias) * gamma + beta, in place on `out`,
+ * both adds rounded to fp16, statistics in fp32 (two-pass), eps inside the
+ * rsqrt.  Replaces add_bias_input_layernorm_kernel_launcher
+ * (bytetransformer/include/layernorm.h:410-428, kernels :114-159,273-296).
+ * gamma/beta are fp32 when gamma_beta_fp32 != 0, else fp16.  hidden_dim % 8 == 0.
+ */
+int bt_add_bias_residual_layernorm(void *out, const void *residual, const void *bias,
+                                   const void *gamma, const void *beta, int gamma_beta_fp32,
+                                   const int *valid_rows, int rows_cap, int hidden_dim,
+                                   float eps, void *stream);
+
+/*
+ * Same LayerNorm, but reading packed rows and writing the padded layout:
+ * out_padded[b, s, :] = LN(out[p] + residual[p] + bias) with p = batch_idx[b]+s
+ * when s < len_b, else zeros.  Replaces
+ * add_bias_input_layernorm_restore_output_kernel_launcher (layernorm.h:430-446,
+ * kernels :334-373).
+ */
+int bt_add_bias_residual_layernorm_restore(const void *out, const void *residual,
+                                           const void *bias, const void *gamma,
+                                           const void *beta, int gamma_beta_fp32,
+                                           void *out_padded, const int *batch_idx,
+                                           int batch_size, int seq_len, int hidden_dim,
+                                           float eps, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* BT_HIP_H_ */

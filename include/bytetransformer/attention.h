@@ -1,0 +1,85 @@
+// Attention<OpType>: parameter structs and the dispatcher between the two
+// fused multi-head-attention kernels.  Public surface follows the reference's
+// bytetransformer/include/attention.h:25-149 (AttentionParam,
+// AttentionInferParam, Attention with ctor / initialize / cal_bufsize / infer).
+#pragma once
+#include "common.h"
+
+namespace bytetransformer {
+
+template <OperationType OpType>
+class AttentionParam {
+ private:
+  using Traits_ = Traits<OpType>;
+  using DataType_ = typename Traits_::DataType;
+
+ public:
+  const DataType_ *attr_bias_QKV = nullptr;  // [3 * hidden_dim]
+  float tao = 1.0f;                          // softmax temperature: scale = 1/sqrt(d)/tao
+  int cublas_Algo[2] = {Traits_::algo, Traits_::algo};  // kept for source compatibility, unused
+};
+
+template <typename T>
+struct AttentionInferParam {
+  // Head-major projections with the QKV bias already added:
+  // [3][head_num][batch_size * seq_len][size_per_head] (written by the QKV GEMM).
+  const T *qkv;
+  const T *atten_mask;  // [batch_size, seq_len, seq_len]; lengths come from et_param.batch_idx
+  T *attention_output;  // token-major [rows, hidden_dim]
+  void *buf;
+  int batch_size = 0;
+  int seq_len = 0;
+  BlasHandle cublas_handle = nullptr;
+  hipStream_t stream = nullptr;
+  ET_Param et_param = {nullptr, nullptr, 0};
+  const T *attention_bias = nullptr;         // [head_num, seq_len, seq_len]; must be null
+  const uint32_t *position_ids = nullptr;    // never read
+  const uint32_t *token_type_ids = nullptr;  // never read
+};
+
+template <OperationType OpType>
+class Attention {
+ protected:
+  typedef Traits<OpType> Traits_;
+  typedef typename Traits_::DataType DataType_;
+  const int max_batch_size_, max_seq_len_, head_num_, size_per_head_;
+  AttentionParam<OpType> param_;
+
+  using AttentionInferParam = struct AttentionInferParam<DataType_>;
+
+  bool use_fused_attention_;
+  const bool is_remove_padding_;
+  const ModelType model_type_;
+
+ public:
+  // Sequences up to this length take the LDS-resident short kernel when
+  // use_fused_attention is set; longer ones (or use_fused_attention = false)
+  // take the streaming grouped kernel.
+  static constexpr int kShortSeqLimit = 256;
+
+  Attention(const int max_batch_size, const int head_num, const int size_per_head,
+            const int max_seq_len, const bool use_fused_attention = true,
+            const bool is_remove_padding = false, const ModelType model_type = ModelType::Bert)
+      : max_batch_size_(max_batch_size),
+        max_seq_len_(max_seq_len),
+        head_num_(head_num),
+        size_per_head_(size_per_head),
+        use_fused_attention_(use_fused_attention),
+        is_remove_padding_(is_remove_padding),
+        model_type_(model_type) {}
+
+  void initialize(AttentionParam<OpType> param) { param_ = param; }
+
+  // Both kernels keep logits and probabilities on chip: no attention scratch.
+  virtual unsigned long long cal_bufsize() const { return 0; }
+
+  bool uses_short_kernel(int seq_len) const {
+    return use_fused_attention_ && seq_len <= kShortSeqLimit;
+  }
+
+  virtual void infer(AttentionInferParam infer_param);
+
+  virtual ~Attention() {}
+};
+
+}  // namespace bytetransformer

@@ -1,0 +1,141 @@
+// BertTransformer<OpType>: one post-LN BERT encoder layer, padded [B,S,H] in,
+// padded [B,S,H] out, optionally running on the packed (padding-free) rows in
+// between.  Public surface follows the reference's
+// bytetransformer/include/bert_transformer.h:30-224: BertTransformerParam,
+// BertTransformerInferParam (same field order, so positional aggregate
+// initialisation keeps working), and BertTransformer with
+// ctor / initialize / cal_bufsize / infer.
+#pragma once
+#include "attention.h"
+#include "common.h"
+
+namespace bytetransformer {
+
+template <OperationType OpType>
+class BertTransformerParam {
+ private:
+  typedef Traits<OpType> Traits_;
+  typedef typename Traits_::DataType DataType_;
+
+ public:
+  AttentionParam<OpType> attention_param;
+
+  const DataType_ *attr_kernel_QKV = nullptr;  // [H, 3H]
+
+  const DataType_ *attr_output_kernel = nullptr;  // [H, H]
+  const DataType_ *attr_output_bias = nullptr;
+  const void *attr_output_layernorm_gamma = nullptr;  // DataType_ or float (use_fp32)
+  const void *attr_output_layernorm_beta = nullptr;
+
+  const DataType_ *inter_kernel = nullptr;  // [H, intermediate_size * H]
+  const DataType_ *inter_bias = nullptr;
+
+  const DataType_ *output_kernel = nullptr;  // [intermediate_size * H, H]
+  const DataType_ *output_bias = nullptr;
+  const void *output_layernorm_gamma = nullptr;
+  const void *output_layernorm_beta = nullptr;
+
+  int intermediate_size = 4;
+
+  int cublas_Algo[3] = {Traits_::algo, Traits_::algo, Traits_::algo};  // unused, kept for callers
+};
+
+template <typename T>
+struct BertTransformerInferParam {
+  const T *input_tensor;  // [batch_size, seq_len, hidden_dim]
+  const T *atten_mask;    // [batch_size, seq_len, seq_len], 1 = attend, 0 = padding
+  T *transformer_output;  // [batch_size, seq_len, hidden_dim]; must not alias input_tensor
+  void *buf;              // >= cal_bufsize() bytes of device memory, 256-byte aligned
+  int batch_size;
+  int seq_len;
+  BlasHandle cublas_handle;  // ignored
+  hipStream_t stream;
+  const T *attention_bias = NULL;         // [head_num, seq_len, seq_len]; must be NULL
+  const uint32_t *position_ids = NULL;    // never read
+  const uint32_t *token_type_ids = NULL;  // never read
+};
+
+template <OperationType OpType>
+class BertTransformer {
+ private:
+  typedef Traits<OpType> Traits_;
+  typedef typename Traits_::DataType DataType_;
+
+  BertTransformerParam<OpType> param_;
+  using BertTransformerInferParam = struct BertTransformerInferParam<DataType_>;
+
+  Attention<OpType> *attention_layer_ = nullptr;
+
+  const int max_batch_size_, max_seq_len_, head_num_, size_per_head_;
+
+  unsigned long long inner_buf_size_ = 0;
+
+  bool use_fused_attention_;
+  bool is_remove_padding_;
+  const bool use_fp32_;  // gamma & beta datatype
+  const ModelType model_type_;
+
+  static unsigned long long align_up(unsigned long long v, unsigned long long a) {
+    return (v + a - 1) / a * a;
+  }
+
+ public:
+  // LayerNorm epsilon of the reference kernels (layernorm.h:35,58,103,133).
+  float layernorm_eps = 1e-6f;
+
+  BertTransformer(const int max_batch_size, const int head_num, const int size_per_head,
+                  const int max_seq_len, const bool use_fused_attention = true,
+                  const bool is_remove_padding = true, const bool use_fp32 = false,
+                  const ModelType model_type = ModelType::Bert)
+      : max_batch_size_(max_batch_size),
+        max_seq_len_(max_seq_len),
+        head_num_(head_num),
+        size_per_head_(size_per_head),
+        use_fused_attention_(use_fused_attention),
+        is_remove_padding_(is_remove_padding),
+        use_fp32_(use_fp32),
+        model_type_(model_type) {
+    // Same side rule as the reference (bert_transformer.h:135-136): tiny batches
+    // run on the padded rows.
+    if (max_batch_size_ <= 2) is_remove_padding_ = false;
+    attention_layer_ =
+        new Attention<OpType>(max_batch_size, head_num, size_per_head, max_seq_len,
+                              use_fused_attention_, is_remove_padding_, model_type_);
+  }
+
+  BertTransformer(const BertTransformer &) = delete;
+  BertTransformer &operator=(const BertTransformer &) = delete;
+
+  void initialize(BertTransformerParam<OpType> param) {
+    param_ = param;
+    attention_layer_->initialize(param_.attention_param);
+  }
+
+  bool is_remove_padding() const { return is_remove_padding_; }
+
+  // Scratch layout (elements of DataType_, T = max_batch*max_seq*hidden):
+  //   [0,3T) qkv heads | [3T,4T) attention out | [4T,5T) projection / LN1 |
+  //   [5T,(5+mult)T) FFN1 | word_idx int[B*S] | batch_idx int[B*S] |
+  //   pre-packed weights (3+1+2*mult)*H*H | attention scratch (none)
+  unsigned long long cal_bufsize() {
+    const unsigned long long rows = (unsigned long long)max_batch_size_ * max_seq_len_;
+    const unsigned long long hidden = (unsigned long long)head_num_ * size_per_head_;
+    const unsigned long long tensor = rows * hidden;
+    inner_buf_size_ = (5 + param_.intermediate_size) * tensor * sizeof(DataType_);
+    inner_buf_size_ = align_up(inner_buf_size_, 256);
+    inner_buf_size_ += align_up(rows * 2 * sizeof(int) + 2 * sizeof(int), 256);
+    inner_buf_size_ += align_up(
+        (4 + 2 * (unsigned long long)param_.intermediate_size) * hidden * hidden *
+            sizeof(DataType_),
+        256);
+    return inner_buf_size_ + attention_layer_->cal_bufsize();
+  }
+
+  void infer(BertTransformerInferParam infer_param) { bert_infer(infer_param); }
+
+  void bert_infer(BertTransformerInferParam infer_param);
+
+  ~BertTransformer() { delete attention_layer_; }
+};
+
+}  // namespace bytetransformer

@@ -1,0 +1,70 @@
+// Shared API types of the BERT encoder-layer library, gfx950 build.
+//
+// Mirrors the public names of the reference's bytetransformer/include/common.h
+// (OperationType, Traits, ET_Param, ModelType, ActType, the runtime-error
+// convention of common.h:130-138) so that caller code written against the
+// reference compiles against this header.  cuBLAS/CUDA types do not exist
+// here: streams are hipStream_t and the BLAS-handle slots are opaque pointers
+// that the library never dereferences (every GEMM is an in-tree MFMA kernel).
+#pragma once
+#include <hip/hip_fp16.h>
+#include <hip/hip_runtime_api.h>
+
+#include <cstdint>
+#include <stdexcept>
+#include <string>
+
+#include "bt_hip.h"
+
+namespace bytetransformer {
+
+enum class OperationType { FP32, HALF };
+
+// Opaque stand-in for the reference's cublasHandle_t members.
+typedef void *BlasHandle;
+
+template <OperationType OpType>
+class Traits;
+
+template <>
+class Traits<OperationType::FP32> {
+ public:
+  typedef float DataType;
+  static const int dtype = BT_F32;
+  static const int algo = -1;
+};
+
+template <>
+class Traits<OperationType::HALF> {
+ public:
+  typedef __half DataType;
+  static const int dtype = BT_F16;
+  static const int algo = 99;
+};
+
+// Packed-token bookkeeping produced by the mask prefix sum.  valid_word_num is
+// only filled in when the caller asked the offsets builder for it; the kernels
+// read the count from batch_idx[batch_size] on the device.
+typedef struct {
+  int *batch_idx;
+  int *word_idx;
+  int valid_word_num;
+} ET_Param;
+
+enum ModelType { Bert };
+
+enum ActType { Relu, Sigmoid, SoftPlus, No };
+
+// Turns a non-zero C-ABI status into the exception the reference's
+// check_cuda_error raises (std::runtime_error, "[BT][ERROR] ..." prefix).
+inline void check_status(int status, const char *file, int line) {
+  if (status != BT_OK) {
+    std::string msg = bt_last_error_string();
+    if (msg.rfind("[BT][ERROR]", 0) != 0) msg = "[BT][ERROR] " + msg;
+    throw std::runtime_error(msg + " " + file + ":" + std::to_string(line) + " \n");
+  }
+}
+
+#define check_bt_error(val) ::bytetransformer::check_status((val), __FILE__, __LINE__)
+
+}  // namespace bytetransformer

@@ -1,0 +1,6 @@
+"""CPU oracle for the padding-free BERT encoder-layer forward.
+
+TEST INFRASTRUCTURE ONLY.  Nothing in the shipped package imports this
+directory; it is used by ``tests/``, by ``__graft_entry__.smoke()`` and by the
+``cpu_baseline`` leg of ``bench.py`` as the checker / reported baseline.
+"""

@@ -1,0 +1,117 @@
+"""CPU-side checks of the boundary: the libraries load, export every symbol the
+headers declare, reject bad arguments before touching the GPU, and the PyTorch
+operator keeps the reference's schema and error behaviour."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+import bytetransformer_amd as bt
+from bytetransformer_amd import _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared(header):
+    text = open(os.path.join(ROOT, "include", header)).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(bt_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_kernel_library_exports_every_declared_symbol():
+    names = _declared("bt_hip.h")
+    assert len(names) >= 12
+    lib = ctypes.CDLL(os.path.join(bt.lib_dir(), "libbt_hip.so"))
+    for n in names:
+        assert hasattr(lib, n), n
+    assert sorted(_lib.KERNEL_ABI) == names       # the ctypes table covers the header
+    assert bt.kernel_lib().bt_version() == 1
+
+
+def test_host_library_exports_every_declared_symbol():
+    names = _declared("bt_encoder.h")
+    bt.kernel_lib()
+    lib = ctypes.CDLL(os.path.join(bt.lib_dir(), "libbytetransformer.so"))
+    for n in names:
+        assert hasattr(lib, n), n
+    assert sorted(_lib.HOST_ABI) == names
+
+
+def test_argument_validation_returns_codes_without_gpu():
+    lib = bt.kernel_lib()
+    err = lambda: lib.bt_last_error_string().decode()
+    assert lib.bt_gemm(None, None, None, None, 4, 8, 64, None) == 1 and "null pointer" in err()
+    p = ctypes.c_void_p(256)   # never dereferenced: validation fails first
+    assert lib.bt_gemm(p, p, p, None, 4, 8, 100, None) == 2 and "multiple of 64" in err()
+    assert lib.bt_gemm(p, p, p, None, 4, 12, 64, None) == 2 and "multiple of 8" in err()
+    assert lib.bt_gemm_qkv_bias_split(p, p, p, p, None, 4, 12, 32, None) == 2
+    assert "size_per_head=32" in err()
+    assert lib.bt_attention_short(p, p, p, 1, 1024, 1024, 12, 64, 0.125, 0, None) == 2
+    assert "exceeds 512" in err()
+    assert lib.bt_attention_grouped(p, p, p, 1, 16, 16, 12, 48, 0.125, 0, None) == 2
+    assert lib.bt_compress(p, p, p, p, 2, 4, 12, None) == 2 and "multiple of 8" in err()
+    assert lib.bt_build_offsets(p, 7, 2, 4, p, p, None, None) == 1 and "dtype" in err()
+    assert lib.bt_build_offsets(p, 1, 0, 4, p, p, None, None) == 1
+    assert lib.bt_add_bias_residual_layernorm(p, p, p, p, p, 0, None, 4, 12, 1e-6, None) == 2
+    assert lib.bt_add_bias_residual_layernorm(p, p, p, p, p, 0, None, 4, 8192, 1e-6, None) == 2
+    assert lib.bt_add_bias_residual_layernorm_restore(p, p, p, p, p, 0, None, p, 2, 4, 64, 1e-6,
+                                                      None) == 1
+    assert lib.bt_transpose_weight(None, p, 8, 8, None) == 1
+
+
+def test_encoder_c_api_validation_and_bufsize():
+    lib = bt.host_lib()
+    cfg = _lib.EncoderConfig(1, 16, 512, 12, 64, 4, 1, 1, 0, 1.0, 1e-6)
+    need = lib.bt_encoder_bufsize(ctypes.byref(cfg))
+    T = 16 * 512 * 768
+    # nine activation tensors + two index arrays + the pre-packed weights
+    assert need >= 9 * T * 2 + 2 * 16 * 512 * 4 + 12 * 768 * 768 * 2
+    assert need < 9 * T * 2 + 2 * 16 * 512 * 4 + 12 * 768 * 768 * 2 + 4096
+    bad = _lib.EncoderConfig(0, 16, 512, 12, 64, 4, 1, 1, 0, 1.0, 1e-6)   # fp32: not implemented
+    assert lib.bt_encoder_bufsize(ctypes.byref(bad)) == 0
+    assert b"BT_F16" in lib.bt_encoder_last_error()
+    w = _lib.LayerWeights()
+    rc = lib.bt_encoder_layer_forward(ctypes.byref(cfg), ctypes.byref(w), None, None, None, None,
+                                      1, 1, None)
+    assert rc != 0 and b"null weight pointer" in lib.bt_encoder_last_error()
+
+
+def _cpu_args(H=128, B=2, S=8, dtype=torch.float16):
+    w = [torch.zeros(H, 3 * H), torch.zeros(3 * H), torch.zeros(H, H), torch.zeros(H),
+         torch.ones(H), torch.zeros(H), torch.zeros(H, 4 * H), torch.zeros(4 * H),
+         torch.zeros(4 * H, H), torch.zeros(H), torch.ones(H), torch.zeros(H)]
+    w = [t.to(dtype) for t in w]
+    return w, torch.zeros(B, S, H, dtype=dtype), torch.ones(B, S, S, dtype=dtype)
+
+
+def test_th_op_schema_matches_reference():
+    bt.load_th_op()
+    schema = str(torch.ops.ByteTransformer.BertTransformer.default._schema)
+    assert schema.startswith("ByteTransformer::BertTransformer(int head_num, int head_size, "
+                             "Tensor qkv_kernel, Tensor qkv_bias, Tensor attr_output_kernel")
+    assert "Tensor input, Tensor attr_mask, bool is_remove_padding=True, " \
+           "bool use_fused_attention=True) -> Tensor" in schema
+
+
+def test_th_op_rejects_host_tensors_like_the_reference():
+    bt.load_th_op()
+    w, x, m = _cpu_args()
+    with pytest.raises(RuntimeError, match="qkv_kernel must be a CUDA tensor"):
+        torch.ops.ByteTransformer.BertTransformer(2, 64, *w, x, m, True, True)
+
+
+def test_missing_library_raises(monkeypatch, tmp_path):
+    monkeypatch.setattr(_lib, "_DIR", str(tmp_path))
+    with pytest.raises(bt.LibraryMissing, match="no fallback"):
+        _lib._path("libbt_hip.so")
+
+
+def test_package_does_not_import_the_oracle():
+    pkg = os.path.join(ROOT, "bytetransformer_amd")
+    for dirpath, _, files in os.walk(pkg):
+        for f in files:
+            if f.endswith((".py", ".cc", ".hip", ".h")):
+                text = open(os.path.join(dirpath, f)).read()
+                assert "oracle" not in text, os.path.join(dirpath, f)

@@ -1,0 +1,303 @@
+"""Per-kernel parity: every C-ABI entry point of libbt_hip.so against the CPU
+oracle on the same seeded inputs.  Integer outputs and copies are bit-exact;
+fp16 results carry the tolerance written in each test."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from bytetransformer_amd import ops, workload
+from oracle import bert_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+
+def _dev(a, device):
+    return torch.from_numpy(np.ascontiguousarray(a)).to(device)
+
+
+def _say(*a):
+    print(*a, flush=True)
+
+
+# ---- offsets (bit-exact) -------------------------------------------------------
+@pytest.mark.parametrize("B,S,dtype", [(1, 256, np.float16), (16, 512, np.float16),
+                                       (3, 7, np.float32), (70, 33, np.float16),
+                                       (130, 100, np.float16), (32, 384, np.float16),
+                                       (16, 1024, np.float32)])
+def test_build_offsets_bit_exact(device, B, S, dtype):
+    _say("offsets", B, S, dtype)
+    rs = np.random.RandomState(B * 1000 + S)
+    lens = rs.randint(0, S + 1, size=B)
+    lens[0] = S
+    if B > 2:
+        lens[1] = 0
+    mask = workload.make_mask(lens, S, dtype)
+    mask[:, 1:, :] = 1 - mask[:, 1:, :]          # rows other than 0 must be ignored
+    bi, wi, M = O.build_offsets(mask)
+    g_bi, g_wi, g_M = ops.build_offsets(_dev(mask, device), want_count=True)
+    assert g_M == M
+    assert g_bi.dtype == torch.int32 and g_wi.dtype == torch.int32
+    assert np.array_equal(g_bi.cpu().numpy(), bi)
+    assert np.array_equal(g_wi.cpu().numpy()[:M], wi)
+
+
+def test_build_offsets_threshold(device):
+    S = 70
+    mask = np.zeros((2, S, S), np.float16)
+    mask[0, 0, :] = np.linspace(0, 1, S)          # crosses 0.5 somewhere in the row
+    mask[1, 0, :5] = [0.5, 0.4999, 1, 0.51, 0]
+    bi, wi, M = O.build_offsets(mask)
+    g_bi, g_wi, g_M = ops.build_offsets(_dev(mask, device), want_count=True)
+    assert g_M == M and np.array_equal(g_bi.cpu().numpy(), bi)
+    assert np.array_equal(g_wi.cpu().numpy()[:M], wi)
+
+
+# ---- compress / restore (bit-exact copies) -------------------------------------
+@pytest.mark.parametrize("B,S,H", [(4, 50, 768), (16, 512, 768), (3, 9, 1024), (2, 5, 8)])
+def test_compress_bit_exact(device, B, S, H):
+    _say("compress", B, S, H)
+    rs = np.random.RandomState(7)
+    lens = rs.randint(0, S + 1, size=B)
+    lens[-1] = S
+    x = rs.standard_normal((B, S, H)).astype(np.float16)
+    mask = workload.make_mask(lens, S, np.float16)
+    bi, wi, M = O.build_offsets(mask)
+    g_bi, g_wi, _ = ops.build_offsets(_dev(mask, device))
+    sentinel = torch.full((B * S, H), 7.0, dtype=torch.float16, device=device)
+    packed = ops.compress(_dev(x, device), g_bi, g_wi, out=sentinel).cpu().numpy()
+    assert np.array_equal(packed[:M].view(np.uint16), O.compress(x, wi).view(np.uint16))
+    assert np.all(packed[M:] == 7.0)               # rows past M are never written
+
+
+# ---- LayerNorm ----------------------------------------------------------------
+@pytest.mark.parametrize("H,gb32", [(768, False), (1024, True), (64, False), (2048, False),
+                                    (4096, True), (264, False)])
+def test_add_bias_residual_layernorm(device, H, gb32):
+    _say("layernorm", H, gb32)
+    rs = np.random.RandomState(H)
+    rows, M = 37, 29
+    out = rs.standard_normal((rows, H)).astype(np.float16)
+    res = (rs.standard_normal((rows, H)) * 2).astype(np.float16)
+    bias = (rs.standard_normal(H) * 0.5).astype(np.float16)
+    gdt = np.float32 if gb32 else np.float16
+    gamma = (1 + 0.2 * rs.standard_normal(H)).astype(gdt)
+    beta = (0.3 * rs.standard_normal(H)).astype(gdt)
+    exp = O.add_bias_residual_layernorm(out, res, bias, gamma, beta, 1e-6)
+    vr = torch.tensor([M], dtype=torch.int32, device=device)
+    g = ops.add_bias_residual_layernorm(_dev(out, device), _dev(res, device), _dev(bias, device),
+                                        _dev(gamma, device), _dev(beta, device), 1e-6,
+                                        valid_rows=vr).cpu().numpy()
+    # rounding of the fp16 result: half an ulp (2^-11 relative) plus fp32 statistics noise
+    err = np.abs(g[:M].astype(np.float64) - exp[:M])
+    assert np.all(err <= 2.0 ** -10 * np.abs(exp[:M]) + 1e-4), err.max()
+    assert np.array_equal(g[M:], out[M:])          # rows past M untouched
+    # all rows live when valid_rows is null
+    g2 = ops.add_bias_residual_layernorm(_dev(out, device), _dev(res, device), _dev(bias, device),
+                                         _dev(gamma, device), _dev(beta, device), 1e-6).cpu().numpy()
+    err = np.abs(g2.astype(np.float64) - exp)
+    assert np.all(err <= 2.0 ** -10 * np.abs(exp) + 1e-4)
+
+
+@pytest.mark.parametrize("B,S,H", [(4, 33, 768), (16, 128, 1024)])
+def test_layernorm_restore_zero_fills_padding(device, B, S, H):
+    _say("layernorm_restore", B, S, H)
+    rs = np.random.RandomState(B + S)
+    lens = rs.randint(0, S + 1, size=B)
+    lens[0], lens[-1] = S, 0
+    mask = workload.make_mask(lens, S, np.float16)
+    bi, wi, M = O.build_offsets(mask)
+    out = rs.standard_normal((B * S, H)).astype(np.float16)
+    res = rs.standard_normal((B * S, H)).astype(np.float16)
+    bias = (rs.standard_normal(H) * 0.5).astype(np.float16)
+    gamma = (1 + 0.2 * rs.standard_normal(H)).astype(np.float16)
+    beta = (0.3 * rs.standard_normal(H)).astype(np.float16)
+    exp = O.restore(O.add_bias_residual_layernorm(out[:M], res[:M], bias, gamma, beta, 1e-6), bi,
+                    B, S)
+    g_bi, _, _ = ops.build_offsets(_dev(mask, device))
+    target = torch.full((B, S, H), float("nan"), dtype=torch.float16, device=device)
+    g = ops.add_bias_residual_layernorm_restore(
+        _dev(out, device), _dev(res, device), _dev(bias, device), _dev(gamma, device),
+        _dev(beta, device), g_bi, B, S, 1e-6, out_padded=target).cpu().numpy()
+    for b in range(B):
+        assert np.all(g[b, lens[b]:].view(np.uint16) == 0)      # exact +0 fill
+    err = np.abs(g.astype(np.float64) - exp)
+    assert np.all(err <= 2.0 ** -10 * np.abs(exp) + 1e-4), err.max()
+
+
+# ---- weight pre-pack -----------------------------------------------------------
+@pytest.mark.parametrize("K,N", [(768, 2304), (3072, 768), (64, 8), (200, 136)])
+def test_transpose_weight_bit_exact(device, K, N):
+    w = np.random.RandomState(K + N).standard_normal((K, N)).astype(np.float16)
+    wt = ops.transpose_weight(_dev(w, device)).cpu().numpy()
+    assert np.array_equal(wt.view(np.uint16), np.ascontiguousarray(w.T).view(np.uint16))
+
+
+# ---- GEMM family ---------------------------------------------------------------
+def _gemm_tol(exp, K, amax, wmax):
+    # one fp16 rounding of the result plus fp32 accumulation noise
+    return 2.0 ** -10 * np.abs(exp) + 4 * K * 2.0 ** -24 * amax * wmax + 1e-6
+
+
+@pytest.mark.parametrize("tile", [0, 1, 2])
+@pytest.mark.parametrize("rows,M,N,K", [(300, 300, 768, 768), (1000, 777, 2304, 768),
+                                        (520, 513, 768, 3072), (64, 1, 136, 64),
+                                        (257, 257, 3072, 768)])
+def test_gemm_plain(device, tile, rows, M, N, K):
+    _say("gemm", tile, rows, M, N, K)
+    rs = np.random.RandomState(rows + N)
+    a = rs.standard_normal((rows, K)).astype(np.float16)
+    w = (rs.standard_normal((K, N)) * 0.05).astype(np.float16)
+    exp = O.gemm(a[:M], w)
+    ops.set_option("gemm_tile", tile)
+    try:
+        wt = ops.transpose_weight(_dev(w, device))
+        vr = torch.tensor([M], dtype=torch.int32, device=device)
+        out = torch.full((rows, N), 3.0, dtype=torch.float16, device=device)
+        g = ops.gemm(_dev(a, device), wt, valid_rows=vr, out=out).cpu().numpy()
+    finally:
+        ops.set_option("gemm_tile", -1)
+    err = np.abs(g[:M].astype(np.float64) - exp)
+    tol = _gemm_tol(exp, K, np.abs(a).max(), np.abs(w).max())
+    assert np.all(err <= tol), (err.max(), np.unravel_index(err.argmax(), err.shape))
+    assert np.all(g[M:] == 3.0)
+
+
+@pytest.mark.parametrize("tile", [0, 1, 2])
+def test_gemm_bias_gelu(device, tile):
+    _say("gemm_bias_gelu", tile)
+    rs = np.random.RandomState(tile)
+    rows, M, N, K = 700, 650, 3072, 768
+    a = rs.standard_normal((rows, K)).astype(np.float16)
+    w = (rs.standard_normal((K, N)) * 0.06).astype(np.float16)
+    bias = (rs.standard_normal(N) * 0.5).astype(np.float16)
+    exp = O.gemm(a[:M], w, bias, "gelu_tanh")
+    ops.set_option("gemm_tile", tile)
+    try:
+        vr = torch.tensor([M], dtype=torch.int32, device=device)
+        g = ops.gemm_bias_gelu(_dev(a, device), ops.transpose_weight(_dev(w, device)),
+                               _dev(bias, device), valid_rows=vr).cpu().numpy()
+    finally:
+        ops.set_option("gemm_tile", -1)
+    err = np.abs(g[:M].astype(np.float64) - exp)
+    # gelu' <= 1.13; fast exp / divide add a few fp32 ulps
+    assert np.all(err <= 2.0 ** -10 * np.abs(exp) + 2e-4), err.max()
+    assert np.all(g[M:] == 0)
+
+
+@pytest.mark.parametrize("tile", [0, 1, 2])
+@pytest.mark.parametrize("heads", [12, 16])
+def test_gemm_qkv_bias_split(device, tile, heads):
+    _say("gemm_qkv", tile, heads)
+    rs = np.random.RandomState(heads)
+    H = heads * 64
+    rows, M = 400, 333
+    a = rs.standard_normal((rows, H)).astype(np.float16)
+    w = (rs.standard_normal((H, 3 * H)) * 0.05).astype(np.float16)
+    bias = (rs.standard_normal(3 * H) * 0.5).astype(np.float16)
+    exp = O.split_heads(O.gemm(a[:M], w, bias), heads, 64)           # [3, heads, M, 64]
+    ops.set_option("gemm_tile", tile)
+    try:
+        vr = torch.tensor([M], dtype=torch.int32, device=device)
+        g = ops.gemm_qkv_bias_split(_dev(a, device), ops.transpose_weight(_dev(w, device)),
+                                    _dev(bias, device), heads, valid_rows=vr).cpu().numpy()
+    finally:
+        ops.set_option("gemm_tile", -1)
+    assert g.shape == (3, heads, rows, 64)
+    err = np.abs(g[:, :, :M].astype(np.float64) - exp)
+    assert np.all(err <= 2.0 ** -10 * np.abs(exp) + 2e-4), err.max()
+    assert np.all(g[:, :, M:] == 0)
+
+
+# ---- attention -----------------------------------------------------------------
+def _attention_case(rs, lens, S, heads, scale_q=1.0):
+    B = len(lens)
+    bi = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    M = int(bi[-1])
+    rows_cap = B * S
+    qkv = np.zeros((3, heads, rows_cap, 64), np.float16)
+    qkv[:, :, :M] = rs.standard_normal((3, heads, M, 64)).astype(np.float16)
+    qkv[0] *= scale_q
+    qkv[:, :, M:] = np.float16("nan")        # rows past M must never be consumed
+    return bi, M, qkv
+
+
+ATT_CASES = [
+    ("short", [154], 256, 12),
+    ("short", [64, 38], 64, 12),
+    ("short", [1, 16, 17, 0, 100, 128], 128, 3),
+    ("short", [300, 384, 77, 5], 384, 4),
+    ("short", [512, 103, 257], 512, 2),
+    ("grouped", [512, 103, 257, 64, 65, 1, 0, 300], 512, 3),
+    ("grouped", [1024, 205, 700], 1024, 2),
+    ("grouped", [154], 256, 12),
+    ("grouped", [33, 2, 47], 47, 5),
+]
+
+
+@pytest.mark.parametrize("qb", [-1, 1, 2])
+@pytest.mark.parametrize("kind,lens,S,heads", ATT_CASES)
+def test_attention_packed(device, kind, lens, S, heads, qb):
+    if kind == "short" and qb != -1:
+        pytest.skip("option only affects the grouped kernel")
+    _say("attention", kind, lens, S, heads, qb)
+    rs = np.random.RandomState(S + heads)
+    bi, M, qkv = _attention_case(rs, lens, S, heads, scale_q=2.0)
+    scale = 1 / math.sqrt(64)
+    exp = O.attention_packed(qkv[0, :, :M], qkv[1, :, :M], qkv[2, :, :M], bi, scale, 1e-6,
+                             round_p_fp16=True)
+    fn = ops.attention_short if kind == "short" else ops.attention_grouped
+    ops.set_option("attention_qb", qb)
+    try:
+        out = torch.full((len(lens) * S, heads * 64), 5.0, dtype=torch.float16, device=device)
+        g = fn(_dev(qkv, device), _dev(bi, device), len(lens), S, scale, False, out=out)
+        g = g.cpu().numpy()
+    finally:
+        ops.set_option("attention_qb", -1)
+    err = np.abs(g[:M].astype(np.float64) - exp)
+    # P is rounded to fp16 (2^-11 relative per term, |V| ~ N(0,1)) and O once more
+    assert err.max() <= 4e-3 and err.mean() <= 4e-4, (err.max(), err.mean())
+    assert np.all(g[M:] == 5.0)
+
+
+@pytest.mark.parametrize("kind", ["short", "grouped"])
+def test_attention_padded_rows_mode(device, kind):
+    """Padded layout: sequence b owns rows [b*S, (b+1)*S); every query row is
+    computed against the len_b valid keys."""
+    _say("attention padded", kind)
+    rs = np.random.RandomState(3)
+    lens, S, heads = [40, 64, 7], 64, 4
+    B = len(lens)
+    bi = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    qkv = rs.standard_normal((3, heads, B * S, 64)).astype(np.float16)
+    scale = 1 / math.sqrt(64)
+    fn = ops.attention_short if kind == "short" else ops.attention_grouped
+    g = fn(_dev(qkv, device), _dev(bi, device), B, S, scale, True).cpu().numpy()
+    for b in range(B):
+        n = lens[b]
+        q = qkv[0, :, b * S:(b + 1) * S].astype(np.float64)
+        k = qkv[1, :, b * S:b * S + n].astype(np.float64)
+        v = qkv[2, :, b * S:b * S + n].astype(np.float64)
+        s = np.einsum("hqd,hkd->hqk", q, k) * scale
+        e = np.exp(s - s.max(-1, keepdims=True))
+        p = O.f16(e / (e.sum(-1, keepdims=True) + 1e-6))
+        exp = np.einsum("hqk,hkd->qhd", p, v).reshape(S, heads * 64)
+        err = np.abs(g[b * S:(b + 1) * S].astype(np.float64) - exp)
+        assert err.max() <= 4e-3, (b, err.max())
+
+
+def test_attention_large_logits_do_not_overflow(device):
+    """Logits of a few hundred in magnitude (fp16 Q.K would overflow at 65504)."""
+    rs = np.random.RandomState(9)
+    lens, S, heads = [96, 200], 256, 2
+    bi, M, qkv = _attention_case(rs, lens, S, heads, scale_q=30.0)
+    qkv[1, :, :M] *= 8
+    scale = 1 / math.sqrt(64)
+    exp = O.attention_packed(qkv[0, :, :M], qkv[1, :, :M], qkv[2, :, :M], bi, scale, 1e-6,
+                             round_p_fp16=True)
+    for fn in (ops.attention_short, ops.attention_grouped):
+        g = fn(_dev(qkv, device), _dev(bi, device), len(lens), S, scale, False).cpu().numpy()
+        assert np.isfinite(g[:M]).all()
+        err = np.abs(g[:M].astype(np.float64) - exp)
+        assert err.max() <= 2e-2, err.max()

@@ -1,0 +1,209 @@
+"""Whole-layer parity on the GPU: the C++ BertTransformer (through
+bt_encoder_layer_forward) and the PyTorch operator against the CPU oracle on
+identical seeded inputs and weights.
+
+Tolerance (fp16 configurations): max-abs <= 2e-2 and mean-abs <= 2e-3 over the
+valid rows, padded rows exactly zero on the remove-padding path.  The oracle is
+the fp32 CPU encoder fed the same fp16-rounded inputs and weights."""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import bytetransformer_amd as bt
+from bytetransformer_amd import workload
+from oracle import bert_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+MAX_ABS, MEAN_ABS = 2e-2, 2e-3
+GOLDEN = os.path.join(os.path.dirname(__file__), "golden")
+
+
+def _say(*a):
+    print(*a, flush=True)
+
+
+def _dev(a, device):
+    return torch.from_numpy(np.ascontiguousarray(a)).to(device)
+
+
+def _oracle(wl, n_layers=None, **kw):
+    layers = wl.layers if n_layers is None else wl.layers[:n_layers]
+    layers32 = [{k: np.asarray(v, np.float32) for k, v in w.items()} for w in layers]
+    out = O.encoder(wl.x.astype(np.float32), wl.mask.astype(np.float32), layers32,
+                    wl.cfg.head_num, **kw)
+    return O.masked_output(out.numpy(), wl.lens)
+
+
+def _gpu_layers(wl, device, n_layers=None, **kw):
+    layers = wl.layers if n_layers is None else wl.layers[:n_layers]
+    return [bt.BertEncoderLayer(wl.cfg.head_num, wl.cfg.head_size,
+                                {k: _dev(v, device) for k, v in w.items()}, **kw)
+            for w in layers]
+
+
+def _run_c_api(wl, device, n_layers=None, **kw):
+    layers = _gpu_layers(wl, device, n_layers, **kw)
+    out = bt.encoder_forward(layers, _dev(wl.x, device), _dev(wl.mask, device))
+    torch.cuda.synchronize()
+    return out.cpu().numpy()
+
+
+def _run_th_op(wl, device, n_layers=None, rm=True, fused=True):
+    bt.load_th_op()
+    layers = wl.layers if n_layers is None else wl.layers[:n_layers]
+    h, mask = _dev(wl.x, device), _dev(wl.mask, device)
+    for w in layers:
+        h = torch.ops.ByteTransformer.BertTransformer(
+            wl.cfg.head_num, wl.cfg.head_size,
+            *[_dev(w[n], device) for n in workload.WEIGHT_NAMES], h, mask, rm, fused)
+    torch.cuda.synchronize()
+    return h.cpu().numpy()
+
+
+def _check(got, exp, lens, pads_must_be_zero=True, tag=""):
+    mx, mean, pads_zero = O.parity_metrics(got, exp, lens)
+    _say("parity %s: max-abs %.3e mean-abs %.3e pads_zero %s" % (tag, mx, mean, pads_zero))
+    assert np.isfinite(np.asarray(got, np.float32)).all()
+    assert mx <= MAX_ABS and mean <= MEAN_ABS, (mx, mean)
+    if pads_must_be_zero:
+        assert pads_zero
+
+
+# ---- committed golden case -------------------------------------------------------
+@pytest.mark.parametrize("path", ["c_api", "th_op"])
+@pytest.mark.parametrize("fused", [True, False])
+def test_small_golden_case(device, path, fused):
+    _say("golden small", path, fused)
+    z = np.load(os.path.join(GOLDEN, "small_fp16_case.npz"))
+    lens = z["lens"]
+    cfg = workload.EncoderConfig("small", 3, 48, 2, layers=1, lens=tuple(int(v) for v in lens))
+    wl = workload.Workload(cfg, lens, z["x"], workload.make_mask(lens, 48, np.float16),
+                           [{n: z[n] for n in workload.WEIGHT_NAMES}])
+    if path == "c_api":
+        got = _run_c_api(wl, device, use_fused_attention=fused)
+    else:
+        got = _run_th_op(wl, device, fused=fused)
+    _check(got, z["expected"], lens, tag="small/%s/fused=%s" % (path, fused))
+
+
+# ---- the named configurations ------------------------------------------------------
+def test_cfg0_shape_fp16_runs_padded_path(device):
+    """B = 2 silently disables remove-padding (as in the reference); padded rows
+    are then not zero, only valid rows are compared, against the committed cfg0
+    golden output (fp32 oracle) with the fp16-rounded inputs of the same seed."""
+    _say("cfg0 fp16")
+    wl32 = workload.make_workload("cfg0")
+    cfg = workload.EncoderConfig("cfg0h", 2, 64, 12, layers=1, dtype="fp16", lens=(64, 38))
+    wl = workload.Workload(cfg, wl32.lens, wl32.x.astype(np.float16),
+                           wl32.mask.astype(np.float16),
+                           [{k: v.astype(np.float16) for k, v in wl32.layers[0].items()}])
+    got = O.masked_output(_run_c_api(wl, device), wl.lens)
+    _check(got, _oracle(wl), wl.lens, tag="cfg0/fp16-inputs")
+    gold = np.load(os.path.join(GOLDEN, "cfg0_out.npy"))
+    _check(got, gold, wl.lens, tag="cfg0/golden-fp32")
+
+
+def test_cfg1_twelve_layers_short_kernel(device):
+    _say("cfg1")
+    wl = workload.make_workload("cfg1")
+    exp = _oracle(wl)
+    got = O.masked_output(_run_th_op(wl, device), wl.lens)   # B = 1: padded path
+    _check(got, exp, wl.lens, tag="cfg1/th_op")
+    got = O.masked_output(_run_c_api(wl, device, use_fused_attention=False), wl.lens)
+    _check(got, exp, wl.lens, tag="cfg1/c_api/grouped")
+
+
+def test_cfg2_one_layer_and_invariants(device):
+    _say("cfg2 one layer")
+    wl = workload.make_workload("cfg2", layers=1, bias_std=0.02, random_affine=True)
+    exp = _oracle(wl)
+    got = _run_c_api(wl, device)
+    _check(got, exp, wl.lens, tag="cfg2/L1/rm")
+    got_op = _run_th_op(wl, device)
+    assert np.array_equal(got_op.view(np.uint16), got.view(np.uint16))   # same kernels, same bits
+    # the result must not depend on what the padded input rows hold
+    x2 = wl.x.copy()
+    for b, n in enumerate(wl.lens):
+        x2[b, n:] = np.float16(300.0)
+    wl2 = workload.Workload(wl.cfg, wl.lens, x2, wl.mask, wl.layers)
+    assert np.array_equal(_run_c_api(wl2, device).view(np.uint16), got.view(np.uint16))
+    # padded path on the same data: valid rows agree with the packed path
+    got_pad = O.masked_output(_run_c_api(wl, device, is_remove_padding=False), wl.lens)
+    _check(got_pad, exp, wl.lens, tag="cfg2/L1/padded")
+    mx, _, _ = O.parity_metrics(got_pad, got, wl.lens)
+    assert mx <= 4e-3, mx
+
+
+def test_cfg2_twelve_layers_headline(device):
+    _say("cfg2 twelve layers")
+    wl = workload.make_workload("cfg2")
+    assert abs(wl.valid_tokens / (16 * 512) - 0.6) < 0.1
+    exp = _oracle(wl)
+    got = _run_th_op(wl, device)
+    _check(got, exp, wl.lens, tag="cfg2/L12/th_op")
+
+
+def test_cfg3_long_sequences_grouped_kernel(device):
+    _say("cfg3 two layers")
+    wl = workload.make_workload("cfg3", layers=2)
+    exp = _oracle(wl)
+    got = _run_c_api(wl, device)
+    _check(got, exp, wl.lens, tag="cfg3/L2")
+
+
+def test_cfg4_bert_large_variable_and_fixed(device):
+    _say("cfg4")
+    wl = workload.make_workload("cfg4", layers=2)
+    _check(_run_c_api(wl, device), _oracle(wl), wl.lens, tag="cfg4/var/L2")
+    # fixed-length twin: the padding-free path must match the padded path
+    wf = workload.make_workload("cfg4_fixed", layers=2)
+    rm = _run_c_api(wf, device, is_remove_padding=True)
+    pad = _run_c_api(wf, device, is_remove_padding=False)
+    _check(rm, _oracle(wf), wf.lens, tag="cfg4/fixed/L2")
+    assert np.abs(rm.astype(np.float32) - pad.astype(np.float32)).max() <= 4e-3
+
+
+def test_fp32_gamma_beta_next_to_fp16_weights(device):
+    _say("fp32 gamma/beta")
+    cfg = workload.EncoderConfig("g32", 4, 96, 4, layers=1, lens=(96, 5, 50, 77), seed=21)
+    wl = workload.make_workload(cfg, bias_std=0.05, random_affine=True)
+    exp = _oracle(wl)
+    for n in workload.WEIGHT_NAMES:
+        if "layernorm" in n:
+            wl.layers[0][n] = wl.layers[0][n].astype(np.float32)
+    _check(_run_th_op(wl, device), exp, wl.lens, tag="g32/th_op")
+    _check(_run_c_api(wl, device), exp, wl.lens, tag="g32/c_api")
+
+
+def test_ragged_edge_cases(device):
+    """Zero-length sequences, length 1, odd seq_len, non-default FFN multiple."""
+    _say("ragged")
+    cfg = workload.EncoderConfig("rag", 5, 37, 3, layers=2, ffn_mult=2, lens=(0, 1, 37, 36, 0),
+                                 seed=33)
+    wl = workload.make_workload(cfg, bias_std=0.05, random_affine=True)
+    _check(_run_c_api(wl, device), _oracle(wl), wl.lens, tag="ragged")
+    _check(_run_th_op(wl, device), _oracle(wl), wl.lens, tag="ragged/th_op")
+
+
+def test_th_op_error_paths_on_gpu(device):
+    bt.load_th_op()
+    cfg = workload.EncoderConfig("e", 3, 16, 2, layers=1, lens=(16, 3, 9))
+    wl = workload.make_workload(cfg)
+    w = [_dev(wl.layers[0][n], device) for n in workload.WEIGHT_NAMES]
+    x, m = _dev(wl.x, device), _dev(wl.mask, device)
+    op = torch.ops.ByteTransformer.BertTransformer
+    with pytest.raises(RuntimeError, match="must be contiguous"):
+        op(2, 64, *w, x.transpose(0, 1), m, True, True)
+    with pytest.raises(RuntimeError, match="Inconsistency of Tensor type"):
+        op(2, 64, *w, x.float(), m, True, True)
+    with pytest.raises(RuntimeError, match="Wrong Tensor type"):
+        op(2, 64, *[t.to(torch.bfloat16) for t in w], x.to(torch.bfloat16),
+           m.to(torch.bfloat16), True, True)
+    with pytest.raises(RuntimeError, match="seq_len too long"):
+        op(2, 64, *w, torch.zeros(1, 1025, 128, dtype=torch.float16, device=device),
+           torch.zeros(1, 1025, 1025, dtype=torch.float16, device=device), True, True)
+    with pytest.raises(RuntimeError, match="only OperationType::HALF"):
+        op(2, 64, *[t.float() for t in w], x.float(), m.float(), True, True)
