@@ -1,0 +1,223 @@
+#!/usr/bin/env python3
+"""Headline benchmark: ms per 12-layer BERT-base forward, fp16, batch 16,
+max seq 512, valid lengths uniform on [103, 512] (mean ~0.6 * max), through the
+PyTorch operator torch.ops.ByteTransformer.BertTransformer - one operator call
+per layer, as the reference's benchmark script drives it
+(unit_test/python_scripts/bert_transformer_test.py:184-208,
+benchmark/bert_bench.sh:21-57).
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg2]
+
+Prints ONE JSON line.  A "step" is one full L-layer forward over the synthetic
+batch; inputs and weights are resident in HBM before the timed region; the
+timed region is bracketed by torch.cuda.synchronize().  The same line carries
+the roofline of the dominant kernel (live HIP-event timing of that kernel at
+the workload's shape) and the CPU baseline (the oracle's PyTorch fp32 encoder on
+the host cores, bounded sample).
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+PUBLISHED_A100_MS = {"cfg1": 1.43, "cfg2": 9.22, "cfg3": 24.70}   # reference README.md:37,63,71
+MFMA_F16_PEAK_TFLOPS = 2500.0
+HBM_PEAK_GBS = 8000.0
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="cfg2",
+                    choices=["cfg1", "cfg2", "cfg3", "cfg4", "cfg4_fixed"])
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--kernel-iters", type=int, default=50)
+    return ap.parse_args()
+
+
+def time_kernel(fn, iters):
+    """Average duration (ms) of `fn`, which enqueues exactly one kernel on the
+    current stream, from HIP events recorded on that stream."""
+    import torch
+    for _ in range(3):
+        fn()
+    beg, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    beg.record()
+    for _ in range(iters):
+        fn()
+    end.record()
+    end.synchronize()
+    return beg.elapsed_time(end) / iters
+
+
+def kernel_table(wl, dev, iters):
+    """Live per-kernel timings at the workload's shape, each against its own
+    roofline: algorithmic flops (GEMMs, attention) or bytes (padding, LN)."""
+    import numpy as np
+    import torch
+    from bytetransformer_amd import ops
+    cfg = wl.cfg
+    B, S, H, F, heads = cfg.batch, cfg.seq_len, cfg.hidden, cfg.ffn_mult * cfg.hidden, cfg.head_num
+    T, M = B * S, wl.valid_tokens
+    sq = int((wl.lens.astype(np.int64) ** 2).sum())
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+    w = {k: t(v) for k, v in wl.layers[0].items()}
+    x, mask = t(wl.x), t(wl.mask)
+    batch_idx, word_idx, _ = ops.build_offsets(mask)
+    vr = batch_idx[B:]
+    packed = ops.compress(x, batch_idx, word_idx)
+    wt_qkv, wt_o = ops.transpose_weight(w["qkv_kernel"]), ops.transpose_weight(w["attr_output_kernel"])
+    wt_1, wt_2 = ops.transpose_weight(w["inter_kernel"]), ops.transpose_weight(w["output_kernel"])
+    qkv = ops.gemm_qkv_bias_split(packed, wt_qkv, w["qkv_bias"], heads, valid_rows=vr)
+    scale = 1.0 / cfg.head_size ** 0.5
+    att_fn = ops.attention_short if S <= 256 else ops.attention_grouped
+    att = att_fn(qkv, batch_idx, B, S, scale)
+    proj = ops.gemm(att, wt_o, valid_rows=vr)
+    inter = ops.gemm_bias_gelu(proj, wt_1, w["inter_bias"], valid_rows=vr)
+    ffn2 = ops.gemm(inter, wt_2, valid_rows=vr)
+    out_pad = torch.empty(B, S, H, dtype=torch.float16, device=dev)
+    ln_buf = proj.clone()
+    g1, b1 = w["attr_output_layernorm_gamma"], w["attr_output_layernorm_beta"]
+
+    rows = [
+        # name, callable, bound, algorithmic work per launch (flops or bytes)
+        ("build_offsets", lambda: ops.build_offsets(mask), "hbm", 2 * B * S + 4 * (B + 1) + 4 * M),
+        ("compress", lambda: ops.compress(x, batch_idx, word_idx, out=packed), "hbm",
+         2 * M * H * 2 + 4 * M),
+        ("gemm_qkv_bias_split", lambda: ops.gemm_qkv_bias_split(packed, wt_qkv, w["qkv_bias"],
+                                                                heads, valid_rows=vr, out=qkv),
+         "mfma", 2 * M * H * 3 * H),
+        ("attention", lambda: att_fn(qkv, batch_idx, B, S, scale, out=att), "mfma", 4 * H * sq),
+        ("gemm_proj", lambda: ops.gemm(att, wt_o, valid_rows=vr, out=proj), "mfma", 2 * M * H * H),
+        ("layernorm", lambda: ops.add_bias_residual_layernorm(ln_buf, packed, w["attr_output_bias"],
+                                                              g1, b1, valid_rows=vr),
+         "hbm", 3 * M * H * 2),
+        ("gemm_bias_gelu", lambda: ops.gemm_bias_gelu(proj, wt_1, w["inter_bias"], valid_rows=vr,
+                                                      out=inter), "mfma", 2 * M * H * F),
+        ("gemm_ffn2", lambda: ops.gemm(inter, wt_2, valid_rows=vr, out=ffn2), "mfma",
+         2 * M * F * H),
+        ("layernorm_restore", lambda: ops.add_bias_residual_layernorm_restore(
+            ffn2, proj, w["output_bias"], g1, b1, batch_idx, B, S, out_padded=out_pad),
+         "hbm", 2 * M * H * 2 + T * H * 2),
+        ("transpose_weights", lambda: ops.transpose_weight(w["inter_kernel"]), "hbm",
+         2 * H * F * 2),
+    ]
+    table = {}
+    for name, fn, bound, work in rows:
+        ms = time_kernel(fn, iters)
+        if bound == "mfma":
+            ach, peak, unit = work / (ms * 1e-3) / 1e12, MFMA_F16_PEAK_TFLOPS, "TFLOP/s"
+        else:
+            ach, peak, unit = work / (ms * 1e-3) / 1e9, HBM_PEAK_GBS, "GB/s"
+        table[name] = {"us": round(ms * 1e3, 2), "bound": bound, "achieved": round(ach, 2),
+                       "peak": peak, "unit": unit, "frac": round(ach / peak, 4)}
+    return table
+
+
+def cpu_baseline(wl, budget_s=25.0):
+    """The oracle's PyTorch fp32 encoder on the padded batch, all host cores,
+    on as many of the L layers as fit the time budget (at least one)."""
+    import numpy as np
+    import torch
+    from oracle import bert_oracle as O
+    cores = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "0")) or 10 ** 6)
+    torch.set_num_threads(cores)
+    x = torch.from_numpy(wl.x.astype(np.float32))
+    mask = torch.from_numpy(wl.mask.astype(np.float32))
+    layers32 = [{k: torch.from_numpy(np.asarray(v, np.float32)) for k, v in w.items()}
+                for w in wl.layers]
+    with torch.no_grad():
+        O.encoder_layer(x, mask, layers32[0], wl.cfg.head_num)       # warm-up
+        done, t0 = 0, time.perf_counter()
+        h = x
+        for w in layers32:
+            h = O.encoder_layer(h, mask, w, wl.cfg.head_num)
+            done += 1
+            if time.perf_counter() - t0 > budget_s:
+                break
+        el = time.perf_counter() - t0
+    ms_full = el / done * len(layers32) * 1e3
+    return {"value": round(ms_full, 1), "unit": "ms", "cores": cores, "kind": "port",
+            "sample": "%d of %d layers of the same padded batch timed (%.1f s), scaled to %d layers; "
+                      "fp32 PyTorch CPU restatement of the reference's encoder script"
+                      % (done, len(layers32), el, len(layers32)),
+            "tokens_per_s": round(wl.valid_tokens / (ms_full * 1e-3), 1)}
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build targets one GPU per process; --gpus %d is not supported "
+                 "(the path shards by batch with no collectives)" % args.gpus)
+    import numpy as np
+    import torch
+    import bytetransformer_amd as bt
+    from bytetransformer_amd import workload
+
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    dev = torch.device("cuda:0")
+    bt.load_th_op()
+    wl = workload.make_workload(args.workload)
+    cfg = wl.cfg
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+    layers = [[t(w[n]) for n in workload.WEIGHT_NAMES] for w in wl.layers]
+    x, mask = t(wl.x), t(wl.mask)
+    op = torch.ops.ByteTransformer.BertTransformer
+
+    def forward():
+        h = x
+        for w in layers:
+            h = op(cfg.head_num, cfg.head_size, *w, h, mask, True, True)
+        return h
+
+    for _ in range(args.warmup):
+        forward()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        forward()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) * 1e3 / args.steps
+
+    gemm_f, attn_f = workload.layer_flops(cfg, wl.lens)
+    kernels = kernel_table(wl, dev, args.kernel_iters)
+    dominant = max((k for k in kernels if kernels[k]["bound"] == "mfma"),
+                   key=lambda k: kernels[k]["us"])
+    d = kernels[dominant]
+    roofline = {"kernel": dominant, "bound": d["bound"], "achieved": d["achieved"],
+                "peak": d["peak"], "unit": d["unit"], "frac": d["frac"], "traffic": None,
+                "launch_us": d["us"]}
+    pub = PUBLISHED_A100_MS.get(args.workload)
+    line = {
+        "metric": "ms per %d-layer BERT fwd, bs%d, avg len 0.6*max (valid-token throughput alongside)"
+                  % (cfg.layers, cfg.batch),
+        "value": round(ms, 4), "unit": "ms", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(ms, 4), "higher_is_better": False,
+        "scaling": "weak", "vs_baseline": round(ms / pub, 4) if pub else None,
+        "dtype": "fp16", "data": "synthetic",
+        "config": {"workload": "%s: %d-layer encoder, hidden %d, heads %d, fp16, batch %d, max seq %d, "
+                               "lens uniform [%d, %d], %d valid tokens, via torch.ops per layer"
+                               % (cfg.name, cfg.layers, cfg.hidden, cfg.head_num, cfg.batch,
+                                  cfg.seq_len, int(wl.lens.min()), int(wl.lens.max()),
+                                  wl.valid_tokens),
+                   "valid_tokens": wl.valid_tokens, "lens": wl.lens.tolist()},
+        "tokens_per_s": round(wl.valid_tokens / (ms * 1e-3), 1),
+        "model_tflops": round(cfg.layers * (gemm_f + attn_f) / (ms * 1e-3) / 1e12, 2),
+        "roofline": roofline,
+        "kernels": kernels,
+    }
+    if not args.no_cpu_baseline:
+        line["cpu_baseline"] = cpu_baseline(wl)
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()
