@@ -107,8 +107,9 @@ def kernel_table(wl, dev, iters):
         ("layernorm_restore", lambda: ops.add_bias_residual_layernorm_restore(
             ffn2, proj, w["output_bias"], g1, b1, batch_idx, B, S, out_padded=out_pad),
          "hbm", 2 * M * H * 2 + T * H * 2),
-        ("transpose_weights", lambda: ops.transpose_weight(w["inter_kernel"]), "hbm",
-         2 * H * F * 2),
+        ("transpose_weights", lambda: ops.transpose_weights(
+            [w["qkv_kernel"], w["attr_output_kernel"], w["inter_kernel"], w["output_kernel"]]),
+         "hbm", 2 * (4 * H * H + 2 * H * F) * 2),
     ]
     table = {}
     for name, fn, bound, work in rows:

@@ -36,6 +36,8 @@ KERNEL_ABI = {
     "bt_build_offsets": (c_int, [_P, c_int, c_int, c_int, _IP, _IP, POINTER(c_int), _P]),
     "bt_compress": (c_int, [_P, _P, _IP, _IP, c_int, c_int, c_int, _P]),
     "bt_transpose_weight": (c_int, [_P, _P, c_int, c_int, _P]),
+    "bt_transpose_weights": (c_int, [c_int, POINTER(c_void_p), POINTER(c_void_p), POINTER(c_int),
+                                     POINTER(c_int), _P]),
     "bt_gemm": (c_int, [_P, _P, _P, _IP, c_int, c_int, c_int, _P]),
     "bt_gemm_bias_gelu": (c_int, [_P, _P, _P, _P, _IP, c_int, c_int, c_int, _P]),
     "bt_gemm_qkv_bias_split": (c_int, [_P, _P, _P, _P, _IP, c_int, c_int, c_int, _P]),

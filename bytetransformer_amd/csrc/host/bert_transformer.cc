@@ -73,11 +73,15 @@ void BertTransformer<OpType>::bert_infer(BertTransformerInferParam infer_param) 
     valid_rows = et_param.batch_idx + batch_size;
   }
 
-  // k-contiguous weight pre-pack
-  check_bt_error(bt_transpose_weight(param_.attr_kernel_QKV, wt_qkv, hidden, 3 * hidden, stream));
-  check_bt_error(bt_transpose_weight(param_.attr_output_kernel, wt_proj, hidden, hidden, stream));
-  check_bt_error(bt_transpose_weight(param_.inter_kernel, wt_inter, hidden, inter, stream));
-  check_bt_error(bt_transpose_weight(param_.output_kernel, wt_out, inter, hidden, stream));
+  // k-contiguous weight pre-pack, all four matrices in one launch
+  {
+    const void *src[4] = {param_.attr_kernel_QKV, param_.attr_output_kernel, param_.inter_kernel,
+                          param_.output_kernel};
+    void *dst[4] = {wt_qkv, wt_proj, wt_inter, wt_out};
+    const int ks[4] = {hidden, hidden, hidden, inter};
+    const int ns[4] = {3 * hidden, hidden, inter, hidden};
+    check_bt_error(bt_transpose_weights(4, src, dst, ks, ns, stream));
+  }
 
   check_bt_error(bt_gemm_qkv_bias_split(from_tensor, wt_qkv, param_.attention_param.attr_bias_QKV,
                                         qkv_buf, valid_rows, rows, head_num_, size_per_head_,

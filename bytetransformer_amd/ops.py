@@ -74,6 +74,20 @@ def transpose_weight(w):
     return wt
 
 
+def transpose_weights(ws):
+    """Pre-pack up to four [K, N] weights in one launch; returns the [N, K] copies."""
+    n = len(ws)
+    wts = [torch.empty(w.shape[1], w.shape[0], dtype=w.dtype, device=w.device) for w in ws]
+    src = (ctypes.c_void_p * n)(*[w.data_ptr() for w in ws])
+    dst = (ctypes.c_void_p * n)(*[w.data_ptr() for w in wts])
+    ks = (ctypes.c_int * n)(*[w.shape[0] for w in ws])
+    ns = (ctypes.c_int * n)(*[w.shape[1] for w in ws])
+    for w in ws:
+        _ptr(w)
+    _check(kernel_lib().bt_transpose_weights(n, src, dst, ks, ns, _stream()))
+    return wts
+
+
 def gemm(a, wt, valid_rows=None, out=None):
     rows, K = a.shape
     N = wt.shape[0]

@@ -44,7 +44,8 @@ const char *bt_last_error_string(void);
 
 /*
  * Tuning knob for experiments and tests; no counterpart in the reference.
- *   "gemm_tile"     -1 heuristic | 0: 256x256 | 1: 256x128 | 2: 128x128 workgroup tile
+ *   "gemm_tile"     -1 heuristic | 0: 256x256 tile, 8 waves | 1: 128x128, 2-stage ring |
+ *                   2: 128x128, 3-stage ring
  *   "attention_qb"  -1 heuristic | 1 | 2: 16-query blocks per wave in the grouped kernel
  * Process-wide; results do not depend on it beyond fp32 summation order.
  */
@@ -78,6 +79,11 @@ int bt_compress(const void *from_tensor, void *to_tensor, const int *batch_idx,
  * once per infer() into scratch.  k % 8 == 0, n % 8 == 0.
  */
 int bt_transpose_weight(const void *w, void *wt, int k, int n, void *stream);
+
+/* The same pre-pack for up to four matrices in ONE launch (a layer has four:
+ * QKV, attention output, FFN1, FFN2): wt[i][n, k] = w[i][k, n]. */
+int bt_transpose_weights(int count, const void *const *w, void *const *wt, const int *k,
+                         const int *n, void *stream);
 
 /*
  * c[rows, n] = a[rows, k] . w[k, n], fp16 in/out, fp32 accumulate on MFMA.

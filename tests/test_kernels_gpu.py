@@ -134,6 +134,16 @@ def test_transpose_weight_bit_exact(device, K, N):
     assert np.array_equal(wt.view(np.uint16), np.ascontiguousarray(w.T).view(np.uint16))
 
 
+def test_transpose_weights_fused_launch(device):
+    rs = np.random.RandomState(5)
+    shapes = [(768, 2304), (768, 768), (768, 3072), (3072, 768)]
+    ws = [rs.standard_normal(sh).astype(np.float16) for sh in shapes]
+    wts = ops.transpose_weights([_dev(w, device) for w in ws])
+    for w, wt in zip(ws, wts):
+        assert np.array_equal(wt.cpu().numpy().view(np.uint16),
+                              np.ascontiguousarray(w.T).view(np.uint16))
+
+
 # ---- GEMM family ---------------------------------------------------------------
 def _gemm_tol(exp, K, amax, wmax):
     # one fp16 rounding of the result plus fp32 accumulation noise
