@@ -5,30 +5,39 @@
 // Both kernels compute the logits TRANSPOSED, S^T = K.Q^T, so that the MFMA
 // accumulator of a 16-key block (lane = query, 4 consecutive keys per lane) is
 // already laid out as the "B" operand of the second product O^T = V^T.P^T: the
-// probabilities never leave registers.  V is staged into LDS transposed
-// ([d][key]) so the "A" operand of that product is two 8-byte LDS reads.
+// probabilities never leave registers.  K and V rows travel global -> LDS with
+// direct-to-LDS 16-byte loads (no staging registers) into XOR-swizzled
+// row-major tiles; the "A" operand of the second product, V^T, is fetched with
+// the LDS transpose read (ds_read_b64_tr_b16), so V is never transposed in
+// memory.
 //
-//   attention_short_kernel    whole K / V^T of the sequence resident in LDS,
+//   attention_short_kernel    whole K / V of the sequence resident in LDS,
 //                             all logits of a query tile in registers, exact
 //                             two-pass softmax: P = exp(s-max)/(sum+1e-6) is
 //                             rounded to fp16 before P.V exactly as
 //                             attention_fused.cu:348-381 does.
-//   attention_grouped_kernel  K / V streamed in 64-key tiles through an LDS
-//                             double buffer with an online softmax; handles
-//                             any length; the [S, S] logits never exist.
+//   attention_grouped_kernel  K / V streamed in 64-key tiles through a 3-stage
+//                             LDS ring with an online softmax; handles any
+//                             length; the [S, S] logits never exist.
 //
 // Keys at or past the sequence length are excluded by index (the mask tensor is
 // not read), the convention of the reference's remove-padding kernels
-// (attention_fused.cu:359, attention_fused_long.cu:254).
+// (attention_fused.cu:359, attention_fused_long.cu:254).  Tile rows past the
+// length are fetched from the last valid row (finite data, never out of
+// bounds) and their probabilities are forced to zero.
 #include "common.h"
+
+#include <type_traits>
 
 namespace bt {
 
 constexpr int kAttThreads = 256;
-constexpr int kKld = 72;   // K tile row stride (halfs): 64 + 8 pad
 constexpr int kHeadDim = 64;
 constexpr float kNegBig = -1.0e30f;
 constexpr float kLog2e = 1.4426950408889634f;
+
+typedef __fp16 fp16x4_t __attribute__((ext_vector_type(4)));
+typedef float float2_t __attribute__((ext_vector_type(2)));
 
 struct AttArgs {
   const half_t *qkv;   // [3][heads][rows_cap][64]
@@ -41,31 +50,56 @@ struct AttArgs {
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
-__device__ __forceinline__ uint4_t zero16() { return uint4_t{0u, 0u, 0u, 0u}; }
+// 16-byte chunk swizzles of a [rows][64] fp16 tile (8 chunks per 128-byte row).
+// K is read with ds_read_b128 by 16 consecutive rows at one chunk: slot =
+// chunk ^ (row>>1 & 7) spreads them over all 64 banks.  V is read with the
+// transpose read, 4 consecutive rows x 32 bytes per 16 lanes: slot =
+// chunk ^ 2*(row>>1 & 3) puts those four rows on distinct banks.
+__device__ __forceinline__ int swz_k(int row) { return (row >> 1) & 7; }
+__device__ __forceinline__ int swz_v(int row) { return ((row >> 1) & 3) << 1; }
 
-// Interleave two 8-half rows (keys 2p and 2p+1) into LDS as V^T[d][key pair].
-__device__ __forceinline__ void store_vt_pair(half_t *sVt, int vld, int d0, int key, uint4_t v0,
-                                              uint4_t v1) {
-  const unsigned short *a = (const unsigned short *)&v0;
-  const unsigned short *b = (const unsigned short *)&v1;
-#pragma unroll
-  for (int i = 0; i < 8; ++i) {
-    unsigned int w = (unsigned int)a[i] | ((unsigned int)b[i] << 16);
-    *(unsigned int *)(sVt + (d0 + i) * vld + key) = w;
-  }
+template <int N>
+__device__ __forceinline__ void att_wait_vmcnt() {
+  __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | 0x0F70);
+}
+
+__device__ __forceinline__ void lds_dma16(const half_t *src, half_t *dst) {
+  __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)src,
+                                   (__attribute__((address_space(3))) void *)dst, 16, 0, 0);
+}
+
+// V^T fragment for d-block db and key pair-block kk of a [keys][64] swizzled V
+// tile: 8 keys {32kk+4g+r, 32kk+16+4g+r} for d = 16db + (lane&15), g = lane>>4.
+__device__ __forceinline__ half8_t load_vt_frag(const half_t *sV, int kk, int db, int lq, int lg) {
+  const int row0 = 32 * kk + 4 * lg + (lq >> 2);
+  const int c = 2 * db + ((lq & 3) >> 1), sub = 4 * (lq & 1);
+  const half_t *p0 = sV + row0 * kHeadDim + ((c ^ swz_v(row0)) << 3) + sub;
+  const int row1 = row0 + 16;
+  const half_t *p1 = sV + row1 * kHeadDim + ((c ^ swz_v(row1)) << 3) + sub;
+  const fp16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4f16(
+      (__attribute__((address_space(3))) fp16x4_t *)p0);
+  const fp16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4f16(
+      (__attribute__((address_space(3))) fp16x4_t *)p1);
+  const half4_t l4 = __builtin_bit_cast(half4_t, lo), h4 = __builtin_bit_cast(half4_t, hi);
+  return half8_t{l4[0], l4[1], l4[2], l4[3], h4[0], h4[1], h4[2], h4[3]};
+}
+
+__device__ __forceinline__ half8_t load_k_frag(const half_t *sK, int kb, int dh, int lq, int lg) {
+  const int row = 16 * kb + lq;
+  return *(const half8_t *)(sK + row * kHeadDim + (((4 * dh + lg) ^ swz_k(row)) << 3));
 }
 
 // ---------------------------------------------------------------------------
 // grouped / streaming kernel
 // ---------------------------------------------------------------------------
-constexpr int kKT = 64;          // keys per streamed tile
-constexpr int kVldT = kKT + 4;   // V^T tile row stride (halfs), 136 B keeps 8-byte alignment
+constexpr int kKT = 64;                          // keys per streamed tile
+constexpr int kTileHalfs = kKT * kHeadDim;       // one K or V tile
+constexpr int kAttStages = 3;
 
 template <int QB>  // 16-query blocks per wave; workgroup covers 4*QB*16 queries
-__global__ __launch_bounds__(kAttThreads) void attention_grouped_kernel(AttArgs p) {
+__global__ __launch_bounds__(kAttThreads, 2) void attention_grouped_kernel(AttArgs p) {
   constexpr int BQ = 4 * QB * 16;
-  __shared__ __attribute__((aligned(16))) half_t sK[2][kKT * kKld];
-  __shared__ __attribute__((aligned(16))) half_t sVt[2][kHeadDim * kVldT];
+  __shared__ __attribute__((aligned(1024))) half_t ring[kAttStages * 2 * kTileHalfs];
 
   const int b = blockIdx.z, head = blockIdx.y;
   const int seq_start = p.batch_idx[b];
@@ -90,138 +124,161 @@ __global__ __launch_bounds__(kAttThreads) void attention_grouped_kernel(AttArgs 
     const int q = q0 + (wave * QB + qb) * 16 + lq;
 #pragma unroll
     for (int dh = 0; dh < 2; ++dh) {
-      uint4_t v = zero16();
+      uint4_t v = {0u, 0u, 0u, 0u};
       if (q < nq) v = *(const uint4_t *)(Q + (size_t)q * kHeadDim + 32 * dh + 8 * lg);
       qf[qb][dh] = __builtin_bit_cast(half8_t, v);
     }
   }
 
-  // staging registers: K 2 chunks/thread (row = tid/8 + 32*i, col = tid%8),
-  //                    V 2 chunks/thread (keys 2*kp, 2*kp+1 ; d chunk = tid%8)
-  const int k_row = tid >> 3, k_col = (tid & 7) * 8;
-  const int v_kp = tid >> 3, v_dc = (tid & 7) * 8;
-  uint4_t rk[2], rv[2];
-
-  auto load_tile = [&](int t) {
+  // Tile copy: 16 load instructions per tile (8 rows each; 0-7 = K, 8-15 = V),
+  // four per wave.  Lane -> (row, slot) and fetches the chunk the swizzle puts
+  // in that slot.
+  const int ld_row = lane >> 3, ld_slot = lane & 7;
+  auto issue_tile = [&](int t, int stage) {
+    half_t *sbase = ring + stage * 2 * kTileHalfs;
     const int k0 = t * kKT;
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
-      const int key = k0 + k_row + 32 * i;
-      rk[i] = key < klen ? *(const uint4_t *)(K + (size_t)key * kHeadDim + k_col) : zero16();
+    for (int i = 0; i < 4; ++i) {
+      const int id = i * 4 + wave;          // 0..15
+      const int row = (id & 7) * 8 + ld_row;
+      const int key = min(k0 + row, klen - 1);
+      if (id < 8)
+        lds_dma16(K + (size_t)key * kHeadDim + ((ld_slot ^ swz_k(row)) << 3),
+                  sbase + (id & 7) * 8 * kHeadDim);
+      else
+        lds_dma16(V + (size_t)key * kHeadDim + ((ld_slot ^ swz_v(row)) << 3),
+                  sbase + kTileHalfs + (id & 7) * 8 * kHeadDim);
     }
-#pragma unroll
-    for (int i = 0; i < 2; ++i) {
-      const int key = k0 + 2 * v_kp + i;
-      rv[i] = key < klen ? *(const uint4_t *)(V + (size_t)key * kHeadDim + v_dc) : zero16();
-    }
-  };
-  auto store_tile = [&](int buf) {
-#pragma unroll
-    for (int i = 0; i < 2; ++i)
-      *(uint4_t *)(&sK[buf][(k_row + 32 * i) * kKld + k_col]) = rk[i];
-    store_vt_pair(sVt[buf], kVldT, v_dc, 2 * v_kp, rv[0], rv[1]);
   };
 
-  float4_t o[4][QB];
-  float m_run[QB], l_run[QB];
+  // o[4] is a fifth "d block" fed with an all-ones V^T fragment: the MFMA then
+  // accumulates the row sums of the (fp16-rounded) probabilities, already
+  // reduced over the wave, in the same rescaled form as O.
+  float4_t o[5][QB];
+  float m_run[QB];
 #pragma unroll
   for (int qb = 0; qb < QB; ++qb) {
     m_run[qb] = kNegBig;
-    l_run[qb] = 0.f;
 #pragma unroll
-    for (int db = 0; db < 4; ++db) o[db][qb] = float4_t{0.f, 0.f, 0.f, 0.f};
+    for (int db = 0; db < 5; ++db) o[db][qb] = float4_t{0.f, 0.f, 0.f, 0.f};
   }
+  const half8_t ones = {1, 1, 1, 1, 1, 1, 1, 1};
 
   const int ntiles = (klen + kKT - 1) / kKT;
-  if (ntiles > 0) {
-    load_tile(0);
-    store_tile(0);
-  }
-  __syncthreads();
+  if (ntiles > 0) issue_tile(0, 0);
+  if (ntiles > 1) issue_tile(1, 1);
 
   const float c = p.scale_log2e;
-  for (int t = 0; t < ntiles; ++t) {
-    const int buf = t & 1;
-    if (t + 1 < ntiles) load_tile(t + 1);
+  int stage = 0;
+
+  auto process_tile = [&](int t, auto masked_tag) {
+    constexpr bool MASKED = decltype(masked_tag)::value;
+    // this wave's share of tile t has landed once only tile t+1's four loads are outstanding
+    if (t + 1 < ntiles)
+      att_wait_vmcnt<4>();
+    else
+      att_wait_vmcnt<0>();
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    if (t + 2 < ntiles) {
+      int ps = stage + 2;
+      if (ps >= kAttStages) ps -= kAttStages;
+      issue_tile(t + 2, ps);
+    }
+    const half_t *sK = ring + stage * 2 * kTileHalfs;
+    const half_t *sV = sK + kTileHalfs;
 
     // S^T = K . Q^T for this tile: 4 key blocks x QB query blocks
     float4_t s[4][QB];
+    const float4_t zero4 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int kb = 0; kb < 4; ++kb) {
+      const half8_t kf0 = load_k_frag(sK, kb, 0, lq, lg), kf1 = load_k_frag(sK, kb, 1, lq, lg);
 #pragma unroll
-      for (int qb = 0; qb < QB; ++qb) s[kb][qb] = float4_t{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-      for (int dh = 0; dh < 2; ++dh) {
-        const half8_t kf =
-            *(const half8_t *)(&sK[buf][(kb * 16 + lq) * kKld + 32 * dh + 8 * lg]);
-#pragma unroll
-        for (int qb = 0; qb < QB; ++qb)
-          s[kb][qb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kf, qf[qb][dh], s[kb][qb], 0, 0, 0);
+      for (int qb = 0; qb < QB; ++qb) {
+        s[kb][qb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kf0, qf[qb][0], zero4, 0, 0, 0);
+        s[kb][qb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kf1, qf[qb][1], s[kb][qb], 0, 0, 0);
       }
     }
-    const int k0 = t * kKT;
-    if (k0 + kKT > klen) {
+    if (MASKED) {
+      const int k0 = t * kKT;
 #pragma unroll
       for (int kb = 0; kb < 4; ++kb)
 #pragma unroll
-        for (int r = 0; r < 4; ++r)
-          if (k0 + kb * 16 + lg * 4 + r >= klen)
+        for (int r = 0; r < 4; ++r) {
+          const bool dead = k0 + kb * 16 + lg * 4 + r >= klen;
 #pragma unroll
-            for (int qb = 0; qb < QB; ++qb) s[kb][qb][r] = kNegBig;
+          for (int qb = 0; qb < QB; ++qb) s[kb][qb][r] = dead ? kNegBig : s[kb][qb][r];
+        }
     }
 
     half8_t pf[2][QB];
 #pragma unroll
     for (int qb = 0; qb < QB; ++qb) {
-      float mx = kNegBig;
+      float mx = fmaxf(s[0][qb][0], s[0][qb][1]);
+      mx = fmaxf(fmaxf(mx, s[0][qb][2]), s[0][qb][3]);
 #pragma unroll
-      for (int kb = 0; kb < 4; ++kb)
-#pragma unroll
-        for (int r = 0; r < 4; ++r) mx = fmaxf(mx, s[kb][qb][r]);
+      for (int kb = 1; kb < 4; ++kb) {
+        mx = fmaxf(fmaxf(mx, s[kb][qb][0]), s[kb][qb][1]);
+        mx = fmaxf(fmaxf(mx, s[kb][qb][2]), s[kb][qb][3]);
+      }
       mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
       mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
       const float m_new = fmaxf(m_run[qb], mx);
-      const float alpha = fast_exp2((m_run[qb] - m_new) * c);
+      const float mc = m_new * c;
+      // rescale the running output only when some query's maximum moved
+      if (__builtin_amdgcn_ballot_w64(m_new != m_run[qb]) != 0) {
+        const float alpha = fast_exp2(m_run[qb] * c - mc);
+#pragma unroll
+        for (int db = 0; db < 5; ++db) o[db][qb] *= alpha;
+      }
       m_run[qb] = m_new;
-      float psum = 0.f;
 #pragma unroll
-      for (int kb = 0; kb < 4; ++kb)
+      for (int kb = 0; kb < 4; ++kb) {
+        float e[4];
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          const float e = fast_exp2((s[kb][qb][r] - m_new) * c);
-          psum += e;
-          pf[kb >> 1][qb][(kb & 1) * 4 + r] = (half_t)e;
-        }
-      l_run[qb] = l_run[qb] * alpha + psum;
-#pragma unroll
-      for (int db = 0; db < 4; ++db) o[db][qb] *= alpha;
+        for (int r = 0; r < 4; ++r) e[r] = fast_exp2(__builtin_fmaf(s[kb][qb][r], c, -mc));
+        const half2_t h01 = __builtin_convertvector(float2_t{e[0], e[1]}, half2_t);
+        const half2_t h23 = __builtin_convertvector(float2_t{e[2], e[3]}, half2_t);
+        pf[kb >> 1][qb][(kb & 1) * 4 + 0] = h01[0];
+        pf[kb >> 1][qb][(kb & 1) * 4 + 1] = h01[1];
+        pf[kb >> 1][qb][(kb & 1) * 4 + 2] = h23[0];
+        pf[kb >> 1][qb][(kb & 1) * 4 + 3] = h23[1];
+      }
     }
 
     // O^T += V^T . P^T ; k-slot (lg, s) <-> key 32*kk + 16*(s>>2) + 4*lg + (s&3)
 #pragma unroll
-    for (int kk = 0; kk < 2; ++kk)
+    for (int kk = 0; kk < 2; ++kk) {
 #pragma unroll
       for (int db = 0; db < 4; ++db) {
-        const half_t *vp = &sVt[buf][(db * 16 + lq) * kVldT + 32 * kk + 4 * lg];
-        const half4_t v0 = *(const half4_t *)vp, v1 = *(const half4_t *)(vp + 16);
-        const half8_t vf = {v0[0], v0[1], v0[2], v0[3], v1[0], v1[1], v1[2], v1[3]};
+        const half8_t vf = load_vt_frag(sV, kk, db, lq, lg);
 #pragma unroll
         for (int qb = 0; qb < QB; ++qb)
           o[db][qb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vf, pf[kk][qb], o[db][qb], 0, 0, 0);
       }
+#pragma unroll
+      for (int qb = 0; qb < QB; ++qb)
+        o[4][qb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ones, pf[kk][qb], o[4][qb], 0, 0, 0);
+    }
+    if (++stage == kAttStages) stage = 0;
+  };
 
-    if (t + 1 < ntiles) store_tile(buf ^ 1);
-    __syncthreads();
+  // every tile but the last is full: no masking code on the steady-state path
+  for (int t = 0; t + 1 < ntiles; ++t) process_tile(t, std::false_type{});
+  if (ntiles > 0) {
+    if (klen % kKT == 0)
+      process_tile(ntiles - 1, std::false_type{});
+    else
+      process_tile(ntiles - 1, std::true_type{});
   }
 
   // O / (l + 1e-6) -> fp16, token-major [row][head*64 + d]
   const int H = p.heads * kHeadDim;
 #pragma unroll
   for (int qb = 0; qb < QB; ++qb) {
-    float l = l_run[qb];
-    l += __shfl_xor(l, 16, 64);
-    l += __shfl_xor(l, 32, 64);
-    const float inv = 1.0f / (l + 1e-6f);
+    const float inv = 1.0f / (o[4][qb][0] + 1e-6f);
     const int q = q0 + (wave * QB + qb) * 16 + lq;
     if (q >= nq) continue;
     half_t *dst = p.out + (size_t)(row_start + q) * H + head * kHeadDim + 4 * lg;
@@ -234,16 +291,15 @@ __global__ __launch_bounds__(kAttThreads) void attention_grouped_kernel(AttArgs 
 }
 
 // ---------------------------------------------------------------------------
-// short kernel: K, V^T resident in LDS, logits of the query tile in registers
+// short kernel: K, V resident in LDS, logits of the query tile in registers
 // ---------------------------------------------------------------------------
 template <int NKB>  // capacity in 16-key blocks (keys <= 16*NKB), NKB even
 __global__ __launch_bounds__(kAttThreads) void attention_short_kernel(AttArgs p) {
   constexpr int KEYS = NKB * 16;
-  constexpr int VLD = KEYS + 4;
   constexpr int BQ = 64;  // 4 waves x 16 queries
-  extern __shared__ __attribute__((aligned(16))) half_t smem[];
-  half_t *sK = smem;                  // [KEYS][kKld]
-  half_t *sVt = smem + KEYS * kKld;   // [64][VLD]
+  extern __shared__ __attribute__((aligned(1024))) half_t att_smem[];
+  half_t *sK = att_smem;                      // [KEYS][64] swizzled
+  half_t *sV = att_smem + KEYS * kHeadDim;    // [KEYS][64] swizzled
 
   const int b = blockIdx.z, head = blockIdx.y;
   const int seq_start = p.batch_idx[b];
@@ -256,7 +312,6 @@ __global__ __launch_bounds__(kAttThreads) void attention_short_kernel(AttArgs p)
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int lq = lane & 15, lg = lane >> 4;
   const int H = p.heads * kHeadDim;
-  half_t *dst_row = nullptr;
   const int q = q0 + wave * 16 + lq;
 
   const size_t head_stride = (size_t)p.rows_cap * kHeadDim;
@@ -264,28 +319,28 @@ __global__ __launch_bounds__(kAttThreads) void attention_short_kernel(AttArgs p)
   const half_t *K = Q + (size_t)p.heads * head_stride;
   const half_t *V = K + (size_t)p.heads * head_stride;
 
+  // copy K and V rows [0, keys32) into LDS, 8 rows per wave instruction
+  const int keys32 = min(((klen + 31) >> 5) << 5, KEYS);
+  if (klen > 0) {
+    const int ld_row = lane >> 3, ld_slot = lane & 7;
+    for (int g8 = wave; g8 < keys32 / 8; g8 += 4) {
+      const int row = g8 * 8 + ld_row;
+      const int key = min(row, klen - 1);
+      lds_dma16(K + (size_t)key * kHeadDim + ((ld_slot ^ swz_k(row)) << 3),
+                sK + g8 * 8 * kHeadDim);
+      lds_dma16(V + (size_t)key * kHeadDim + ((ld_slot ^ swz_v(row)) << 3),
+                sV + g8 * 8 * kHeadDim);
+    }
+  }
   half8_t qf[2];
 #pragma unroll
   for (int dh = 0; dh < 2; ++dh) {
-    uint4_t v = zero16();
+    uint4_t v = {0u, 0u, 0u, 0u};
     if (q < nq) v = *(const uint4_t *)(Q + (size_t)q * kHeadDim + 32 * dh + 8 * lg);
     qf[dh] = __builtin_bit_cast(half8_t, v);
   }
-
-  // stage K rows and V^T columns for keys [0, keys32), zero past klen
-  const int keys32 = min(((klen + 31) >> 5) << 5, KEYS);
-  const int col = (tid & 7) * 8;
-  for (int key = tid >> 3; key < keys32; key += 32) {
-    uint4_t v = key < klen ? *(const uint4_t *)(K + (size_t)key * kHeadDim + col) : zero16();
-    *(uint4_t *)(sK + key * kKld + col) = v;
-  }
-  for (int kp = tid >> 3; kp < keys32 / 2; kp += 32) {
-    const int key = 2 * kp;
-    uint4_t v0 = key < klen ? *(const uint4_t *)(V + (size_t)key * kHeadDim + col) : zero16();
-    uint4_t v1 =
-        key + 1 < klen ? *(const uint4_t *)(V + (size_t)(key + 1) * kHeadDim + col) : zero16();
-    store_vt_pair(sVt, VLD, col, key, v0, v1);
-  }
+  att_wait_vmcnt<0>();
+  asm volatile("" ::: "memory");
   __syncthreads();
 
   const int nkb = keys32 >> 4;  // even
@@ -295,10 +350,9 @@ __global__ __launch_bounds__(kAttThreads) void attention_short_kernel(AttArgs p)
     s[kb] = float4_t{0.f, 0.f, 0.f, 0.f};
     if (kb < nkb) {
 #pragma unroll
-      for (int dh = 0; dh < 2; ++dh) {
-        const half8_t kf = *(const half8_t *)(sK + (kb * 16 + lq) * kKld + 32 * dh + 8 * lg);
-        s[kb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kf, qf[dh], s[kb], 0, 0, 0);
-      }
+      for (int dh = 0; dh < 2; ++dh)
+        s[kb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(load_k_frag(sK, kb, dh, lq, lg), qf[dh],
+                                                       s[kb], 0, 0, 0);
     }
   }
 
@@ -314,12 +368,13 @@ __global__ __launch_bounds__(kAttThreads) void attention_short_kernel(AttArgs p)
   mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
   mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
   const float c = p.scale_log2e;
+  const float mc = mx * c;
   float sum = 0.f;
 #pragma unroll
   for (int kb = 0; kb < NKB; ++kb)
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
-      s[kb][r] = fast_exp2((s[kb][r] - mx) * c);
+      s[kb][r] = fast_exp2(__builtin_fmaf(s[kb][r], c, -mc));
       sum += s[kb][r];
     }
   sum += __shfl_xor(sum, 16, 64);
@@ -339,17 +394,14 @@ __global__ __launch_bounds__(kAttThreads) void attention_short_kernel(AttArgs p)
         pf[4 + r] = (half_t)(s[2 * kk + 1][r] * inv);
       }
 #pragma unroll
-      for (int db = 0; db < 4; ++db) {
-        const half_t *vp = sVt + (db * 16 + lq) * VLD + 32 * kk + 4 * lg;
-        const half4_t v0 = *(const half4_t *)vp, v1 = *(const half4_t *)(vp + 16);
-        const half8_t vf = {v0[0], v0[1], v0[2], v0[3], v1[0], v1[1], v1[2], v1[3]};
-        o[db] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vf, pf, o[db], 0, 0, 0);
-      }
+      for (int db = 0; db < 4; ++db)
+        o[db] = __builtin_amdgcn_mfma_f32_16x16x32_f16(load_vt_frag(sV, kk, db, lq, lg), pf, o[db],
+                                                       0, 0, 0);
     }
   }
 
   if (q < nq) {
-    dst_row = p.out + (size_t)(row_start + q) * H + head * kHeadDim + 4 * lg;
+    half_t *dst_row = p.out + (size_t)(row_start + q) * H + head * kHeadDim + 4 * lg;
 #pragma unroll
     for (int db = 0; db < 4; ++db)
       *(half4_t *)(dst_row + 16 * db) =
@@ -371,7 +423,8 @@ static int check_att_args(const char *who, const void *qkv, const void *out, con
 
 template <int NKB>
 static int launch_short(const AttArgs &a, hipStream_t s) {
-  constexpr size_t smem = ((size_t)NKB * 16 * kKld + (size_t)kHeadDim * (NKB * 16 + 4)) * 2;
+  constexpr size_t smem = (size_t)2 * NKB * 16 * kHeadDim * sizeof(half_t);
+  static_assert(smem <= 160 * 1024, "LDS budget");
   static bool configured = false;
   if (!configured) {
     hipError_t e = hipFuncSetAttribute((const void *)attention_short_kernel<NKB>,
