@@ -111,6 +111,16 @@ def kernel_table(wl, dev, iters):
             [w["qkv_kernel"], w["attr_output_kernel"], w["inter_kernel"], w["output_kernel"]]),
          "hbm", 2 * (4 * H * H + 2 * H * F) * 2),
     ]
+    # plain device copy of known size: the reference dispatch that the rocprofv3
+    # FETCH_SIZE / WRITE_SIZE counters are scaled by
+    # (the row gather on an all-valid [64, 256, 2048] batch: a 64 MiB copy)
+    cB, cS, cH = 64, 256, 2048
+    calib_src = torch.empty(cB, cS, cH, dtype=torch.float16, device=dev).normal_()
+    calib_dst = torch.empty(cB * cS, cH, dtype=torch.float16, device=dev)
+    c_bi, c_wi, _ = ops.build_offsets(torch.ones(cB, cS, cS, dtype=torch.float16, device=dev))
+    rows.append(("copy_calibration_64MiB",
+                 lambda: ops.compress(calib_src, c_bi, c_wi, out=calib_dst), "hbm",
+                 2 * calib_src.numel() * 2))
     table = {}
     for name, fn, bound, work in rows:
         ms = time_kernel(fn, iters)
@@ -121,6 +131,18 @@ def kernel_table(wl, dev, iters):
         table[name] = {"us": round(ms * 1e3, 2), "bound": bound, "achieved": round(ach, 2),
                        "peak": peak, "unit": unit, "frac": round(ach / peak, 4)}
     return table
+
+
+def measured_traffic(workload_name, kernel):
+    """HBM bytes per launch of `kernel` from the committed rocprofv3 --pmc runs
+    (profiles/traffic.json: FETCH_SIZE and WRITE_SIZE, each scaled by what the same
+    counter reads for the 64 MiB calibration copy); None when not recorded."""
+    path = os.path.join(ROOT, "profiles", "traffic.json")
+    try:
+        with open(path) as f:
+            return json.load(f)[workload_name][kernel]["hbm_bytes_per_launch"]
+    except (OSError, KeyError, ValueError):
+        return None
 
 
 def cpu_baseline(wl, budget_s=25.0):
@@ -194,8 +216,8 @@ def main():
                    key=lambda k: kernels[k]["us"])
     d = kernels[dominant]
     roofline = {"kernel": dominant, "bound": d["bound"], "achieved": d["achieved"],
-                "peak": d["peak"], "unit": d["unit"], "frac": d["frac"], "traffic": None,
-                "launch_us": d["us"]}
+                "peak": d["peak"], "unit": d["unit"], "frac": d["frac"],
+                "traffic": measured_traffic(args.workload, dominant), "launch_us": d["us"]}
     pub = PUBLISHED_A100_MS.get(args.workload)
     line = {
         "metric": "ms per %d-layer BERT fwd, bs%d, avg len 0.6*max (valid-token throughput alongside)"

@@ -295,9 +295,10 @@ static int launch_gemm_tile(GemmArgs p, hipStream_t s) {
 template <int EPI>
 static int launch_gemm(GemmArgs p, hipStream_t s) {
   // 256x256 tiles (8 waves) when the output is wide enough to give every CU a
-  // tile, else 128x128 (4 waves, two workgroups per CU).
+  // tile, else 128x128 (4 waves, two workgroups per CU), with a deeper ring
+  // when the k loop is long.
   int choice = option_gemm_tile();
-  if (choice < 0) choice = (p.N >= 3072 && p.rows_cap >= 2048) ? 0 : 1;
+  if (choice < 0) choice = (p.N >= 3072 && p.rows_cap >= 2048) ? 0 : (p.K >= 2048 ? 2 : 1);
   switch (choice) {
     case 0:
       return launch_gemm_tile<256, 256, 2, 2, 4, EPI>(p, s);
