@@ -62,7 +62,7 @@ __device__ __forceinline__ void wait_vmcnt() {
   __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | 0x0F70);
 }
 
-template <int BM, int BN, int STAGES, int WM, int WN, int EPI>
+template <int BM, int BN, int STAGES, int WM, int WN, int SCHED, int EPI>
 __global__ __launch_bounds__(WM *WN * 64) void gemm_kernel(GemmArgs p) {
   constexpr int NW = WM * WN;
   constexpr int WTM = BM / WM, WTN = BN / WN;   // wave tile
@@ -161,6 +161,9 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_kernel(GemmArgs p) {
       }
     };
     load_frags(0, 0);
+    // compiler scheduling strategy that interleaves the LDS reads with the MFMAs
+    if (SCHED == 0) __builtin_amdgcn_iglp_opt(0);
+    if (SCHED == 1) __builtin_amdgcn_iglp_opt(1);
 #pragma unroll
     for (int ks = 0; ks < kBK / 16; ++ks) {
       if (ks + 1 < kBK / 16) load_frags(ks + 1, (ks + 1) & 1);
@@ -214,6 +217,7 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_kernel(GemmArgs p) {
 #pragma unroll
     for (int r0 = 0; r0 < 32; r0 += RPS) {
       const int r = r0 + sr;
+      if (sr >= RPS || r >= 32) continue;   // lanes left over when 64 % CPRW != 0
       const int m = m0 + wm * WTM + j * 32 + r, n = n0 + wn * WTN + sc;
       const uint4_t v = *(const uint4_t *)(st + r * EP + sc);
       if (m < M && n < p.N) {
@@ -273,13 +277,13 @@ __global__ __launch_bounds__(256) void transpose_kernel(TransposeArgs a) {
   }
 }
 
-template <int BM, int BN, int STAGES, int WM, int WN, int EPI>
+template <int BM, int BN, int STAGES, int WM, int WN, int SCHED, int EPI>
 static int launch_gemm_tile(GemmArgs p, hipStream_t s) {
   constexpr size_t smem = (size_t)STAGES * (BM + BN) * kBK * sizeof(half_t);
   static_assert(smem <= 160 * 1024, "LDS budget");
   static bool configured = false;  // benign race: setting the attribute is idempotent
   if (!configured) {
-    hipError_t e = hipFuncSetAttribute((const void *)gemm_kernel<BM, BN, STAGES, WM, WN, EPI>,
+    hipError_t e = hipFuncSetAttribute((const void *)gemm_kernel<BM, BN, STAGES, WM, WN, SCHED, EPI>,
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
     if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute(gemm_kernel)");
     configured = true;
@@ -287,25 +291,37 @@ static int launch_gemm_tile(GemmArgs p, hipStream_t s) {
   const int tiles_m = (p.rows_cap + BM - 1) / BM;
   p.tiles_n = (p.N + BN - 1) / BN;
   const int grid = (tiles_m * p.tiles_n + 7) / 8 * 8;
-  gemm_kernel<BM, BN, STAGES, WM, WN, EPI><<<grid, WM * WN * 64, smem, s>>>(p);
+  gemm_kernel<BM, BN, STAGES, WM, WN, SCHED, EPI><<<grid, WM * WN * 64, smem, s>>>(p);
   BT_CHECK_LAUNCH("gemm_kernel");
   return BT_OK;
 }
 
 template <int EPI>
 static int launch_gemm(GemmArgs p, hipStream_t s) {
-  // 256x256 tiles (8 waves) when the output is wide enough to give every CU a
-  // tile, else 128x128 (4 waves, two workgroups per CU), with a deeper ring
-  // when the k loop is long.
+  // Tile table (rows x cols, ring depth, wave grid):
+  //   0: 256x256, 2, 2x4   wide outputs (FFN1): one tile per CU
+  //   1: 128x128, 2, 2x2   narrow outputs, short k loop (projection)
+  //   2: 128x128, 3, 4x2   narrow outputs, long k loop (FFN2)
+  //   3: 256x192, 2, 4x2   outputs that split into 192-wide panels but not into a
+  //                        full wave of 256-wide ones (QKV at hidden 768)
   int choice = option_gemm_tile();
-  if (choice < 0) choice = (p.N >= 3072 && p.rows_cap >= 2048) ? 0 : (p.K >= 2048 ? 2 : 1);
+  if (choice < 0) {
+    if (p.N >= 3072 && p.N % 256 == 0 && p.rows_cap >= 2048)
+      choice = 0;
+    else if (p.N >= 1536 && p.N % 192 == 0 && p.rows_cap >= 2048)
+      choice = 3;
+    else
+      choice = p.K >= 2048 ? 2 : 1;
+  }
   switch (choice) {
     case 0:
-      return launch_gemm_tile<256, 256, 2, 2, 4, EPI>(p, s);
+      return launch_gemm_tile<256, 256, 2, 2, 4, 1, EPI>(p, s);
     case 2:
-      return launch_gemm_tile<128, 128, 3, 2, 2, EPI>(p, s);
+      return launch_gemm_tile<128, 128, 3, 4, 2, 1, EPI>(p, s);
+    case 3:
+      return launch_gemm_tile<256, 192, 2, 4, 2, 1, EPI>(p, s);
     default:
-      return launch_gemm_tile<128, 128, 2, 2, 2, EPI>(p, s);
+      return launch_gemm_tile<128, 128, 2, 2, 2, 0, EPI>(p, s);
   }
 }
 

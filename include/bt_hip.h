@@ -44,8 +44,8 @@ const char *bt_last_error_string(void);
 
 /*
  * Tuning knob for experiments and tests; no counterpart in the reference.
- *   "gemm_tile"     -1 heuristic | 0: 256x256 tile, 8 waves | 1: 128x128, 2-stage ring |
- *                   2: 128x128, 3-stage ring
+ *   "gemm_tile"     -1 heuristic | 0: 256x256 tile, 8 waves | 1: 128x128, 4 waves, 2-stage ring |
+ *                   2: 128x128, 8 waves, 3-stage ring | 3: 256x192, 8 waves
  *   "attention_qb"  -1 heuristic | 1 | 2: 16-query blocks per wave in the grouped kernel
  * Process-wide; results do not depend on it beyond fp32 summation order.
  */
