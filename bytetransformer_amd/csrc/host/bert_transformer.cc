@@ -28,9 +28,6 @@ void BertTransformer<OpType>::bert_infer(BertTransformerInferParam infer_param) 
         "[BT][ERROR] BertTransformer: batch_size/seq_len outside the constructed maximum");
   if (infer_param.attention_bias != nullptr)
     throw std::runtime_error("[BT][ERROR] BertTransformer: attention_bias is not supported");
-  if (from_tensor == transformer_out && is_remove_padding_)
-    throw std::runtime_error(
-        "[BT][ERROR] BertTransformer: transformer_output must not alias input_tensor");
 
   const int hidden = head_num_ * size_per_head_;
   const int inter = hidden * param_.intermediate_size;
@@ -62,12 +59,13 @@ void BertTransformer<OpType>::bert_infer(BertTransformerInferParam infer_param) 
   check_bt_error(bt_build_offsets(atten_mask, Traits_::dtype, batch_size, seq_len,
                                   et_param.batch_idx, et_param.word_idx, nullptr, stream));
   const int *valid_rows = nullptr;
+  const int *gather = nullptr;
   DataType_ *restore_target = nullptr;
   if (is_remove_padding_) {
-    // packed x lives in the caller's output buffer until the final restore
-    check_bt_error(bt_compress(from_tensor, transformer_out, et_param.batch_idx,
-                               et_param.word_idx, batch_size, seq_len, hidden, stream));
-    from_tensor = transformer_out;
+    // The packed copy of the input is never materialised: the QKV GEMM and the
+    // first LayerNorm read valid token t from the padded input at row word_idx[t]
+    // (the compress step of bert_transformer.cu:68-78 folded into its consumers).
+    gather = et_param.word_idx;
     restore_target = transformer_out;
     transformer_out = inner_buf;  // FFN2 output reuses the dead qkv region
     valid_rows = et_param.batch_idx + batch_size;
@@ -83,9 +81,9 @@ void BertTransformer<OpType>::bert_infer(BertTransformerInferParam infer_param) 
     check_bt_error(bt_transpose_weights(4, src, dst, ks, ns, stream));
   }
 
-  check_bt_error(bt_gemm_qkv_bias_split(from_tensor, wt_qkv, param_.attention_param.attr_bias_QKV,
-                                        qkv_buf, valid_rows, rows, head_num_, size_per_head_,
-                                        stream));
+  check_bt_error(bt_gemm_qkv_bias_split(from_tensor, gather, wt_qkv,
+                                        param_.attention_param.attr_bias_QKV, qkv_buf, valid_rows,
+                                        rows, head_num_, size_per_head_, stream));
 
   struct AttentionInferParam<DataType_> attention_infer_param {
     qkv_buf, atten_mask, attr_out_buf, base + inner_buf_size_, batch_size, seq_len,
@@ -98,7 +96,7 @@ void BertTransformer<OpType>::bert_infer(BertTransformerInferParam infer_param) 
       bt_gemm(attr_out_buf, wt_proj, attr_matmul_buf, valid_rows, rows, hidden, hidden, stream));
 
   check_bt_error(bt_add_bias_residual_layernorm(
-      attr_matmul_buf, from_tensor, param_.attr_output_bias, param_.attr_output_layernorm_gamma,
+      attr_matmul_buf, from_tensor, gather, param_.attr_output_bias, param_.attr_output_layernorm_gamma,
       param_.attr_output_layernorm_beta, use_fp32_ ? 1 : 0, valid_rows, rows, hidden,
       layernorm_eps, stream));
 
@@ -115,7 +113,7 @@ void BertTransformer<OpType>::bert_infer(BertTransformerInferParam infer_param) 
         batch_size, seq_len, hidden, layernorm_eps, stream));
   else
     check_bt_error(bt_add_bias_residual_layernorm(
-        transformer_out, attr_matmul_buf, param_.output_bias, param_.output_layernorm_gamma,
+        transformer_out, attr_matmul_buf, nullptr, param_.output_bias, param_.output_layernorm_gamma,
         param_.output_layernorm_beta, use_fp32_ ? 1 : 0, nullptr, rows, hidden, layernorm_eps,
         stream));
 }

@@ -40,6 +40,7 @@ struct GemmArgs {
   const half_t *bias;   // [N] or null
   half_t *c;            // [rows_cap, N]  (or [3][heads][rows_cap][64] for the QKV split)
   const int *valid_rows;
+  const int *a_row_index;   // optional gather: A row r is a[a_row_index[r]] (null = identity)
   int rows_cap, N, K;
   int tiles_n;
 };
@@ -100,9 +101,11 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_kernel(GemmArgs p) {
   for (int i = 0; i < NI; ++i) {
     const int r = (i * NW + wave) * 8 + (lane >> 3);
     const int kc = (lane & 7) ^ swz(r);
-    if (r < BM)
-      gsrc[i] = p.a + (size_t)min(m0 + r, p.rows_cap - 1) * p.K + kc * 8;
-    else
+    if (r < BM) {
+      int ar = min(m0 + r, p.rows_cap - 1);
+      if (p.a_row_index) ar = p.a_row_index[min(ar, M - 1)];   // live rows only hold valid indices
+      gsrc[i] = p.a + (size_t)ar * p.K + kc * 8;
+    } else
       gsrc[i] = p.wt + (size_t)min(n0 + r - BM, p.N - 1) * p.K + kc * 8;
   }
   auto issue_loads = [&](int kt, int stage) {
@@ -374,7 +377,7 @@ extern "C" int bt_gemm(const void *a, const void *wt, void *c, const int *valid_
   int rc = check_gemm_args("bt_gemm", a, wt, c, rows_cap, n, k);
   if (rc) return rc;
   if (rows_cap == 0) return BT_OK;
-  GemmArgs p{(const half_t *)a, (const half_t *)wt, nullptr, (half_t *)c, valid_rows,
+  GemmArgs p{(const half_t *)a, (const half_t *)wt, nullptr, (half_t *)c, valid_rows, nullptr,
              rows_cap,          n,                  k,       0};
   return launch_gemm<kEpiPlain>(p, as_stream(stream));
 }
@@ -387,13 +390,14 @@ extern "C" int bt_gemm_bias_gelu(const void *a, const void *wt, const void *bias
   BT_REQUIRE(bias, BT_ERR_INVALID_ARGUMENT, "bt_gemm_bias_gelu: null bias");
   if (rows_cap == 0) return BT_OK;
   GemmArgs p{(const half_t *)a, (const half_t *)wt, (const half_t *)bias, (half_t *)c, valid_rows,
-             rows_cap,          n,                  k,                    0};
+             nullptr,           rows_cap,           n,                    k,           0};
   return launch_gemm<kEpiBiasGelu>(p, as_stream(stream));
 }
 
-extern "C" int bt_gemm_qkv_bias_split(const void *a, const void *wt_qkv, const void *bias_qkv,
-                                      void *qkv_heads, const int *valid_rows, int rows_cap,
-                                      int head_num, int size_per_head, void *stream) {
+extern "C" int bt_gemm_qkv_bias_split(const void *a, const int *a_row_index, const void *wt_qkv,
+                                      const void *bias_qkv, void *qkv_heads,
+                                      const int *valid_rows, int rows_cap, int head_num,
+                                      int size_per_head, void *stream) {
   BT_REQUIRE(head_num > 0, BT_ERR_INVALID_ARGUMENT, "bt_gemm_qkv_bias_split: head_num=%d",
              head_num);
   BT_REQUIRE(size_per_head == 64, BT_ERR_UNSUPPORTED,
@@ -403,7 +407,9 @@ extern "C" int bt_gemm_qkv_bias_split(const void *a, const void *wt_qkv, const v
   if (rc) return rc;
   BT_REQUIRE(bias_qkv, BT_ERR_INVALID_ARGUMENT, "bt_gemm_qkv_bias_split: null bias");
   if (rows_cap == 0) return BT_OK;
+  BT_REQUIRE(!a_row_index || valid_rows, BT_ERR_INVALID_ARGUMENT,
+             "bt_gemm_qkv_bias_split: a_row_index needs valid_rows (only live rows are indexed)");
   GemmArgs p{(const half_t *)a, (const half_t *)wt_qkv, (const half_t *)bias_qkv,
-             (half_t *)qkv_heads, valid_rows, rows_cap, 3 * H, H, 0};
+             (half_t *)qkv_heads, valid_rows, a_row_index, rows_cap, 3 * H, H, 0};
   return launch_gemm<kEpiQkvSplit>(p, as_stream(stream));
 }

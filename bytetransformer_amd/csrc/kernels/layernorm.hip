@@ -17,7 +17,8 @@ __global__ __launch_bounds__(kLnRowsPerBlock *kWave) void layernorm_kernel(
     const half8_t *src, const half8_t *__restrict__ residual,
     const half8_t *__restrict__ bias, const void *__restrict__ gamma,
     const void *__restrict__ beta, half8_t *dst, const int *__restrict__ idx,
-    int B, int S, int rows_cap, int chunks, float inv_n, float eps) {
+    const int *__restrict__ residual_row_index, int B, int S, int rows_cap, int chunks,
+    float inv_n, float eps) {
   const int r = blockIdx.x * kLnRowsPerBlock + (threadIdx.x >> 6);
   const int lane = threadIdx.x & 63;
   if (r >= rows_cap) return;
@@ -41,7 +42,8 @@ __global__ __launch_bounds__(kLnRowsPerBlock *kWave) void layernorm_kernel(
   }
 
   const half8_t *a = src + src_row * chunks;
-  const half8_t *b = residual + src_row * chunks;
+  const size_t res_row = residual_row_index ? (size_t)residual_row_index[src_row] : src_row;
+  const half8_t *b = residual + res_row * chunks;
   float v[NC][8];
   float sum = 0.f;
 #pragma unroll
@@ -109,8 +111,9 @@ __global__ __launch_bounds__(kLnRowsPerBlock *kWave) void layernorm_kernel(
 
 template <bool RESTORE>
 static int launch_ln(const void *src, const void *residual, const void *bias, const void *gamma,
-                     const void *beta, int gb32, void *dst, const int *idx, int B, int S,
-                     int rows_cap, int H, float eps, hipStream_t s, const char *who) {
+                     const void *beta, int gb32, void *dst, const int *idx,
+                     const int *residual_row_index, int B, int S, int rows_cap, int H, float eps,
+                     hipStream_t s, const char *who) {
   BT_REQUIRE(H > 0 && H % 8 == 0, BT_ERR_UNSUPPORTED, "%s: hidden_dim %d must be a multiple of 8",
              who, H);
   const int chunks = H / 8;
@@ -122,7 +125,7 @@ static int launch_ln(const void *src, const void *residual, const void *bias, co
 #define BT_LN_LAUNCH(NC_, GB_)                                                                  \
   layernorm_kernel<NC_, RESTORE, GB_><<<grid, kLnRowsPerBlock * kWave, 0, s>>>(                 \
       (const half8_t *)src, (const half8_t *)residual, (const half8_t *)bias, gamma, beta,      \
-      (half8_t *)dst, idx, B, S, rows_cap, chunks, inv_n, eps)
+      (half8_t *)dst, idx, residual_row_index, B, S, rows_cap, chunks, inv_n, eps)
 #define BT_LN_NC(NC_)              \
   do {                             \
     if (gb32)                      \
@@ -148,7 +151,8 @@ static int launch_ln(const void *src, const void *residual, const void *bias, co
 
 using namespace bt;
 
-extern "C" int bt_add_bias_residual_layernorm(void *out, const void *residual, const void *bias,
+extern "C" int bt_add_bias_residual_layernorm(void *out, const void *residual,
+                                              const int *residual_row_index, const void *bias,
                                               const void *gamma, const void *beta,
                                               int gamma_beta_fp32, const int *valid_rows,
                                               int rows_cap, int hidden_dim, float eps,
@@ -157,8 +161,10 @@ extern "C" int bt_add_bias_residual_layernorm(void *out, const void *residual, c
              "bt_add_bias_residual_layernorm: null pointer argument");
   BT_REQUIRE(rows_cap >= 0, BT_ERR_INVALID_ARGUMENT,
              "bt_add_bias_residual_layernorm: negative rows_cap");
-  return launch_ln<false>(out, residual, bias, gamma, beta, gamma_beta_fp32, out, valid_rows, 0,
-                          1, rows_cap, hidden_dim, eps, as_stream(stream),
+  BT_REQUIRE(!residual_row_index || valid_rows, BT_ERR_INVALID_ARGUMENT,
+             "bt_add_bias_residual_layernorm: residual_row_index needs valid_rows");
+  return launch_ln<false>(out, residual, bias, gamma, beta, gamma_beta_fp32, out, valid_rows,
+                          residual_row_index, 0, 1, rows_cap, hidden_dim, eps, as_stream(stream),
                           "bt_add_bias_residual_layernorm");
 }
 
@@ -174,6 +180,6 @@ extern "C" int bt_add_bias_residual_layernorm_restore(
   BT_REQUIRE((long long)batch_size * seq_len < (1ll << 31), BT_ERR_UNSUPPORTED,
              "bt_add_bias_residual_layernorm_restore: too many rows");
   return launch_ln<true>(out, residual, bias, gamma, beta, gamma_beta_fp32, out_padded, batch_idx,
-                         batch_size, seq_len, batch_size * seq_len, hidden_dim, eps,
+                         nullptr, batch_size, seq_len, batch_size * seq_len, hidden_dim, eps,
                          as_stream(stream), "bt_add_bias_residual_layernorm_restore");
 }

@@ -46,11 +46,14 @@ def set_option(name, value):
     _check(kernel_lib().bt_set_option(name.encode(), int(value)))
 
 
-def build_offsets(mask, want_count=False):
+def build_offsets(mask, want_count=False, out=None):
     """mask [B,S,S] -> (batch_idx int32[B+1], word_idx int32[B*S], M or None)."""
     B, S = mask.shape[0], mask.shape[1]
-    batch_idx = torch.empty(B + 1, dtype=torch.int32, device=mask.device)
-    word_idx = torch.empty(B * S, dtype=torch.int32, device=mask.device)
+    if out is None:
+        batch_idx = torch.empty(B + 1, dtype=torch.int32, device=mask.device)
+        word_idx = torch.empty(B * S, dtype=torch.int32, device=mask.device)
+    else:
+        batch_idx, word_idx = out
     cnt = ctypes.c_int(-1)
     _check(kernel_lib().bt_build_offsets(_ptr(mask), _dtype_code(mask), B, S, _ptr(batch_idx),
                                          _ptr(word_idx),
@@ -74,10 +77,11 @@ def transpose_weight(w):
     return wt
 
 
-def transpose_weights(ws):
+def transpose_weights(ws, out=None):
     """Pre-pack up to four [K, N] weights in one launch; returns the [N, K] copies."""
     n = len(ws)
-    wts = [torch.empty(w.shape[1], w.shape[0], dtype=w.dtype, device=w.device) for w in ws]
+    wts = out if out is not None else [
+        torch.empty(w.shape[1], w.shape[0], dtype=w.dtype, device=w.device) for w in ws]
     src = (ctypes.c_void_p * n)(*[w.data_ptr() for w in ws])
     dst = (ctypes.c_void_p * n)(*[w.data_ptr() for w in wts])
     ks = (ctypes.c_int * n)(*[w.shape[0] for w in ws])
@@ -109,11 +113,12 @@ def gemm_bias_gelu(a, wt, bias, valid_rows=None, out=None):
 
 
 def gemm_qkv_bias_split(a, wt_qkv, bias_qkv, head_num, size_per_head=64, valid_rows=None,
-                        out=None):
-    rows = a.shape[0]
+                        out=None, a_row_index=None, rows_cap=None):
+    rows = a.shape[0] if rows_cap is None else rows_cap
     if out is None:
         out = torch.zeros(3, head_num, rows, size_per_head, dtype=a.dtype, device=a.device)
-    _check(kernel_lib().bt_gemm_qkv_bias_split(_ptr(a), _ptr(wt_qkv), _ptr(bias_qkv), _ptr(out),
+    _check(kernel_lib().bt_gemm_qkv_bias_split(_ptr(a), _ptr(a_row_index), _ptr(wt_qkv),
+                                               _ptr(bias_qkv), _ptr(out),
                                                _ptr(valid_rows), rows, head_num, size_per_head,
                                                _stream()))
     return out
@@ -139,10 +144,11 @@ def attention_grouped(qkv_heads, batch_idx, batch_size, seq_len, scale, padded_r
                       seq_len, scale, padded_rows, out)
 
 
-def add_bias_residual_layernorm(out, residual, bias, gamma, beta, eps=1e-6, valid_rows=None):
+def add_bias_residual_layernorm(out, residual, bias, gamma, beta, eps=1e-6, valid_rows=None,
+                                residual_row_index=None):
     rows, H = out.shape
     _check(kernel_lib().bt_add_bias_residual_layernorm(
-        _ptr(out), _ptr(residual), _ptr(bias), _ptr(gamma), _ptr(beta),
+        _ptr(out), _ptr(residual), _ptr(residual_row_index), _ptr(bias), _ptr(gamma), _ptr(beta),
         int(gamma.dtype == torch.float32), _ptr(valid_rows), rows, H, float(eps), _stream()))
     return out
 

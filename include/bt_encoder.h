@@ -52,7 +52,8 @@ unsigned long long bt_encoder_bufsize(const bt_encoder_config *cfg);
 
 /* One encoder layer: padded input [B,S,H] + mask [B,S,S] -> padded output
  * [B,S,H] (rows past each sequence's length are zero on the remove-padding
- * path).  `output` must not alias `input`. */
+ * path).  `output` may alias `input` (the input is fully consumed before the
+ * final LayerNorm writes). */
 int bt_encoder_layer_forward(const bt_encoder_config *cfg, const bt_layer_weights *weights,
                              const void *input, const void *atten_mask, void *output, void *buf,
                              int batch_size, int seq_len, void *stream);

@@ -111,10 +111,13 @@ int bt_gemm_bias_gelu(const void *a, const void *wt, const void *bias, void *c,
  * dense_layer_kernel_launcher call (bert_transformer.cu:85-87) plus
  * add_QKV_bias_padding (attention_nofused_utils.cu:143-184) / the in-kernel
  * bias add of attention_fused.cu:318-325.  size_per_head must be 64.
+ * a_row_index (nullable, needs valid_rows): live row t of A is a[a_row_index[t], :] -
+ * passing word_idx reads the valid tokens straight out of the padded input, which
+ * folds compressBertInput (remove_padding.h:104-121) into this GEMM's operand fetch.
  */
-int bt_gemm_qkv_bias_split(const void *a, const void *wt_qkv, const void *bias_qkv,
-                           void *qkv_heads, const int *valid_rows, int rows_cap, int head_num,
-                           int size_per_head, void *stream);
+int bt_gemm_qkv_bias_split(const void *a, const int *a_row_index, const void *wt_qkv,
+                           const void *bias_qkv, void *qkv_heads, const int *valid_rows,
+                           int rows_cap, int head_num, int size_per_head, void *stream);
 
 /*
  * Fused multi-head attention over the head-major Q/K/V written by
@@ -151,8 +154,11 @@ int bt_attention_grouped(const void *qkv_heads, void *attention_output, const in
  * rsqrt.  Replaces add_bias_input_layernorm_kernel_launcher
  * (bytetransformer/include/layernorm.h:410-428, kernels :114-159,273-296).
  * gamma/beta are fp32 when gamma_beta_fp32 != 0, else fp16.  hidden_dim % 8 == 0.
+ * residual_row_index (nullable, needs valid_rows): row t adds residual[residual_row_index[t], :]
+ * instead of residual[t, :] (word_idx: the residual is read from the padded input).
  */
-int bt_add_bias_residual_layernorm(void *out, const void *residual, const void *bias,
+int bt_add_bias_residual_layernorm(void *out, const void *residual,
+                                   const int *residual_row_index, const void *bias,
                                    const void *gamma, const void *beta, int gamma_beta_fp32,
                                    const int *valid_rows, int rows_cap, int hidden_dim,
                                    float eps, void *stream);

@@ -44,7 +44,7 @@ template <typename T>
 struct BertTransformerInferParam {
   const T *input_tensor;  // [batch_size, seq_len, hidden_dim]
   const T *atten_mask;    // [batch_size, seq_len, seq_len], 1 = attend, 0 = padding
-  T *transformer_output;  // [batch_size, seq_len, hidden_dim]; must not alias input_tensor
+  T *transformer_output;  // [batch_size, seq_len, hidden_dim]; may alias input_tensor
   void *buf;              // >= cal_bufsize() bytes of device memory, 256-byte aligned
   int batch_size;
   int seq_len;

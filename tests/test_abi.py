@@ -46,16 +46,18 @@ def test_argument_validation_returns_codes_without_gpu():
     p = ctypes.c_void_p(256)   # never dereferenced: validation fails first
     assert lib.bt_gemm(p, p, p, None, 4, 8, 100, None) == 2 and "multiple of 64" in err()
     assert lib.bt_gemm(p, p, p, None, 4, 12, 64, None) == 2 and "multiple of 8" in err()
-    assert lib.bt_gemm_qkv_bias_split(p, p, p, p, None, 4, 12, 32, None) == 2
+    assert lib.bt_gemm_qkv_bias_split(p, None, p, p, p, None, 4, 12, 32, None) == 2
     assert "size_per_head=32" in err()
+    assert lib.bt_gemm_qkv_bias_split(p, p, p, p, p, None, 4, 12, 64, None) == 1
+    assert "needs valid_rows" in err()
     assert lib.bt_attention_short(p, p, p, 1, 1024, 1024, 12, 64, 0.125, 0, None) == 2
     assert "exceeds 512" in err()
     assert lib.bt_attention_grouped(p, p, p, 1, 16, 16, 12, 48, 0.125, 0, None) == 2
     assert lib.bt_compress(p, p, p, p, 2, 4, 12, None) == 2 and "multiple of 8" in err()
     assert lib.bt_build_offsets(p, 7, 2, 4, p, p, None, None) == 1 and "dtype" in err()
     assert lib.bt_build_offsets(p, 1, 0, 4, p, p, None, None) == 1
-    assert lib.bt_add_bias_residual_layernorm(p, p, p, p, p, 0, None, 4, 12, 1e-6, None) == 2
-    assert lib.bt_add_bias_residual_layernorm(p, p, p, p, p, 0, None, 4, 8192, 1e-6, None) == 2
+    assert lib.bt_add_bias_residual_layernorm(p, p, None, p, p, p, 0, None, 4, 12, 1e-6, None) == 2
+    assert lib.bt_add_bias_residual_layernorm(p, p, None, p, p, p, 0, None, 4, 8192, 1e-6, None) == 2
     assert lib.bt_add_bias_residual_layernorm_restore(p, p, p, p, p, 0, None, p, 2, 4, 64, 1e-6,
                                                       None) == 1
     assert lib.bt_transpose_weight(None, p, 8, 8, None) == 1

@@ -220,6 +220,42 @@ def test_gemm_qkv_bias_split(device, tile, heads):
     assert np.all(g[:, :, M:] == 0)
 
 
+def test_gather_fused_into_qkv_gemm_and_layernorm(device):
+    """a_row_index / residual_row_index = word_idx reads the valid tokens straight from
+    the padded input: bit-identical to compress followed by the plain call."""
+    _say("gather fusion")
+    rs = np.random.RandomState(17)
+    B, S, heads = 5, 70, 2
+    H = heads * 64
+    lens = np.array([70, 0, 33, 1, 64])
+    x = rs.standard_normal((B, S, H)).astype(np.float16)
+    mask = workload.make_mask(lens, S, np.float16)
+    w = (rs.standard_normal((H, 3 * H)) * 0.05).astype(np.float16)
+    bias = (rs.standard_normal(3 * H) * 0.5).astype(np.float16)
+    g_bi, g_wi, M = ops.build_offsets(_dev(mask, device), want_count=True)
+    vr = g_bi[B:]
+    xd, wt = _dev(x, device), ops.transpose_weight(_dev(w, device))
+    packed = ops.compress(xd, g_bi, g_wi)
+    ref = ops.gemm_qkv_bias_split(packed, wt, _dev(bias, device), heads, valid_rows=vr)
+    got = ops.gemm_qkv_bias_split(xd.view(B * S, H), wt, _dev(bias, device), heads, valid_rows=vr,
+                                  a_row_index=g_wi)
+    assert torch.equal(ref[:, :, :M], got[:, :, :M])
+    exp = O.split_heads(O.gemm(O.compress(x, g_wi.cpu().numpy()[:M]), w, bias), heads, 64)
+    err = np.abs(got.cpu().numpy()[:, :, :M].astype(np.float64) - exp)
+    assert np.all(err <= 2.0 ** -10 * np.abs(exp) + 2e-4)
+    # LayerNorm with the residual gathered from the padded input
+    out = rs.standard_normal((B * S, H)).astype(np.float16)
+    b2 = (rs.standard_normal(H) * 0.5).astype(np.float16)
+    gamma = (1 + 0.2 * rs.standard_normal(H)).astype(np.float16)
+    beta = (0.3 * rs.standard_normal(H)).astype(np.float16)
+    a = ops.add_bias_residual_layernorm(_dev(out, device), packed, _dev(b2, device),
+                                        _dev(gamma, device), _dev(beta, device), valid_rows=vr)
+    b = ops.add_bias_residual_layernorm(_dev(out, device), xd.view(B * S, H), _dev(b2, device),
+                                        _dev(gamma, device), _dev(beta, device), valid_rows=vr,
+                                        residual_row_index=g_wi)
+    assert torch.equal(a, b)
+
+
 # ---- attention -----------------------------------------------------------------
 def _attention_case(rs, lens, S, heads, scale_q=1.0):
     B = len(lens)
