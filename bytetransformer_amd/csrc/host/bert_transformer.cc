@@ -71,8 +71,16 @@ void BertTransformer<OpType>::bert_infer(BertTransformerInferParam infer_param) 
     valid_rows = et_param.batch_idx + batch_size;
   }
 
-  // k-contiguous weight pre-pack, all four matrices in one launch
-  {
+  // k-contiguous weight pre-pack: all four matrices in one launch, unless the
+  // caller handed in copies it already made
+  const bool have_prepack = param_.prepacked_kernels[0] && param_.prepacked_kernels[1] &&
+                            param_.prepacked_kernels[2] && param_.prepacked_kernels[3];
+  if (have_prepack) {
+    wt_qkv = const_cast<DataType_ *>(param_.prepacked_kernels[0]);
+    wt_proj = const_cast<DataType_ *>(param_.prepacked_kernels[1]);
+    wt_inter = const_cast<DataType_ *>(param_.prepacked_kernels[2]);
+    wt_out = const_cast<DataType_ *>(param_.prepacked_kernels[3]);
+  } else {
     const void *src[4] = {param_.attr_kernel_QKV, param_.attr_output_kernel, param_.inter_kernel,
                           param_.output_kernel};
     void *dst[4] = {wt_qkv, wt_proj, wt_inter, wt_out};

@@ -3,6 +3,7 @@
 // bytetransformer/th_op/bert_transformer_ext.h:30-117.
 #pragma once
 #include "bytetransformer/bert_transformer.h"
+#include "prepack_cache.h"
 #include "util.h"
 
 namespace bytetransformer {
@@ -66,13 +67,18 @@ class BTEncoder : public IBTEncoder {
     TORCH_CHECK(!attention_bias.defined(), "attention_bias is not supported");
     c10::DeviceGuard device_guard(input.device());
 
+    hipStream_t stream = c10::hip::getCurrentHIPStream(input.device().index()).stream();
+    BertTransformerParam<kOp> param = param_;
+    std::vector<Tensor> packed = prepacked_weights(stream);   // keeps the copies alive
+    if (packed.size() == 4)
+      for (int i = 0; i < 4; ++i) param.prepacked_kernels[i] = get_ptr<T>(packed[i]);
+
     BertTransformer<kOp> encoder(batch_size, head_num_, head_size_, seq_len, use_fused_attention,
                                  is_remove_padding, use_fp32_, model_type);
-    encoder.initialize(param_);
+    encoder.initialize(param);
     const unsigned long long buf_size = encoder.cal_bufsize();
     auto buf_tensor = torch::empty({(int64_t)buf_size},
                                    torch::dtype(torch::kInt8).device(input.device()));
-    hipStream_t stream = c10::hip::getCurrentHIPStream(input.device().index()).stream();
     struct BertTransformerInferParam<T> infer_param {
       get_ptr<T>(input), get_ptr<T>(attr_mask), get_ptr<T>(output), get_ptr<void>(buf_tensor),
           batch_size, seq_len, nullptr, stream
@@ -81,6 +87,37 @@ class BTEncoder : public IBTEncoder {
   }
 
  private:
+  // The four [N, K] weight copies, from the process-wide cache when the same
+  // tensors were seen before, else packed now (one launch) and remembered.
+  // Empty for dtypes the kernels do not run (infer() raises for those).
+  std::vector<Tensor> prepacked_weights(hipStream_t stream) {
+    std::vector<Tensor> out;
+    if (kOp != OperationType::HALF) return out;
+    auto &cache = PrepackCache::instance();
+    if (!cache.enabled()) return out;
+    static const int kIdx[4] = {0, 2, 6, 8};
+    for (int i = 0; i < 4; ++i)
+      if (weights_[kIdx[i]].dim() != 2) return out;
+    out.resize(4);
+    bool all_hit = true;
+    for (int i = 0; i < 4; ++i) all_hit = cache.lookup(weights_[kIdx[i]], stream, &out[i]) && all_hit;
+    if (all_hit) return out;
+    const void *src[4];
+    void *dst[4];
+    int ks[4], ns[4];
+    for (int i = 0; i < 4; ++i) {
+      const Tensor &w = weights_[kIdx[i]];
+      out[i] = torch::empty({w.size(1), w.size(0)}, w.options());
+      src[i] = w.data_ptr();
+      dst[i] = out[i].data_ptr();
+      ks[i] = (int)w.size(0);
+      ns[i] = (int)w.size(1);
+    }
+    check_bt_error(bt_transpose_weights(4, src, dst, ks, ns, stream));
+    for (int i = 0; i < 4; ++i) cache.store(weights_[kIdx[i]], stream, out[i]);
+    return out;
+  }
+
   const int head_num_, head_size_;
   bool use_fp32_ = false;
   std::vector<Tensor> weights_;

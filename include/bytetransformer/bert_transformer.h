@@ -38,6 +38,13 @@ class BertTransformerParam {
   int intermediate_size = 4;
 
   int cublas_Algo[3] = {Traits_::algo, Traits_::algo, Traits_::algo};  // unused, kept for callers
+
+  // Extension (no counterpart in the reference): the four weight matrices already
+  // pre-packed k-contiguous by bt_transpose_weights, in the order QKV [3H,H],
+  // attention output [H,H], FFN1 [F,H], FFN2 [H,F].  When all four are set,
+  // infer() uses them and skips its own pre-pack launch; the caller vouches that
+  // they match the *_kernel tensors above.
+  const DataType_ *prepacked_kernels[4] = {nullptr, nullptr, nullptr, nullptr};
 };
 
 template <typename T>

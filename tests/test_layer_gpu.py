@@ -188,6 +188,38 @@ def test_ragged_edge_cases(device):
     _check(_run_th_op(wl, device), _oracle(wl), wl.lens, tag="ragged/th_op")
 
 
+def test_th_op_prepack_cache_tracks_weight_updates(device):
+    """The operator caches the k-contiguous weight copies per tensor object; an
+    in-place update of a weight (version counter bump) must be picked up, and a
+    new tensor at a recycled address must not hit a stale entry."""
+    _say("prepack cache")
+    bt.load_th_op()
+    cfg = workload.EncoderConfig("pc", 4, 64, 2, layers=1, lens=(64, 20, 33, 50), seed=3)
+    wl = workload.make_workload(cfg, bias_std=0.05, random_affine=True)
+    w = [_dev(wl.layers[0][n], device) for n in workload.WEIGHT_NAMES]
+    x, m = _dev(wl.x, device), _dev(wl.mask, device)
+    op = torch.ops.ByteTransformer.BertTransformer
+    a = op(2, 64, *w, x, m, True, True)
+    b = op(2, 64, *w, x, m, True, True)              # second call: cache hit
+    assert torch.equal(a, b)
+    _check(a.cpu().numpy(), _oracle(wl), wl.lens, tag="cache/first")
+    # in-place update of FFN2's weight
+    w[8].mul_(0.5)
+    wl.layers[0]["output_kernel"] = (wl.layers[0]["output_kernel"].astype(np.float32) * 0.5).astype(np.float16)
+    c = op(2, 64, *w, x, m, True, True)
+    assert not torch.equal(a, c)
+    _check(c.cpu().numpy(), _oracle(wl), wl.lens, tag="cache/after-inplace-update")
+    # brand-new tensors (old ones freed, addresses may be recycled)
+    for _ in range(3):
+        wl2 = workload.make_workload(workload.EncoderConfig("pc2", 4, 64, 2, layers=1,
+                                                            lens=(64, 20, 33, 50), seed=4 + _),
+                                     bias_std=0.05, random_affine=True)
+        del w
+        w = [_dev(wl2.layers[0][n], device) for n in workload.WEIGHT_NAMES]
+        d = op(2, 64, *w, _dev(wl2.x, device), m, True, True)
+        _check(d.cpu().numpy(), _oracle(wl2), wl2.lens, tag="cache/new-tensors")
+
+
 def test_th_op_error_paths_on_gpu(device):
     bt.load_th_op()
     cfg = workload.EncoderConfig("e", 3, 16, 2, layers=1, lens=(16, 3, 9))
