@@ -104,6 +104,14 @@ def test_th_op_rejects_host_tensors_like_the_reference():
         torch.ops.ByteTransformer.BertTransformer(2, 64, *w, x, m, True, True)
 
 
+def test_torchscript_class_is_registered_and_checks_arguments():
+    bt.load_th_op()
+    w, _, _ = _cpu_args()
+    cls = torch.classes.ByteTransformer.BertTransformer
+    with pytest.raises(RuntimeError, match="qkv_kernel must be a CUDA tensor"):
+        cls(2, 64, *w)
+
+
 def test_missing_library_raises(monkeypatch, tmp_path):
     monkeypatch.setattr(_lib, "_DIR", str(tmp_path))
     with pytest.raises(bt.LibraryMissing, match="no fallback"):

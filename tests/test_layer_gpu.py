@@ -220,6 +220,44 @@ def test_th_op_prepack_cache_tracks_weight_updates(device):
         _check(d.cpu().numpy(), _oracle(wl2), wl2.lens, tag="cache/new-tensors")
 
 
+def test_torchscript_class_forward_and_pickle(device):
+    """torch.classes.ByteTransformer.BertTransformer: forward == functional
+    operator, forwardv2 flags, TorchScript save/load round trip (pickle state =
+    12 tensors + head_info)."""
+    _say("torchscript class")
+    import io
+    bt.load_th_op()
+    cfg = workload.EncoderConfig("ts", 4, 80, 2, layers=1, lens=(80, 20, 33, 50), seed=8)
+    wl = workload.make_workload(cfg, bias_std=0.05, random_affine=True)
+    w = [_dev(wl.layers[0][n], device) for n in workload.WEIGHT_NAMES]
+    x, m = _dev(wl.x, device), _dev(wl.mask, device)
+    layer = torch.classes.ByteTransformer.BertTransformer(2, 64, *w)
+    ref = torch.ops.ByteTransformer.BertTransformer(2, 64, *w, x, m, True, True)
+    out = layer.forward(x, m)
+    assert torch.equal(out, ref)
+    _check(out.cpu().numpy(), _oracle(wl), wl.lens, tag="class/forward")
+    padded = layer.forwardv2(x, m, False, False)
+    _check(O.masked_output(padded.cpu().numpy(), wl.lens), _oracle(wl), wl.lens,
+           tag="class/forwardv2-padded")
+
+    class Wrap(torch.nn.Module):
+        def __init__(self, inner):
+            super().__init__()
+            self.inner = inner
+
+        def forward(self, a, b):
+            return self.inner.forward(a, b)
+
+    scripted = torch.jit.script(Wrap(layer))
+    buf = io.BytesIO()
+    torch.jit.save(scripted, buf)
+    buf.seek(0)
+    loaded = torch.jit.load(buf, map_location=device)
+    assert torch.equal(loaded(x, m), ref)
+    with pytest.raises(RuntimeError, match="Inconsistency of Tensor type"):
+        layer.forward(x.float(), m)
+
+
 def test_th_op_error_paths_on_gpu(device):
     bt.load_th_op()
     cfg = workload.EncoderConfig("e", 3, 16, 2, layers=1, lens=(16, 3, 9))
