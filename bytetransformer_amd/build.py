@@ -4,7 +4,9 @@
     libbytetransformer.so      host C++ BertTransformer API (g++,   include/bytetransformer/, bt_encoder.h)
     libths_bytetransformer.so  PyTorch operator             (g++ against the installed PyTorch-ROCm)
 
-Run `python -m bytetransformer_amd.build [kernels|host|th_op|all]`.  Outputs
+    bert_transformer_test      stand-alone C++ driver       (g++, text fixtures)
+
+Run `python -m bytetransformer_amd.build [kernels|host|th_op|unit_test|all]`.  Outputs
 land in bytetransformer_amd/lib/.
 """
 import os
@@ -108,10 +110,24 @@ def build_th_op():
     return out
 
 
+def build_unit_test():
+    """The stand-alone C++ driver (text fixtures in, max diff and timing out)."""
+    os.makedirs(LIB, exist_ok=True)
+    out = os.path.join(LIB, "bert_transformer_test")
+    _run(["g++"] + HOST_FLAGS + ["-I", INC, "-I", os.path.join(ROCM, "include"),
+                                 os.path.join(CSRC, "unit_test", "bert_transformer_test.cc"),
+                                 "-L", LIB, "-lbytetransformer", "-lbt_hip",
+                                 "-L", os.path.join(ROCM, "lib"), "-lamdhip64",
+                                 "-Wl,-rpath,$ORIGIN", "-Wl,-rpath," + os.path.join(ROCM, "lib"),
+                                 "-o", out])
+    return out
+
+
 def build_all():
-    return [build_kernels(), build_host(), build_th_op()]
+    return [build_kernels(), build_host(), build_th_op(), build_unit_test()]
 
 
 if __name__ == "__main__":
     what = sys.argv[1] if len(sys.argv) > 1 else "all"
-    {"kernels": build_kernels, "host": build_host, "th_op": build_th_op, "all": build_all}[what]()
+    {"kernels": build_kernels, "host": build_host, "th_op": build_th_op,
+     "unit_test": build_unit_test, "all": build_all}[what]()
