@@ -38,9 +38,10 @@ KERNEL_ABI = {
     "bt_transpose_weight": (c_int, [_P, _P, c_int, c_int, _P]),
     "bt_transpose_weights": (c_int, [c_int, POINTER(c_void_p), POINTER(c_void_p), POINTER(c_int),
                                      POINTER(c_int), _P]),
-    "bt_gemm": (c_int, [_P, _P, _P, _IP, c_int, c_int, c_int, _P]),
-    "bt_gemm_bias_gelu": (c_int, [_P, _P, _P, _P, _IP, c_int, c_int, c_int, _P]),
-    "bt_gemm_qkv_bias_split": (c_int, [_P, _IP, _P, _P, _P, _IP, c_int, c_int, c_int, _P]),
+    "bt_gemm": (c_int, [_P, _P, _P, _IP, c_int, c_int, c_int, c_int, _P]),
+    "bt_gemm_bias_gelu": (c_int, [_P, _P, _P, _P, _IP, c_int, c_int, c_int, c_int, _P]),
+    "bt_gemm_qkv_bias_split": (c_int, [_P, _IP, _P, _P, _P, _IP, c_int, c_int, c_int, c_int,
+                                       _P]),
     "bt_attention_short": (c_int, [_P, _P, _IP, c_int, c_int, c_int, c_int, c_int, c_float,
                                    c_int, _P]),
     "bt_attention_grouped": (c_int, [_P, _P, _IP, c_int, c_int, c_int, c_int, c_int, c_float,

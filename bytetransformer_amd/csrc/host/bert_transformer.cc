@@ -55,9 +55,16 @@ void BertTransformer<OpType>::bert_infer(BertTransformerInferParam infer_param) 
   DataType_ *wt_inter = wt_proj + (size_t)hidden * hidden;
   DataType_ *wt_out = wt_inter + (size_t)hidden * inter;
 
-  // lengths from the mask (needed on both paths: keys past len_b are excluded)
-  check_bt_error(bt_build_offsets(atten_mask, Traits_::dtype, batch_size, seq_len,
-                                  et_param.batch_idx, et_param.word_idx, nullptr, stream));
+  // lengths from the mask (needed on both paths: keys past len_b are excluded),
+  // unless the caller already holds the offsets of this mask
+  int rows_hint = 0;
+  if (infer_param.offsets && infer_param.offsets->batch_idx && infer_param.offsets->word_idx) {
+    et_param = *infer_param.offsets;
+    rows_hint = et_param.valid_word_num;
+  } else {
+    check_bt_error(bt_build_offsets(atten_mask, Traits_::dtype, batch_size, seq_len,
+                                    et_param.batch_idx, et_param.word_idx, nullptr, stream));
+  }
   const int *valid_rows = nullptr;
   const int *gather = nullptr;
   DataType_ *restore_target = nullptr;
@@ -91,7 +98,7 @@ void BertTransformer<OpType>::bert_infer(BertTransformerInferParam infer_param) 
 
   check_bt_error(bt_gemm_qkv_bias_split(from_tensor, gather, wt_qkv,
                                         param_.attention_param.attr_bias_QKV, qkv_buf, valid_rows,
-                                        rows, head_num_, size_per_head_, stream));
+                                        rows, rows_hint, head_num_, size_per_head_, stream));
 
   struct AttentionInferParam<DataType_> attention_infer_param {
     qkv_buf, atten_mask, attr_out_buf, base + inner_buf_size_, batch_size, seq_len,
@@ -101,7 +108,8 @@ void BertTransformer<OpType>::bert_infer(BertTransformerInferParam infer_param) 
   attention_layer_->infer(attention_infer_param);
 
   check_bt_error(
-      bt_gemm(attr_out_buf, wt_proj, attr_matmul_buf, valid_rows, rows, hidden, hidden, stream));
+      bt_gemm(attr_out_buf, wt_proj, attr_matmul_buf, valid_rows, rows, rows_hint, hidden, hidden,
+              stream));
 
   check_bt_error(bt_add_bias_residual_layernorm(
       attr_matmul_buf, from_tensor, gather, param_.attr_output_bias, param_.attr_output_layernorm_gamma,
@@ -109,10 +117,11 @@ void BertTransformer<OpType>::bert_infer(BertTransformerInferParam infer_param) 
       layernorm_eps, stream));
 
   check_bt_error(bt_gemm_bias_gelu(attr_matmul_buf, wt_inter, param_.inter_bias, inter_matmul_buf,
-                                   valid_rows, rows, inter, hidden, stream));
+                                   valid_rows, rows, rows_hint, inter, hidden, stream));
 
   check_bt_error(
-      bt_gemm(inter_matmul_buf, wt_out, transformer_out, valid_rows, rows, hidden, inter, stream));
+      bt_gemm(inter_matmul_buf, wt_out, transformer_out, valid_rows, rows, rows_hint, hidden, inter,
+              stream));
 
   if (is_remove_padding_)
     check_bt_error(bt_add_bias_residual_layernorm_restore(

@@ -43,6 +43,7 @@ struct GemmArgs {
   const int *a_row_index;   // optional gather: A row r is a[a_row_index[r]] (null = identity)
   int rows_cap, N, K;
   int tiles_n;
+  int rows_hint;        // host-side estimate of the live rows (0 = unknown); tile choice only
 };
 
 __device__ __forceinline__ float gelu_tanh_f32(float x) {
@@ -302,19 +303,43 @@ static int launch_gemm_tile(GemmArgs p, hipStream_t s) {
 template <int EPI>
 static int launch_gemm(GemmArgs p, hipStream_t s) {
   // Tile table (rows x cols, ring depth, wave grid):
-  //   0: 256x256, 2, 2x4   wide outputs (FFN1): one tile per CU
+  //   0: 256x256, 2, 2x4   wide outputs (FFN1 at hidden 768): one tile per CU
   //   1: 128x128, 2, 2x2   narrow outputs, short k loop (projection)
   //   2: 128x128, 3, 4x2   narrow outputs, long k loop (FFN2)
   //   3: 256x192, 2, 4x2   outputs that split into 192-wide panels but not into a
   //                        full wave of 256-wide ones (QKV at hidden 768)
+  // The choice minimises (tiles per CU, rounded up) x (measured time of one tile)
+  // for the estimated live rows: the exact count when every row is live, the
+  // caller's hint when it has one, else 60 % of the capacity (the fill the
+  // padding-free path is built for).
   int choice = option_gemm_tile();
   if (choice < 0) {
-    if (p.N >= 3072 && p.N % 256 == 0 && p.rows_cap >= 2048)
-      choice = 0;
-    else if (p.N >= 1536 && p.N % 192 == 0 && p.rows_cap >= 2048)
-      choice = 3;
-    else
-      choice = p.K >= 2048 ? 2 : 1;
+    static const int cus = [] {
+      int dev = 0, n = 0;
+      if (hipGetDevice(&dev) != hipSuccess ||
+          hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
+          n <= 0)
+        n = 256;
+      return n;
+    }();
+    const long long m_est = !p.valid_rows ? p.rows_cap
+                            : p.rows_hint > 0 ? (p.rows_hint < p.rows_cap ? p.rows_hint : p.rows_cap)
+                                              : (p.rows_cap * 3LL + 4) / 5;
+    struct Cand {
+      int id, bm, bn;
+      float tile_time;   // relative time of one tile of this shape per k-step
+    };
+    const Cand cands[3] = {{0, 256, 256, 24.0f}, {3, 256, 192, 19.5f},
+                           {p.K >= 2048 ? 2 : 1, 128, 128, 7.5f}};
+    float best = 0.f;
+    for (const Cand &c : cands) {
+      const long long tiles = ((m_est + c.bm - 1) / c.bm) * ((p.N + c.bn - 1) / c.bn);
+      const float t = (float)((tiles + cus - 1) / cus) * c.tile_time;
+      if (choice < 0 || t < best) {
+        best = t;
+        choice = c.id;
+      }
+    }
   }
   switch (choice) {
     case 0:
@@ -373,31 +398,32 @@ extern "C" int bt_transpose_weight(const void *w, void *wt, int k, int n, void *
 }
 
 extern "C" int bt_gemm(const void *a, const void *wt, void *c, const int *valid_rows,
-                       int rows_cap, int n, int k, void *stream) {
+                       int rows_cap, int rows_hint, int n, int k, void *stream) {
   int rc = check_gemm_args("bt_gemm", a, wt, c, rows_cap, n, k);
   if (rc) return rc;
   if (rows_cap == 0) return BT_OK;
   GemmArgs p{(const half_t *)a, (const half_t *)wt, nullptr, (half_t *)c, valid_rows, nullptr,
-             rows_cap,          n,                  k,       0};
+             rows_cap,          n,                  k,       0,           rows_hint};
   return launch_gemm<kEpiPlain>(p, as_stream(stream));
 }
 
 extern "C" int bt_gemm_bias_gelu(const void *a, const void *wt, const void *bias, void *c,
-                                 const int *valid_rows, int rows_cap, int n, int k,
+                                 const int *valid_rows, int rows_cap, int rows_hint, int n, int k,
                                  void *stream) {
   int rc = check_gemm_args("bt_gemm_bias_gelu", a, wt, c, rows_cap, n, k);
   if (rc) return rc;
   BT_REQUIRE(bias, BT_ERR_INVALID_ARGUMENT, "bt_gemm_bias_gelu: null bias");
   if (rows_cap == 0) return BT_OK;
   GemmArgs p{(const half_t *)a, (const half_t *)wt, (const half_t *)bias, (half_t *)c, valid_rows,
-             nullptr,           rows_cap,           n,                    k,           0};
+             nullptr,           rows_cap,           n,                    k,           0,
+             rows_hint};
   return launch_gemm<kEpiBiasGelu>(p, as_stream(stream));
 }
 
 extern "C" int bt_gemm_qkv_bias_split(const void *a, const int *a_row_index, const void *wt_qkv,
                                       const void *bias_qkv, void *qkv_heads,
-                                      const int *valid_rows, int rows_cap, int head_num,
-                                      int size_per_head, void *stream) {
+                                      const int *valid_rows, int rows_cap, int rows_hint,
+                                      int head_num, int size_per_head, void *stream) {
   BT_REQUIRE(head_num > 0, BT_ERR_INVALID_ARGUMENT, "bt_gemm_qkv_bias_split: head_num=%d",
              head_num);
   BT_REQUIRE(size_per_head == 64, BT_ERR_UNSUPPORTED,
@@ -410,6 +436,6 @@ extern "C" int bt_gemm_qkv_bias_split(const void *a, const int *a_row_index, con
   BT_REQUIRE(!a_row_index || valid_rows, BT_ERR_INVALID_ARGUMENT,
              "bt_gemm_qkv_bias_split: a_row_index needs valid_rows (only live rows are indexed)");
   GemmArgs p{(const half_t *)a, (const half_t *)wt_qkv, (const half_t *)bias_qkv,
-             (half_t *)qkv_heads, valid_rows, a_row_index, rows_cap, 3 * H, H, 0};
+             (half_t *)qkv_heads, valid_rows, a_row_index, rows_cap, 3 * H, H, 0, rows_hint};
   return launch_gemm<kEpiQkvSplit>(p, as_stream(stream));
 }

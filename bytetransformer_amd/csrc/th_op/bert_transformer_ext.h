@@ -6,6 +6,8 @@
 #include "prepack_cache.h"
 #include "util.h"
 
+#include <hip/hip_runtime_api.h>
+
 namespace bytetransformer {
 namespace torch_ext {
 using torch::Tensor;
@@ -83,6 +85,16 @@ class BTEncoder : public IBTEncoder {
       get_ptr<T>(input), get_ptr<T>(attr_mask), get_ptr<T>(output), get_ptr<void>(buf_tensor),
           batch_size, seq_len, nullptr, stream
     };
+    // offsets of this mask: cached per mask tensor (never while the stream is being
+    // captured into a graph, where the host may not wait for the token count)
+    MaskPlanCache::Plan plan;
+    ET_Param offsets{nullptr, nullptr, 0};
+    if (mask_plan(attr_mask, batch_size, seq_len, stream, &plan)) {
+      offsets.batch_idx = plan.batch_idx.data_ptr<int>();
+      offsets.word_idx = plan.word_idx.data_ptr<int>();
+      offsets.valid_word_num = plan.valid_word_num;
+      infer_param.offsets = &offsets;
+    }
     encoder.infer(infer_param);
   }
 
@@ -116,6 +128,26 @@ class BTEncoder : public IBTEncoder {
     check_bt_error(bt_transpose_weights(4, src, dst, ks, ns, stream));
     for (int i = 0; i < 4; ++i) cache.store(weights_[kIdx[i]], stream, out[i]);
     return out;
+  }
+
+  bool mask_plan(const Tensor &mask, int batch_size, int seq_len, hipStream_t stream,
+                 MaskPlanCache::Plan *plan) {
+    if (kOp != OperationType::HALF || !PrepackCache::instance().enabled() || mask.is_inference())
+      return false;
+    hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(stream, &capturing) != hipSuccess ||
+        capturing != hipStreamCaptureStatusNone)
+      return false;
+    auto &cache = MaskPlanCache::instance();
+    if (cache.lookup(mask, stream, plan)) return true;
+    auto opts = torch::dtype(torch::kInt32).device(mask.device());
+    plan->batch_idx = torch::empty({(int64_t)batch_size + 1}, opts);
+    plan->word_idx = torch::empty({(int64_t)batch_size * seq_len}, opts);
+    check_bt_error(bt_build_offsets(mask.data_ptr(), BT_F16, batch_size, seq_len,
+                                    plan->batch_idx.data_ptr<int>(), plan->word_idx.data_ptr<int>(),
+                                    &plan->valid_word_num, stream));
+    cache.store(mask, stream, *plan);
+    return true;
   }
 
   const int head_num_, head_size_;

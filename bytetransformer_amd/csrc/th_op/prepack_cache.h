@@ -17,6 +17,7 @@
 #include <cstdlib>
 #include <mutex>
 #include <unordered_map>
+#include <vector>
 
 #include "bt_hip.h"
 
@@ -102,6 +103,72 @@ class PrepackCache {
   }
 
   bool enabled_ = true;
+  std::mutex mu_;
+  std::unordered_map<const c10::TensorImpl *, Entry> map_;
+};
+
+// Offsets of an attention mask (batch_idx, word_idx, valid-token count), cached
+// per mask tensor under the same validity rules as the weight copies.  A model
+// calls the operator once per layer with one mask, so the prefix sum - and the
+// one host synchronisation that fetches the token count used to pick GEMM tile
+// shapes - happens once per mask instead of once per layer.
+class MaskPlanCache {
+ public:
+  struct Plan {
+    torch::Tensor batch_idx, word_idx;
+    int valid_word_num = 0;
+  };
+
+  static MaskPlanCache &instance() {
+    static MaskPlanCache c;
+    return c;
+  }
+
+  bool lookup(const torch::Tensor &mask, void *stream, Plan *plan) {
+    std::lock_guard<std::mutex> g(mu_);
+    auto it = map_.find(mask.unsafeGetTensorImpl());
+    if (it == map_.end()) return false;
+    Entry &e = it->second;
+    auto alive = e.owner.lock();
+    if (!alive || alive.get() != mask.unsafeGetTensorImpl() || e.version != mask._version() ||
+        e.data != mask.data_ptr() || e.stream != stream || e.sizes != mask.sizes().vec() ||
+        e.device != mask.device()) {
+      map_.erase(it);
+      return false;
+    }
+    *plan = e.plan;
+    return true;
+  }
+
+  void store(const torch::Tensor &mask, void *stream, const Plan &plan) {
+    std::lock_guard<std::mutex> g(mu_);
+    if (map_.size() >= kMaxEntries) {
+      for (auto it = map_.begin(); it != map_.end();)
+        it = it->second.owner.expired() ? map_.erase(it) : std::next(it);
+      if (map_.size() >= kMaxEntries) map_.clear();
+    }
+    Entry e;
+    e.owner = c10::weak_intrusive_ptr<c10::TensorImpl>(mask.getIntrusivePtr());
+    e.version = mask._version();
+    e.data = mask.data_ptr();
+    e.stream = stream;
+    e.sizes = mask.sizes().vec();
+    e.device = mask.device();
+    e.plan = plan;
+    map_[mask.unsafeGetTensorImpl()] = std::move(e);
+  }
+
+ private:
+  struct Entry {
+    c10::weak_intrusive_ptr<c10::TensorImpl> owner{c10::intrusive_ptr<c10::TensorImpl>()};
+    int64_t version = 0;
+    void *data = nullptr;
+    void *stream = nullptr;
+    std::vector<int64_t> sizes;
+    c10::Device device{c10::kCPU};
+    Plan plan;
+  };
+  static constexpr size_t kMaxEntries = 64;
   std::mutex mu_;
   std::unordered_map<const c10::TensorImpl *, Entry> map_;
 };

@@ -92,35 +92,36 @@ def transpose_weights(ws, out=None):
     return wts
 
 
-def gemm(a, wt, valid_rows=None, out=None):
+def gemm(a, wt, valid_rows=None, out=None, rows_hint=0):
     rows, K = a.shape
     N = wt.shape[0]
     if out is None:
         out = torch.zeros(rows, N, dtype=a.dtype, device=a.device)
-    _check(kernel_lib().bt_gemm(_ptr(a), _ptr(wt), _ptr(out), _ptr(valid_rows), rows, N, K,
-                                _stream()))
+    _check(kernel_lib().bt_gemm(_ptr(a), _ptr(wt), _ptr(out), _ptr(valid_rows), rows,
+                                int(rows_hint), N, K, _stream()))
     return out
 
 
-def gemm_bias_gelu(a, wt, bias, valid_rows=None, out=None):
+def gemm_bias_gelu(a, wt, bias, valid_rows=None, out=None, rows_hint=0):
     rows, K = a.shape
     N = wt.shape[0]
     if out is None:
         out = torch.zeros(rows, N, dtype=a.dtype, device=a.device)
     _check(kernel_lib().bt_gemm_bias_gelu(_ptr(a), _ptr(wt), _ptr(bias), _ptr(out),
-                                          _ptr(valid_rows), rows, N, K, _stream()))
+                                          _ptr(valid_rows), rows, int(rows_hint), N, K,
+                                          _stream()))
     return out
 
 
 def gemm_qkv_bias_split(a, wt_qkv, bias_qkv, head_num, size_per_head=64, valid_rows=None,
-                        out=None, a_row_index=None, rows_cap=None):
+                        out=None, a_row_index=None, rows_cap=None, rows_hint=0):
     rows = a.shape[0] if rows_cap is None else rows_cap
     if out is None:
         out = torch.zeros(3, head_num, rows, size_per_head, dtype=a.dtype, device=a.device)
     _check(kernel_lib().bt_gemm_qkv_bias_split(_ptr(a), _ptr(a_row_index), _ptr(wt_qkv),
                                                _ptr(bias_qkv), _ptr(out),
-                                               _ptr(valid_rows), rows, head_num, size_per_head,
-                                               _stream()))
+                                               _ptr(valid_rows), rows, int(rows_hint), head_num,
+                                               size_per_head, _stream()))
     return out
 
 

@@ -16,6 +16,8 @@
  *     number of live rows M (normally batch_idx + batch_size); kernels size
  *     their grids for `rows_cap` rows and retire rows >= M on the device, so
  *     the host never waits for M.  NULL means all rows_cap rows are live.
+ *   - `rows_hint` arguments are the host's estimate of M (0 = none); they only
+ *     steer the choice of tile shape and never affect results.
  *
  * Each declaration cites the reference interface it replaces (paths relative
  * to the ByteTransformer tree).
@@ -92,8 +94,8 @@ int bt_transpose_weights(int count, const void *const *w, void *const *wt, const
  * (bert_transformer.cu:102-104,115-117).  `wt` is the [n, k] pre-packed weight.
  * k % 64 == 0, n % 8 == 0.
  */
-int bt_gemm(const void *a, const void *wt, void *c, const int *valid_rows, int rows_cap, int n,
-            int k, void *stream);
+int bt_gemm(const void *a, const void *wt, void *c, const int *valid_rows, int rows_cap,
+            int rows_hint, int n, int k, void *stream);
 
 /*
  * c = gelu_tanh(a . w + bias).  Replaces gemm_bias_gelu
@@ -101,7 +103,8 @@ int bt_gemm(const void *a, const void *wt, void *c, const int *valid_rows, int r
  * gemm_bias_act.h:80-87).
  */
 int bt_gemm_bias_gelu(const void *a, const void *wt, const void *bias, void *c,
-                      const int *valid_rows, int rows_cap, int n, int k, void *stream);
+                      const int *valid_rows, int rows_cap, int rows_hint, int n, int k,
+                      void *stream);
 
 /*
  * QKV projection with the bias add and the head split fused into the store:
@@ -117,7 +120,8 @@ int bt_gemm_bias_gelu(const void *a, const void *wt, const void *bias, void *c,
  */
 int bt_gemm_qkv_bias_split(const void *a, const int *a_row_index, const void *wt_qkv,
                            const void *bias_qkv, void *qkv_heads, const int *valid_rows,
-                           int rows_cap, int head_num, int size_per_head, void *stream);
+                           int rows_cap, int rows_hint, int head_num, int size_per_head,
+                           void *stream);
 
 /*
  * Fused multi-head attention over the head-major Q/K/V written by

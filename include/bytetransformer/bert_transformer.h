@@ -60,6 +60,11 @@ struct BertTransformerInferParam {
   const T *attention_bias = NULL;         // [head_num, seq_len, seq_len]; must be NULL
   const uint32_t *position_ids = NULL;    // never read
   const uint32_t *token_type_ids = NULL;  // never read
+  // Extension (no counterpart in the reference): offsets already built from this
+  // very atten_mask by bt_build_offsets (batch_idx int[batch_size+1], word_idx
+  // int[batch_size*seq_len], valid_word_num = their total).  When set, infer()
+  // skips its own mask prefix sum and uses valid_word_num to pick tile shapes.
+  const ET_Param *offsets = NULL;
 };
 
 template <OperationType OpType>

@@ -42,13 +42,13 @@ def test_host_library_exports_every_declared_symbol():
 def test_argument_validation_returns_codes_without_gpu():
     lib = bt.kernel_lib()
     err = lambda: lib.bt_last_error_string().decode()
-    assert lib.bt_gemm(None, None, None, None, 4, 8, 64, None) == 1 and "null pointer" in err()
+    assert lib.bt_gemm(None, None, None, None, 4, 0, 8, 64, None) == 1 and "null pointer" in err()
     p = ctypes.c_void_p(256)   # never dereferenced: validation fails first
-    assert lib.bt_gemm(p, p, p, None, 4, 8, 100, None) == 2 and "multiple of 64" in err()
-    assert lib.bt_gemm(p, p, p, None, 4, 12, 64, None) == 2 and "multiple of 8" in err()
-    assert lib.bt_gemm_qkv_bias_split(p, None, p, p, p, None, 4, 12, 32, None) == 2
+    assert lib.bt_gemm(p, p, p, None, 4, 0, 8, 100, None) == 2 and "multiple of 64" in err()
+    assert lib.bt_gemm(p, p, p, None, 4, 0, 12, 64, None) == 2 and "multiple of 8" in err()
+    assert lib.bt_gemm_qkv_bias_split(p, None, p, p, p, None, 4, 0, 12, 32, None) == 2
     assert "size_per_head=32" in err()
-    assert lib.bt_gemm_qkv_bias_split(p, p, p, p, p, None, 4, 12, 64, None) == 1
+    assert lib.bt_gemm_qkv_bias_split(p, p, p, p, p, None, 4, 0, 12, 64, None) == 1
     assert "needs valid_rows" in err()
     assert lib.bt_attention_short(p, p, p, 1, 1024, 1024, 12, 64, 0.125, 0, None) == 2
     assert "exceeds 512" in err()

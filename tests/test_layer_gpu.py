@@ -209,6 +209,14 @@ def test_th_op_prepack_cache_tracks_weight_updates(device):
     c = op(2, 64, *w, x, m, True, True)
     assert not torch.equal(a, c)
     _check(c.cpu().numpy(), _oracle(wl), wl.lens, tag="cache/after-inplace-update")
+    # in-place change of the mask: the cached offsets of that mask tensor must go
+    new_lens = np.array([30, 64, 10, 50])
+    m.copy_(_dev(workload.make_mask(new_lens, 64, np.float16), device))
+    wl_m = workload.Workload(wl.cfg, new_lens, wl.x, workload.make_mask(new_lens, 64, np.float16),
+                             wl.layers)
+    e = op(2, 64, *w, x, m, True, True)
+    _check(e.cpu().numpy(), _oracle(wl_m), new_lens, tag="cache/after-mask-update")
+    m.copy_(_dev(wl.mask, device))
     # brand-new tensors (old ones freed, addresses may be recycled)
     for _ in range(3):
         wl2 = workload.make_workload(workload.EncoderConfig("pc2", 4, 64, 2, layers=1,
