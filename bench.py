@@ -113,16 +113,19 @@ def kernel_table(wl, dev, iters):
         ("compress", lambda: ops.compress(x, batch_idx, word_idx, out=packed), "hbm",
          2 * M * H * 2 + 4 * M),
         ("gemm_qkv_bias_split", lambda: ops.gemm_qkv_bias_split(
-            x2d, wt_qkv, w["qkv_bias"], heads, valid_rows=vr, out=qkv, a_row_index=word_idx),
+            x2d, wt_qkv, w["qkv_bias"], heads, valid_rows=vr, out=qkv, a_row_index=word_idx,
+            rows_hint=M),
          "mfma", 2 * M * H * 3 * H),
         ("attention", lambda: att_fn(qkv, batch_idx, B, S, scale, out=att), "mfma", 4 * H * sq),
-        ("gemm_proj", lambda: ops.gemm(att, wt_o, valid_rows=vr, out=proj), "mfma", 2 * M * H * H),
+        ("gemm_proj", lambda: ops.gemm(att, wt_o, valid_rows=vr, out=proj, rows_hint=M), "mfma",
+         2 * M * H * H),
         ("layernorm", lambda: ops.add_bias_residual_layernorm(
             ln_buf, x2d, w["attr_output_bias"], g1, b1, valid_rows=vr, residual_row_index=word_idx),
          "hbm", 3 * M * H * 2),
         ("gemm_bias_gelu", lambda: ops.gemm_bias_gelu(proj, wt_1, w["inter_bias"], valid_rows=vr,
-                                                      out=inter), "mfma", 2 * M * H * F),
-        ("gemm_ffn2", lambda: ops.gemm(inter, wt_2, valid_rows=vr, out=ffn2), "mfma",
+                                                      out=inter, rows_hint=M), "mfma",
+         2 * M * H * F),
+        ("gemm_ffn2", lambda: ops.gemm(inter, wt_2, valid_rows=vr, out=ffn2, rows_hint=M), "mfma",
          2 * M * F * H),
         ("layernorm_restore", lambda: ops.add_bias_residual_layernorm_restore(
             ffn2, proj, w["output_bias"], g1, b1, batch_idx, B, S, out_padded=out_pad),
