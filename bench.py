@@ -88,7 +88,8 @@ def kernel_table(wl, dev, iters):
     t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dev)
     w = {k: t(v) for k, v in wl.layers[0].items()}
     x, mask = t(wl.x), t(wl.mask)
-    batch_idx, word_idx, _ = ops.build_offsets(mask)
+    seq_order = torch.empty(B, dtype=torch.int32, device=dev)
+    batch_idx, word_idx, _ = ops.build_offsets(mask, seq_order=seq_order)
     vr = batch_idx[B:]
     packed = ops.compress(x, batch_idx, word_idx)
     wt_qkv, wt_o = ops.transpose_weight(w["qkv_kernel"]), ops.transpose_weight(w["attr_output_kernel"])
@@ -116,7 +117,8 @@ def kernel_table(wl, dev, iters):
             x2d, wt_qkv, w["qkv_bias"], heads, valid_rows=vr, out=qkv, a_row_index=word_idx,
             rows_hint=M),
          "mfma", 2 * M * H * 3 * H),
-        ("attention", lambda: att_fn(qkv, batch_idx, B, S, scale, out=att), "mfma", 4 * H * sq),
+        ("attention", lambda: att_fn(qkv, batch_idx, B, S, scale, out=att, seq_order=seq_order),
+         "mfma", 4 * H * sq),
         ("gemm_proj", lambda: ops.gemm(att, wt_o, valid_rows=vr, out=proj, rows_hint=M), "mfma",
          2 * M * H * H),
         ("layernorm", lambda: ops.add_bias_residual_layernorm(

@@ -33,7 +33,7 @@ KERNEL_ABI = {
     "bt_version": (c_int, []),
     "bt_last_error_string": (c_char_p, []),
     "bt_set_option": (c_int, [c_char_p, c_int]),
-    "bt_build_offsets": (c_int, [_P, c_int, c_int, c_int, _IP, _IP, POINTER(c_int), _P]),
+    "bt_build_offsets": (c_int, [_P, c_int, c_int, c_int, _IP, _IP, _IP, POINTER(c_int), _P]),
     "bt_compress": (c_int, [_P, _P, _IP, _IP, c_int, c_int, c_int, _P]),
     "bt_transpose_weight": (c_int, [_P, _P, c_int, c_int, _P]),
     "bt_transpose_weights": (c_int, [c_int, POINTER(c_void_p), POINTER(c_void_p), POINTER(c_int),
@@ -42,9 +42,9 @@ KERNEL_ABI = {
     "bt_gemm_bias_gelu": (c_int, [_P, _P, _P, _P, _IP, c_int, c_int, c_int, c_int, _P]),
     "bt_gemm_qkv_bias_split": (c_int, [_P, _IP, _P, _P, _P, _IP, c_int, c_int, c_int, c_int,
                                        _P]),
-    "bt_attention_short": (c_int, [_P, _P, _IP, c_int, c_int, c_int, c_int, c_int, c_float,
+    "bt_attention_short": (c_int, [_P, _P, _IP, _IP, c_int, c_int, c_int, c_int, c_int, c_float,
                                    c_int, _P]),
-    "bt_attention_grouped": (c_int, [_P, _P, _IP, c_int, c_int, c_int, c_int, c_int, c_float,
+    "bt_attention_grouped": (c_int, [_P, _P, _IP, _IP, c_int, c_int, c_int, c_int, c_int, c_float,
                                      c_int, _P]),
     "bt_add_bias_residual_layernorm": (c_int, [_P, _P, _IP, _P, _P, _P, c_int, _IP, c_int, c_int,
                                                c_float, _P]),

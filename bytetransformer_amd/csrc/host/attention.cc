@@ -24,13 +24,13 @@ void Attention<OpType>::infer(AttentionInferParam infer_param) {
   const int padded_rows = is_remove_padding_ ? 0 : 1;
   if (uses_short_kernel(infer_param.seq_len))
     check_bt_error(bt_attention_short(infer_param.qkv, infer_param.attention_output,
-                                      infer_param.et_param.batch_idx, infer_param.batch_size,
-                                      infer_param.seq_len, rows_cap, head_num_, size_per_head_,
+                                      infer_param.et_param.batch_idx, infer_param.seq_order,
+                                      infer_param.batch_size, infer_param.seq_len, rows_cap, head_num_, size_per_head_,
                                       scale, padded_rows, infer_param.stream));
   else
     check_bt_error(bt_attention_grouped(infer_param.qkv, infer_param.attention_output,
-                                        infer_param.et_param.batch_idx, infer_param.batch_size,
-                                        infer_param.seq_len, rows_cap, head_num_, size_per_head_,
+                                        infer_param.et_param.batch_idx, infer_param.seq_order,
+                                        infer_param.batch_size, infer_param.seq_len, rows_cap, head_num_, size_per_head_,
                                         scale, padded_rows, infer_param.stream));
 }
 

@@ -49,7 +49,8 @@ void BertTransformer<OpType>::bert_infer(BertTransformerInferParam infer_param) 
   et_param.word_idx = (int *)(base + off);
   et_param.batch_idx = et_param.word_idx + max_rows;
   et_param.valid_word_num = rows;
-  off += align_up(max_rows * 2 * sizeof(int) + 2 * sizeof(int), 256);
+  int *seq_order = et_param.batch_idx + max_rows;   // int[max_batch_size]
+  off += align_up((max_rows * 2 + 2 * (unsigned long long)max_batch_size_ + 2) * sizeof(int), 256);
   DataType_ *wt_qkv = (DataType_ *)(base + off);
   DataType_ *wt_proj = wt_qkv + (size_t)3 * hidden * hidden;
   DataType_ *wt_inter = wt_proj + (size_t)hidden * hidden;
@@ -61,9 +62,11 @@ void BertTransformer<OpType>::bert_infer(BertTransformerInferParam infer_param) 
   if (infer_param.offsets && infer_param.offsets->batch_idx && infer_param.offsets->word_idx) {
     et_param = *infer_param.offsets;
     rows_hint = et_param.valid_word_num;
+    seq_order = const_cast<int *>(infer_param.seq_order);
   } else {
     check_bt_error(bt_build_offsets(atten_mask, Traits_::dtype, batch_size, seq_len,
-                                    et_param.batch_idx, et_param.word_idx, nullptr, stream));
+                                    et_param.batch_idx, et_param.word_idx, seq_order, nullptr,
+                                    stream));
   }
   const int *valid_rows = nullptr;
   const int *gather = nullptr;
@@ -105,6 +108,7 @@ void BertTransformer<OpType>::bert_infer(BertTransformerInferParam infer_param) 
         infer_param.cublas_handle, stream, et_param
   };
   attention_infer_param.attention_bias = infer_param.attention_bias;
+  attention_infer_param.seq_order = seq_order;
   attention_layer_->infer(attention_infer_param);
 
   check_bt_error(

@@ -43,6 +43,7 @@ struct AttArgs {
   const half_t *qkv;   // [3][heads][rows_cap][64]
   half_t *out;         // [rows, heads*64]
   const int *batch_idx;
+  const int *seq_order;   // optional: grid z -> sequence, longest first (null = identity)
   int B, S, rows_cap, heads;
   float scale_log2e;   // scale * log2(e)
   int padded_rows;
@@ -101,7 +102,7 @@ __global__ __launch_bounds__(kAttThreads, 2) void attention_grouped_kernel(AttAr
   constexpr int BQ = 4 * QB * 16;
   __shared__ __attribute__((aligned(1024))) half_t ring[kAttStages * 2 * kTileHalfs];
 
-  const int b = blockIdx.z, head = blockIdx.y;
+  const int b = p.seq_order ? p.seq_order[blockIdx.z] : blockIdx.z, head = blockIdx.y;
   const int seq_start = p.batch_idx[b];
   const int klen = p.batch_idx[b + 1] - seq_start;
   const int row_start = p.padded_rows ? b * p.S : seq_start;
@@ -301,7 +302,7 @@ __global__ __launch_bounds__(kAttThreads) void attention_short_kernel(AttArgs p)
   half_t *sK = att_smem;                      // [KEYS][64] swizzled
   half_t *sV = att_smem + KEYS * kHeadDim;    // [KEYS][64] swizzled
 
-  const int b = blockIdx.z, head = blockIdx.y;
+  const int b = p.seq_order ? p.seq_order[blockIdx.z] : blockIdx.z, head = blockIdx.y;
   const int seq_start = p.batch_idx[b];
   const int klen = p.batch_idx[b + 1] - seq_start;
   const int row_start = p.padded_rows ? b * p.S : seq_start;
@@ -443,7 +444,8 @@ static int launch_short(const AttArgs &a, hipStream_t s) {
 using namespace bt;
 
 extern "C" int bt_attention_short(const void *qkv_heads, void *attention_output,
-                                  const int *batch_idx, int batch_size, int seq_len, int rows_cap,
+                                  const int *batch_idx, const int *seq_order, int batch_size,
+                                  int seq_len, int rows_cap,
                                   int head_num, int size_per_head, float scale, int padded_rows,
                                   void *stream) {
   int rc = check_att_args("bt_attention_short", qkv_heads, attention_output, batch_idx,
@@ -451,7 +453,7 @@ extern "C" int bt_attention_short(const void *qkv_heads, void *attention_output,
   if (rc) return rc;
   BT_REQUIRE(seq_len <= 512, BT_ERR_UNSUPPORTED,
              "bt_attention_short: seq_len=%d exceeds 512, use bt_attention_grouped", seq_len);
-  AttArgs a{(const half_t *)qkv_heads, (half_t *)attention_output, batch_idx, batch_size, seq_len,
+  AttArgs a{(const half_t *)qkv_heads, (half_t *)attention_output, batch_idx, seq_order, batch_size, seq_len,
             rows_cap, head_num, scale * kLog2e, padded_rows};
   hipStream_t s = as_stream(stream);
   if (seq_len <= 64) return launch_short<4>(a, s);
@@ -462,13 +464,13 @@ extern "C" int bt_attention_short(const void *qkv_heads, void *attention_output,
 }
 
 extern "C" int bt_attention_grouped(const void *qkv_heads, void *attention_output,
-                                    const int *batch_idx, int batch_size, int seq_len,
-                                    int rows_cap, int head_num, int size_per_head, float scale,
+                                    const int *batch_idx, const int *seq_order, int batch_size,
+                                    int seq_len, int rows_cap, int head_num, int size_per_head, float scale,
                                     int padded_rows, void *stream) {
   int rc = check_att_args("bt_attention_grouped", qkv_heads, attention_output, batch_idx,
                           batch_size, seq_len, rows_cap, head_num, size_per_head);
   if (rc) return rc;
-  AttArgs a{(const half_t *)qkv_heads, (half_t *)attention_output, batch_idx, batch_size, seq_len,
+  AttArgs a{(const half_t *)qkv_heads, (half_t *)attention_output, batch_idx, seq_order, batch_size, seq_len,
             rows_cap, head_num, scale * kLog2e, padded_rows};
   hipStream_t s = as_stream(stream);
   // 128-query tiles once there is enough work to fill the chip, else 64

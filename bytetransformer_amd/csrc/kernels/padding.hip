@@ -42,8 +42,8 @@ constexpr int kOffsetWaves = kOffsetThreads / kWave;
 // as the batch.
 template <typename T>
 __global__ __launch_bounds__(kOffsetThreads) void build_offsets_kernel(
-    const T *__restrict__ mask, int *__restrict__ batch_idx, int *__restrict__ word_idx, int B,
-    int S) {
+    const T *__restrict__ mask, int *__restrict__ batch_idx, int *__restrict__ word_idx,
+    int *__restrict__ seq_order, int B, int S) {
   extern __shared__ int smem[];
   int *s_len = smem;          // [B]
   int *s_off = smem + B;      // [B + 1]
@@ -78,8 +78,20 @@ __global__ __launch_bounds__(kOffsetThreads) void build_offsets_kernel(
   }
   __syncthreads();
 
-  if (blockIdx.x == 0)
+  if (blockIdx.x == 0) {
     for (int i = tid; i <= B; i += kOffsetThreads) batch_idx[i] = s_off[i];
+    // sequences by descending length (ties by index): rank by counting
+    if (seq_order)
+      for (int b = tid; b < B; b += kOffsetThreads) {
+        const int len = s_len[b];
+        int rank = 0;
+        for (int o = 0; o < B; ++o) {
+          const int lo = s_len[o];
+          rank += (lo > len) || (lo == len && o < b);
+        }
+        seq_order[rank] = b;
+      }
+  }
 
   for (int b = blockIdx.x; b < B; b += gridDim.x) {
     const int off = s_off[b], len = s_len[b];
@@ -130,7 +142,7 @@ extern "C" int bt_set_option(const char *name, int value) {
 }
 
 extern "C" int bt_build_offsets(const void *atten_mask, int mask_dtype, int batch_size,
-                                int seq_len, int *batch_idx, int *word_idx,
+                                int seq_len, int *batch_idx, int *word_idx, int *seq_order,
                                 int *valid_word_num_host, void *stream) {
   BT_REQUIRE(atten_mask && batch_idx && word_idx, BT_ERR_INVALID_ARGUMENT,
              "bt_build_offsets: null pointer argument");
@@ -147,10 +159,10 @@ extern "C" int bt_build_offsets(const void *atten_mask, int mask_dtype, int batc
   const int grid = batch_size < 64 ? batch_size : 64;
   if (mask_dtype == BT_F16)
     build_offsets_kernel<half_t><<<grid, kOffsetThreads, smem, s>>>(
-        (const half_t *)atten_mask, batch_idx, word_idx, batch_size, seq_len);
+        (const half_t *)atten_mask, batch_idx, word_idx, seq_order, batch_size, seq_len);
   else
     build_offsets_kernel<float><<<grid, kOffsetThreads, smem, s>>>(
-        (const float *)atten_mask, batch_idx, word_idx, batch_size, seq_len);
+        (const float *)atten_mask, batch_idx, word_idx, seq_order, batch_size, seq_len);
   BT_CHECK_LAUNCH("build_offsets_kernel");
   if (valid_word_num_host) {
     hipError_t e = hipMemcpyAsync(valid_word_num_host, batch_idx + batch_size, sizeof(int),

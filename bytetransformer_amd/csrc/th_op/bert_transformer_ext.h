@@ -94,6 +94,7 @@ class BTEncoder : public IBTEncoder {
       offsets.word_idx = plan.word_idx.data_ptr<int>();
       offsets.valid_word_num = plan.valid_word_num;
       infer_param.offsets = &offsets;
+      infer_param.seq_order = plan.seq_order.data_ptr<int>();
     }
     encoder.infer(infer_param);
   }
@@ -143,9 +144,11 @@ class BTEncoder : public IBTEncoder {
     auto opts = torch::dtype(torch::kInt32).device(mask.device());
     plan->batch_idx = torch::empty({(int64_t)batch_size + 1}, opts);
     plan->word_idx = torch::empty({(int64_t)batch_size * seq_len}, opts);
+    plan->seq_order = torch::empty({(int64_t)batch_size}, opts);
     check_bt_error(bt_build_offsets(mask.data_ptr(), BT_F16, batch_size, seq_len,
                                     plan->batch_idx.data_ptr<int>(), plan->word_idx.data_ptr<int>(),
-                                    &plan->valid_word_num, stream));
+                                    plan->seq_order.data_ptr<int>(), &plan->valid_word_num,
+                                    stream));
     cache.store(mask, stream, *plan);
     return true;
   }

@@ -115,7 +115,7 @@ class PrepackCache {
 class MaskPlanCache {
  public:
   struct Plan {
-    torch::Tensor batch_idx, word_idx;
+    torch::Tensor batch_idx, word_idx, seq_order;
     int valid_word_num = 0;
   };
 

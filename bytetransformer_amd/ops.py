@@ -46,7 +46,7 @@ def set_option(name, value):
     _check(kernel_lib().bt_set_option(name.encode(), int(value)))
 
 
-def build_offsets(mask, want_count=False, out=None):
+def build_offsets(mask, want_count=False, out=None, seq_order=None):
     """mask [B,S,S] -> (batch_idx int32[B+1], word_idx int32[B*S], M or None)."""
     B, S = mask.shape[0], mask.shape[1]
     if out is None:
@@ -56,7 +56,7 @@ def build_offsets(mask, want_count=False, out=None):
         batch_idx, word_idx = out
     cnt = ctypes.c_int(-1)
     _check(kernel_lib().bt_build_offsets(_ptr(mask), _dtype_code(mask), B, S, _ptr(batch_idx),
-                                         _ptr(word_idx),
+                                         _ptr(word_idx), _ptr(seq_order),
                                          ctypes.byref(cnt) if want_count else None, _stream()))
     return batch_idx, word_idx, (cnt.value if want_count else None)
 
@@ -125,24 +125,27 @@ def gemm_qkv_bias_split(a, wt_qkv, bias_qkv, head_num, size_per_head=64, valid_r
     return out
 
 
-def _attention(fn, qkv_heads, batch_idx, batch_size, seq_len, scale, padded_rows, out):
+def _attention(fn, qkv_heads, batch_idx, batch_size, seq_len, scale, padded_rows, out,
+               seq_order=None):
     _, head_num, rows_cap, d = qkv_heads.shape
     if out is None:
         out = torch.zeros(rows_cap, head_num * d, dtype=qkv_heads.dtype, device=qkv_heads.device)
-    _check(fn(_ptr(qkv_heads), _ptr(out), _ptr(batch_idx), batch_size, seq_len, rows_cap,
+    _check(fn(_ptr(qkv_heads), _ptr(out), _ptr(batch_idx), _ptr(seq_order), batch_size, seq_len,
+              rows_cap,
               head_num, d, float(scale), int(padded_rows), _stream()))
     return out
 
 
-def attention_short(qkv_heads, batch_idx, batch_size, seq_len, scale, padded_rows=False, out=None):
+def attention_short(qkv_heads, batch_idx, batch_size, seq_len, scale, padded_rows=False, out=None,
+                    seq_order=None):
     return _attention(kernel_lib().bt_attention_short, qkv_heads, batch_idx, batch_size, seq_len,
-                      scale, padded_rows, out)
+                      scale, padded_rows, out, seq_order)
 
 
 def attention_grouped(qkv_heads, batch_idx, batch_size, seq_len, scale, padded_rows=False,
-                      out=None):
+                      out=None, seq_order=None):
     return _attention(kernel_lib().bt_attention_grouped, qkv_heads, batch_idx, batch_size,
-                      seq_len, scale, padded_rows, out)
+                      seq_len, scale, padded_rows, out, seq_order)
 
 
 def add_bias_residual_layernorm(out, residual, bias, gamma, beta, eps=1e-6, valid_rows=None,

@@ -60,11 +60,15 @@ int bt_set_option(const char *name, int value);
  *               only row 0 of each batch is read; an element counts when >= 0.5
  *   batch_idx   int[batch_size + 1]  exclusive prefix sum of the lengths, total last
  *   word_idx    int[batch_size * seq_len]; first M entries = b*seq_len + i, i < len_b
+ *   seq_order   NULL, or int[batch_size]: the sequence indices by descending
+ *               length (ties by index); the attention kernels use it to start the
+ *               longest sequences first (no counterpart in the reference)
  *   valid_word_num_host  NULL, or a host int that receives M; passing it makes
  *               the call wait for the stream (the reference always does)
  */
 int bt_build_offsets(const void *atten_mask, int mask_dtype, int batch_size, int seq_len,
-                     int *batch_idx, int *word_idx, int *valid_word_num_host, void *stream);
+                     int *batch_idx, int *word_idx, int *seq_order, int *valid_word_num_host,
+                     void *stream);
 
 /*
  * Gather valid rows: to_tensor[t, :] = from_tensor[word_idx[t], :], t < M.
@@ -132,6 +136,9 @@ int bt_gemm_qkv_bias_split(const void *a, const int *a_row_index, const void *wt
  *   padded_rows == 0: sequence b owns packed rows [batch_idx[b], batch_idx[b+1])
  *   padded_rows != 0: sequence b owns rows [b*seq_len, (b+1)*seq_len), all
  *                     seq_len query rows are computed against the len_b keys
+ *   seq_order (nullable): a permutation of the sequence indices from
+ *                     bt_build_offsets; workgroups are issued in that order so the
+ *                     longest sequences start first.  Results do not depend on it.
  *
  * bt_attention_short keeps the whole logits row of a query tile in registers
  * (exact two-pass softmax, seq_len <= 512).  Replaces wmma_attention[_rm]_kernel
@@ -145,12 +152,14 @@ int bt_gemm_qkv_bias_split(const void *a, const int *a_row_index, const void *wt
  * the logits round trip through HBM.
  */
 int bt_attention_short(const void *qkv_heads, void *attention_output, const int *batch_idx,
-                       int batch_size, int seq_len, int rows_cap, int head_num,
-                       int size_per_head, float scale, int padded_rows, void *stream);
+                       const int *seq_order, int batch_size, int seq_len, int rows_cap,
+                       int head_num, int size_per_head, float scale, int padded_rows,
+                       void *stream);
 
 int bt_attention_grouped(const void *qkv_heads, void *attention_output, const int *batch_idx,
-                         int batch_size, int seq_len, int rows_cap, int head_num,
-                         int size_per_head, float scale, int padded_rows, void *stream);
+                         const int *seq_order, int batch_size, int seq_len, int rows_cap,
+                         int head_num, int size_per_head, float scale, int padded_rows,
+                         void *stream);
 
 /*
  * out = LayerNorm((out + residual) + bias) * gamma + beta, in place on `out`,

@@ -35,6 +35,9 @@ struct AttentionInferParam {
   const T *attention_bias = nullptr;         // [head_num, seq_len, seq_len]; must be null
   const uint32_t *position_ids = nullptr;    // never read
   const uint32_t *token_type_ids = nullptr;  // never read
+  // Extension: sequence indices by descending length from bt_build_offsets; the
+  // kernels then start the longest sequences first.  May be null.
+  const int *seq_order = nullptr;
 };
 
 template <OperationType OpType>

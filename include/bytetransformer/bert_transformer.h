@@ -65,6 +65,8 @@ struct BertTransformerInferParam {
   // int[batch_size*seq_len], valid_word_num = their total).  When set, infer()
   // skips its own mask prefix sum and uses valid_word_num to pick tile shapes.
   const ET_Param *offsets = NULL;
+  // ... and the matching sequence order (int[batch_size], longest first), or NULL.
+  const int *seq_order = NULL;
 };
 
 template <OperationType OpType>
@@ -127,7 +129,7 @@ class BertTransformer {
 
   // Scratch layout (elements of DataType_, T = max_batch*max_seq*hidden):
   //   [0,3T) qkv heads | [3T,4T) attention out | [4T,5T) projection / LN1 |
-  //   [5T,(5+mult)T) FFN1 | word_idx int[B*S] | batch_idx int[B*S] |
+  //   [5T,(5+mult)T) FFN1 | word_idx int[B*S] | batch_idx int[B*S] | seq order int[B] |
   //   pre-packed weights (3+1+2*mult)*H*H | attention scratch (none)
   unsigned long long cal_bufsize() {
     const unsigned long long rows = (unsigned long long)max_batch_size_ * max_seq_len_;
@@ -135,7 +137,7 @@ class BertTransformer {
     const unsigned long long tensor = rows * hidden;
     inner_buf_size_ = (5 + param_.intermediate_size) * tensor * sizeof(DataType_);
     inner_buf_size_ = align_up(inner_buf_size_, 256);
-    inner_buf_size_ += align_up(rows * 2 * sizeof(int) + 2 * sizeof(int), 256);
+    inner_buf_size_ += align_up((rows * 2 + 2 * max_batch_size_ + 2) * sizeof(int), 256);
     inner_buf_size_ += align_up(
         (4 + 2 * (unsigned long long)param_.intermediate_size) * hidden * hidden *
             sizeof(DataType_),

@@ -50,12 +50,12 @@ def test_argument_validation_returns_codes_without_gpu():
     assert "size_per_head=32" in err()
     assert lib.bt_gemm_qkv_bias_split(p, p, p, p, p, None, 4, 0, 12, 64, None) == 1
     assert "needs valid_rows" in err()
-    assert lib.bt_attention_short(p, p, p, 1, 1024, 1024, 12, 64, 0.125, 0, None) == 2
+    assert lib.bt_attention_short(p, p, p, None, 1, 1024, 1024, 12, 64, 0.125, 0, None) == 2
     assert "exceeds 512" in err()
-    assert lib.bt_attention_grouped(p, p, p, 1, 16, 16, 12, 48, 0.125, 0, None) == 2
+    assert lib.bt_attention_grouped(p, p, p, None, 1, 16, 16, 12, 48, 0.125, 0, None) == 2
     assert lib.bt_compress(p, p, p, p, 2, 4, 12, None) == 2 and "multiple of 8" in err()
-    assert lib.bt_build_offsets(p, 7, 2, 4, p, p, None, None) == 1 and "dtype" in err()
-    assert lib.bt_build_offsets(p, 1, 0, 4, p, p, None, None) == 1
+    assert lib.bt_build_offsets(p, 7, 2, 4, p, p, None, None, None) == 1 and "dtype" in err()
+    assert lib.bt_build_offsets(p, 1, 0, 4, p, p, None, None, None) == 1
     assert lib.bt_add_bias_residual_layernorm(p, p, None, p, p, p, 0, None, 4, 12, 1e-6, None) == 2
     assert lib.bt_add_bias_residual_layernorm(p, p, None, p, p, p, 0, None, 4, 8192, 1e-6, None) == 2
     assert lib.bt_add_bias_residual_layernorm_restore(p, p, p, p, p, 0, None, p, 2, 4, 64, 1e-6,
@@ -70,7 +70,7 @@ def test_encoder_c_api_validation_and_bufsize():
     T = 16 * 512 * 768
     # nine activation tensors + two index arrays + the pre-packed weights
     assert need >= 9 * T * 2 + 2 * 16 * 512 * 4 + 12 * 768 * 768 * 2
-    assert need < 9 * T * 2 + 2 * 16 * 512 * 4 + 12 * 768 * 768 * 2 + 4096
+    assert need < 9 * T * 2 + 2 * 16 * 512 * 4 + 12 * 768 * 768 * 2 + 8192
     bad = _lib.EncoderConfig(0, 16, 512, 12, 64, 4, 1, 1, 0, 1.0, 1e-6)   # fp32: not implemented
     assert lib.bt_encoder_bufsize(ctypes.byref(bad)) == 0
     assert b"BT_F16" in lib.bt_encoder_last_error()

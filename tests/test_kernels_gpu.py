@@ -36,8 +36,11 @@ def test_build_offsets_bit_exact(device, B, S, dtype):
     mask = workload.make_mask(lens, S, dtype)
     mask[:, 1:, :] = 1 - mask[:, 1:, :]          # rows other than 0 must be ignored
     bi, wi, M = O.build_offsets(mask)
-    g_bi, g_wi, g_M = ops.build_offsets(_dev(mask, device), want_count=True)
+    order = torch.full((B,), -1, dtype=torch.int32, device=device)
+    g_bi, g_wi, g_M = ops.build_offsets(_dev(mask, device), want_count=True, seq_order=order)
     assert g_M == M
+    # longest first, ties by index: the stable argsort of the negated lengths
+    assert order.cpu().numpy().tolist() == np.argsort(-lens.astype(np.int64), kind="stable").tolist()
     assert g_bi.dtype == torch.int32 and g_wi.dtype == torch.int32
     assert np.array_equal(g_bi.cpu().numpy(), bi)
     assert np.array_equal(g_wi.cpu().numpy()[:M], wi)
@@ -298,6 +301,10 @@ def test_attention_packed(device, kind, lens, S, heads, qb):
     try:
         out = torch.full((len(lens) * S, heads * 64), 5.0, dtype=torch.float16, device=device)
         g = fn(_dev(qkv, device), _dev(bi, device), len(lens), S, scale, False, out=out)
+        # issuing the workgroups longest-sequence-first must not change a bit
+        order = _dev(np.argsort(-np.asarray(lens), kind="stable").astype(np.int32), device)
+        g2 = fn(_dev(qkv, device), _dev(bi, device), len(lens), S, scale, False, seq_order=order)
+        assert torch.equal(g[:M], g2[:M])
         g = g.cpu().numpy()
     finally:
         ops.set_option("attention_qb", -1)
