@@ -22,14 +22,17 @@ void Attention<OpType>::infer(AttentionInferParam infer_param) {
   const int rows_cap = infer_param.batch_size * infer_param.seq_len;
   const float scale = 1.0f / std::sqrt((float)size_per_head_) / param_.tao;
   const int padded_rows = is_remove_padding_ ? 0 : 1;
+  // on padded rows the mask tensor itself is applied (any 0/1 pattern), as in the
+  // reference's non-remove-padding kernels; packed rows use the prefix lengths
+  const void *mask = is_remove_padding_ ? nullptr : (const void *)infer_param.atten_mask;
   if (uses_short_kernel(infer_param.seq_len))
     check_bt_error(bt_attention_short(infer_param.qkv, infer_param.attention_output,
-                                      infer_param.et_param.batch_idx, infer_param.seq_order,
+                                      infer_param.et_param.batch_idx, infer_param.seq_order, mask,
                                       infer_param.batch_size, infer_param.seq_len, rows_cap, head_num_, size_per_head_,
                                       scale, padded_rows, infer_param.stream));
   else
     check_bt_error(bt_attention_grouped(infer_param.qkv, infer_param.attention_output,
-                                        infer_param.et_param.batch_idx, infer_param.seq_order,
+                                        infer_param.et_param.batch_idx, infer_param.seq_order, mask,
                                         infer_param.batch_size, infer_param.seq_len, rows_cap, head_num_, size_per_head_,
                                         scale, padded_rows, infer_param.stream));
 }

@@ -44,6 +44,8 @@ struct AttArgs {
   half_t *out;         // [rows, heads*64]
   const int *batch_idx;
   const int *seq_order;   // optional: grid z -> sequence, longest first (null = identity)
+  const half_t *mask;     // optional [B,S,S] 0/1 mask, padded rows only: every key of the
+                          // sequence's S rows takes part, shifted by (mask-1)*10000
   int B, S, rows_cap, heads;
   float scale_log2e;   // scale * log2(e)
   int padded_rows;
@@ -90,6 +92,25 @@ __device__ __forceinline__ half8_t load_k_frag(const half_t *sK, int kb, int dh,
   return *(const half8_t *)(sK + row * kHeadDim + (((4 * dh + lg) ^ swz_k(row)) << 3));
 }
 
+// Additive mask term of four consecutive keys of one query row, in the exp2
+// domain: (mask - 1) * 10000 * log2(e)  (the reference's non-remove-padding
+// kernels, attention_fused.cu:234-237).  Keys at or past S get no term here; the
+// caller excludes them by index.
+__device__ __forceinline__ float4_t mask_bias4(const half_t *mask_row, int key, int S, bool vec) {
+  constexpr float kShift = 10000.0f * kLog2e;
+  float4_t m = {1.f, 1.f, 1.f, 1.f};
+  if (vec && key + 3 < S) {
+    const half4_t h = *(const half4_t *)(mask_row + key);
+#pragma unroll
+    for (int r = 0; r < 4; ++r) m[r] = (float)h[r];
+  } else {
+#pragma unroll
+    for (int r = 0; r < 4; ++r)
+      if (key + r < S) m[r] = (float)mask_row[key + r];
+  }
+  return (m - 1.0f) * kShift;
+}
+
 // ---------------------------------------------------------------------------
 // grouped / streaming kernel
 // ---------------------------------------------------------------------------
@@ -97,14 +118,15 @@ constexpr int kKT = 64;                          // keys per streamed tile
 constexpr int kTileHalfs = kKT * kHeadDim;       // one K or V tile
 constexpr int kAttStages = 3;
 
-template <int QB>  // 16-query blocks per wave; workgroup covers 4*QB*16 queries
+template <int QB, bool FULLMASK>  // QB 16-query blocks per wave; workgroup covers 4*QB*16 queries
 __global__ __launch_bounds__(kAttThreads, 2) void attention_grouped_kernel(AttArgs p) {
   constexpr int BQ = 4 * QB * 16;
   __shared__ __attribute__((aligned(1024))) half_t ring[kAttStages * 2 * kTileHalfs];
 
   const int b = p.seq_order ? p.seq_order[blockIdx.z] : blockIdx.z, head = blockIdx.y;
   const int seq_start = p.batch_idx[b];
-  const int klen = p.batch_idx[b + 1] - seq_start;
+  // with a full mask every one of the S key rows takes part
+  const int klen = FULLMASK ? p.S : p.batch_idx[b + 1] - seq_start;
   const int row_start = p.padded_rows ? b * p.S : seq_start;
   const int nq = p.padded_rows ? p.S : klen;
   const int q0 = blockIdx.x * BQ;
@@ -170,6 +192,9 @@ __global__ __launch_bounds__(kAttThreads, 2) void attention_grouped_kernel(AttAr
   if (ntiles > 1) issue_tile(1, 1);
 
   const float c = p.scale_log2e;
+  // after the mask term is folded in, the logits already are in the exp2 domain
+  const float cs = FULLMASK ? 1.0f : c;
+  const bool mask_vec = (p.S & 3) == 0;
   int stage = 0;
 
   auto process_tile = [&](int t, auto masked_tag) {
@@ -202,6 +227,20 @@ __global__ __launch_bounds__(kAttThreads, 2) void attention_grouped_kernel(AttAr
         s[kb][qb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kf1, qf[qb][1], s[kb][qb], 0, 0, 0);
       }
     }
+    if (FULLMASK) {
+      const int k0 = t * kKT;
+#pragma unroll
+      for (int qb = 0; qb < QB; ++qb) {
+        const int q = min(q0 + (wave * QB + qb) * 16 + lq, p.S - 1);
+        const half_t *mrow = p.mask + ((size_t)b * p.S + q) * p.S;
+#pragma unroll
+        for (int kb = 0; kb < 4; ++kb) {
+          const float4_t bias = mask_bias4(mrow, k0 + kb * 16 + lg * 4, p.S, mask_vec);
+#pragma unroll
+          for (int r = 0; r < 4; ++r) s[kb][qb][r] = __builtin_fmaf(s[kb][qb][r], c, bias[r]);
+        }
+      }
+    }
     if (MASKED) {
       const int k0 = t * kKT;
 #pragma unroll
@@ -227,10 +266,10 @@ __global__ __launch_bounds__(kAttThreads, 2) void attention_grouped_kernel(AttAr
       mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
       mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
       const float m_new = fmaxf(m_run[qb], mx);
-      const float mc = m_new * c;
+      const float mc = m_new * cs;
       // rescale the running output only when some query's maximum moved
       if (__builtin_amdgcn_ballot_w64(m_new != m_run[qb]) != 0) {
-        const float alpha = fast_exp2(m_run[qb] * c - mc);
+        const float alpha = fast_exp2(m_run[qb] * cs - mc);
 #pragma unroll
         for (int db = 0; db < 5; ++db) o[db][qb] *= alpha;
       }
@@ -239,7 +278,7 @@ __global__ __launch_bounds__(kAttThreads, 2) void attention_grouped_kernel(AttAr
       for (int kb = 0; kb < 4; ++kb) {
         float e[4];
 #pragma unroll
-        for (int r = 0; r < 4; ++r) e[r] = fast_exp2(__builtin_fmaf(s[kb][qb][r], c, -mc));
+        for (int r = 0; r < 4; ++r) e[r] = fast_exp2(__builtin_fmaf(s[kb][qb][r], cs, -mc));
         const half2_t h01 = __builtin_convertvector(float2_t{e[0], e[1]}, half2_t);
         const half2_t h23 = __builtin_convertvector(float2_t{e[2], e[3]}, half2_t);
         pf[kb >> 1][qb][(kb & 1) * 4 + 0] = h01[0];
@@ -294,7 +333,7 @@ __global__ __launch_bounds__(kAttThreads, 2) void attention_grouped_kernel(AttAr
 // ---------------------------------------------------------------------------
 // short kernel: K, V resident in LDS, logits of the query tile in registers
 // ---------------------------------------------------------------------------
-template <int NKB>  // capacity in 16-key blocks (keys <= 16*NKB), NKB even
+template <int NKB, bool FULLMASK>  // capacity in 16-key blocks (keys <= 16*NKB), NKB even
 __global__ __launch_bounds__(kAttThreads) void attention_short_kernel(AttArgs p) {
   constexpr int KEYS = NKB * 16;
   constexpr int BQ = 64;  // 4 waves x 16 queries
@@ -304,7 +343,7 @@ __global__ __launch_bounds__(kAttThreads) void attention_short_kernel(AttArgs p)
 
   const int b = p.seq_order ? p.seq_order[blockIdx.z] : blockIdx.z, head = blockIdx.y;
   const int seq_start = p.batch_idx[b];
-  const int klen = p.batch_idx[b + 1] - seq_start;
+  const int klen = FULLMASK ? p.S : p.batch_idx[b + 1] - seq_start;
   const int row_start = p.padded_rows ? b * p.S : seq_start;
   const int nq = p.padded_rows ? p.S : klen;
   const int q0 = blockIdx.x * BQ;
@@ -357,6 +396,18 @@ __global__ __launch_bounds__(kAttThreads) void attention_short_kernel(AttArgs p)
     }
   }
 
+  const float c = p.scale_log2e;
+  const float cs = FULLMASK ? 1.0f : c;
+  if (FULLMASK) {
+    const half_t *mrow = p.mask + ((size_t)b * p.S + min(q, p.S - 1)) * p.S;
+    const bool mask_vec = (p.S & 3) == 0;
+#pragma unroll
+    for (int kb = 0; kb < NKB; ++kb) {
+      const float4_t bias = mask_bias4(mrow, kb * 16 + lg * 4, p.S, mask_vec);
+#pragma unroll
+      for (int r = 0; r < 4; ++r) s[kb][r] = __builtin_fmaf(s[kb][r], c, bias[r]);
+    }
+  }
   // exact softmax over the row: mask by index, max, exp, sum, normalise, round
   float mx = kNegBig;
 #pragma unroll
@@ -368,14 +419,13 @@ __global__ __launch_bounds__(kAttThreads) void attention_short_kernel(AttArgs p)
     }
   mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
   mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-  const float c = p.scale_log2e;
-  const float mc = mx * c;
+  const float mc = mx * cs;
   float sum = 0.f;
 #pragma unroll
   for (int kb = 0; kb < NKB; ++kb)
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
-      s[kb][r] = fast_exp2(__builtin_fmaf(s[kb][r], c, -mc));
+      s[kb][r] = fast_exp2(__builtin_fmaf(s[kb][r], cs, -mc));
       sum += s[kb][r];
     }
   sum += __shfl_xor(sum, 16, 64);
@@ -411,7 +461,10 @@ __global__ __launch_bounds__(kAttThreads) void attention_short_kernel(AttArgs p)
 }
 
 static int check_att_args(const char *who, const void *qkv, const void *out, const int *batch_idx,
-                          int B, int S, int rows_cap, int heads, int d) {
+                          const void *mask, int padded_rows, int B, int S, int rows_cap,
+                          int heads, int d) {
+  BT_REQUIRE(!mask || padded_rows, BT_ERR_INVALID_ARGUMENT,
+             "%s: atten_mask is only applied on padded rows (padded_rows != 0)", who);
   BT_REQUIRE(qkv && out && batch_idx, BT_ERR_INVALID_ARGUMENT, "%s: null pointer argument", who);
   BT_REQUIRE(B > 0 && S > 0 && heads > 0 && rows_cap > 0, BT_ERR_INVALID_ARGUMENT,
              "%s: batch_size=%d seq_len=%d head_num=%d rows_cap=%d must be positive", who, B, S,
@@ -422,21 +475,26 @@ static int check_att_args(const char *who, const void *qkv, const void *out, con
   return BT_OK;
 }
 
-template <int NKB>
-static int launch_short(const AttArgs &a, hipStream_t s) {
+template <int NKB, bool FULLMASK>
+static int launch_short_impl(const AttArgs &a, hipStream_t s) {
   constexpr size_t smem = (size_t)2 * NKB * 16 * kHeadDim * sizeof(half_t);
   static_assert(smem <= 160 * 1024, "LDS budget");
   static bool configured = false;
   if (!configured) {
-    hipError_t e = hipFuncSetAttribute((const void *)attention_short_kernel<NKB>,
+    hipError_t e = hipFuncSetAttribute((const void *)attention_short_kernel<NKB, FULLMASK>,
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
     if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute(attention_short_kernel)");
     configured = true;
   }
   dim3 grid((a.S + 63) / 64, a.heads, a.B);
-  attention_short_kernel<NKB><<<grid, kAttThreads, smem, s>>>(a);
+  attention_short_kernel<NKB, FULLMASK><<<grid, kAttThreads, smem, s>>>(a);
   BT_CHECK_LAUNCH("attention_short_kernel");
   return BT_OK;
+}
+
+template <int NKB>
+static int launch_short(const AttArgs &a, hipStream_t s) {
+  return a.mask ? launch_short_impl<NKB, true>(a, s) : launch_short_impl<NKB, false>(a, s);
 }
 
 }  // namespace bt
@@ -444,16 +502,18 @@ static int launch_short(const AttArgs &a, hipStream_t s) {
 using namespace bt;
 
 extern "C" int bt_attention_short(const void *qkv_heads, void *attention_output,
-                                  const int *batch_idx, const int *seq_order, int batch_size,
-                                  int seq_len, int rows_cap,
+                                  const int *batch_idx, const int *seq_order,
+                                  const void *atten_mask, int batch_size, int seq_len,
+                                  int rows_cap,
                                   int head_num, int size_per_head, float scale, int padded_rows,
                                   void *stream) {
-  int rc = check_att_args("bt_attention_short", qkv_heads, attention_output, batch_idx,
-                          batch_size, seq_len, rows_cap, head_num, size_per_head);
+  int rc = check_att_args("bt_attention_short", qkv_heads, attention_output, batch_idx, atten_mask,
+                          padded_rows, batch_size, seq_len, rows_cap, head_num, size_per_head);
   if (rc) return rc;
   BT_REQUIRE(seq_len <= 512, BT_ERR_UNSUPPORTED,
              "bt_attention_short: seq_len=%d exceeds 512, use bt_attention_grouped", seq_len);
-  AttArgs a{(const half_t *)qkv_heads, (half_t *)attention_output, batch_idx, seq_order, batch_size, seq_len,
+  AttArgs a{(const half_t *)qkv_heads, (half_t *)attention_output, batch_idx, seq_order,
+            (const half_t *)atten_mask, batch_size, seq_len,
             rows_cap, head_num, scale * kLog2e, padded_rows};
   hipStream_t s = as_stream(stream);
   if (seq_len <= 64) return launch_short<4>(a, s);
@@ -464,13 +524,16 @@ extern "C" int bt_attention_short(const void *qkv_heads, void *attention_output,
 }
 
 extern "C" int bt_attention_grouped(const void *qkv_heads, void *attention_output,
-                                    const int *batch_idx, const int *seq_order, int batch_size,
-                                    int seq_len, int rows_cap, int head_num, int size_per_head, float scale,
+                                    const int *batch_idx, const int *seq_order,
+                                    const void *atten_mask, int batch_size, int seq_len,
+                                    int rows_cap, int head_num, int size_per_head, float scale,
                                     int padded_rows, void *stream) {
   int rc = check_att_args("bt_attention_grouped", qkv_heads, attention_output, batch_idx,
-                          batch_size, seq_len, rows_cap, head_num, size_per_head);
+                          atten_mask, padded_rows, batch_size, seq_len, rows_cap, head_num,
+                          size_per_head);
   if (rc) return rc;
-  AttArgs a{(const half_t *)qkv_heads, (half_t *)attention_output, batch_idx, seq_order, batch_size, seq_len,
+  AttArgs a{(const half_t *)qkv_heads, (half_t *)attention_output, batch_idx, seq_order,
+            (const half_t *)atten_mask, batch_size, seq_len,
             rows_cap, head_num, scale * kLog2e, padded_rows};
   hipStream_t s = as_stream(stream);
   // 128-query tiles once there is enough work to fill the chip, else 64
@@ -478,10 +541,16 @@ extern "C" int bt_attention_grouped(const void *qkv_heads, void *attention_outpu
   const int qb = option_attention_qb();
   if (qb == 2 || (qb < 0 && blocks128 >= 512)) {
     dim3 grid((seq_len + 127) / 128, head_num, batch_size);
-    attention_grouped_kernel<2><<<grid, kAttThreads, 0, s>>>(a);
+    if (a.mask)
+      attention_grouped_kernel<2, true><<<grid, kAttThreads, 0, s>>>(a);
+    else
+      attention_grouped_kernel<2, false><<<grid, kAttThreads, 0, s>>>(a);
   } else {
     dim3 grid((seq_len + 63) / 64, head_num, batch_size);
-    attention_grouped_kernel<1><<<grid, kAttThreads, 0, s>>>(a);
+    if (a.mask)
+      attention_grouped_kernel<1, true><<<grid, kAttThreads, 0, s>>>(a);
+    else
+      attention_grouped_kernel<1, false><<<grid, kAttThreads, 0, s>>>(a);
   }
   BT_CHECK_LAUNCH("attention_grouped_kernel");
   return BT_OK;

@@ -126,26 +126,26 @@ def gemm_qkv_bias_split(a, wt_qkv, bias_qkv, head_num, size_per_head=64, valid_r
 
 
 def _attention(fn, qkv_heads, batch_idx, batch_size, seq_len, scale, padded_rows, out,
-               seq_order=None):
+               seq_order=None, mask=None):
     _, head_num, rows_cap, d = qkv_heads.shape
     if out is None:
         out = torch.zeros(rows_cap, head_num * d, dtype=qkv_heads.dtype, device=qkv_heads.device)
-    _check(fn(_ptr(qkv_heads), _ptr(out), _ptr(batch_idx), _ptr(seq_order), batch_size, seq_len,
-              rows_cap,
+    _check(fn(_ptr(qkv_heads), _ptr(out), _ptr(batch_idx), _ptr(seq_order), _ptr(mask), batch_size,
+              seq_len, rows_cap,
               head_num, d, float(scale), int(padded_rows), _stream()))
     return out
 
 
 def attention_short(qkv_heads, batch_idx, batch_size, seq_len, scale, padded_rows=False, out=None,
-                    seq_order=None):
+                    seq_order=None, mask=None):
     return _attention(kernel_lib().bt_attention_short, qkv_heads, batch_idx, batch_size, seq_len,
-                      scale, padded_rows, out, seq_order)
+                      scale, padded_rows, out, seq_order, mask)
 
 
 def attention_grouped(qkv_heads, batch_idx, batch_size, seq_len, scale, padded_rows=False,
-                      out=None, seq_order=None):
+                      out=None, seq_order=None, mask=None):
     return _attention(kernel_lib().bt_attention_grouped, qkv_heads, batch_idx, batch_size,
-                      seq_len, scale, padded_rows, out, seq_order)
+                      seq_len, scale, padded_rows, out, seq_order, mask)
 
 
 def add_bias_residual_layernorm(out, residual, bias, gamma, beta, eps=1e-6, valid_rows=None,

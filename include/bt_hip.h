@@ -136,6 +136,12 @@ int bt_gemm_qkv_bias_split(const void *a, const int *a_row_index, const void *wt
  *   padded_rows == 0: sequence b owns packed rows [batch_idx[b], batch_idx[b+1])
  *   padded_rows != 0: sequence b owns rows [b*seq_len, (b+1)*seq_len), all
  *                     seq_len query rows are computed against the len_b keys
+ *   atten_mask (nullable, padded rows only): the fp16 [batch_size, seq_len, seq_len]
+ *                     0/1 mask.  When given, ALL seq_len keys of the sequence take
+ *                     part and every logit is shifted by (mask[b,q,k] - 1) * 10000
+ *                     before the softmax - the arbitrary-mask semantics of the
+ *                     reference's non-remove-padding kernels (attention_fused.cu:234-237,
+ *                     attention_fused_long.cu) - instead of the prefix-length rule.
  *   seq_order (nullable): a permutation of the sequence indices from
  *                     bt_build_offsets; workgroups are issued in that order so the
  *                     longest sequences start first.  Results do not depend on it.
@@ -152,14 +158,14 @@ int bt_gemm_qkv_bias_split(const void *a, const int *a_row_index, const void *wt
  * the logits round trip through HBM.
  */
 int bt_attention_short(const void *qkv_heads, void *attention_output, const int *batch_idx,
-                       const int *seq_order, int batch_size, int seq_len, int rows_cap,
-                       int head_num, int size_per_head, float scale, int padded_rows,
-                       void *stream);
+                       const int *seq_order, const void *atten_mask, int batch_size, int seq_len,
+                       int rows_cap, int head_num, int size_per_head, float scale,
+                       int padded_rows, void *stream);
 
 int bt_attention_grouped(const void *qkv_heads, void *attention_output, const int *batch_idx,
-                         const int *seq_order, int batch_size, int seq_len, int rows_cap,
-                         int head_num, int size_per_head, float scale, int padded_rows,
-                         void *stream);
+                         const int *seq_order, const void *atten_mask, int batch_size,
+                         int seq_len, int rows_cap, int head_num, int size_per_head, float scale,
+                         int padded_rows, void *stream);
 
 /*
  * out = LayerNorm((out + residual) + bias) * gamma + beta, in place on `out`,

@@ -340,6 +340,38 @@ def test_attention_padded_rows_mode(device, kind):
         assert err.max() <= 4e-3, (b, err.max())
 
 
+@pytest.mark.parametrize("kind,S", [("short", 64), ("short", 200), ("grouped", 200),
+                                     ("grouped", 70), ("short", 37), ("grouped", 640)])
+def test_attention_arbitrary_mask_on_padded_rows(device, kind, S):
+    """With the mask tensor given, every (query, key) pair follows mask[b,q,k]:
+    logits are shifted by (mask-1)*10000 as in the reference's non-remove-padding
+    kernels - banded, random and fully-masked rows included."""
+    _say("attention full mask", kind, S)
+    rs = np.random.RandomState(S)
+    B, heads = 3, 2
+    qkv = rs.standard_normal((3, heads, B * S, 64)).astype(np.float16)
+    mask = (rs.rand(B, S, S) < 0.6).astype(np.float16)
+    i, j = np.indices((S, S))
+    mask[1] = (np.abs(i - j) <= 5).astype(np.float16)          # banded
+    mask[2, 3, :] = 0                                          # a fully masked query row
+    mask[2, :, S // 2:] = 0                                    # a prefix-style block
+    bi = np.arange(B + 1, dtype=np.int32) * S                  # lengths are not used here
+    scale = 1 / math.sqrt(64)
+    fn = ops.attention_short if kind == "short" else ops.attention_grouped
+    g = fn(_dev(qkv, device), _dev(bi, device), B, S, scale, True, mask=_dev(mask, device))
+    g = g.cpu().numpy().astype(np.float64)
+    for b in range(B):
+        q = qkv[0, :, b * S:(b + 1) * S].astype(np.float64)
+        k = qkv[1, :, b * S:(b + 1) * S].astype(np.float64)
+        v = qkv[2, :, b * S:(b + 1) * S].astype(np.float64)
+        sc = np.einsum("hqd,hkd->hqk", q, k) * scale - 10000.0 * (1.0 - mask[b].astype(np.float64))
+        e = np.exp(sc - sc.max(-1, keepdims=True))
+        p = O.f16(e / (e.sum(-1, keepdims=True) + 1e-6))
+        exp = np.einsum("hqk,hkd->qhd", p, v).reshape(S, heads * 64)
+        err = np.abs(g[b * S:(b + 1) * S] - exp)
+        assert err.max() <= 4e-3, (b, err.max())
+
+
 def test_attention_large_logits_do_not_overflow(device):
     """Logits of a few hundred in magnitude (fp16 Q.K would overflow at 65504)."""
     rs = np.random.RandomState(9)

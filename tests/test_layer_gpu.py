@@ -166,6 +166,30 @@ def test_cfg4_bert_large_variable_and_fixed(device):
     assert np.abs(rm.astype(np.float32) - pad.astype(np.float32)).max() <= 4e-3
 
 
+def test_padded_path_applies_arbitrary_masks(device):
+    """Batch <= 2 (or is_remove_padding = False) runs on the padded rows and must
+    honour any 0/1 mask pattern, not only prefixes - every row is compared."""
+    _say("padded path, arbitrary mask")
+    rs = np.random.RandomState(12)
+    cfg = workload.EncoderConfig("am", 2, 72, 4, layers=2, lens=(72, 72), seed=9)
+    wl = workload.make_workload(cfg, bias_std=0.05, random_affine=True)
+    mask = (rs.rand(2, 72, 72) < 0.7).astype(np.float16)
+    i, j = np.indices((72, 72))
+    mask[1] = (j <= i).astype(np.float16)                       # causal
+    wl = workload.Workload(cfg, wl.lens, wl.x, mask, wl.layers)
+    exp = _oracle(wl)
+    _check(_run_th_op(wl, device), exp, wl.lens, pads_must_be_zero=False, tag="mask/th_op")
+    _check(_run_c_api(wl, device, use_fused_attention=False), exp, wl.lens,
+           pads_must_be_zero=False, tag="mask/c_api/grouped")
+    cfg5 = workload.EncoderConfig("am5", 5, 40, 2, layers=1, lens=(40,) * 5, seed=10)
+    wl5 = workload.make_workload(cfg5, bias_std=0.05, random_affine=True)
+    m5 = (rs.rand(5, 40, 40) < 0.5).astype(np.float16)
+    m5[:, :, 0] = 1
+    wl5 = workload.Workload(cfg5, wl5.lens, wl5.x, m5, wl5.layers)
+    _check(_run_c_api(wl5, device, is_remove_padding=False), _oracle(wl5), wl5.lens,
+           pads_must_be_zero=False, tag="mask/c_api/no-rm")
+
+
 def test_fp32_gamma_beta_next_to_fp16_weights(device):
     _say("fp32 gamma/beta")
     cfg = workload.EncoderConfig("g32", 4, 96, 4, layers=1, lens=(96, 5, 50, 77), seed=21)
