@@ -4,9 +4,11 @@
 // A as stored, W through the [N, K] pre-pack made by bt_transpose_weights.
 //
 // Structure of one workgroup (tile BM x BN, BK = 64):
-//   * global -> LDS copies are direct-to-LDS 16-byte loads (global_load_lds):
-//     no staging registers, no ds_write; each wave instruction lands 1 KB = 8
-//     tile rows back to back in LDS;
+//   * global -> LDS copies are 16-byte buffer loads with an LDS destination: no
+//     staging registers, no ds_write; each wave instruction lands 1 KB = 8 tile
+//     rows back to back in LDS.  Small tiles give this job to dedicated loader
+//     waves so the computing waves' instruction streams hold MFMAs and LDS
+//     reads only;
 //   * the LDS image is XOR-swizzled on 16-byte chunks (slot = chunk ^ (row>>1 & 7));
 //     the swizzle is applied by choosing which global chunk each lane fetches,
 //     and makes the ds_read_b128 operand fetches conflict-free on the 64 banks;
@@ -30,7 +32,6 @@
 
 namespace bt {
 
-constexpr int kBK = 64;   // k extent of one LDS tile (halfs) = 8 chunks of 16 bytes
 
 enum Epilogue { kEpiPlain = 0, kEpiBiasGelu = 1, kEpiQkvSplit = 2 };
 
@@ -55,7 +56,12 @@ __device__ __forceinline__ float gelu_tanh_f32(float x) {
   return x * __builtin_amdgcn_rcpf(1.0f + e);
 }
 
+// XOR swizzle of the 16-byte chunk slot inside a 128-byte tile row: rows r and r+1
+// differ by half of the 256-byte bank window, so 16 consecutive rows need 8 distinct
+// slots.  The 16 lanes that one ds_read_b128 pass serves then touch every bank once.
 __device__ __forceinline__ int swz(int row) { return (row >> 1) & 7; }
+
+constexpr int kBK = 64;   // k extent of one LDS tile (halfs) = 8 chunks of 16 bytes
 
 template <int N>
 __device__ __forceinline__ void wait_vmcnt() {
@@ -64,22 +70,62 @@ __device__ __forceinline__ void wait_vmcnt() {
   __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | 0x0F70);
 }
 
-template <int BM, int BN, int STAGES, int WM, int WN, int SCHED, int EPI>
-__global__ __launch_bounds__(WM *WN * 64) void gemm_kernel(GemmArgs p) {
-  constexpr int NW = WM * WN;
+// Wait until at most `younger` whole stages (NI loads each) are still in flight.
+template <int NI, int MAXY>
+__device__ __forceinline__ void wait_stages(int younger) {
+  if constexpr (MAXY == 0) {
+    wait_vmcnt<0>();
+  } else {
+    if (younger >= MAXY)
+      wait_vmcnt<MAXY * NI>();
+    else
+      wait_stages<NI, MAXY - 1>(younger);
+  }
+}
+
+// The buffer-descriptor type exists in the device pass only; the host pass sees the
+// kernel as an empty stub.
+#if defined(__HIP_DEVICE_COMPILE__)
+// Untyped buffer descriptor (stride 0) over [base, base + bytes): loads past the end
+// return 0.
+typedef __amdgpu_buffer_rsrc_t rsrc_t;
+__device__ __forceinline__ rsrc_t make_rsrc(const void *base, size_t bytes) {
+  const int recs = bytes > 0x7fffffffull ? 0x7fffffff : (int)bytes;
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, recs, 0x00020000);
+}
+
+// One stage's loads of one wave: instruction i lands 8 tile rows (1 KB) at
+// lds + i * lds_step; the first NIA instructions read A, the rest W.
+template <int NI, int NIA>
+__device__ __forceinline__ void issue_stage_loads(rsrc_t rs_a, rsrc_t rs_w, const int (&voff)[NI],
+                                                  half_t *lds, int lds_step, int k_bytes) {
+#pragma unroll
+  for (int i = 0; i < NI; ++i)
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(i < NIA ? rs_a : rs_w,
+                                             (__attribute__((address_space(3))) void *)(lds + i * lds_step),
+                                             16, voff[i], k_bytes, 0, 0);
+}
+
+template <int BM, int BN, int STAGES, int WM, int WN, int NP, int SCHED, int EPI>
+__device__ __forceinline__ void gemm_tile(const GemmArgs &p) {
+  constexpr int BK = kBK;
+  constexpr int NW = WM * WN;                   // waves that run the MFMAs
+  constexpr int NL = NP > 0 ? NP : NW;          // waves that issue the global loads
   constexpr int WTM = BM / WM, WTN = BN / WN;   // wave tile
   constexpr int TM = WTM / 32, TN = WTN / 32;   // 32x32 MFMA blocks per wave
   constexpr int ROWS = BM + BN;                 // A rows then W rows in one stage
-  constexpr int NI = ROWS / 8 / NW;             // load instructions per wave per stage
-  constexpr int STAGE_HALFS = ROWS * kBK;
-  static_assert(ROWS % (8 * NW) == 0, "tile rows must split evenly over the waves");
-  static_assert(STAGES >= 2 && STAGES <= 3, "pipeline depth");
+  constexpr int NI = ROWS / 8 / NL;             // load instructions per loading wave per stage
+  constexpr int NIA = BM / 8 / NL;              // ... of which the first NIA fetch A rows
+  constexpr int STAGE_HALFS = ROWS * BK;
+  static_assert(BM % (8 * NL) == 0 && BN % (8 * NL) == 0, "tile rows must split evenly over the loading waves");
+  static_assert(STAGES >= 2 && STAGES <= 5 && (STAGES - 2) * NI < 64, "pipeline depth");
+  constexpr int YOUNG = STAGES - 2;   // stages that may still be in flight at a barrier
 
   extern __shared__ __attribute__((aligned(1024))) half_t gemm_smem[];
   half_t *smem = gemm_smem;
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int wm = wave / WN, wn = wave % WN;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int M = p.valid_rows ? min(*p.valid_rows, p.rows_cap) : p.rows_cap;
 
   // XCD-aware tile order over the live tiles
@@ -93,32 +139,72 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_kernel(GemmArgs p) {
     tile_n = L - tile_m * p.tiles_n;
   }
   const int m0 = tile_m * BM, n0 = tile_n * BN;
+  const int nk = p.K / BK;
 
-  // Per-lane source of each load instruction: instruction i of this wave fills
-  // tile rows [(i*NW + wave)*8, +8); lane -> (row, slot), fetching the chunk
-  // that the swizzle places in that slot.
-  const half_t *gsrc[NI];
-#pragma unroll
-  for (int i = 0; i < NI; ++i) {
-    const int r = (i * NW + wave) * 8 + (lane >> 3);
-    const int kc = (lane & 7) ^ swz(r);
-    if (r < BM) {
-      int ar = min(m0 + r, p.rows_cap - 1);
-      if (p.a_row_index) ar = p.a_row_index[min(ar, M - 1)];   // live rows only hold valid indices
-      gsrc[i] = p.a + (size_t)ar * p.K + kc * 8;
-    } else
-      gsrc[i] = p.wt + (size_t)min(n0 + r - BM, p.N - 1) * p.K + kc * 8;
-  }
-  auto issue_loads = [&](int kt, int stage) {
+  // ---- loading side ---------------------------------------------------------
+  // Global -> LDS copies are buffer loads with the LDS destination: descriptor and
+  // k offset in scalar registers, one fixed 32-bit byte offset per lane and load.
+  // (Beside a wave that keeps the MFMA pipe full this form issues at the full
+  // 64 B/clk of the vector memory path; the flat-address form drops to half.)
+  // Load instruction i of loading wave w fills tile rows [(i*NL + w)*8, +8); a lane
+  // fetches the chunk that the swizzle places in its slot.  Rows past the end of
+  // either operand fall outside the descriptor and read as zero.
+  //
+  // With NP == 0 every wave loads its share and then computes.  With NP > 0 the
+  // last NP waves only load: the vector-memory unit accepts one 1 KB instruction
+  // per 16 clocks, and a wave that has to push its loads through that queue at the
+  // top of every k-step cannot feed the MFMA pipe meanwhile; for small tiles
+  // (load clocks ~ MFMA clocks) that serialisation costs half of the throughput.
+  const bool loader = NP == 0 || wave >= NW;
+  const int lw = NP == 0 ? wave : wave - NW;    // index among the loading waves
+  const bool gather = p.a_row_index != nullptr;
+  const rsrc_t rs_a =
+      gather ? make_rsrc(p.a, (size_t)p.rows_cap * p.K * sizeof(half_t))
+             : make_rsrc(p.a + (size_t)m0 * p.K, (size_t)(p.rows_cap - m0) * p.K * sizeof(half_t));
+  const rsrc_t rs_w =
+      make_rsrc(p.wt + (size_t)n0 * p.K, (size_t)(p.N - n0) * p.K * sizeof(half_t));
+  int voff[NI];
+  if (loader) {
 #pragma unroll
     for (int i = 0; i < NI; ++i) {
-      half_t *dst = smem + stage * STAGE_HALFS + (i * NW + wave) * 8 * kBK;
-      __builtin_amdgcn_global_load_lds(
-          (const __attribute__((address_space(1))) void *)(gsrc[i] + kt * kBK),
-          (__attribute__((address_space(3))) void *)dst, 16, 0, 0);
+      const int r = (i * NL + lw) * 8 + (lane >> 3);
+      const int kc = (lane & 7) ^ swz(r);
+      int row = i < NIA ? r : r - BM;
+      if (i < NIA && gather) row = p.a_row_index[min(m0 + r, M - 1)];   // live rows only hold valid indices
+      voff[i] = (row * p.K + kc * 8) * (int)sizeof(half_t);
     }
-  };
+  }
+#define BT_ISSUE_LOADS(kt, stage)                                                        \
+  issue_stage_loads<NI, NIA>(rs_a, rs_w, voff, smem + (stage)*STAGE_HALFS + lw * 8 * BK, \
+                             NL * 8 * BK, (kt)*BK * (int)sizeof(half_t))
 
+  if (loader) {
+#pragma unroll
+    for (int s = 0; s < STAGES - 1; ++s)
+      if (s < nk) BT_ISSUE_LOADS(s, s);
+  }
+
+  if (NP > 0 && wave >= NW) {
+    // pure loader: one barrier per k-step, in step with the computing waves
+    int stage = 0;
+    for (int kt = 0; kt < nk; ++kt) {
+      wait_stages<NI, YOUNG>(nk - 1 - kt);       // this wave's part of tile kt has landed
+      asm volatile("" ::: "memory");
+      __builtin_amdgcn_s_barrier();               // tile kt is complete; stage of tile kt-1 is free
+      asm volatile("" ::: "memory");
+      if (kt + STAGES - 1 < nk) {
+        int ps = stage + STAGES - 1;
+        if (ps >= STAGES) ps -= STAGES;
+        BT_ISSUE_LOADS(kt + STAGES - 1, ps);
+      }
+      if (++stage == STAGES) stage = 0;
+    }
+    __builtin_amdgcn_s_barrier();                 // pairs with the barrier before the epilogue
+    return;
+  }
+
+  // ---- computing side -------------------------------------------------------
+  const int wm = wave / WN, wn = wave % WN;
   float16_t acc[TN][TM];
 #pragma unroll
   for (int i = 0; i < TN; ++i)
@@ -127,50 +213,41 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_kernel(GemmArgs p) {
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
 
-  const int nk = p.K / kBK;
-#pragma unroll
-  for (int s = 0; s < STAGES - 1; ++s)
-    if (s < nk) issue_loads(s, s);
-
   const int fr_row = lane & 31, fr_kc = lane >> 5;
+  half8_t fw[2][TN], fa[2][TM];
+  auto load_frags = [&](int st, int ks, int b) {
+    const half_t *sA = smem + st * STAGE_HALFS;
+    const half_t *sB = sA + BM * BK;
+#pragma unroll
+    for (int i = 0; i < TN; ++i) {
+      const int r = wn * WTN + i * 32 + fr_row;
+      fw[b][i] = *(const half8_t *)(sB + r * BK + (((2 * ks + fr_kc) ^ swz(r + BM)) * 8));
+    }
+#pragma unroll
+    for (int j = 0; j < TM; ++j) {
+      const int r = wm * WTM + j * 32 + fr_row;
+      fa[b][j] = *(const half8_t *)(sA + r * BK + (((2 * ks + fr_kc) ^ swz(r)) * 8));
+    }
+  };
   int stage = 0;
   for (int kt = 0; kt < nk; ++kt) {
     // tile kt has landed for this wave once only the younger stages' loads are outstanding
-    if (STAGES == 3 && kt + 1 < nk)
-      wait_vmcnt<NI>();
-    else
-      wait_vmcnt<0>();
+    if (NP == 0) wait_stages<NI, YOUNG>(nk - 1 - kt);
     asm volatile("" ::: "memory");
-    __builtin_amdgcn_s_barrier();   // everyone's tile kt is in LDS; stage (kt-1) is free again
+    __builtin_amdgcn_s_barrier();   // everyone's tile is in LDS; stage (kt-1) is free again
     asm volatile("" ::: "memory");
-    if (kt + STAGES - 1 < nk) {
+    if (NP == 0 && kt + STAGES - 1 < nk) {
       int ps = stage + STAGES - 1;
       if (ps >= STAGES) ps -= STAGES;
-      issue_loads(kt + STAGES - 1, ps);
+      BT_ISSUE_LOADS(kt + STAGES - 1, ps);
     }
-    const half_t *sA = smem + stage * STAGE_HALFS;
-    const half_t *sB = sA + BM * kBK;
-
-    half8_t fw[2][TN], fa[2][TM];
-    auto load_frags = [&](int ks, int b) {
-#pragma unroll
-      for (int i = 0; i < TN; ++i) {
-        const int r = wn * WTN + i * 32 + fr_row;
-        fw[b][i] = *(const half8_t *)(sB + r * kBK + (((2 * ks + fr_kc) ^ swz(r + BM)) * 8));
-      }
-#pragma unroll
-      for (int j = 0; j < TM; ++j) {
-        const int r = wm * WTM + j * 32 + fr_row;
-        fa[b][j] = *(const half8_t *)(sA + r * kBK + (((2 * ks + fr_kc) ^ swz(r)) * 8));
-      }
-    };
-    load_frags(0, 0);
+    load_frags(stage, 0, 0);
     // compiler scheduling strategy that interleaves the LDS reads with the MFMAs
     if (SCHED == 0) __builtin_amdgcn_iglp_opt(0);
     if (SCHED == 1) __builtin_amdgcn_iglp_opt(1);
 #pragma unroll
-    for (int ks = 0; ks < kBK / 16; ++ks) {
-      if (ks + 1 < kBK / 16) load_frags(ks + 1, (ks + 1) & 1);
+    for (int ks = 0; ks < BK / 16; ++ks) {
+      if (ks + 1 < BK / 16) load_frags(stage, ks + 1, (ks + 1) & 1);
 #pragma unroll
       for (int i = 0; i < TN; ++i)
 #pragma unroll
@@ -181,12 +258,13 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_kernel(GemmArgs p) {
     if (++stage == STAGES) stage = 0;
   }
 
+#undef BT_ISSUE_LOADS
   // ---- epilogue -------------------------------------------------------------
   // accumulator block (i, j), quad q: columns n..n+3 of row m with
   //   n = n0 + wn*WTN + i*32 + q*8 + (lane>>5)*4,  m = m0 + wm*WTM + j*32 + (lane&31)
   constexpr int EP = WTN + 8;   // pitch (halfs) of the wave-private staging tile
   static_assert((size_t)NW * 32 * EP <= (size_t)STAGES * STAGE_HALFS, "staging fits the ring");
-  __syncthreads();              // all waves are done with the last stage
+  __builtin_amdgcn_s_barrier();   // all waves are done with the last stage
   half_t *st = smem + wave * 32 * EP;
   const int row_in = lane & 31, col_in = (lane >> 5) * 4;
   constexpr int CPRW = WTN / 8;   // 16-byte chunks per staged row
@@ -236,6 +314,15 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_kernel(GemmArgs p) {
   }
 }
 
+#endif  // __HIP_DEVICE_COMPILE__
+
+template <int BM, int BN, int STAGES, int WM, int WN, int NP, int SCHED, int EPI>
+__global__ __launch_bounds__((WM * WN + NP) * 64) void gemm_kernel(GemmArgs p) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  gemm_tile<BM, BN, STAGES, WM, WN, NP, SCHED, EPI>(p);
+#endif
+}
+
 // ---- weight pre-pack: wt[n][k] = w[k][n] for up to four matrices in one launch ---
 struct TransposeJob {
   const half_t *w;
@@ -281,13 +368,13 @@ __global__ __launch_bounds__(256) void transpose_kernel(TransposeArgs a) {
   }
 }
 
-template <int BM, int BN, int STAGES, int WM, int WN, int SCHED, int EPI>
+template <int BM, int BN, int STAGES, int WM, int WN, int NP, int SCHED, int EPI>
 static int launch_gemm_tile(GemmArgs p, hipStream_t s) {
   constexpr size_t smem = (size_t)STAGES * (BM + BN) * kBK * sizeof(half_t);
   static_assert(smem <= 160 * 1024, "LDS budget");
   static bool configured = false;  // benign race: setting the attribute is idempotent
   if (!configured) {
-    hipError_t e = hipFuncSetAttribute((const void *)gemm_kernel<BM, BN, STAGES, WM, WN, SCHED, EPI>,
+    hipError_t e = hipFuncSetAttribute((const void *)gemm_kernel<BM, BN, STAGES, WM, WN, NP, SCHED, EPI>,
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
     if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute(gemm_kernel)");
     configured = true;
@@ -295,23 +382,23 @@ static int launch_gemm_tile(GemmArgs p, hipStream_t s) {
   const int tiles_m = (p.rows_cap + BM - 1) / BM;
   p.tiles_n = (p.N + BN - 1) / BN;
   const int grid = (tiles_m * p.tiles_n + 7) / 8 * 8;
-  gemm_kernel<BM, BN, STAGES, WM, WN, SCHED, EPI><<<grid, WM * WN * 64, smem, s>>>(p);
+  gemm_kernel<BM, BN, STAGES, WM, WN, NP, SCHED, EPI><<<grid, (WM * WN + NP) * 64, smem, s>>>(p);
   BT_CHECK_LAUNCH("gemm_kernel");
   return BT_OK;
 }
 
 template <int EPI>
 static int launch_gemm(GemmArgs p, hipStream_t s) {
-  // Tile table (rows x cols, ring depth, wave grid):
-  //   0: 256x256, 2, 2x4   wide outputs (FFN1 at hidden 768): one tile per CU
-  //   1: 128x128, 2, 2x2   narrow outputs, short k loop (projection)
-  //   2: 128x128, 3, 4x2   narrow outputs, long k loop (FFN2)
-  //   3: 256x192, 2, 4x2   outputs that split into 192-wide panels but not into a
-  //                        full wave of 256-wide ones (QKV at hidden 768)
-  // The choice minimises (tiles per CU, rounded up) x (measured time of one tile)
-  // for the estimated live rows: the exact count when every row is live, the
-  // caller's hint when it has one, else 60 % of the capacity (the fill the
-  // padding-free path is built for).
+  // Tile table (rows x cols, ring depth, computing wave grid, loader waves):
+  //   0: 256x256, 2, 2x4, 0   wide outputs: one tile per CU, every wave loads and computes
+  //   1: 128x128, 3, 2x2, 4   narrow outputs (projection, FFN2) and small problems
+  //   2: 256x128, 3, 4x2, 4   narrow outputs with enough rows to fill the chip
+  //   3: 256x192, 2, 4x2, 0   outputs that split into 192-wide panels but not into a
+  //                           full wave of 256-wide ones (QKV at hidden 768)
+  // The choice minimises rounds x (k-steps x time of one k-step + fill and epilogue)
+  // with the measured per-shape times below, for the estimated live rows: the exact
+  // count when every row is live, the caller's hint when it has one, else 60 % of
+  // the capacity (the fill the padding-free path is built for).
   int choice = option_gemm_tile();
   if (choice < 0) {
     static const int cus = [] {
@@ -327,14 +414,17 @@ static int launch_gemm(GemmArgs p, hipStream_t s) {
                                               : (p.rows_cap * 3LL + 4) / 5;
     struct Cand {
       int id, bm, bn;
-      float tile_time;   // relative time of one tile of this shape per k-step
+      float step_us, fixed_us;   // one k-step of one tile; fill + epilogue of one tile
     };
-    const Cand cands[3] = {{0, 256, 256, 24.0f}, {3, 256, 192, 19.5f},
-                           {p.K >= 2048 ? 2 : 1, 128, 128, 7.5f}};
+    const Cand cands[4] = {{0, 256, 256, 1.29f, 3.4f},
+                           {3, 256, 192, 1.04f, 2.8f},
+                           {2, 256, 128, 0.62f, 2.3f},
+                           {1, 128, 128, 0.43f, 1.8f}};
+    const float nk = (float)(p.K / kBK);
     float best = 0.f;
     for (const Cand &c : cands) {
       const long long tiles = ((m_est + c.bm - 1) / c.bm) * ((p.N + c.bn - 1) / c.bn);
-      const float t = (float)((tiles + cus - 1) / cus) * c.tile_time;
+      const float t = (float)((tiles + cus - 1) / cus) * (nk * c.step_us + c.fixed_us);
       if (choice < 0 || t < best) {
         best = t;
         choice = c.id;
@@ -343,13 +433,13 @@ static int launch_gemm(GemmArgs p, hipStream_t s) {
   }
   switch (choice) {
     case 0:
-      return launch_gemm_tile<256, 256, 2, 2, 4, 1, EPI>(p, s);
+      return launch_gemm_tile<256, 256, 2, 2, 4, 0, 1, EPI>(p, s);
     case 2:
-      return launch_gemm_tile<128, 128, 3, 4, 2, 1, EPI>(p, s);
+      return launch_gemm_tile<256, 128, 3, 4, 2, 4, 1, EPI>(p, s);
     case 3:
-      return launch_gemm_tile<256, 192, 2, 4, 2, 1, EPI>(p, s);
+      return launch_gemm_tile<256, 192, 2, 4, 2, 0, 1, EPI>(p, s);
     default:
-      return launch_gemm_tile<128, 128, 2, 2, 2, 0, EPI>(p, s);
+      return launch_gemm_tile<128, 128, 3, 2, 2, 4, 0, EPI>(p, s);
   }
 }
 
@@ -358,8 +448,10 @@ static int check_gemm_args(const char *who, const void *a, const void *wt, const
   BT_REQUIRE(a && wt && c, BT_ERR_INVALID_ARGUMENT, "%s: null pointer argument", who);
   BT_REQUIRE(rows_cap >= 0 && n > 0 && k > 0, BT_ERR_INVALID_ARGUMENT,
              "%s: rows_cap=%d n=%d k=%d out of range", who, rows_cap, n, k);
-  BT_REQUIRE(k % kBK == 0, BT_ERR_UNSUPPORTED, "%s: k=%d must be a multiple of %d", who, k, kBK);
+  BT_REQUIRE(k % 64 == 0, BT_ERR_UNSUPPORTED, "%s: k=%d must be a multiple of 64", who, k);
   BT_REQUIRE(n % 8 == 0, BT_ERR_UNSUPPORTED, "%s: n=%d must be a multiple of 8", who, n);
+  // a 256-row tile is addressed with 32-bit byte offsets from its first row
+  BT_REQUIRE(k <= (1 << 21), BT_ERR_UNSUPPORTED, "%s: k=%d is beyond 2^21", who, k);
   return BT_OK;
 }
 
@@ -435,6 +527,9 @@ extern "C" int bt_gemm_qkv_bias_split(const void *a, const int *a_row_index, con
   if (rows_cap == 0) return BT_OK;
   BT_REQUIRE(!a_row_index || valid_rows, BT_ERR_INVALID_ARGUMENT,
              "bt_gemm_qkv_bias_split: a_row_index needs valid_rows (only live rows are indexed)");
+  // gathered rows are addressed with 32-bit byte offsets from the start of `a`
+  BT_REQUIRE(!a_row_index || (long long)rows_cap * H * 2 <= 0x7fffffffLL, BT_ERR_UNSUPPORTED,
+             "bt_gemm_qkv_bias_split: a gathered input of %d x %d halfs is beyond 2 GiB", rows_cap, H);
   GemmArgs p{(const half_t *)a, (const half_t *)wt_qkv, (const half_t *)bias_qkv,
              (half_t *)qkv_heads, valid_rows, a_row_index, rows_cap, 3 * H, H, 0, rows_hint};
   return launch_gemm<kEpiQkvSplit>(p, as_stream(stream));
