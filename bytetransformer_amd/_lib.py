@@ -42,9 +42,9 @@ KERNEL_ABI = {
     "bt_gemm_bias_gelu": (c_int, [_P, _P, _P, _P, _IP, c_int, c_int, c_int, c_int, _P]),
     "bt_gemm_qkv_bias_split": (c_int, [_P, _IP, _P, _P, _P, _IP, c_int, c_int, c_int, c_int,
                                        _P]),
-    "bt_attention_short": (c_int, [_P, _P, _IP, _IP, _P, c_int, c_int, c_int, c_int, c_int,
+    "bt_attention_short": (c_int, [_P, _P, _IP, _IP, _P, _P, c_int, c_int, c_int, c_int, c_int,
                                    c_float, c_int, _P]),
-    "bt_attention_grouped": (c_int, [_P, _P, _IP, _IP, _P, c_int, c_int, c_int, c_int, c_int,
+    "bt_attention_grouped": (c_int, [_P, _P, _IP, _IP, _P, _P, c_int, c_int, c_int, c_int, c_int,
                                      c_float, c_int, _P]),
     "bt_add_bias_residual_layernorm": (c_int, [_P, _P, _IP, _P, _P, _P, c_int, _IP, c_int, c_int,
                                                c_float, _P]),
@@ -74,6 +74,8 @@ HOST_ABI = {
     "bt_encoder_bufsize": (c_ulonglong, [POINTER(EncoderConfig)]),
     "bt_encoder_layer_forward": (c_int, [POINTER(EncoderConfig), POINTER(LayerWeights), _P, _P,
                                          _P, _P, c_int, c_int, _P]),
+    "bt_encoder_layer_forward_bias": (c_int, [POINTER(EncoderConfig), POINTER(LayerWeights), _P,
+                                              _P, _P, _P, _P, c_int, c_int, _P]),
     "bt_encoder_last_error": (c_char_p, []),
 }
 

@@ -12,8 +12,6 @@ template <OperationType OpType>
 void Attention<OpType>::infer(AttentionInferParam infer_param) {
   if (OpType != OperationType::HALF)
     throw std::runtime_error("[BT][ERROR] Attention: only OperationType::HALF is implemented");
-  if (infer_param.attention_bias != nullptr)
-    throw std::runtime_error("[BT][ERROR] Attention: attention_bias is not supported");
   if (infer_param.et_param.batch_idx == nullptr)
     throw std::runtime_error("[BT][ERROR] Attention: et_param.batch_idx must be set");
   if (infer_param.batch_size > max_batch_size_ || infer_param.seq_len > max_seq_len_)
@@ -28,12 +26,12 @@ void Attention<OpType>::infer(AttentionInferParam infer_param) {
   if (uses_short_kernel(infer_param.seq_len))
     check_bt_error(bt_attention_short(infer_param.qkv, infer_param.attention_output,
                                       infer_param.et_param.batch_idx, infer_param.seq_order, mask,
-                                      infer_param.batch_size, infer_param.seq_len, rows_cap, head_num_, size_per_head_,
+                                      infer_param.attention_bias, infer_param.batch_size, infer_param.seq_len, rows_cap, head_num_, size_per_head_,
                                       scale, padded_rows, infer_param.stream));
   else
     check_bt_error(bt_attention_grouped(infer_param.qkv, infer_param.attention_output,
                                         infer_param.et_param.batch_idx, infer_param.seq_order, mask,
-                                        infer_param.batch_size, infer_param.seq_len, rows_cap, head_num_, size_per_head_,
+                                        infer_param.attention_bias, infer_param.batch_size, infer_param.seq_len, rows_cap, head_num_, size_per_head_,
                                         scale, padded_rows, infer_param.stream));
 }
 

@@ -26,8 +26,6 @@ void BertTransformer<OpType>::bert_infer(BertTransformerInferParam infer_param) 
   if (batch_size <= 0 || seq_len <= 0 || batch_size > max_batch_size_ || seq_len > max_seq_len_)
     throw std::runtime_error(
         "[BT][ERROR] BertTransformer: batch_size/seq_len outside the constructed maximum");
-  if (infer_param.attention_bias != nullptr)
-    throw std::runtime_error("[BT][ERROR] BertTransformer: attention_bias is not supported");
 
   const int hidden = head_num_ * size_per_head_;
   const int inter = hidden * param_.intermediate_size;

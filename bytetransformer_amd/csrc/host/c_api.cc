@@ -66,6 +66,15 @@ extern "C" int bt_encoder_layer_forward(const bt_encoder_config *cfg,
                                         const bt_layer_weights *weights, const void *input,
                                         const void *atten_mask, void *output, void *buf,
                                         int batch_size, int seq_len, void *stream) {
+  return bt_encoder_layer_forward_bias(cfg, weights, input, atten_mask, nullptr, output, buf,
+                                       batch_size, seq_len, stream);
+}
+
+extern "C" int bt_encoder_layer_forward_bias(const bt_encoder_config *cfg,
+                                             const bt_layer_weights *weights, const void *input,
+                                             const void *atten_mask, const void *attention_bias,
+                                             void *output, void *buf, int batch_size,
+                                             int seq_len, void *stream) {
   int rc = validate(cfg);
   if (rc != BT_OK) return rc;
   if (!weights) {
@@ -93,6 +102,7 @@ extern "C" int bt_encoder_layer_forward(const bt_encoder_config *cfg,
                                          seq_len,
                                          nullptr,
                                          (hipStream_t)stream};
+    ip.attention_bias = (const __half *)attention_bias;
     enc.infer(ip);
   } catch (const std::exception &e) {
     g_error = e.what();

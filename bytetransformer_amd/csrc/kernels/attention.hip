@@ -46,6 +46,7 @@ struct AttArgs {
   const int *seq_order;   // optional: grid z -> sequence, longest first (null = identity)
   const half_t *mask;     // optional [B,S,S] 0/1 mask, padded rows only: every key of the
                           // sequence's S rows takes part, shifted by (mask-1)*10000
+  const half_t *bias;     // optional [heads,S,S] term added to the scaled logits
   int B, S, rows_cap, heads;
   float scale_log2e;   // scale * log2(e)
   int padded_rows;
@@ -96,19 +97,32 @@ __device__ __forceinline__ half8_t load_k_frag(const half_t *sK, int kb, int dh,
 // domain: (mask - 1) * 10000 * log2(e)  (the reference's non-remove-padding
 // kernels, attention_fused.cu:234-237).  Keys at or past S get no term here; the
 // caller excludes them by index.
-__device__ __forceinline__ float4_t mask_bias4(const half_t *mask_row, int key, int S, bool vec) {
-  constexpr float kShift = 10000.0f * kLog2e;
-  float4_t m = {1.f, 1.f, 1.f, 1.f};
+__device__ __forceinline__ float4_t row4(const half_t *row, int key, int S, bool vec, float fill) {
+  float4_t m = {fill, fill, fill, fill};
   if (vec && key + 3 < S) {
-    const half4_t h = *(const half4_t *)(mask_row + key);
+    const half4_t h = *(const half4_t *)(row + key);
 #pragma unroll
     for (int r = 0; r < 4; ++r) m[r] = (float)h[r];
   } else {
 #pragma unroll
     for (int r = 0; r < 4; ++r)
-      if (key + r < S) m[r] = (float)mask_row[key + r];
+      if (key + r < S) m[r] = (float)row[key + r];
   }
-  return (m - 1.0f) * kShift;
+  return m;
+}
+__device__ __forceinline__ float4_t mask_bias4(const half_t *mask_row, int key, int S, bool vec) {
+  constexpr float kShift = 10000.0f * kLog2e;
+  return (row4(mask_row, key, S, vec, 1.f) - 1.0f) * kShift;
+}
+// Additive term of four consecutive keys in the exp2 domain: the mask shift (when a
+// mask row is given) plus the attention bias (softmax.h:41-46 adds it to the
+// scaled logits before the mask term).
+__device__ __forceinline__ float4_t add_terms4(const half_t *mask_row, const half_t *bias_row,
+                                               int key, int S, bool vec) {
+  float4_t t = {0.f, 0.f, 0.f, 0.f};
+  if (mask_row) t = mask_bias4(mask_row, key, S, vec);
+  if (bias_row) t += row4(bias_row, key, S, vec, 0.f) * kLog2e;
+  return t;
 }
 
 // ---------------------------------------------------------------------------
@@ -118,15 +132,17 @@ constexpr int kKT = 64;                          // keys per streamed tile
 constexpr int kTileHalfs = kKT * kHeadDim;       // one K or V tile
 constexpr int kAttStages = 3;
 
-template <int QB, bool FULLMASK>  // QB 16-query blocks per wave; workgroup covers 4*QB*16 queries
+// QB 16-query blocks per wave; workgroup covers 4*QB*16 queries.  ADD: a mask tensor and / or an
+// attention bias contribute additive terms to the logits.
+template <int QB, bool ADD>
 __global__ __launch_bounds__(kAttThreads, 2) void attention_grouped_kernel(AttArgs p) {
   constexpr int BQ = 4 * QB * 16;
   __shared__ __attribute__((aligned(1024))) half_t ring[kAttStages * 2 * kTileHalfs];
 
   const int b = p.seq_order ? p.seq_order[blockIdx.z] : blockIdx.z, head = blockIdx.y;
   const int seq_start = p.batch_idx[b];
-  // with a full mask every one of the S key rows takes part
-  const int klen = FULLMASK ? p.S : p.batch_idx[b + 1] - seq_start;
+  // with a mask tensor every one of the S key rows takes part
+  const int klen = ADD && p.mask ? p.S : p.batch_idx[b + 1] - seq_start;
   const int row_start = p.padded_rows ? b * p.S : seq_start;
   const int nq = p.padded_rows ? p.S : klen;
   const int q0 = blockIdx.x * BQ;
@@ -193,7 +209,7 @@ __global__ __launch_bounds__(kAttThreads, 2) void attention_grouped_kernel(AttAr
 
   const float c = p.scale_log2e;
   // after the mask term is folded in, the logits already are in the exp2 domain
-  const float cs = FULLMASK ? 1.0f : c;
+  const float cs = ADD ? 1.0f : c;
   const bool mask_vec = (p.S & 3) == 0;
   int stage = 0;
 
@@ -227,15 +243,16 @@ __global__ __launch_bounds__(kAttThreads, 2) void attention_grouped_kernel(AttAr
         s[kb][qb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kf1, qf[qb][1], s[kb][qb], 0, 0, 0);
       }
     }
-    if (FULLMASK) {
+    if (ADD) {
       const int k0 = t * kKT;
 #pragma unroll
       for (int qb = 0; qb < QB; ++qb) {
         const int q = min(q0 + (wave * QB + qb) * 16 + lq, p.S - 1);
-        const half_t *mrow = p.mask + ((size_t)b * p.S + q) * p.S;
+        const half_t *mrow = p.mask ? p.mask + ((size_t)b * p.S + q) * p.S : nullptr;
+        const half_t *brow = p.bias ? p.bias + ((size_t)head * p.S + q) * p.S : nullptr;
 #pragma unroll
         for (int kb = 0; kb < 4; ++kb) {
-          const float4_t bias = mask_bias4(mrow, k0 + kb * 16 + lg * 4, p.S, mask_vec);
+          const float4_t bias = add_terms4(mrow, brow, k0 + kb * 16 + lg * 4, p.S, mask_vec);
 #pragma unroll
           for (int r = 0; r < 4; ++r) s[kb][qb][r] = __builtin_fmaf(s[kb][qb][r], c, bias[r]);
         }
@@ -333,7 +350,7 @@ __global__ __launch_bounds__(kAttThreads, 2) void attention_grouped_kernel(AttAr
 // ---------------------------------------------------------------------------
 // short kernel: K, V resident in LDS, logits of the query tile in registers
 // ---------------------------------------------------------------------------
-template <int NKB, bool FULLMASK>  // capacity in 16-key blocks (keys <= 16*NKB), NKB even
+template <int NKB, bool ADD>  // capacity in 16-key blocks (keys <= 16*NKB), NKB even; ADD as above
 __global__ __launch_bounds__(kAttThreads) void attention_short_kernel(AttArgs p) {
   constexpr int KEYS = NKB * 16;
   constexpr int BQ = 64;  // 4 waves x 16 queries
@@ -343,7 +360,7 @@ __global__ __launch_bounds__(kAttThreads) void attention_short_kernel(AttArgs p)
 
   const int b = p.seq_order ? p.seq_order[blockIdx.z] : blockIdx.z, head = blockIdx.y;
   const int seq_start = p.batch_idx[b];
-  const int klen = FULLMASK ? p.S : p.batch_idx[b + 1] - seq_start;
+  const int klen = ADD && p.mask ? p.S : p.batch_idx[b + 1] - seq_start;
   const int row_start = p.padded_rows ? b * p.S : seq_start;
   const int nq = p.padded_rows ? p.S : klen;
   const int q0 = blockIdx.x * BQ;
@@ -397,13 +414,15 @@ __global__ __launch_bounds__(kAttThreads) void attention_short_kernel(AttArgs p)
   }
 
   const float c = p.scale_log2e;
-  const float cs = FULLMASK ? 1.0f : c;
-  if (FULLMASK) {
-    const half_t *mrow = p.mask + ((size_t)b * p.S + min(q, p.S - 1)) * p.S;
+  const float cs = ADD ? 1.0f : c;
+  if (ADD) {
+    const int qc = min(q, p.S - 1);
+    const half_t *mrow = p.mask ? p.mask + ((size_t)b * p.S + qc) * p.S : nullptr;
+    const half_t *brow = p.bias ? p.bias + ((size_t)head * p.S + qc) * p.S : nullptr;
     const bool mask_vec = (p.S & 3) == 0;
 #pragma unroll
     for (int kb = 0; kb < NKB; ++kb) {
-      const float4_t bias = mask_bias4(mrow, kb * 16 + lg * 4, p.S, mask_vec);
+      const float4_t bias = add_terms4(mrow, brow, kb * 16 + lg * 4, p.S, mask_vec);
 #pragma unroll
       for (int r = 0; r < 4; ++r) s[kb][r] = __builtin_fmaf(s[kb][r], c, bias[r]);
     }
@@ -475,26 +494,26 @@ static int check_att_args(const char *who, const void *qkv, const void *out, con
   return BT_OK;
 }
 
-template <int NKB, bool FULLMASK>
+template <int NKB, bool ADD>
 static int launch_short_impl(const AttArgs &a, hipStream_t s) {
   constexpr size_t smem = (size_t)2 * NKB * 16 * kHeadDim * sizeof(half_t);
   static_assert(smem <= 160 * 1024, "LDS budget");
   static bool configured = false;
   if (!configured) {
-    hipError_t e = hipFuncSetAttribute((const void *)attention_short_kernel<NKB, FULLMASK>,
+    hipError_t e = hipFuncSetAttribute((const void *)attention_short_kernel<NKB, ADD>,
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
     if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute(attention_short_kernel)");
     configured = true;
   }
   dim3 grid((a.S + 63) / 64, a.heads, a.B);
-  attention_short_kernel<NKB, FULLMASK><<<grid, kAttThreads, smem, s>>>(a);
+  attention_short_kernel<NKB, ADD><<<grid, kAttThreads, smem, s>>>(a);
   BT_CHECK_LAUNCH("attention_short_kernel");
   return BT_OK;
 }
 
 template <int NKB>
 static int launch_short(const AttArgs &a, hipStream_t s) {
-  return a.mask ? launch_short_impl<NKB, true>(a, s) : launch_short_impl<NKB, false>(a, s);
+  return a.mask || a.bias ? launch_short_impl<NKB, true>(a, s) : launch_short_impl<NKB, false>(a, s);
 }
 
 }  // namespace bt
@@ -503,17 +522,16 @@ using namespace bt;
 
 extern "C" int bt_attention_short(const void *qkv_heads, void *attention_output,
                                   const int *batch_idx, const int *seq_order,
-                                  const void *atten_mask, int batch_size, int seq_len,
-                                  int rows_cap,
-                                  int head_num, int size_per_head, float scale, int padded_rows,
-                                  void *stream) {
+                                  const void *atten_mask, const void *attention_bias,
+                                  int batch_size, int seq_len, int rows_cap, int head_num,
+                                  int size_per_head, float scale, int padded_rows, void *stream) {
   int rc = check_att_args("bt_attention_short", qkv_heads, attention_output, batch_idx, atten_mask,
                           padded_rows, batch_size, seq_len, rows_cap, head_num, size_per_head);
   if (rc) return rc;
   BT_REQUIRE(seq_len <= 512, BT_ERR_UNSUPPORTED,
              "bt_attention_short: seq_len=%d exceeds 512, use bt_attention_grouped", seq_len);
   AttArgs a{(const half_t *)qkv_heads, (half_t *)attention_output, batch_idx, seq_order,
-            (const half_t *)atten_mask, batch_size, seq_len,
+            (const half_t *)atten_mask, (const half_t *)attention_bias, batch_size, seq_len,
             rows_cap, head_num, scale * kLog2e, padded_rows};
   hipStream_t s = as_stream(stream);
   if (seq_len <= 64) return launch_short<4>(a, s);
@@ -525,15 +543,16 @@ extern "C" int bt_attention_short(const void *qkv_heads, void *attention_output,
 
 extern "C" int bt_attention_grouped(const void *qkv_heads, void *attention_output,
                                     const int *batch_idx, const int *seq_order,
-                                    const void *atten_mask, int batch_size, int seq_len,
-                                    int rows_cap, int head_num, int size_per_head, float scale,
-                                    int padded_rows, void *stream) {
+                                    const void *atten_mask, const void *attention_bias,
+                                    int batch_size, int seq_len, int rows_cap, int head_num,
+                                    int size_per_head, float scale, int padded_rows,
+                                    void *stream) {
   int rc = check_att_args("bt_attention_grouped", qkv_heads, attention_output, batch_idx,
                           atten_mask, padded_rows, batch_size, seq_len, rows_cap, head_num,
                           size_per_head);
   if (rc) return rc;
   AttArgs a{(const half_t *)qkv_heads, (half_t *)attention_output, batch_idx, seq_order,
-            (const half_t *)atten_mask, batch_size, seq_len,
+            (const half_t *)atten_mask, (const half_t *)attention_bias, batch_size, seq_len,
             rows_cap, head_num, scale * kLog2e, padded_rows};
   hipStream_t s = as_stream(stream);
   // 128-query tiles once there is enough work to fill the chip, else 64
@@ -541,13 +560,13 @@ extern "C" int bt_attention_grouped(const void *qkv_heads, void *attention_outpu
   const int qb = option_attention_qb();
   if (qb == 2 || (qb < 0 && blocks128 >= 512)) {
     dim3 grid((seq_len + 127) / 128, head_num, batch_size);
-    if (a.mask)
+    if (a.mask || a.bias)
       attention_grouped_kernel<2, true><<<grid, kAttThreads, 0, s>>>(a);
     else
       attention_grouped_kernel<2, false><<<grid, kAttThreads, 0, s>>>(a);
   } else {
     dim3 grid((seq_len + 63) / 64, head_num, batch_size);
-    if (a.mask)
+    if (a.mask || a.bias)
       attention_grouped_kernel<1, true><<<grid, kAttThreads, 0, s>>>(a);
     else
       attention_grouped_kernel<1, false><<<grid, kAttThreads, 0, s>>>(a);

@@ -66,7 +66,12 @@ class BTEncoder : public IBTEncoder {
                const ModelType model_type = ModelType::Bert,
                const Tensor attention_bias = Tensor()) override {
     CHECK_SEQ_LEN(seq_len);
-    TORCH_CHECK(!attention_bias.defined(), "attention_bias is not supported");
+    if (attention_bias.defined()) {
+      CHECK_INPUT(attention_bias, input.scalar_type());
+      TORCH_CHECK(attention_bias.dim() == 3 && attention_bias.size(0) == head_num_ &&
+                      attention_bias.size(1) == seq_len && attention_bias.size(2) == seq_len,
+                  "attention_bias must be [head_num, seq_len, seq_len]");
+    }
     c10::DeviceGuard device_guard(input.device());
 
     hipStream_t stream = c10::hip::getCurrentHIPStream(input.device().index()).stream();
@@ -85,6 +90,7 @@ class BTEncoder : public IBTEncoder {
       get_ptr<T>(input), get_ptr<T>(attr_mask), get_ptr<T>(output), get_ptr<void>(buf_tensor),
           batch_size, seq_len, nullptr, stream
     };
+    infer_param.attention_bias = attention_bias.defined() ? get_ptr<T>(attention_bias) : NULL;
     // offsets of this mask: cached per mask tensor (never while the stream is being
     // captured into a graph, where the host may not wait for the token count)
     MaskPlanCache::Plan plan;

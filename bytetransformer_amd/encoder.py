@@ -40,7 +40,7 @@ class BertEncoderLayer:
                              int(self.weights[10].dtype == torch.float32), self.tao,
                              self.layernorm_eps)
 
-    def __call__(self, x, mask, out=None):
+    def __call__(self, x, mask, out=None, attention_bias=None):
         lib = host_lib()
         if x.dtype != torch.float16:
             raise RuntimeError("only fp16 activations are implemented")
@@ -53,9 +53,16 @@ class BertEncoderLayer:
             self._buf = torch.empty(need, dtype=torch.int8, device=x.device)
         if out is None:
             out = torch.empty_like(x)
-        rc = lib.bt_encoder_layer_forward(
+        if attention_bias is not None:
+            if (attention_bias.dtype != x.dtype or not attention_bias.is_contiguous()
+                    or tuple(attention_bias.shape) != (self.head_num, S, S)):
+                raise ValueError("attention_bias must be a contiguous [head_num, S, S] tensor "
+                                 "of the activation dtype")
+        rc = lib.bt_encoder_layer_forward_bias(
             ctypes.byref(cfg), ctypes.byref(self._w), ctypes.c_void_p(x.data_ptr()),
-            ctypes.c_void_p(mask.data_ptr()), ctypes.c_void_p(out.data_ptr()),
+            ctypes.c_void_p(mask.data_ptr()),
+            ctypes.c_void_p(attention_bias.data_ptr() if attention_bias is not None else None),
+            ctypes.c_void_p(out.data_ptr()),
             ctypes.c_void_p(self._buf.data_ptr()), B, S,
             ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
         if rc != 0:

@@ -126,26 +126,28 @@ def gemm_qkv_bias_split(a, wt_qkv, bias_qkv, head_num, size_per_head=64, valid_r
 
 
 def _attention(fn, qkv_heads, batch_idx, batch_size, seq_len, scale, padded_rows, out,
-               seq_order=None, mask=None):
+               seq_order=None, mask=None, bias=None):
     _, head_num, rows_cap, d = qkv_heads.shape
     if out is None:
         out = torch.zeros(rows_cap, head_num * d, dtype=qkv_heads.dtype, device=qkv_heads.device)
-    _check(fn(_ptr(qkv_heads), _ptr(out), _ptr(batch_idx), _ptr(seq_order), _ptr(mask), batch_size,
-              seq_len, rows_cap,
-              head_num, d, float(scale), int(padded_rows), _stream()))
+    if bias is not None and tuple(bias.shape) != (head_num, seq_len, seq_len):
+        raise ValueError("attention bias must be [head_num, seq_len, seq_len]")
+    _check(fn(_ptr(qkv_heads), _ptr(out), _ptr(batch_idx), _ptr(seq_order), _ptr(mask), _ptr(bias),
+              batch_size, seq_len, rows_cap, head_num, d, float(scale), int(padded_rows),
+              _stream()))
     return out
 
 
 def attention_short(qkv_heads, batch_idx, batch_size, seq_len, scale, padded_rows=False, out=None,
-                    seq_order=None, mask=None):
+                    seq_order=None, mask=None, bias=None):
     return _attention(kernel_lib().bt_attention_short, qkv_heads, batch_idx, batch_size, seq_len,
-                      scale, padded_rows, out, seq_order, mask)
+                      scale, padded_rows, out, seq_order, mask, bias)
 
 
 def attention_grouped(qkv_heads, batch_idx, batch_size, seq_len, scale, padded_rows=False,
-                      out=None, seq_order=None, mask=None):
+                      out=None, seq_order=None, mask=None, bias=None):
     return _attention(kernel_lib().bt_attention_grouped, qkv_heads, batch_idx, batch_size,
-                      seq_len, scale, padded_rows, out, seq_order, mask)
+                      seq_len, scale, padded_rows, out, seq_order, mask, bias)
 
 
 def add_bias_residual_layernorm(out, residual, bias, gamma, beta, eps=1e-6, valid_rows=None,

@@ -58,6 +58,14 @@ int bt_encoder_layer_forward(const bt_encoder_config *cfg, const bt_layer_weight
                              const void *input, const void *atten_mask, void *output, void *buf,
                              int batch_size, int seq_len, void *stream);
 
+/* The same with the optional attention bias of the reference's infer parameters
+ * (bert_transformer.h:93, attention.h:56): fp16 [head_num, seq_len, seq_len],
+ * added to the scaled logits before the mask term (softmax.h:41-46).  NULL = none. */
+int bt_encoder_layer_forward_bias(const bt_encoder_config *cfg, const bt_layer_weights *weights,
+                                  const void *input, const void *atten_mask,
+                                  const void *attention_bias, void *output, void *buf,
+                                  int batch_size, int seq_len, void *stream);
+
 const char *bt_encoder_last_error(void);
 
 #ifdef __cplusplus

@@ -142,6 +142,11 @@ int bt_gemm_qkv_bias_split(const void *a, const int *a_row_index, const void *wt
  *                     before the softmax - the arbitrary-mask semantics of the
  *                     reference's non-remove-padding kernels (attention_fused.cu:234-237,
  *                     attention_fused_long.cu) - instead of the prefix-length rule.
+ *   attention_bias (nullable): fp16 [head_num, seq_len, seq_len], added to the scaled
+ *                     logit of (head, query position, key position) before the mask
+ *                     term, as the reference's unfused softmax does (softmax.h:41-46,
+ *                     attention_nofused.cu:78-95); positions are relative to the
+ *                     start of the sequence in both row layouts.
  *   seq_order (nullable): a permutation of the sequence indices from
  *                     bt_build_offsets; workgroups are issued in that order so the
  *                     longest sequences start first.  Results do not depend on it.
@@ -158,14 +163,14 @@ int bt_gemm_qkv_bias_split(const void *a, const int *a_row_index, const void *wt
  * the logits round trip through HBM.
  */
 int bt_attention_short(const void *qkv_heads, void *attention_output, const int *batch_idx,
-                       const int *seq_order, const void *atten_mask, int batch_size, int seq_len,
-                       int rows_cap, int head_num, int size_per_head, float scale,
-                       int padded_rows, void *stream);
+                       const int *seq_order, const void *atten_mask, const void *attention_bias,
+                       int batch_size, int seq_len, int rows_cap, int head_num, int size_per_head,
+                       float scale, int padded_rows, void *stream);
 
 int bt_attention_grouped(const void *qkv_heads, void *attention_output, const int *batch_idx,
-                         const int *seq_order, const void *atten_mask, int batch_size,
-                         int seq_len, int rows_cap, int head_num, int size_per_head, float scale,
-                         int padded_rows, void *stream);
+                         const int *seq_order, const void *atten_mask, const void *attention_bias,
+                         int batch_size, int seq_len, int rows_cap, int head_num,
+                         int size_per_head, float scale, int padded_rows, void *stream);
 
 /*
  * out = LayerNorm((out + residual) + bias) * gamma + beta, in place on `out`,

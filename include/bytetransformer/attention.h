@@ -32,7 +32,7 @@ struct AttentionInferParam {
   BlasHandle cublas_handle = nullptr;
   hipStream_t stream = nullptr;
   ET_Param et_param = {nullptr, nullptr, 0};
-  const T *attention_bias = nullptr;         // [head_num, seq_len, seq_len]; must be null
+  const T *attention_bias = nullptr;         // [head_num, seq_len, seq_len], added to the scaled logits
   const uint32_t *position_ids = nullptr;    // never read
   const uint32_t *token_type_ids = nullptr;  // never read
   // Extension: sequence indices by descending length from bt_build_offsets; the

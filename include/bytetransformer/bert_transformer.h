@@ -57,7 +57,7 @@ struct BertTransformerInferParam {
   int seq_len;
   BlasHandle cublas_handle;  // ignored
   hipStream_t stream;
-  const T *attention_bias = NULL;         // [head_num, seq_len, seq_len]; must be NULL
+  const T *attention_bias = NULL;         // [head_num, seq_len, seq_len], added to the scaled logits
   const uint32_t *position_ids = NULL;    // never read
   const uint32_t *token_type_ids = NULL;  // never read
   // Extension (no counterpart in the reference): offsets already built from this

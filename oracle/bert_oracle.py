@@ -193,13 +193,16 @@ def _t(a, dtype):
 
 
 def encoder_layer(x, mask, w, head_num, eps=1e-6, gelu="tanh", softmax_eps=1e-6, tao=1.0,
-                  dtype=torch.float32):
+                  dtype=torch.float32, attention_bias=None):
     """One post-LN encoder layer on the PADDED [B, S, H] batch, on CPU torch
     (bert_transformer_test.py:120-158).  `w` maps WEIGHT_NAMES to arrays.
 
     eps / gelu / softmax_eps select between the three conventions the
     reference itself mixes: CUDA kernels (1e-6, tanh, 1e-6), its PyTorch
-    script (1e-5, erf, 0) and the stated config (1e-12)."""
+    script (1e-5, erf, 0) and the stated config (1e-12).
+
+    attention_bias [head_num, S, S] is added to the scaled logits before the
+    mask term (softmax.h:41-46; the reference's script has no such input)."""
     x = _t(x, dtype)
     mask = _t(mask, dtype)
     W = {n: _t(w[n], dtype) for n in WEIGHT_NAMES}
@@ -212,6 +215,8 @@ def encoder_layer(x, mask, w, head_num, eps=1e-6, gelu="tanh", softmax_eps=1e-6,
     qkv = x @ W["qkv_kernel"] + W["qkv_bias"]
     q, k, v = qkv.chunk(3, dim=-1)
     scores = heads(q) @ heads(k).transpose(-2, -1) / (d ** 0.5) / tao
+    if attention_bias is not None:
+        scores = scores + _t(attention_bias, dtype).unsqueeze(0)
     scores = scores - 10000.0 * (1.0 - mask.unsqueeze(1))
     if softmax_eps == 0.0:
         probs = F.softmax(scores, dim=-1)

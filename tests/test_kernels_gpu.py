@@ -372,6 +372,54 @@ def test_attention_arbitrary_mask_on_padded_rows(device, kind, S):
         assert err.max() <= 4e-3, (b, err.max())
 
 
+@pytest.mark.parametrize("kind,S,padded,with_mask", [("short", 64, True, True), ("grouped", 200, True, True),
+                                                    ("short", 100, False, False), ("grouped", 300, False, False),
+                                                    ("grouped", 130, True, False)])
+def test_attention_bias(device, kind, S, padded, with_mask):
+    """attention_bias[h, q, k] is added to the scaled logits (positions relative to
+    the sequence start) in the packed and the padded row layout, with and without
+    the mask tensor."""
+    _say("attention bias", kind, S, padded, with_mask)
+    rs = np.random.RandomState(S + 7)
+    B, heads = 3, 2
+    lens = np.array([S, max(1, S // 3), S - 5])
+    bias = rs.standard_normal((heads, S, S)).astype(np.float16)
+    scale = 1 / math.sqrt(64)
+    if padded:
+        T = B * S
+        starts = np.arange(B) * S
+        bi = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    else:
+        T = int(lens.sum())
+        bi = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+        starts = bi[:-1]
+    qkv = rs.standard_normal((3, heads, T, 64)).astype(np.float16)
+    mask = None
+    if with_mask:
+        mask = (rs.rand(B, S, S) < 0.6).astype(np.float16)
+        mask[:, :, 0] = 1
+    fn = ops.attention_short if kind == "short" else ops.attention_grouped
+    g = fn(_dev(qkv, device), _dev(bi, device), B, S, scale, padded,
+           mask=_dev(mask, device) if with_mask else None, bias=_dev(bias, device))
+    g = g.cpu().numpy().astype(np.float64)
+    for b in range(B):
+        n = int(lens[b])
+        nq = S if padded else n
+        nk = S if with_mask else n
+        t0 = int(starts[b])
+        q = qkv[0, :, t0:t0 + nq].astype(np.float64)
+        k = qkv[1, :, t0:t0 + nk].astype(np.float64)
+        v = qkv[2, :, t0:t0 + nk].astype(np.float64)
+        sc = np.einsum("hqd,hkd->hqk", q, k) * scale + bias[:, :nq, :nk].astype(np.float64)
+        if with_mask:
+            sc = sc - 10000.0 * (1.0 - mask[b, :nq, :nk].astype(np.float64))
+        e = np.exp(sc - sc.max(-1, keepdims=True))
+        p = O.f16(e / (e.sum(-1, keepdims=True) + 1e-6))
+        exp = np.einsum("hqk,hkd->qhd", p, v).reshape(nq, heads * 64)
+        err = np.abs(g[t0:t0 + nq] - exp)
+        assert err.max() <= 4e-3, (b, err.max())
+
+
 def test_attention_large_logits_do_not_overflow(device):
     """Logits of a few hundred in magnitude (fp16 Q.K would overflow at 65504)."""
     rs = np.random.RandomState(9)

@@ -190,6 +190,32 @@ def test_padded_path_applies_arbitrary_masks(device):
            pads_must_be_zero=False, tag="mask/c_api/no-rm")
 
 
+@pytest.mark.parametrize("rm,S,lens", [(True, 48, (48, 20, 33, 7)), (False, 40, (40, 12, 40)),
+                                       (True, 300, (300, 120, 211))])
+def test_attention_bias_through_the_layer(device, rm, S, lens):
+    """The optional [head_num, S, S] bias of the infer parameters reaches the logits
+    on the packed path, the padded path and the streaming kernel."""
+    _say("attention bias, layer", rm, S)
+    rs = np.random.RandomState(21)
+    cfg = workload.EncoderConfig("ab", len(lens), S, 2, layers=1, lens=tuple(lens), seed=13)
+    wl = workload.make_workload(cfg, bias_std=0.05, random_affine=True)
+    bias = (0.5 * rs.standard_normal((2, S, S))).astype(np.float16)
+    w32 = {k: np.asarray(v, np.float32) for k, v in wl.layers[0].items()}
+    exp = O.encoder_layer(wl.x.astype(np.float32), wl.mask.astype(np.float32), w32, 2,
+                          attention_bias=bias.astype(np.float32)).numpy()
+    layer = _gpu_layers(wl, device, is_remove_padding=rm)[0]
+    got = layer(_dev(wl.x, device), _dev(wl.mask, device), attention_bias=_dev(bias, device))
+    torch.cuda.synchronize()
+    got = got.cpu().numpy()
+    if rm:
+        exp = O.masked_output(exp, wl.lens)
+    _check(got, exp, wl.lens, pads_must_be_zero=rm, tag="bias rm=%s S=%d" % (rm, S))
+    plain = layer(_dev(wl.x, device), _dev(wl.mask, device)).cpu().numpy()
+    assert np.abs(plain.astype(np.float32) - got.astype(np.float32)).max() > 1e-2   # not a no-op
+    with pytest.raises(ValueError):
+        layer(_dev(wl.x, device), _dev(wl.mask, device), attention_bias=_dev(bias[:, :-1], device))
+
+
 def test_fp32_gamma_beta_next_to_fp16_weights(device):
     _say("fp32 gamma/beta")
     cfg = workload.EncoderConfig("g32", 4, 96, 4, layers=1, lens=(96, 5, 50, 77), seed=21)

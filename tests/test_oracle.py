@@ -179,6 +179,45 @@ def test_encoder_layer_matches_torch_transformer_encoder_layer():
     assert mx < 1e-9, mx
 
 
+def test_encoder_layer_attention_bias_and_arbitrary_mask_match_torch_float_mask():
+    """Bias and a non-prefix 0/1 mask enter as additive terms: the same layer through
+    nn.TransformerEncoderLayer with the float attention mask bias - 10000 (1 - mask)."""
+    wl = _small_workload(lens=(16, 16), S=16)
+    rs = np.random.RandomState(8)
+    H, heads, S, B = wl.cfg.hidden, wl.cfg.head_num, wl.cfg.seq_len, wl.cfg.batch
+    w = wl.layers[0]
+    mask = (rs.rand(B, S, S) < 0.7).astype(np.float64)
+    mask[:, :, 0] = 1
+    bias = rs.standard_normal((heads, S, S))
+    ours = O.encoder_layer(wl.x, mask, w, heads, eps=1e-5, gelu="erf", softmax_eps=0.0,
+                           dtype=torch.float64, attention_bias=bias).numpy()
+    layer = torch.nn.TransformerEncoderLayer(H, heads, dim_feedforward=4 * H, dropout=0.0,
+                                             activation="gelu", layer_norm_eps=1e-5,
+                                             batch_first=True, norm_first=False).double().eval()
+    t = lambda a: torch.tensor(np.asarray(a, np.float64))
+    with torch.no_grad():
+        layer.self_attn.in_proj_weight.copy_(t(w["qkv_kernel"]).T)
+        layer.self_attn.in_proj_bias.copy_(t(w["qkv_bias"]))
+        layer.self_attn.out_proj.weight.copy_(t(w["attr_output_kernel"]).T)
+        layer.self_attn.out_proj.bias.copy_(t(w["attr_output_bias"]))
+        layer.norm1.weight.copy_(t(w["attr_output_layernorm_gamma"]))
+        layer.norm1.bias.copy_(t(w["attr_output_layernorm_beta"]))
+        layer.linear1.weight.copy_(t(w["inter_kernel"]).T)
+        layer.linear1.bias.copy_(t(w["inter_bias"]))
+        layer.linear2.weight.copy_(t(w["output_kernel"]).T)
+        layer.linear2.bias.copy_(t(w["output_bias"]))
+        layer.norm2.weight.copy_(t(w["output_layernorm_gamma"]))
+        layer.norm2.bias.copy_(t(w["output_layernorm_beta"]))
+        add = bias[None] - 10000.0 * (1.0 - mask[:, None])          # [B, heads, S, S]
+        torch.backends.mha.set_fastpath_enabled(False)
+        ref = layer(t(wl.x), src_mask=t(add.reshape(B * heads, S, S))).numpy()
+    assert np.abs(ours - ref).max() < 1e-9
+    # and the bias is not a no-op
+    plain = O.encoder_layer(wl.x, mask, w, heads, eps=1e-5, gelu="erf", softmax_eps=0.0,
+                            dtype=torch.float64).numpy()
+    assert np.abs(ours - plain).max() > 1e-3
+
+
 def test_encoder_layer_padded_torch_vs_packed_numpy_f64():
     wl = _small_workload()
     for eps, gelu, seps in [(1e-6, "tanh", 1e-6), (1e-5, "erf", 0.0), (1e-12, "tanh", 0.0)]:
