@@ -236,6 +236,29 @@ def main():
     torch.cuda.synchronize()
     ms = (time.perf_counter() - t0) * 1e3 / args.steps
 
+    def timed(fn):
+        for _ in range(args.warmup):
+            fn()
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        for _ in range(args.steps):
+            fn()
+        torch.cuda.synchronize()
+        return round((time.perf_counter() - t1) * 1e3 / args.steps, 4)
+
+    # the same forward through the other entry points (reported beside `value`, which
+    # stays the reference's protocol: one operator call per layer)
+    per_layer = [bt.BertEncoderLayer(cfg.head_num, cfg.head_size, w) for w in layers]
+    whole = bt.BertEncoder(cfg.head_num, cfg.head_size, layers)
+    graphed = whole.graph(cfg.batch, cfg.seq_len, valid_rows_hint=wl.valid_tokens)
+    graphed.input.copy_(x)
+    graphed.mask.copy_(mask)
+    other = {
+        "c_api_per_layer_ms": timed(lambda: bt.encoder_forward(per_layer, x, mask)),
+        "whole_encoder_ms": timed(lambda: whole(x, mask, valid_rows_hint=wl.valid_tokens)),
+        "whole_encoder_graph_ms": timed(graphed.replay),
+    }
+
     gemm_f, attn_f = workload.layer_flops(cfg, wl.lens)
     kernels = kernel_table(wl, dev, args.kernel_iters)
     dominant = max((k for k in kernels if kernels[k]["bound"] == "mfma"),
@@ -261,6 +284,7 @@ def main():
         "tokens_per_s": round(wl.valid_tokens / (ms * 1e-3), 1),
         "model_tflops": round(cfg.layers * (gemm_f + attn_f) / (ms * 1e-3) / 1e12, 2),
         "roofline": roofline,
+        "other_entry_points": other,
         "kernels": kernels,
     }
     if not args.no_cpu_baseline:

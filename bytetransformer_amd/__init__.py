@@ -9,4 +9,4 @@ implementation to fall back to - a missing library raises.
 from ._lib import (LibraryMissing, host_lib, kernel_lib, lib_dir, load_th_op,  # noqa: F401
                    th_op_path)
 from . import ops  # noqa: F401
-from .encoder import BertEncoderLayer, encoder_forward  # noqa: F401
+from .encoder import BertEncoder, BertEncoderLayer, GraphedBertEncoder, encoder_forward  # noqa: F401

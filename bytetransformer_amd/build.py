@@ -23,7 +23,7 @@ ROCM = os.environ.get("ROCM_PATH", "/opt/rocm")
 HIPCC = os.path.join(ROCM, "bin", "hipcc")
 
 KERNEL_SOURCES = ["padding.hip", "layernorm.hip", "gemm.hip", "attention.hip"]
-HOST_SOURCES = ["attention.cc", "bert_transformer.cc", "c_api.cc"]
+HOST_SOURCES = ["attention.cc", "bert_transformer.cc", "bert_encoder.cc", "c_api.cc"]
 TH_OP_SOURCES = ["ths_op_f.cc", "ths_op.cc"]
 
 # Packed-fp32 VALU ops are switched off for every device compile.

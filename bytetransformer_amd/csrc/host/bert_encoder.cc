@@ -1,0 +1,135 @@
+// BertEncoder<OpType>::infer - a stack of encoder layers over the C ABI with the
+// hidden state kept packed between layers.  Per layer the operation order and
+// residual choices are those of one reference layer (bert_transformer.cu:28-130);
+// the compress / restore pair of every inner layer is dropped.
+#include "bytetransformer/bert_encoder.h"
+
+namespace bytetransformer {
+
+template <OperationType OpType>
+void BertEncoder<OpType>::prepack(void *prepacked, hipStream_t stream) const {
+  if (OpType != OperationType::HALF)
+    throw std::runtime_error("[BT][ERROR] BertEncoder: only OperationType::HALF is implemented");
+  if (!prepacked) throw std::runtime_error("[BT][ERROR] BertEncoder::prepack: null destination");
+  const int hidden = head_num_ * size_per_head_, inter = hidden * intermediate_size_;
+  DataType_ *dst = (DataType_ *)prepacked;
+  for (const auto &l : layers_) {
+    DataType_ *wt_qkv = dst, *wt_proj = wt_qkv + (size_t)3 * hidden * hidden;
+    DataType_ *wt_inter = wt_proj + (size_t)hidden * hidden, *wt_out = wt_inter + (size_t)hidden * inter;
+    const void *src[4] = {l.attr_kernel_QKV, l.attr_output_kernel, l.inter_kernel, l.output_kernel};
+    void *out[4] = {wt_qkv, wt_proj, wt_inter, wt_out};
+    const int ks[4] = {hidden, hidden, hidden, inter};
+    const int ns[4] = {3 * hidden, hidden, inter, hidden};
+    check_bt_error(bt_transpose_weights(4, src, out, ks, ns, stream));
+    dst += layer_weight_elems();
+  }
+}
+
+template <OperationType OpType>
+void BertEncoder<OpType>::infer(BertEncoderInferParam<DataType_> ip) {
+  if (OpType != OperationType::HALF)
+    throw std::runtime_error("[BT][ERROR] BertEncoder: only OperationType::HALF is implemented");
+  if (layers_.empty()) throw std::runtime_error("[BT][ERROR] BertEncoder: initialize() first");
+  if (!ip.input_tensor || !ip.atten_mask || !ip.transformer_output || !ip.buf)
+    throw std::runtime_error("[BT][ERROR] BertEncoder: null input/mask/output/buf pointer");
+  const int batch_size = ip.batch_size, seq_len = ip.seq_len;
+  if (batch_size <= 0 || seq_len <= 0 || batch_size > max_batch_size_ || seq_len > max_seq_len_)
+    throw std::runtime_error(
+        "[BT][ERROR] BertEncoder: batch_size/seq_len outside the constructed maximum");
+  hipStream_t stream = ip.stream;
+
+  const int hidden = head_num_ * size_per_head_, inter = hidden * intermediate_size_;
+  const int rows = batch_size * seq_len;
+  const size_t tensor = (size_t)rows * hidden;
+  const unsigned long long max_rows = (unsigned long long)max_batch_size_ * max_seq_len_;
+  const unsigned long long max_tensor = max_rows * hidden;
+
+  uint8_t *base = (uint8_t *)ip.buf;
+  DataType_ *qkv_buf = (DataType_ *)base;
+  DataType_ *attr_out_buf = qkv_buf + 3 * tensor;
+  DataType_ *attr_matmul_buf = qkv_buf + 4 * tensor;   // projection, then LN1 in place
+  DataType_ *hidden_buf = qkv_buf + 5 * tensor;        // FFN2 out, then LN2 in place = next input
+  DataType_ *inter_matmul_buf = qkv_buf + 6 * tensor;
+  unsigned long long off = align_up((6 + intermediate_size_) * max_tensor * sizeof(DataType_), 256);
+  ET_Param et_param;
+  et_param.word_idx = (int *)(base + off);
+  et_param.batch_idx = et_param.word_idx + max_rows;
+  et_param.valid_word_num = rows;
+  int *seq_order = et_param.batch_idx + max_rows;
+  off += align_up((max_rows * 2 + 2 * (unsigned long long)max_batch_size_ + 2) * sizeof(int), 256);
+  DataType_ *staging = (DataType_ *)(base + off);      // one layer's weights when none were passed
+
+  check_bt_error(bt_build_offsets(ip.atten_mask, Traits_::dtype, batch_size, seq_len,
+                                  et_param.batch_idx, et_param.word_idx, seq_order, nullptr,
+                                  stream));
+  const int *valid_rows = is_remove_padding_ ? et_param.batch_idx + batch_size : nullptr;
+  const int rows_hint = ip.valid_rows_hint;
+  const int L = (int)layers_.size();
+
+  for (int l = 0; l < L; ++l) {
+    const auto &w = layers_[l];
+    // layer 0 reads the caller's padded input (valid token t at row word_idx[t] when
+    // packing), every later layer the packed hidden state
+    const DataType_ *x = l == 0 ? ip.input_tensor : hidden_buf;
+    const int *gather = (l == 0 && is_remove_padding_) ? et_param.word_idx : nullptr;
+
+    const DataType_ *wt_qkv;
+    if (ip.prepacked) {
+      wt_qkv = (const DataType_ *)ip.prepacked + (size_t)l * layer_weight_elems();
+    } else {
+      DataType_ *d = staging;
+      const void *src[4] = {w.attr_kernel_QKV, w.attr_output_kernel, w.inter_kernel, w.output_kernel};
+      void *dst[4] = {d, d + (size_t)3 * hidden * hidden, d + (size_t)4 * hidden * hidden,
+                      d + (size_t)4 * hidden * hidden + (size_t)hidden * inter};
+      const int ks[4] = {hidden, hidden, hidden, inter};
+      const int ns[4] = {3 * hidden, hidden, inter, hidden};
+      check_bt_error(bt_transpose_weights(4, src, dst, ks, ns, stream));
+      wt_qkv = staging;
+    }
+    const DataType_ *wt_proj = wt_qkv + (size_t)3 * hidden * hidden;
+    const DataType_ *wt_inter = wt_proj + (size_t)hidden * hidden;
+    const DataType_ *wt_out = wt_inter + (size_t)hidden * inter;
+
+    check_bt_error(bt_gemm_qkv_bias_split(x, gather, wt_qkv, w.attention_param.attr_bias_QKV,
+                                          qkv_buf, valid_rows, rows, rows_hint, head_num_,
+                                          size_per_head_, stream));
+
+    attention_layer_->initialize(w.attention_param);
+    struct AttentionInferParam<DataType_> att {
+      qkv_buf, ip.atten_mask, attr_out_buf, nullptr, batch_size, seq_len, nullptr, stream, et_param
+    };
+    att.attention_bias = ip.attention_bias;
+    att.seq_order = seq_order;
+    attention_layer_->infer(att);
+
+    check_bt_error(bt_gemm(attr_out_buf, wt_proj, attr_matmul_buf, valid_rows, rows, rows_hint,
+                           hidden, hidden, stream));
+    check_bt_error(bt_add_bias_residual_layernorm(
+        attr_matmul_buf, x, gather, w.attr_output_bias, w.attr_output_layernorm_gamma,
+        w.attr_output_layernorm_beta, use_fp32_ ? 1 : 0, valid_rows, rows, hidden, layernorm_eps,
+        stream));
+    check_bt_error(bt_gemm_bias_gelu(attr_matmul_buf, wt_inter, w.inter_bias, inter_matmul_buf,
+                                     valid_rows, rows, rows_hint, inter, hidden, stream));
+
+    const bool last = l == L - 1;
+    // the last layer of the padded path writes straight into the caller's output
+    DataType_ *ffn2_out = (last && !is_remove_padding_) ? ip.transformer_output : hidden_buf;
+    check_bt_error(bt_gemm(inter_matmul_buf, wt_out, ffn2_out, valid_rows, rows, rows_hint, hidden,
+                           inter, stream));
+    if (last && is_remove_padding_)
+      check_bt_error(bt_add_bias_residual_layernorm_restore(
+          ffn2_out, attr_matmul_buf, w.output_bias, w.output_layernorm_gamma,
+          w.output_layernorm_beta, use_fp32_ ? 1 : 0, ip.transformer_output, et_param.batch_idx,
+          batch_size, seq_len, hidden, layernorm_eps, stream));
+    else
+      check_bt_error(bt_add_bias_residual_layernorm(
+          ffn2_out, attr_matmul_buf, nullptr, w.output_bias, w.output_layernorm_gamma,
+          w.output_layernorm_beta, use_fp32_ ? 1 : 0, valid_rows, rows, hidden, layernorm_eps,
+          stream));
+  }
+}
+
+template class BertEncoder<OperationType::FP32>;
+template class BertEncoder<OperationType::HALF>;
+
+}  // namespace bytetransformer

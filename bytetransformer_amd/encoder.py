@@ -77,3 +77,132 @@ def encoder_forward(layers, x, mask):
     for i, layer in enumerate(layers):
         h = layer(h, mask, out=bufs[i & 1])
     return h
+
+
+class BertEncoder:
+    """Every layer of an encoder in one call (bt_encoder_forward): the hidden
+    state stays on the packed rows between layers, the weights are pre-packed
+    once at construction.  The reference has no such interface (one layer per
+    call); the result equals running the layers one by one.
+
+    `layers` is a list of 12-tensor weight sets (dicts by WEIGHT_NAMES or
+    sequences in operator-argument order)."""
+
+    def __init__(self, head_num, head_size, layers, is_remove_padding=True,
+                 use_fused_attention=True, layernorm_eps=1e-6, tao=1.0):
+        sets = []
+        for w in layers:
+            if isinstance(w, dict):
+                w = [w[n] for n in WEIGHT_NAMES]
+            if len(w) != 12:
+                raise ValueError("expected 12 weight tensors per layer")
+            for t in w:
+                if not (t.is_cuda and t.is_contiguous()):
+                    raise ValueError("weights must be contiguous GPU tensors")
+            sets.append(list(w))
+        if not sets:
+            raise ValueError("expected at least one layer")
+        self.weights = sets
+        self.head_num, self.head_size = head_num, head_size
+        self.hidden = head_num * head_size
+        self.is_remove_padding = is_remove_padding
+        self.use_fused_attention = use_fused_attention
+        self.layernorm_eps, self.tao = layernorm_eps, tao
+        self._w = (LayerWeights * len(sets))(
+            *[LayerWeights(*[ctypes.c_void_p(t.data_ptr()) for t in w]) for w in sets])
+        self._prepacked = None
+        self._buf = None
+
+    def _config(self, B, S):
+        w0 = self.weights[0]
+        return EncoderConfig(1, B, S, self.head_num, self.head_size,
+                             w0[6].shape[1] // self.hidden, int(self.use_fused_attention),
+                             int(self.is_remove_padding), int(w0[10].dtype == torch.float32),
+                             self.tao, self.layernorm_eps)
+
+    def prepack(self):
+        """(Re)builds the k-contiguous weight copies; call again after changing weights."""
+        lib = host_lib()
+        cfg = self._config(1, 1)
+        n = lib.bt_encoder_prepack_bytes(ctypes.byref(cfg), len(self.weights))
+        dev = self.weights[0][0].device
+        with torch.cuda.device(dev):
+            buf = torch.empty(n, dtype=torch.int8, device=dev)
+            rc = lib.bt_encoder_prepack(ctypes.byref(cfg), len(self.weights), self._w,
+                                        ctypes.c_void_p(buf.data_ptr()),
+                                        ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+        if rc != 0:
+            raise RuntimeError(lib.bt_encoder_last_error().decode())
+        self._prepacked = buf
+
+    def __call__(self, x, mask, out=None, attention_bias=None, valid_rows_hint=0):
+        lib = host_lib()
+        if x.dtype != torch.float16:
+            raise RuntimeError("only fp16 activations are implemented")
+        B, S, H = x.shape
+        if attention_bias is not None and (
+                attention_bias.dtype != x.dtype or not attention_bias.is_contiguous()
+                or tuple(attention_bias.shape) != (self.head_num, S, S)):
+            raise ValueError("attention_bias must be a contiguous [head_num, S, S] tensor "
+                             "of the activation dtype")
+        if self._prepacked is None:
+            self.prepack()
+        cfg = self._config(B, S)
+        need = lib.bt_encoder_forward_bufsize(ctypes.byref(cfg))
+        if need == 0:
+            raise RuntimeError(lib.bt_encoder_last_error().decode())
+        if self._buf is None or self._buf.numel() < need or self._buf.device != x.device:
+            self._buf = torch.empty(need, dtype=torch.int8, device=x.device)
+        if out is None:
+            out = torch.empty_like(x)
+        rc = lib.bt_encoder_forward(
+            ctypes.byref(cfg), len(self.weights), self._w,
+            ctypes.c_void_p(self._prepacked.data_ptr()), ctypes.c_void_p(x.data_ptr()),
+            ctypes.c_void_p(mask.data_ptr()),
+            ctypes.c_void_p(attention_bias.data_ptr() if attention_bias is not None else None),
+            ctypes.c_void_p(out.data_ptr()), ctypes.c_void_p(self._buf.data_ptr()), B, S,
+            int(valid_rows_hint), ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+        if rc != 0:
+            raise RuntimeError(lib.bt_encoder_last_error().decode())
+        return out
+
+    def graph(self, batch_size, seq_len, valid_rows_hint=0):
+        """Captures one forward for a fixed [batch_size, seq_len] into a HIP graph."""
+        return GraphedBertEncoder(self, batch_size, seq_len, valid_rows_hint)
+
+
+class GraphedBertEncoder:
+    """A captured BertEncoder forward.  `input`, `mask` and `output` are the
+    static tensors the graph reads and writes: fill input / mask (any lengths -
+    the offsets are rebuilt on the device inside the graph), call replay(), read
+    output.  Calling the object copies its arguments in and returns `output`."""
+
+    def __init__(self, encoder, batch_size, seq_len, valid_rows_hint=0):
+        dev = encoder.weights[0][0].device
+        self.encoder = encoder
+        with torch.cuda.device(dev):
+            self.input = torch.zeros(batch_size, seq_len, encoder.hidden, dtype=torch.float16,
+                                     device=dev)
+            self.mask = torch.ones(batch_size, seq_len, seq_len, dtype=torch.float16, device=dev)
+            self.output = torch.empty_like(self.input)
+            # first call outside the capture: one-time kernel attribute set-up, pre-pack, scratch
+            side = torch.cuda.Stream(device=dev)
+            side.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(side):
+                encoder(self.input, self.mask, out=self.output, valid_rows_hint=valid_rows_hint)
+            torch.cuda.current_stream().wait_stream(side)
+            torch.cuda.synchronize(dev)
+            self._graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(self._graph):
+                encoder(self.input, self.mask, out=self.output, valid_rows_hint=valid_rows_hint)
+            # the graph holds raw pointers into these: keep them alive with it
+            self._buf, self._prepacked = encoder._buf, encoder._prepacked
+
+    def replay(self):
+        self._graph.replay()
+        return self.output
+
+    def __call__(self, x, mask):
+        self.input.copy_(x)
+        self.mask.copy_(mask)
+        return self.replay()

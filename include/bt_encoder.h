@@ -66,6 +66,34 @@ int bt_encoder_layer_forward_bias(const bt_encoder_config *cfg, const bt_layer_w
                                   const void *attention_bias, void *output, void *buf,
                                   int batch_size, int seq_len, void *stream);
 
+/*
+ * Whole encoder in one call: num_layers layers (weights[l] = layer l) over one padded
+ * batch, hidden state kept on the packed rows between layers.  No counterpart in the
+ * reference, whose interface is one layer per call: the mask prefix sum runs once,
+ * layer 0 gathers from the padded input, the last layer scatters to the padded output
+ * (rows past each length zero), inner layers neither compress nor restore.  Never
+ * waits for the device and never allocates, so a caller may capture it into a HIP
+ * graph and replay it with other lengths written into the same mask buffer.
+ *
+ *   bt_encoder_forward_bufsize  bytes of scratch `buf` (independent of num_layers)
+ *   bt_encoder_prepack_bytes    bytes of the pre-packed weight area of all layers
+ *   bt_encoder_prepack          fills that area (one launch per layer); do it once per
+ *                               weight set and pass it to every forward
+ *   bt_encoder_forward          prepacked == NULL: each layer's weights are pre-packed
+ *                               inside the call; attention_bias nullable, shared by
+ *                               all layers; valid_rows_hint = expected number of valid
+ *                               tokens or 0 (steers tile shapes only)
+ * cfg->max_batch_size <= 2 or is_remove_padding == 0 runs every layer on the padded rows.
+ */
+unsigned long long bt_encoder_forward_bufsize(const bt_encoder_config *cfg);
+unsigned long long bt_encoder_prepack_bytes(const bt_encoder_config *cfg, int num_layers);
+int bt_encoder_prepack(const bt_encoder_config *cfg, int num_layers,
+                       const bt_layer_weights *weights, void *prepacked, void *stream);
+int bt_encoder_forward(const bt_encoder_config *cfg, int num_layers,
+                       const bt_layer_weights *weights, const void *prepacked, const void *input,
+                       const void *atten_mask, const void *attention_bias, void *output,
+                       void *buf, int batch_size, int seq_len, int valid_rows_hint, void *stream);
+
 const char *bt_encoder_last_error(void);
 
 #ifdef __cplusplus

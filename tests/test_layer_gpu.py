@@ -216,6 +216,74 @@ def test_attention_bias_through_the_layer(device, rm, S, lens):
         layer(_dev(wl.x, device), _dev(wl.mask, device), attention_bias=_dev(bias[:, :-1], device))
 
 
+# ---- whole encoder in one call ---------------------------------------------------
+def _whole_encoder(wl, device, **kw):
+    return bt.BertEncoder(wl.cfg.head_num, wl.cfg.head_size,
+                          [{k: _dev(v, device) for k, v in w.items()} for w in wl.layers], **kw)
+
+
+@pytest.mark.parametrize("name", ["cfg1", "cfg2", "cfg4"])
+def test_whole_encoder_matches_oracle_and_layer_by_layer(device, name):
+    """bt_encoder_forward (hidden state packed between layers) against the oracle and
+    against the per-layer entry point on the same inputs."""
+    _say("whole encoder", name)
+    wl = workload.make_workload(name)
+    n = min(wl.cfg.layers, 4)
+    wl4 = workload.Workload(wl.cfg, wl.lens, wl.x, wl.mask, wl.layers[:n])
+    enc = _whole_encoder(wl4, device)
+    got = enc(_dev(wl.x, device), _dev(wl.mask, device), valid_rows_hint=wl.valid_tokens)
+    torch.cuda.synchronize()
+    got = got.cpu().numpy()
+    rm = wl.cfg.batch > 2
+    _check(got, _oracle(wl4), wl.lens, pads_must_be_zero=rm, tag="whole/" + name)
+    per_layer = _run_c_api(wl4, device)
+    d = np.abs(got.astype(np.float32) - per_layer.astype(np.float32))
+    for b, ln in enumerate(wl.lens):
+        assert d[b, :int(ln)].max() <= 2e-3, d[b, :int(ln)].max()     # same kernels, same order
+
+
+def test_whole_encoder_graph_replays_with_changing_lengths(device):
+    """One captured graph serves any lengths: the offsets are rebuilt on the device
+    inside it.  Replays alternate with eager work and are checked every time."""
+    _say("whole encoder graph")
+    cfg = workload.EncoderConfig("g", 6, 96, 4, layers=3, lens=(96, 40, 77, 5, 60, 31), seed=3)
+    wl = workload.make_workload(cfg, bias_std=0.05, random_affine=True)
+    enc = _whole_encoder(wl, device)
+    g = enc.graph(cfg.batch, cfg.seq_len)
+    rs = np.random.RandomState(0)
+    for it in range(4):
+        lens = np.array(cfg.lens) if it == 0 else rs.randint(1, cfg.seq_len + 1, cfg.batch)
+        mask = workload.make_mask(lens, cfg.seq_len, np.float16)
+        x = (wl.x if it == 0 else rs.standard_normal(wl.x.shape)).astype(np.float16)
+        cur = workload.Workload(cfg, lens, x, mask, wl.layers)
+        out = g(_dev(x, device), _dev(mask, device))
+        torch.cuda.synchronize()
+        got = out.cpu().numpy()
+        eager = enc(_dev(x, device), _dev(mask, device))         # eager work between replays
+        torch.cuda.synchronize()
+        _check(got, _oracle(cur), lens, tag="graph replay %d" % it)
+        assert np.array_equal(got, eager.cpu().numpy())
+
+
+def test_whole_encoder_padded_path_bias_and_errors(device):
+    _say("whole encoder padded / bias / errors")
+    rs = np.random.RandomState(4)
+    cfg = workload.EncoderConfig("p", 2, 40, 2, layers=2, lens=(40, 17), seed=5)
+    wl = workload.make_workload(cfg, bias_std=0.05, random_affine=True)
+    bias = (0.5 * rs.standard_normal((2, 40, 40))).astype(np.float16)
+    enc = _whole_encoder(wl, device)
+    got = enc(_dev(wl.x, device), _dev(wl.mask, device), attention_bias=_dev(bias, device))
+    torch.cuda.synchronize()
+    layers32 = [{k: np.asarray(v, np.float32) for k, v in w.items()} for w in wl.layers]
+    exp = O.encoder(wl.x.astype(np.float32), wl.mask.astype(np.float32), layers32, 2,
+                    attention_bias=bias.astype(np.float32)).numpy()
+    _check(got.cpu().numpy(), exp, wl.lens, pads_must_be_zero=False, tag="whole/padded+bias")
+    with pytest.raises(ValueError):
+        bt.BertEncoder(2, 64, [])
+    with pytest.raises(RuntimeError):
+        enc(_dev(wl.x, device).float(), _dev(wl.mask, device))
+
+
 def test_fp32_gamma_beta_next_to_fp16_weights(device):
     _say("fp32 gamma/beta")
     cfg = workload.EncoderConfig("g32", 4, 96, 4, layers=1, lens=(96, 5, 50, 77), seed=21)
