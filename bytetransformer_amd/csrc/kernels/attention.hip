@@ -54,6 +54,41 @@ struct AttArgs {
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
+// Reductions over the four 16-lane rows of a wave (lanes l, l^16, l^32, l^48) with the
+// row-swap VALU instructions: after a swap of two copies of x, the pair holds x of
+// rows {0,0,2,2} / {1,1,3,3} (16-lane swap) or {0,1,0,1} / {2,3,2,3} (32-lane swap),
+// so one max / add per step folds the partner row in - no LDS round trip.  The empty
+// asm keeps the optimiser from treating the two results of a swap of equal inputs as
+// equal (it then drops the max / add).
+__device__ __forceinline__ void swap_rows16(float x, float &lo, float &hi) {
+  const unsigned u = __builtin_bit_cast(unsigned, x);
+  auto r = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+  unsigned r0 = r[0], r1 = r[1];
+  asm volatile("" : "+v"(r0), "+v"(r1));
+  lo = __builtin_bit_cast(float, r0);
+  hi = __builtin_bit_cast(float, r1);
+}
+__device__ __forceinline__ void swap_rows32(float x, float &lo, float &hi) {
+  const unsigned u = __builtin_bit_cast(unsigned, x);
+  auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  unsigned r0 = r[0], r1 = r[1];
+  asm volatile("" : "+v"(r0), "+v"(r1));
+  lo = __builtin_bit_cast(float, r0);
+  hi = __builtin_bit_cast(float, r1);
+}
+__device__ __forceinline__ float rows_max(float x) {
+  float a, b;
+  swap_rows16(x, a, b);
+  swap_rows32(fmaxf(a, b), a, b);
+  return fmaxf(a, b);
+}
+__device__ __forceinline__ float rows_sum(float x) {
+  float a, b;
+  swap_rows16(x, a, b);
+  swap_rows32(a + b, a, b);
+  return a + b;
+}
+
 // 16-byte chunk swizzles of a [rows][64] fp16 tile (8 chunks per 128-byte row).
 // K is read with ds_read_b128 by 16 consecutive rows at one chunk: slot =
 // chunk ^ (row>>1 & 7) spreads them over all 64 banks.  V is read with the
@@ -280,8 +315,7 @@ __global__ __launch_bounds__(kAttThreads, 2) void attention_grouped_kernel(AttAr
         mx = fmaxf(fmaxf(mx, s[kb][qb][0]), s[kb][qb][1]);
         mx = fmaxf(fmaxf(mx, s[kb][qb][2]), s[kb][qb][3]);
       }
-      mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+      mx = rows_max(mx);
       const float m_new = fmaxf(m_run[qb], mx);
       const float mc = m_new * cs;
       // rescale the running output only when some query's maximum moved
@@ -335,7 +369,7 @@ __global__ __launch_bounds__(kAttThreads, 2) void attention_grouped_kernel(AttAr
   const int H = p.heads * kHeadDim;
 #pragma unroll
   for (int qb = 0; qb < QB; ++qb) {
-    const float inv = 1.0f / (o[4][qb][0] + 1e-6f);
+    const float inv = __builtin_amdgcn_rcpf(o[4][qb][0] + 1e-6f);
     const int q = q0 + (wave * QB + qb) * 16 + lq;
     if (q >= nq) continue;
     half_t *dst = p.out + (size_t)(row_start + q) * H + head * kHeadDim + 4 * lg;
@@ -436,8 +470,7 @@ __global__ __launch_bounds__(kAttThreads) void attention_short_kernel(AttArgs p)
       if (kb * 16 + lg * 4 + r >= klen) s[kb][r] = kNegBig;
       mx = fmaxf(mx, s[kb][r]);
     }
-  mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-  mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+  mx = rows_max(mx);
   const float mc = mx * cs;
   float sum = 0.f;
 #pragma unroll
@@ -447,8 +480,7 @@ __global__ __launch_bounds__(kAttThreads) void attention_short_kernel(AttArgs p)
       s[kb][r] = fast_exp2(__builtin_fmaf(s[kb][r], cs, -mc));
       sum += s[kb][r];
     }
-  sum += __shfl_xor(sum, 16, 64);
-  sum += __shfl_xor(sum, 32, 64);
+  sum = rows_sum(sum);
   const float inv = 1.0f / (sum + 1e-6f);
 
   float4_t o[4];
