@@ -27,12 +27,14 @@ void Attention<OpType>::infer(AttentionInferParam infer_param) {
     check_bt_error(bt_attention_short(infer_param.qkv, infer_param.attention_output,
                                       infer_param.et_param.batch_idx, infer_param.seq_order, mask,
                                       infer_param.attention_bias, infer_param.batch_size, infer_param.seq_len, rows_cap, head_num_, size_per_head_,
-                                      scale, padded_rows, infer_param.stream));
+                                      scale, padded_rows, infer_param.prefetch,
+                                      infer_param.prefetch_bytes, infer_param.stream));
   else
     check_bt_error(bt_attention_grouped(infer_param.qkv, infer_param.attention_output,
                                         infer_param.et_param.batch_idx, infer_param.seq_order, mask,
                                         infer_param.attention_bias, infer_param.batch_size, infer_param.seq_len, rows_cap, head_num_, size_per_head_,
-                                        scale, padded_rows, infer_param.stream));
+                                        scale, padded_rows, infer_param.prefetch,
+                                      infer_param.prefetch_bytes, infer_param.stream));
 }
 
 template class Attention<OperationType::FP32>;

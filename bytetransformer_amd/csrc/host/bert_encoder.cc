@@ -100,6 +100,12 @@ void BertEncoder<OpType>::infer(BertEncoderInferParam<DataType_> ip) {
     };
     att.attention_bias = ip.attention_bias;
     att.seq_order = seq_order;
+    // warm the memory-side cache with what follows in memory order: the rest of this
+    // layer's weights and, when all layers are pre-packed back to back, the next
+    // layer's QKV matrix
+    att.prefetch = wt_proj;
+    att.prefetch_bytes = ((size_t)hidden * hidden + 2 * (size_t)hidden * inter) * sizeof(DataType_);
+    if (ip.prepacked && l + 1 < L) att.prefetch_bytes += (size_t)3 * hidden * hidden * sizeof(DataType_);
     attention_layer_->infer(att);
 
     check_bt_error(bt_gemm(attr_out_buf, wt_proj, attr_matmul_buf, valid_rows, rows, rows_hint,

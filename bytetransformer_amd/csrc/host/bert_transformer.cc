@@ -107,6 +107,13 @@ void BertTransformer<OpType>::bert_infer(BertTransformerInferParam infer_param) 
   };
   attention_infer_param.attention_bias = infer_param.attention_bias;
   attention_infer_param.seq_order = seq_order;
+  // the three weight matrices the rest of the layer reads, when they lie back to back:
+  // the attention kernel pulls them into the memory-side cache while it runs
+  if (wt_inter == wt_proj + (size_t)hidden * hidden && wt_out == wt_inter + (size_t)hidden * inter) {
+    attention_infer_param.prefetch = wt_proj;
+    attention_infer_param.prefetch_bytes =
+        ((size_t)hidden * hidden + 2 * (size_t)hidden * inter) * sizeof(DataType_);
+  }
   attention_layer_->infer(attention_infer_param);
 
   check_bt_error(

@@ -47,6 +47,8 @@ struct AttArgs {
   const half_t *mask;     // optional [B,S,S] 0/1 mask, padded rows only: every key of the
                           // sequence's S rows takes part, shifted by (mask-1)*10000
   const half_t *bias;     // optional [heads,S,S] term added to the scaled logits
+  const char *prefetch;   // optional: memory the NEXT kernels will read (weights); touched
+  unsigned long long prefetch_bytes;   // line by line so it sits in the memory-side cache
   int B, S, rows_cap, heads;
   float scale_log2e;   // scale * log2(e)
   int padded_rows;
@@ -87,6 +89,29 @@ __device__ __forceinline__ float rows_sum(float x) {
   swap_rows16(x, a, b);
   swap_rows32(a + b, a, b);
   return a + b;
+}
+
+// Cache warm-up on behalf of later kernels: the workgroups of the second half of the
+// issue order (short sequences and dead tiles, which retire early) each touch one
+// dword per 128-byte line of their slice of [prefetch, prefetch + bytes).  The loads
+// are the wave's last instructions; nothing reads their results.
+__device__ __forceinline__ void prefetch_slice(const AttArgs &p) {
+  if (!p.prefetch) return;
+  const unsigned z0 = gridDim.z / 2;
+  if (blockIdx.z < z0) return;
+  const unsigned long long duty = (unsigned long long)gridDim.x * gridDim.y * (gridDim.z - z0);
+  const unsigned long long me =
+      ((unsigned long long)(blockIdx.z - z0) * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x;
+  const unsigned long long lines = (p.prefetch_bytes + 127) / 128;
+  const unsigned long long per = (lines + duty - 1) / duty;
+  const unsigned long long first = me * per;
+  const unsigned long long last = first + per < lines ? first + per : lines;
+  for (unsigned long long l = first + threadIdx.x; l < last; l += blockDim.x) {
+    unsigned sink;
+    const char *addr = p.prefetch + l * 128;
+    asm volatile("global_load_dword %0, %1, off" : "=v"(sink) : "v"(addr) : "memory");
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 }
 
 // 16-byte chunk swizzles of a [rows][64] fp16 tile (8 chunks per 128-byte row).
@@ -181,7 +206,10 @@ __global__ __launch_bounds__(kAttThreads, 2) void attention_grouped_kernel(AttAr
   const int row_start = p.padded_rows ? b * p.S : seq_start;
   const int nq = p.padded_rows ? p.S : klen;
   const int q0 = blockIdx.x * BQ;
-  if (q0 >= nq) return;
+  if (q0 >= nq) {
+    prefetch_slice(p);
+    return;
+  }
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int lq = lane & 15, lg = lane >> 4;
@@ -379,6 +407,7 @@ __global__ __launch_bounds__(kAttThreads, 2) void attention_grouped_kernel(AttAr
       *(half4_t *)(dst + 16 * db) = half4_t{(half_t)v[0], (half_t)v[1], (half_t)v[2], (half_t)v[3]};
     }
   }
+  prefetch_slice(p);
 }
 
 // ---------------------------------------------------------------------------
@@ -398,7 +427,10 @@ __global__ __launch_bounds__(kAttThreads) void attention_short_kernel(AttArgs p)
   const int row_start = p.padded_rows ? b * p.S : seq_start;
   const int nq = p.padded_rows ? p.S : klen;
   const int q0 = blockIdx.x * BQ;
-  if (q0 >= nq) return;
+  if (q0 >= nq) {
+    prefetch_slice(p);
+    return;
+  }
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int lq = lane & 15, lg = lane >> 4;
@@ -509,6 +541,7 @@ __global__ __launch_bounds__(kAttThreads) void attention_short_kernel(AttArgs p)
       *(half4_t *)(dst_row + 16 * db) =
           half4_t{(half_t)o[db][0], (half_t)o[db][1], (half_t)o[db][2], (half_t)o[db][3]};
   }
+  prefetch_slice(p);
 }
 
 static int check_att_args(const char *who, const void *qkv, const void *out, const int *batch_idx,
@@ -556,14 +589,17 @@ extern "C" int bt_attention_short(const void *qkv_heads, void *attention_output,
                                   const int *batch_idx, const int *seq_order,
                                   const void *atten_mask, const void *attention_bias,
                                   int batch_size, int seq_len, int rows_cap, int head_num,
-                                  int size_per_head, float scale, int padded_rows, void *stream) {
+                                  int size_per_head, float scale, int padded_rows,
+                                  const void *prefetch, unsigned long long prefetch_bytes,
+                                  void *stream) {
   int rc = check_att_args("bt_attention_short", qkv_heads, attention_output, batch_idx, atten_mask,
                           padded_rows, batch_size, seq_len, rows_cap, head_num, size_per_head);
   if (rc) return rc;
   BT_REQUIRE(seq_len <= 512, BT_ERR_UNSUPPORTED,
              "bt_attention_short: seq_len=%d exceeds 512, use bt_attention_grouped", seq_len);
   AttArgs a{(const half_t *)qkv_heads, (half_t *)attention_output, batch_idx, seq_order,
-            (const half_t *)atten_mask, (const half_t *)attention_bias, batch_size, seq_len,
+            (const half_t *)atten_mask, (const half_t *)attention_bias,
+            prefetch_bytes && option_prefetch() ? (const char *)prefetch : nullptr, prefetch_bytes, batch_size, seq_len,
             rows_cap, head_num, scale * kLog2e, padded_rows};
   hipStream_t s = as_stream(stream);
   if (seq_len <= 64) return launch_short<4>(a, s);
@@ -578,13 +614,15 @@ extern "C" int bt_attention_grouped(const void *qkv_heads, void *attention_outpu
                                     const void *atten_mask, const void *attention_bias,
                                     int batch_size, int seq_len, int rows_cap, int head_num,
                                     int size_per_head, float scale, int padded_rows,
+                                    const void *prefetch, unsigned long long prefetch_bytes,
                                     void *stream) {
   int rc = check_att_args("bt_attention_grouped", qkv_heads, attention_output, batch_idx,
                           atten_mask, padded_rows, batch_size, seq_len, rows_cap, head_num,
                           size_per_head);
   if (rc) return rc;
   AttArgs a{(const half_t *)qkv_heads, (half_t *)attention_output, batch_idx, seq_order,
-            (const half_t *)atten_mask, (const half_t *)attention_bias, batch_size, seq_len,
+            (const half_t *)atten_mask, (const half_t *)attention_bias,
+            prefetch_bytes && option_prefetch() ? (const char *)prefetch : nullptr, prefetch_bytes, batch_size, seq_len,
             rows_cap, head_num, scale * kLog2e, padded_rows};
   hipStream_t s = as_stream(stream);
   // 128-query tiles once there is enough work to fill the chip, else 64

@@ -44,6 +44,7 @@ int hip_fail(hipError_t e, const char *what);
 // ---- tuning options (bt_set_option) ----------------------------------------
 int option_gemm_tile();      // -1 = heuristic, else index into the tile table
 int option_attention_qb();   // -1 = heuristic, 1 or 2 = query blocks per wave
+int option_prefetch();       // 1 = honour the prefetch hints of the attention entries (default), 0 = ignore
 
 inline hipStream_t as_stream(void *s) { return reinterpret_cast<hipStream_t>(s); }
 

@@ -124,9 +124,16 @@ class BTEncoder : public IBTEncoder {
     const void *src[4];
     void *dst[4];
     int ks[4], ns[4];
+    // one allocation for the four copies: the layer hands the last three to the
+    // attention kernel as one range to warm the cache with
+    int64_t total = 0;
+    for (int i = 0; i < 4; ++i) total += weights_[kIdx[i]].numel();
+    Tensor block = torch::empty({total}, weights_[kIdx[0]].options());
+    int64_t at = 0;
     for (int i = 0; i < 4; ++i) {
       const Tensor &w = weights_[kIdx[i]];
-      out[i] = torch::empty({w.size(1), w.size(0)}, w.options());
+      out[i] = block.narrow(0, at, w.numel()).view({w.size(1), w.size(0)});
+      at += w.numel();
       src[i] = w.data_ptr();
       dst[i] = out[i].data_ptr();
       ks[i] = (int)w.size(0);

@@ -126,7 +126,7 @@ def gemm_qkv_bias_split(a, wt_qkv, bias_qkv, head_num, size_per_head=64, valid_r
 
 
 def _attention(fn, qkv_heads, batch_idx, batch_size, seq_len, scale, padded_rows, out,
-               seq_order=None, mask=None, bias=None):
+               seq_order=None, mask=None, bias=None, prefetch=None):
     _, head_num, rows_cap, d = qkv_heads.shape
     if out is None:
         out = torch.zeros(rows_cap, head_num * d, dtype=qkv_heads.dtype, device=qkv_heads.device)
@@ -134,20 +134,21 @@ def _attention(fn, qkv_heads, batch_idx, batch_size, seq_len, scale, padded_rows
         raise ValueError("attention bias must be [head_num, seq_len, seq_len]")
     _check(fn(_ptr(qkv_heads), _ptr(out), _ptr(batch_idx), _ptr(seq_order), _ptr(mask), _ptr(bias),
               batch_size, seq_len, rows_cap, head_num, d, float(scale), int(padded_rows),
+              _ptr(prefetch), prefetch.numel() * prefetch.element_size() if prefetch is not None else 0,
               _stream()))
     return out
 
 
 def attention_short(qkv_heads, batch_idx, batch_size, seq_len, scale, padded_rows=False, out=None,
-                    seq_order=None, mask=None, bias=None):
+                    seq_order=None, mask=None, bias=None, prefetch=None):
     return _attention(kernel_lib().bt_attention_short, qkv_heads, batch_idx, batch_size, seq_len,
-                      scale, padded_rows, out, seq_order, mask, bias)
+                      scale, padded_rows, out, seq_order, mask, bias, prefetch)
 
 
 def attention_grouped(qkv_heads, batch_idx, batch_size, seq_len, scale, padded_rows=False,
-                      out=None, seq_order=None, mask=None, bias=None):
+                      out=None, seq_order=None, mask=None, bias=None, prefetch=None):
     return _attention(kernel_lib().bt_attention_grouped, qkv_heads, batch_idx, batch_size,
-                      seq_len, scale, padded_rows, out, seq_order, mask, bias)
+                      seq_len, scale, padded_rows, out, seq_order, mask, bias, prefetch)
 
 
 def add_bias_residual_layernorm(out, residual, bias, gamma, beta, eps=1e-6, valid_rows=None,

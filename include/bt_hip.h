@@ -46,9 +46,10 @@ const char *bt_last_error_string(void);
 
 /*
  * Tuning knob for experiments and tests; no counterpart in the reference.
- *   "gemm_tile"     -1 heuristic | 0: 256x256 tile, 8 waves | 1: 128x128, 4 waves, 2-stage ring |
- *                   2: 128x128, 8 waves, 3-stage ring | 3: 256x192, 8 waves
+ *   "gemm_tile"     -1 heuristic | 0: 256x256 tile, 8 waves | 1: 128x128, 4 computing + 4 loader
+ *                   waves | 2: 256x128, 8 + 4 waves | 3: 256x192, 8 waves
  *   "attention_qb"  -1 heuristic | 1 | 2: 16-query blocks per wave in the grouped kernel
+ *   "prefetch"      1 (default) | 0: honour / ignore the prefetch hint of the attention entries
  * Process-wide; results do not depend on it beyond fp32 summation order.
  */
 int bt_set_option(const char *name, int value);
@@ -147,6 +148,11 @@ int bt_gemm_qkv_bias_split(const void *a, const int *a_row_index, const void *wt
  *                     term, as the reference's unfused softmax does (softmax.h:41-46,
  *                     attention_nofused.cu:78-95); positions are relative to the
  *                     start of the sequence in both row layouts.
+ *   prefetch, prefetch_bytes (nullable / 0): a readable device range that LATER kernels
+ *                     of the stream will read, typically the layer's remaining weight
+ *                     matrices.  Workgroups that retire early touch it line by line so
+ *                     that it sits in the memory-side cache by then; purely a hint, the
+ *                     results do not depend on it.  No counterpart in the reference.
  *   seq_order (nullable): a permutation of the sequence indices from
  *                     bt_build_offsets; workgroups are issued in that order so the
  *                     longest sequences start first.  Results do not depend on it.
@@ -165,12 +171,14 @@ int bt_gemm_qkv_bias_split(const void *a, const int *a_row_index, const void *wt
 int bt_attention_short(const void *qkv_heads, void *attention_output, const int *batch_idx,
                        const int *seq_order, const void *atten_mask, const void *attention_bias,
                        int batch_size, int seq_len, int rows_cap, int head_num, int size_per_head,
-                       float scale, int padded_rows, void *stream);
+                       float scale, int padded_rows, const void *prefetch,
+                       unsigned long long prefetch_bytes, void *stream);
 
 int bt_attention_grouped(const void *qkv_heads, void *attention_output, const int *batch_idx,
                          const int *seq_order, const void *atten_mask, const void *attention_bias,
                          int batch_size, int seq_len, int rows_cap, int head_num,
-                         int size_per_head, float scale, int padded_rows, void *stream);
+                         int size_per_head, float scale, int padded_rows, const void *prefetch,
+                         unsigned long long prefetch_bytes, void *stream);
 
 /*
  * out = LayerNorm((out + residual) + bias) * gamma + beta, in place on `out`,

@@ -38,6 +38,10 @@ struct AttentionInferParam {
   // Extension: sequence indices by descending length from bt_build_offsets; the
   // kernels then start the longest sequences first.  May be null.
   const int *seq_order = nullptr;
+  // Extension: a device range later kernels of the stream will read (the layer's
+  // remaining weights); the attention kernel warms the memory-side cache with it.
+  const void *prefetch = nullptr;
+  unsigned long long prefetch_bytes = 0;
 };
 
 template <OperationType OpType>

@@ -420,6 +420,30 @@ def test_attention_bias(device, kind, S, padded, with_mask):
         assert err.max() <= 4e-3, (b, err.max())
 
 
+@pytest.mark.parametrize("kind,lens,S", [("short", [100, 7, 64], 128), ("grouped", [300, 40, 129, 5], 320),
+                                        ("grouped", [77], 96)])
+def test_attention_prefetch_hint_changes_nothing(device, kind, lens, S):
+    """The cache warm-up range is only read: same output bits with and without it, for
+    sizes that are not multiples of a line and for a single-sequence grid."""
+    _say("attention prefetch", kind, lens, S)
+    rs = np.random.RandomState(len(lens) + S)
+    bi, M, qkv = _attention_case(rs, lens, S, 2, scale_q=1.0)
+    fn = ops.attention_short if kind == "short" else ops.attention_grouped
+    base = fn(_dev(qkv, device), _dev(bi, device), len(lens), S, 0.125, False)
+    for nbytes in (1, 127, 128, 1000003, 8 << 20):
+        warm = torch.full((nbytes,), 7, dtype=torch.uint8, device=device)
+        got = fn(_dev(qkv, device), _dev(bi, device), len(lens), S, 0.125, False, prefetch=warm)
+        torch.cuda.synchronize()
+        assert torch.equal(got[:M], base[:M])
+        assert bool((warm == 7).all())
+    ops.set_option("prefetch", 0)
+    try:
+        got = fn(_dev(qkv, device), _dev(bi, device), len(lens), S, 0.125, False, prefetch=warm)
+        assert torch.equal(got[:M], base[:M])
+    finally:
+        ops.set_option("prefetch", 1)
+
+
 def test_attention_large_logits_do_not_overflow(device):
     """Logits of a few hundred in magnitude (fp16 Q.K would overflow at 65504)."""
     rs = np.random.RandomState(9)
