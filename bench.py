@@ -171,9 +171,10 @@ def measured_traffic(workload_name, kernel):
         return None
 
 
-def cpu_baseline(wl, budget_s=25.0):
-    """The oracle's PyTorch fp32 encoder on the padded batch, all host cores,
-    on as many of the L layers as fit the time budget (at least one)."""
+def cpu_baseline(wl, budget_s=25.0, target_s=10.0):
+    """The oracle's PyTorch fp32 encoder on the padded batch, all host cores: whole
+    forwards repeated until about target_s of CPU work is done, cut off inside a
+    forward at budget_s (at least one layer is timed)."""
     import numpy as np
     import torch
     from oracle import bert_oracle as O
@@ -186,18 +187,22 @@ def cpu_baseline(wl, budget_s=25.0):
     with torch.no_grad():
         O.encoder_layer(x, mask, layers32[0], wl.cfg.head_num)       # warm-up
         done, t0 = 0, time.perf_counter()
-        h = x
-        for w in layers32:
-            h = O.encoder_layer(h, mask, w, wl.cfg.head_num)
-            done += 1
-            if time.perf_counter() - t0 > budget_s:
+        while True:
+            h = x
+            for w in layers32:
+                h = O.encoder_layer(h, mask, w, wl.cfg.head_num)
+                done += 1
+                if time.perf_counter() - t0 > budget_s:
+                    break
+            if time.perf_counter() - t0 > target_s:
                 break
         el = time.perf_counter() - t0
     ms_full = el / done * len(layers32) * 1e3
     return {"value": round(ms_full, 1), "unit": "ms", "cores": cores, "kind": "port",
-            "sample": "%d of %d layers of the same padded batch timed (%.1f s), scaled to %d layers; "
-                      "fp32 PyTorch CPU restatement of the reference's encoder script"
-                      % (done, len(layers32), el, len(layers32)),
+            "sample": "%d layer passes (%.1f forwards of %d layers) of the same padded batch timed "
+                      "in %.1f s, scaled to one forward; fp32 PyTorch CPU restatement of the "
+                      "reference's encoder script"
+                      % (done, done / len(layers32), len(layers32), el),
             "tokens_per_s": round(wl.valid_tokens / (ms_full * 1e-3), 1)}
 
 
