@@ -2,6 +2,8 @@
 // reductions, error plumbing for the C ABI.
 #pragma once
 #include <hip/hip_runtime.h>
+
+#include <atomic>
 #include <hip/hip_fp16.h>
 
 #include <cstdarg>
@@ -42,6 +44,30 @@ int hip_fail(hipError_t e, const char *what);
   } while (0)
 
 // ---- tuning options (bt_set_option) ----------------------------------------
+// Once-per-device set-up of a kernel's dynamic LDS limit (the attribute belongs to the
+// function on one device).  `done` is the kernel's own flag array; a lost race only
+// repeats an idempotent call.
+constexpr int kMaxDevices = 64;
+template <typename Kernel>
+inline int allow_dynamic_lds(Kernel kernel, size_t bytes, std::atomic<bool> (&done)[kMaxDevices],
+                             const char *what) {
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return hip_fail(e, "hipGetDevice");
+  if (dev < 0 || dev >= kMaxDevices) {
+    e = hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+                            (int)bytes);
+    return e == hipSuccess ? BT_OK : hip_fail(e, what);
+  }
+  if (!done[dev].load(std::memory_order_acquire)) {
+    e = hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+                            (int)bytes);
+    if (e != hipSuccess) return hip_fail(e, what);
+    done[dev].store(true, std::memory_order_release);
+  }
+  return BT_OK;
+}
+
 int option_gemm_tile();      // -1 = heuristic, else index into the tile table
 int option_attention_qb();   // -1 = heuristic, 1 or 2 = query blocks per wave
 int option_prefetch();       // 1 = honour the prefetch hints of the attention entries (default), 0 = ignore

@@ -372,13 +372,10 @@ template <int BM, int BN, int STAGES, int WM, int WN, int NP, int SCHED, int EPI
 static int launch_gemm_tile(GemmArgs p, hipStream_t s) {
   constexpr size_t smem = (size_t)STAGES * (BM + BN) * kBK * sizeof(half_t);
   static_assert(smem <= 160 * 1024, "LDS budget");
-  static bool configured = false;  // benign race: setting the attribute is idempotent
-  if (!configured) {
-    hipError_t e = hipFuncSetAttribute((const void *)gemm_kernel<BM, BN, STAGES, WM, WN, NP, SCHED, EPI>,
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
-    if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute(gemm_kernel)");
-    configured = true;
-  }
+  static std::atomic<bool> configured[kMaxDevices];
+  const int rc = allow_dynamic_lds(gemm_kernel<BM, BN, STAGES, WM, WN, NP, SCHED, EPI>, smem,
+                                   configured, "hipFuncSetAttribute(gemm_kernel)");
+  if (rc != BT_OK) return rc;
   const int tiles_m = (p.rows_cap + BM - 1) / BM;
   p.tiles_n = (p.N + BN - 1) / BN;
   const int grid = (tiles_m * p.tiles_n + 7) / 8 * 8;
@@ -395,6 +392,8 @@ static int launch_gemm(GemmArgs p, hipStream_t s) {
   //   2: 256x128, 3, 4x2, 4   narrow outputs with enough rows to fill the chip
   //   3: 256x192, 2, 4x2, 0   outputs that split into 192-wide panels but not into a
   //                           full wave of 256-wide ones (QKV at hidden 768)
+  //   4:  32x64,  4, 1x2, 2   a few hundred rows or fewer: the k loop of one tile is the
+  //                           whole run time, and a small tile has the shortest k-step
   // The choice minimises rounds x (k-steps x time of one k-step + fill and epilogue)
   // with the measured per-shape times below, for the estimated live rows: the exact
   // count when every row is live, the caller's hint when it has one, else 60 % of
@@ -415,16 +414,24 @@ static int launch_gemm(GemmArgs p, hipStream_t s) {
     struct Cand {
       int id, bm, bn;
       float step_us, fixed_us;   // one k-step of one tile; fill + epilogue of one tile
+      bool shares_cu;            // several workgroups per CU: time grows with tiles / CUs, not in rounds
     };
-    const Cand cands[4] = {{0, 256, 256, 1.29f, 3.4f},
-                           {3, 256, 192, 1.04f, 2.8f},
-                           {2, 256, 128, 0.62f, 2.3f},
-                           {1, 128, 128, 0.43f, 1.8f}};
+    const Cand cands[5] = {{0, 256, 256, 1.29f, 3.4f, false},
+                           {3, 256, 192, 1.04f, 2.8f, false},
+                           {2, 256, 128, 0.62f, 2.3f, false},
+                           {1, 128, 128, 0.43f, 1.8f, false},
+                           {4, 32, 64, 0.16f, 2.6f, true}};
     const float nk = (float)(p.K / kBK);
     float best = 0.f;
     for (const Cand &c : cands) {
       const long long tiles = ((m_est + c.bm - 1) / c.bm) * ((p.N + c.bn - 1) / c.bn);
-      const float t = (float)((tiles + cus - 1) / cus) * (nk * c.step_us + c.fixed_us);
+      float t;
+      if (c.shares_cu) {
+        const float load = (float)tiles / (float)cus;
+        t = c.fixed_us + nk * c.step_us * (load > 1.f ? load : 1.f);
+      } else {
+        t = (float)((tiles + cus - 1) / cus) * (nk * c.step_us + c.fixed_us);
+      }
       if (choice < 0 || t < best) {
         best = t;
         choice = c.id;
@@ -438,6 +445,8 @@ static int launch_gemm(GemmArgs p, hipStream_t s) {
       return launch_gemm_tile<256, 128, 3, 4, 2, 4, 1, EPI>(p, s);
     case 3:
       return launch_gemm_tile<256, 192, 2, 4, 2, 0, 1, EPI>(p, s);
+    case 4:
+      return launch_gemm_tile<32, 64, 4, 1, 2, 2, 0, EPI>(p, s);
     default:
       return launch_gemm_tile<128, 128, 3, 2, 2, 4, 0, EPI>(p, s);
   }
