@@ -42,15 +42,6 @@ KERNEL_ABI = {
     "bt_gemm_bias_gelu": (c_int, [_P, _P, _P, _P, _IP, c_int, c_int, c_int, c_int, _P]),
     "bt_gemm_qkv_bias_split": (c_int, [_P, _IP, _P, _P, _P, _IP, c_int, c_int, c_int, c_int,
                                        _P]),
-    "bt_gemm_bias_residual_stats": (c_int, [_P, _P, _P, _P, _IP, _P, _P, _IP, c_int, c_int, c_int,
-                                            c_int, _P]),
-    "bt_fold_layernorm": (c_int, [_P, _P, _P, c_int, _P, _P, _P, c_int, c_int, _P]),
-    "bt_gemm_layernorm_bias_gelu": (c_int, [_P, _P, _P, _P, _P, c_float, _P, _IP, c_int, c_int,
-                                            c_int, c_int, _P]),
-    "bt_add_bias_lnresidual_layernorm": (c_int, [_P, _P, _P, _P, _P, _P, _P, _P, c_int, _IP, c_int,
-                                                 c_int, c_float, _P]),
-    "bt_add_bias_lnresidual_layernorm_restore": (c_int, [_P, _P, _P, _P, _P, _P, _P, _P, c_int, _P,
-                                                         _IP, c_int, c_int, c_int, c_float, _P]),
     "bt_attention_short": (c_int, [_P, _P, _IP, _IP, _P, _P, c_int, c_int, c_int, c_int, c_int,
                                    c_float, c_int, _P, c_ulonglong, _P]),
     "bt_attention_grouped": (c_int, [_P, _P, _IP, _IP, _P, _P, c_int, c_int, c_int, c_int, c_int,

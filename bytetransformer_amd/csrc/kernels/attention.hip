@@ -56,6 +56,28 @@ struct AttArgs {
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
+// Reductions over the four 16-lane rows of a wave (lanes l, l^16, l^32, l^48) with the
+// row-swap VALU instructions: after a swap of two copies of x, the pair holds x of
+// rows {0,0,2,2} / {1,1,3,3} (16-lane swap) or {0,1,0,1} / {2,3,2,3} (32-lane swap),
+// so one max / add per step folds the partner row in - no LDS round trip.  The empty
+// asm keeps the optimiser from treating the two results of a swap of equal inputs as
+// equal (it then drops the max / add).
+__device__ __forceinline__ void swap_rows16(float x, float &lo, float &hi) {
+  const unsigned u = __builtin_bit_cast(unsigned, x);
+  auto r = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+  unsigned r0 = r[0], r1 = r[1];
+  asm volatile("" : "+v"(r0), "+v"(r1));
+  lo = __builtin_bit_cast(float, r0);
+  hi = __builtin_bit_cast(float, r1);
+}
+__device__ __forceinline__ void swap_rows32(float x, float &lo, float &hi) {
+  const unsigned u = __builtin_bit_cast(unsigned, x);
+  auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  unsigned r0 = r[0], r1 = r[1];
+  asm volatile("" : "+v"(r0), "+v"(r1));
+  lo = __builtin_bit_cast(float, r0);
+  hi = __builtin_bit_cast(float, r1);
+}
 __device__ __forceinline__ float rows_max(float x) {
   float a, b;
   swap_rows16(x, a, b);

@@ -33,13 +33,7 @@
 namespace bt {
 
 
-enum Epilogue {
-  kEpiPlain = 0,
-  kEpiBiasGelu = 1,
-  kEpiQkvSplit = 2,
-  kEpiResidualStats = 3,   // + bias + residual, and per-row sums for a LayerNorm applied later
-  kEpiLnBiasGelu = 4       // LayerNorm of the A rows folded in (statistics given), + bias, GELU
-};
+enum Epilogue { kEpiPlain = 0, kEpiBiasGelu = 1, kEpiQkvSplit = 2 };
 
 struct GemmArgs {
   const half_t *a;      // [rows_cap, K]
@@ -51,18 +45,6 @@ struct GemmArgs {
   int rows_cap, N, K;
   int tiles_n;
   int rows_hint;        // host-side estimate of the live rows (0 = unknown); tile choice only
-  // kEpiResidualStats: x = fp16(fp16(acc + residual row) + bias) is stored, and per row the sums
-  // (sum x, sum x^2) over each workgroup's columns go to stats[row][n0 / 64] (the other
-  // 64-column slots the workgroup covers are zeroed), so sum over the N/64 slots = whole row
-  const half_t *residual;       // [*, N]
-  const int *res_row_index;     // optional gather of the residual rows (live rows only)
-  float2 *stats_out;            // [rows_cap][N / 64]
-  // kEpiLnBiasGelu: C = gelu(rstd * (A.W' - mean * g) + b), W' = diag(gamma).W pre-scaled,
-  // g[n] = sum_k W'[k][n], b[n] = sum_k beta[k] W[k][n] + bias[n]; mean / rstd of A's rows
-  // from stats_in[row][K / 64]
-  const float2 *stats_in;
-  const float *fold_g, *fold_b;
-  float eps;
 };
 
 __device__ __forceinline__ float gelu_tanh_f32(float x) {
@@ -218,31 +200,11 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs &p) {
       if (++stage == STAGES) stage = 0;
     }
     __builtin_amdgcn_s_barrier();                 // pairs with the barrier before the epilogue
-    if (EPI == kEpiResidualStats) __builtin_amdgcn_s_barrier();   // ... and the one inside it
     return;
   }
 
   // ---- computing side -------------------------------------------------------
   const int wm = wave / WN, wn = wave % WN;
-  // mean and 1/std of this tile's A rows, from the per-slot sums (visible to all
-  // computing waves after the first barrier of the k loop)
-  float2 *rowstat = (float2 *)(smem + (size_t)STAGES * STAGE_HALFS);
-  if (EPI == kEpiLnBiasGelu) {
-    const int slots = p.K >> 6;
-    const float inv_k = 1.0f / (float)p.K;
-    for (int r = tid; r < BM; r += NW * 64) {
-      const int m = min(m0 + r, p.rows_cap - 1);
-      float s1 = 0.f, s2 = 0.f;
-      for (int sl = 0; sl < slots; ++sl) {
-        const float2 v = p.stats_in[(size_t)m * slots + sl];
-        s1 += v.x;
-        s2 += v.y;
-      }
-      const float mean = s1 * inv_k;
-      const float var = fmaxf(s2 * inv_k - mean * mean, 0.f);
-      rowstat[r] = make_float2(mean, rsqrtf(var + p.eps));
-    }
-  }
   float16_t acc[TN][TM];
 #pragma unroll
   for (int i = 0; i < TN; ++i)
@@ -308,56 +270,15 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs &p) {
   constexpr int CPRW = WTN / 8;   // 16-byte chunks per staged row
   constexpr int RPS = 64 / CPRW;  // rows per store instruction
   const int sr = lane / CPRW, sc = (lane % CPRW) * 8;
-  // per-wave row sums of the stats epilogue, behind the staging tiles
-  float2 *wstat = (float2 *)(smem + (((size_t)NW * 32 * EP + 3) & ~(size_t)3));
-  static_assert(EPI != kEpiResidualStats ||
-                    (((size_t)NW * 32 * EP + 3) & ~(size_t)3) * sizeof(half_t) +
-                            (size_t)NW * TM * 32 * sizeof(float2) <=
-                        (size_t)STAGES * STAGE_HALFS * sizeof(half_t),
-                "row sums fit behind the staging tiles");
 #pragma unroll
   for (int j = 0; j < TM; ++j) {
-    float s1 = 0.f, s2 = 0.f;
-    const half_t *res_row = nullptr;
-    float2 ms = {0.f, 1.f};
-    if (EPI == kEpiResidualStats) {
-      const int m = m0 + wm * WTM + j * 32 + row_in;
-      const int mc = min(m, max(M - 1, 0));
-      const size_t rr = p.res_row_index ? (size_t)p.res_row_index[mc] : (size_t)min(m, p.rows_cap - 1);
-      res_row = p.residual + rr * p.N;
-    }
-    if (EPI == kEpiLnBiasGelu) ms = rowstat[wm * WTM + j * 32 + row_in];
 #pragma unroll
     for (int i = 0; i < TN; ++i) {
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
         float v0 = acc[i][j][4 * q + 0], v1 = acc[i][j][4 * q + 1];
         float v2 = acc[i][j][4 * q + 2], v3 = acc[i][j][4 * q + 3];
-        if (EPI == kEpiResidualStats) {
-          const int nn = n0 + wn * WTN + i * 32 + q * 8 + col_in;
-          const int n = min(nn, p.N - 4);
-          const half4_t b = *(const half4_t *)(p.bias + n);
-          const half4_t r = *(const half4_t *)(res_row + n);
-          // the two fp16-rounded adds of the LayerNorm kernel it replaces
-          const half4_t a16 = {(half_t)v0, (half_t)v1, (half_t)v2, (half_t)v3};
-          const half4_t x = (a16 + r) + b;
-          v0 = (float)x[0];
-          v1 = (float)x[1];
-          v2 = (float)x[2];
-          v3 = (float)x[3];
-          if (nn < p.N) {
-            s1 += (v0 + v1) + (v2 + v3);
-            s2 += (v0 * v0 + v1 * v1) + (v2 * v2 + v3 * v3);
-          }
-        } else if (EPI == kEpiLnBiasGelu) {
-          const int n = min(n0 + wn * WTN + i * 32 + q * 8 + col_in, p.N - 4);
-          const float4_t g = *(const float4_t *)(p.fold_g + n);
-          const float4_t b = *(const float4_t *)(p.fold_b + n);
-          v0 = gelu_tanh_f32(ms.y * (v0 - ms.x * g[0]) + b[0]);
-          v1 = gelu_tanh_f32(ms.y * (v1 - ms.x * g[1]) + b[1]);
-          v2 = gelu_tanh_f32(ms.y * (v2 - ms.x * g[2]) + b[2]);
-          v3 = gelu_tanh_f32(ms.y * (v3 - ms.x * g[3]) + b[3]);
-        } else if (EPI != kEpiPlain) {
+        if (EPI != kEpiPlain) {
           const int n = min(n0 + wn * WTN + i * 32 + q * 8 + col_in, p.N - 4);
           const half4_t b = *(const half4_t *)(p.bias + n);
           v0 += (float)b[0];
@@ -375,15 +296,6 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs &p) {
             half4_t{(half_t)v0, (half_t)v1, (half_t)v2, (half_t)v3};
       }
     }
-    if (EPI == kEpiResidualStats) {
-      // lanes l and l + 32 hold the two column halves of the same row
-      float a, b;
-      swap_rows32(s1, a, b);
-      s1 = a + b;
-      swap_rows32(s2, a, b);
-      s2 = a + b;
-      if (lane < 32) wstat[(wave * TM + j) * 32 + lane] = make_float2(s1, s2);
-    }
 #pragma unroll
     for (int r0 = 0; r0 < 32; r0 += RPS) {
       const int r = r0 + sr;
@@ -398,27 +310,6 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs &p) {
           *(uint4_t *)(p.c + (size_t)m * p.N + n) = v;
         }
       }
-    }
-  }
-  if (EPI == kEpiResidualStats) {
-    asm volatile("" ::: "memory");
-    __builtin_amdgcn_s_barrier();   // every wave's row sums are in LDS
-    asm volatile("" ::: "memory");
-    const int slots = p.N >> 6;
-    for (int r = tid; r < BM; r += NW * 64) {
-      const int m = m0 + r;
-      if (m >= M) continue;
-      const int rwm = r / WTM, rj = (r % WTM) / 32, rl = r % 32;
-      float t1 = 0.f, t2 = 0.f;
-#pragma unroll
-      for (int w = 0; w < WN; ++w) {
-        const float2 v = wstat[((rwm * WN + w) * TM + rj) * 32 + rl];
-        t1 += v.x;
-        t2 += v.y;
-      }
-      float2 *dst = p.stats_out + (size_t)m * slots + (n0 >> 6);
-      dst[0] = make_float2(t1, t2);
-      for (int sl = 1; sl < BN / 64 && (n0 >> 6) + sl < slots; ++sl) dst[sl] = make_float2(0.f, 0.f);
     }
   }
 }
@@ -477,46 +368,9 @@ __global__ __launch_bounds__(256) void transpose_kernel(TransposeArgs a) {
   }
 }
 
-// ---- LayerNorm folded into the GEMM that consumes it ---------------------------
-// y = LN(x) . W + bias with LN(x) = (x - mean) rstd gamma + beta equals
-//   rstd (x . W' - mean g) + b,   W' = diag(gamma) W,  g[n] = sum_k W'[k][n],
-//   b[n] = sum_k beta[k] W[k][n] + bias[n].
-// One wave per output column n (a row of the [N, K] pre-pack): scales the row by gamma
-// in place (rounded to fp16; g sums the rounded values, which are what the MFMAs see)
-// and emits g[n], b[n] in fp32.
-template <bool GB32>
-__global__ __launch_bounds__(256) void fold_layernorm_kernel(half_t *wt, const void *gamma,
-                                                             const void *beta, const half_t *bias,
-                                                             float *g, float *b, int N, int K) {
-  const int n = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
-  if (n >= N) return;
-  half_t *row = wt + (size_t)n * K;
-  float gs = 0.f, bs = 0.f;
-  for (int c = lane * 8; c < K; c += 64 * 8) {
-    half8_t w = *(const half8_t *)(row + c);
-    half8_t o;
-#pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      const float ga = GB32 ? ((const float *)gamma)[c + e] : (float)((const half_t *)gamma)[c + e];
-      const float be = GB32 ? ((const float *)beta)[c + e] : (float)((const half_t *)beta)[c + e];
-      o[e] = (half_t)((float)w[e] * ga);
-      gs += (float)o[e];
-      bs += be * (float)w[e];
-    }
-    *(half8_t *)(row + c) = o;
-  }
-  gs = wave_sum(gs);
-  bs = wave_sum(bs);
-  if (lane == 0) {
-    g[n] = gs;
-    b[n] = bs + (bias ? (float)bias[n] : 0.f);
-  }
-}
-
 template <int BM, int BN, int STAGES, int WM, int WN, int NP, int SCHED, int EPI>
 static int launch_gemm_tile(GemmArgs p, hipStream_t s) {
-  constexpr size_t smem = (size_t)STAGES * (BM + BN) * kBK * sizeof(half_t) +
-                          (EPI == kEpiLnBiasGelu ? (size_t)BM * sizeof(float2) : 0);
+  constexpr size_t smem = (size_t)STAGES * (BM + BN) * kBK * sizeof(half_t);
   static_assert(smem <= 160 * 1024, "LDS budget");
   static std::atomic<bool> configured[kMaxDevices];
   const int rc = allow_dynamic_lds(gemm_kernel<BM, BN, STAGES, WM, WN, NP, SCHED, EPI>, smem,
@@ -688,78 +542,4 @@ extern "C" int bt_gemm_qkv_bias_split(const void *a, const int *a_row_index, con
   GemmArgs p{(const half_t *)a, (const half_t *)wt_qkv, (const half_t *)bias_qkv,
              (half_t *)qkv_heads, valid_rows, a_row_index, rows_cap, 3 * H, H, 0, rows_hint};
   return launch_gemm<kEpiQkvSplit>(p, as_stream(stream));
-}
-
-extern "C" int bt_gemm_bias_residual_stats(const void *a, const void *wt, const void *bias,
-                                           const void *residual, const int *residual_row_index,
-                                           void *c, void *stats, const int *valid_rows,
-                                           int rows_cap, int rows_hint, int n, int k,
-                                           void *stream) {
-  int rc = check_gemm_args("bt_gemm_bias_residual_stats", a, wt, c, rows_cap, n, k);
-  if (rc) return rc;
-  BT_REQUIRE(bias && residual && stats, BT_ERR_INVALID_ARGUMENT,
-             "bt_gemm_bias_residual_stats: null bias / residual / stats");
-  BT_REQUIRE(n % 64 == 0, BT_ERR_UNSUPPORTED,
-             "bt_gemm_bias_residual_stats: n=%d must be a multiple of 64", n);
-  BT_REQUIRE(!residual_row_index || valid_rows, BT_ERR_INVALID_ARGUMENT,
-             "bt_gemm_bias_residual_stats: residual_row_index needs valid_rows");
-  if (rows_cap == 0) return BT_OK;
-  GemmArgs p{};
-  p.a = (const half_t *)a;
-  p.wt = (const half_t *)wt;
-  p.bias = (const half_t *)bias;
-  p.c = (half_t *)c;
-  p.valid_rows = valid_rows;
-  p.rows_cap = rows_cap;
-  p.N = n;
-  p.K = k;
-  p.rows_hint = rows_hint;
-  p.residual = (const half_t *)residual;
-  p.res_row_index = residual_row_index;
-  p.stats_out = (float2 *)stats;
-  return launch_gemm<kEpiResidualStats>(p, as_stream(stream));
-}
-
-extern "C" int bt_gemm_layernorm_bias_gelu(const void *a, const void *wt_folded,
-                                           const void *stats, const float *fold_g,
-                                           const float *fold_b, float eps, void *c,
-                                           const int *valid_rows, int rows_cap, int rows_hint,
-                                           int n, int k, void *stream) {
-  int rc = check_gemm_args("bt_gemm_layernorm_bias_gelu", a, wt_folded, c, rows_cap, n, k);
-  if (rc) return rc;
-  BT_REQUIRE(stats && fold_g && fold_b, BT_ERR_INVALID_ARGUMENT,
-             "bt_gemm_layernorm_bias_gelu: null stats / fold_g / fold_b");
-  if (rows_cap == 0) return BT_OK;
-  GemmArgs p{};
-  p.a = (const half_t *)a;
-  p.wt = (const half_t *)wt_folded;
-  p.c = (half_t *)c;
-  p.valid_rows = valid_rows;
-  p.rows_cap = rows_cap;
-  p.N = n;
-  p.K = k;
-  p.rows_hint = rows_hint;
-  p.stats_in = (const float2 *)stats;
-  p.fold_g = fold_g;
-  p.fold_b = fold_b;
-  p.eps = eps;
-  return launch_gemm<kEpiLnBiasGelu>(p, as_stream(stream));
-}
-
-extern "C" int bt_fold_layernorm(void *wt, const void *gamma, const void *beta,
-                                 int gamma_beta_fp32, const void *bias, float *fold_g,
-                                 float *fold_b, int n, int k, void *stream) {
-  BT_REQUIRE(wt && gamma && beta && fold_g && fold_b, BT_ERR_INVALID_ARGUMENT,
-             "bt_fold_layernorm: null pointer argument");
-  BT_REQUIRE(n > 0 && k > 0 && k % 8 == 0, BT_ERR_UNSUPPORTED,
-             "bt_fold_layernorm: n=%d k=%d (k must be a positive multiple of 8)", n, k);
-  const int grid = (n + 3) / 4;
-  if (gamma_beta_fp32)
-    fold_layernorm_kernel<true><<<grid, 256, 0, as_stream(stream)>>>(
-        (half_t *)wt, gamma, beta, (const half_t *)bias, fold_g, fold_b, n, k);
-  else
-    fold_layernorm_kernel<false><<<grid, 256, 0, as_stream(stream)>>>(
-        (half_t *)wt, gamma, beta, (const half_t *)bias, fold_g, fold_b, n, k);
-  BT_CHECK_LAUNCH("fold_layernorm_kernel");
-  return BT_OK;
 }

@@ -12,46 +12,13 @@ namespace bt {
 
 constexpr int kLnRowsPerBlock = 4;
 
-// The residual may itself be a LayerNorm that was never materialised: `residual`
-// then holds its input x, and (res_stats, res_gamma, res_beta) its per-row slot sums
-// (sum x, sum x^2 per 64 columns) and affine parameters; the row is normalised on the
-// fly, rounded to fp16, and used as the residual.
-struct LnResidualNorm {
-  const float2 *stats;   // [rows][chunks / 8] or null
-  const void *gamma, *beta;
-};
-
-template <bool GB32>
-__device__ __forceinline__ void load_gb8(const void *gamma, const void *beta, int c, float (&g)[8],
-                                         float (&b)[8]) {
-  if (GB32) {
-    const float4_t *gp = (const float4_t *)gamma + 2 * c;
-    const float4_t *bp = (const float4_t *)beta + 2 * c;
-    float4_t g0 = gp[0], g1 = gp[1], b0 = bp[0], b1 = bp[1];
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      g[j] = g0[j];
-      g[4 + j] = g1[j];
-      b[j] = b0[j];
-      b[4 + j] = b1[j];
-    }
-  } else {
-    half8_t gh = ((const half8_t *)gamma)[c], bh = ((const half8_t *)beta)[c];
-#pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      g[j] = (float)gh[j];
-      b[j] = (float)bh[j];
-    }
-  }
-}
-
-template <int NC, bool RESTORE, bool GB32, bool RESNORM>
+template <int NC, bool RESTORE, bool GB32>
 __global__ __launch_bounds__(kLnRowsPerBlock *kWave) void layernorm_kernel(
     const half8_t *src, const half8_t *__restrict__ residual,
     const half8_t *__restrict__ bias, const void *__restrict__ gamma,
     const void *__restrict__ beta, half8_t *dst, const int *__restrict__ idx,
     const int *__restrict__ residual_row_index, int B, int S, int rows_cap, int chunks,
-    float inv_n, float eps, LnResidualNorm rn) {
+    float inv_n, float eps) {
   const int r = blockIdx.x * kLnRowsPerBlock + (threadIdx.x >> 6);
   const int lane = threadIdx.x & 63;
   if (r >= rows_cap) return;
@@ -77,33 +44,13 @@ __global__ __launch_bounds__(kLnRowsPerBlock *kWave) void layernorm_kernel(
   const half8_t *a = src + src_row * chunks;
   const size_t res_row = residual_row_index ? (size_t)residual_row_index[src_row] : src_row;
   const half8_t *b = residual + res_row * chunks;
-  float r_mean = 0.f, r_rstd = 1.f;
-  if (RESNORM) {
-    const int slots = chunks >> 3;
-    float s1 = 0.f, s2 = 0.f;
-    for (int sl = 0; sl < slots; ++sl) {
-      const float2 t = rn.stats[res_row * slots + sl];
-      s1 += t.x;
-      s2 += t.y;
-    }
-    r_mean = s1 * inv_n;
-    r_rstd = rsqrtf(fmaxf(s2 * inv_n - r_mean * r_mean, 0.f) + eps);
-  }
   float v[NC][8];
   float sum = 0.f;
 #pragma unroll
   for (int i = 0; i < NC; ++i) {
     const int c = lane + i * kWave;
     if (c < chunks) {
-      half8_t res = b[c];
-      if (RESNORM) {
-        float g[8], bt_[8];
-        load_gb8<GB32>(rn.gamma, rn.beta, c, g, bt_);
-#pragma unroll
-        for (int j = 0; j < 8; ++j)
-          res[j] = (half_t)(((float)res[j] - r_mean) * r_rstd * g[j] + bt_[j]);
-      }
-      half8_t x = (a[c] + res) + bias[c];  // two fp16-rounded adds
+      half8_t x = (a[c] + b[c]) + bias[c];  // two fp16-rounded adds
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
         v[i][j] = (float)x[j];
@@ -135,7 +82,25 @@ __global__ __launch_bounds__(kLnRowsPerBlock *kWave) void layernorm_kernel(
     const int c = lane + i * kWave;
     if (c < chunks) {
       float g[8], bt_[8];
-      load_gb8<GB32>(gamma, beta, c, g, bt_);
+      if (GB32) {
+        const float4_t *gp = (const float4_t *)gamma + 2 * c;
+        const float4_t *bp = (const float4_t *)beta + 2 * c;
+        float4_t g0 = gp[0], g1 = gp[1], b0 = bp[0], b1 = bp[1];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          g[j] = g0[j];
+          g[4 + j] = g1[j];
+          bt_[j] = b0[j];
+          bt_[4 + j] = b1[j];
+        }
+      } else {
+        half8_t gh = ((const half8_t *)gamma)[c], bh = ((const half8_t *)beta)[c];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          g[j] = (float)gh[j];
+          bt_[j] = (float)bh[j];
+        }
+      }
       half8_t y;
 #pragma unroll
       for (int j = 0; j < 8; ++j) y[j] = (half_t)(v[i][j] * rstd * g[j] + bt_[j]);
@@ -148,35 +113,25 @@ template <bool RESTORE>
 static int launch_ln(const void *src, const void *residual, const void *bias, const void *gamma,
                      const void *beta, int gb32, void *dst, const int *idx,
                      const int *residual_row_index, int B, int S, int rows_cap, int H, float eps,
-                     hipStream_t s, const char *who, LnResidualNorm rn = {nullptr, nullptr, nullptr}) {
+                     hipStream_t s, const char *who) {
   BT_REQUIRE(H > 0 && H % 8 == 0, BT_ERR_UNSUPPORTED, "%s: hidden_dim %d must be a multiple of 8",
              who, H);
   const int chunks = H / 8;
   const int nc = (chunks + kWave - 1) / kWave;
   BT_REQUIRE(nc <= 8, BT_ERR_UNSUPPORTED, "%s: hidden_dim %d exceeds 4096", who, H);
-  if (rn.stats) {
-    BT_REQUIRE(H % 64 == 0, BT_ERR_UNSUPPORTED,
-               "%s: hidden_dim %d must be a multiple of 64 with residual statistics", who, H);
-    BT_REQUIRE(rn.gamma && rn.beta, BT_ERR_INVALID_ARGUMENT,
-               "%s: residual statistics need the residual's gamma and beta", who);
-  }
   if (rows_cap == 0) return BT_OK;
   const int grid = (rows_cap + kLnRowsPerBlock - 1) / kLnRowsPerBlock;
   const float inv_n = 1.0f / (float)H;
-#define BT_LN_LAUNCH(NC_, GB_, RN_)                                                             \
-  layernorm_kernel<NC_, RESTORE, GB_, RN_><<<grid, kLnRowsPerBlock * kWave, 0, s>>>(            \
+#define BT_LN_LAUNCH(NC_, GB_)                                                                  \
+  layernorm_kernel<NC_, RESTORE, GB_><<<grid, kLnRowsPerBlock * kWave, 0, s>>>(                 \
       (const half8_t *)src, (const half8_t *)residual, (const half8_t *)bias, gamma, beta,      \
-      (half8_t *)dst, idx, residual_row_index, B, S, rows_cap, chunks, inv_n, eps, rn)
-#define BT_LN_NC(NC_)                      \
-  do {                                     \
-    if (gb32 && rn.stats)                  \
-      BT_LN_LAUNCH(NC_, true, true);       \
-    else if (gb32)                         \
-      BT_LN_LAUNCH(NC_, true, false);      \
-    else if (rn.stats)                     \
-      BT_LN_LAUNCH(NC_, false, true);      \
-    else                                   \
-      BT_LN_LAUNCH(NC_, false, false);     \
+      (half8_t *)dst, idx, residual_row_index, B, S, rows_cap, chunks, inv_n, eps)
+#define BT_LN_NC(NC_)              \
+  do {                             \
+    if (gb32)                      \
+      BT_LN_LAUNCH(NC_, true);     \
+    else                           \
+      BT_LN_LAUNCH(NC_, false);    \
   } while (0)
   if (nc <= 1)
     BT_LN_NC(1);
@@ -227,44 +182,4 @@ extern "C" int bt_add_bias_residual_layernorm_restore(
   return launch_ln<true>(out, residual, bias, gamma, beta, gamma_beta_fp32, out_padded, batch_idx,
                          nullptr, batch_size, seq_len, batch_size * seq_len, hidden_dim, eps,
                          as_stream(stream), "bt_add_bias_residual_layernorm_restore");
-}
-
-extern "C" int bt_add_bias_lnresidual_layernorm(void *out, const void *residual_x,
-                                                const void *residual_stats,
-                                                const void *residual_gamma,
-                                                const void *residual_beta, const void *bias,
-                                                const void *gamma, const void *beta,
-                                                int gamma_beta_fp32, const int *valid_rows,
-                                                int rows_cap, int hidden_dim, float eps,
-                                                void *stream) {
-  BT_REQUIRE(out && residual_x && residual_stats && bias && gamma && beta,
-             BT_ERR_INVALID_ARGUMENT, "bt_add_bias_lnresidual_layernorm: null pointer argument");
-  BT_REQUIRE(rows_cap >= 0, BT_ERR_INVALID_ARGUMENT,
-             "bt_add_bias_lnresidual_layernorm: negative rows_cap");
-  return launch_ln<false>(out, residual_x, bias, gamma, beta, gamma_beta_fp32, out, valid_rows,
-                          nullptr, 0, 1, rows_cap, hidden_dim, eps, as_stream(stream),
-                          "bt_add_bias_lnresidual_layernorm",
-                          LnResidualNorm{(const float2 *)residual_stats, residual_gamma,
-                                         residual_beta});
-}
-
-extern "C" int bt_add_bias_lnresidual_layernorm_restore(
-    const void *out, const void *residual_x, const void *residual_stats,
-    const void *residual_gamma, const void *residual_beta, const void *bias, const void *gamma,
-    const void *beta, int gamma_beta_fp32, void *out_padded, const int *batch_idx,
-    int batch_size, int seq_len, int hidden_dim, float eps, void *stream) {
-  BT_REQUIRE(out && residual_x && residual_stats && bias && gamma && beta && out_padded &&
-                 batch_idx,
-             BT_ERR_INVALID_ARGUMENT,
-             "bt_add_bias_lnresidual_layernorm_restore: null pointer argument");
-  BT_REQUIRE(batch_size > 0 && seq_len > 0, BT_ERR_INVALID_ARGUMENT,
-             "bt_add_bias_lnresidual_layernorm_restore: sizes must be positive");
-  BT_REQUIRE((long long)batch_size * seq_len < (1ll << 31), BT_ERR_UNSUPPORTED,
-             "bt_add_bias_lnresidual_layernorm_restore: too many rows");
-  return launch_ln<true>(out, residual_x, bias, gamma, beta, gamma_beta_fp32, out_padded,
-                         batch_idx, nullptr, batch_size, seq_len, batch_size * seq_len,
-                         hidden_dim, eps, as_stream(stream),
-                         "bt_add_bias_lnresidual_layernorm_restore",
-                         LnResidualNorm{(const float2 *)residual_stats, residual_gamma,
-                                        residual_beta});
 }

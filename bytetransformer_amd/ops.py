@@ -125,68 +125,6 @@ def gemm_qkv_bias_split(a, wt_qkv, bias_qkv, head_num, size_per_head=64, valid_r
     return out
 
 
-def gemm_bias_residual_stats(a, wt, bias, residual, valid_rows=None, residual_row_index=None,
-                             out=None, stats=None, rows_hint=0):
-    """-> (x = fp16(fp16(a.wt^T + residual) + bias), stats float32 [rows, n/64, 2])."""
-    rows, k = a.shape
-    n = wt.shape[0]
-    if out is None:
-        out = torch.zeros(rows, n, dtype=a.dtype, device=a.device)
-    if stats is None:
-        stats = torch.zeros(rows, n // 64, 2, dtype=torch.float32, device=a.device)
-    _check(kernel_lib().bt_gemm_bias_residual_stats(
-        _ptr(a), _ptr(wt), _ptr(bias), _ptr(residual), _ptr(residual_row_index), _ptr(out),
-        _ptr(stats), _ptr(valid_rows), rows, int(rows_hint), n, k, _stream()))
-    return out, stats
-
-
-def fold_layernorm(wt, gamma, beta, bias):
-    """Scales the pre-packed wt [n, k] by gamma[k] in place -> (fold_g, fold_b) float32 [n]."""
-    n, k = wt.shape
-    g = torch.empty(n, dtype=torch.float32, device=wt.device)
-    b = torch.empty(n, dtype=torch.float32, device=wt.device)
-    _check(kernel_lib().bt_fold_layernorm(_ptr(wt), _ptr(gamma), _ptr(beta),
-                                          int(gamma.dtype == torch.float32), _ptr(bias), _ptr(g),
-                                          _ptr(b), n, k, _stream()))
-    return g, b
-
-
-def gemm_layernorm_bias_gelu(a, wt_folded, stats, fold_g, fold_b, eps=1e-6, valid_rows=None,
-                             out=None, rows_hint=0):
-    rows, k = a.shape
-    n = wt_folded.shape[0]
-    if out is None:
-        out = torch.zeros(rows, n, dtype=a.dtype, device=a.device)
-    _check(kernel_lib().bt_gemm_layernorm_bias_gelu(
-        _ptr(a), _ptr(wt_folded), _ptr(stats), _ptr(fold_g), _ptr(fold_b), float(eps), _ptr(out),
-        _ptr(valid_rows), rows, int(rows_hint), n, k, _stream()))
-    return out
-
-
-def add_bias_lnresidual_layernorm(out, residual_x, residual_stats, residual_gamma, residual_beta,
-                                  bias, gamma, beta, eps=1e-6, valid_rows=None):
-    rows, H = out.shape
-    _check(kernel_lib().bt_add_bias_lnresidual_layernorm(
-        _ptr(out), _ptr(residual_x), _ptr(residual_stats), _ptr(residual_gamma),
-        _ptr(residual_beta), _ptr(bias), _ptr(gamma), _ptr(beta),
-        int(gamma.dtype == torch.float32), _ptr(valid_rows), rows, H, float(eps), _stream()))
-    return out
-
-
-def add_bias_lnresidual_layernorm_restore(out, residual_x, residual_stats, residual_gamma,
-                                          residual_beta, bias, gamma, beta, batch_idx,
-                                          batch_size, seq_len, eps=1e-6, out_padded=None):
-    H = out.shape[-1]
-    if out_padded is None:
-        out_padded = torch.empty(batch_size, seq_len, H, dtype=out.dtype, device=out.device)
-    _check(kernel_lib().bt_add_bias_lnresidual_layernorm_restore(
-        _ptr(out), _ptr(residual_x), _ptr(residual_stats), _ptr(residual_gamma),
-        _ptr(residual_beta), _ptr(bias), _ptr(gamma), _ptr(beta),
-        int(gamma.dtype == torch.float32), _ptr(out_padded), _ptr(batch_idx), batch_size,
-        seq_len, H, float(eps), _stream()))
-    return out_padded
-
-
 def _attention(fn, qkv_heads, batch_idx, batch_size, seq_len, scale, padded_rows, out,
                seq_order=None, mask=None, bias=None, prefetch=None):
     _, head_num, rows_cap, d = qkv_heads.shape

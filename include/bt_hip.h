@@ -129,54 +129,6 @@ int bt_gemm_qkv_bias_split(const void *a, const int *a_row_index, const void *wt
                            void *stream);
 
 /*
- * A LayerNorm folded into the two GEMMs around it (no counterpart in the reference,
- * which runs add_bias_input_layernorm, layernorm.h:273-296, as a kernel of its own
- * between them).  For y = LN(x) . W + bias with LN(x) = (x - mean) rstd gamma + beta:
- *   y = rstd (x . W' - mean g) + b,  W' = diag(gamma) W,  g[n] = sum_k W'[k][n],
- *   b[n] = sum_k beta[k] W[k][n] + bias[n].
- *
- * bt_gemm_bias_residual_stats  the producer: c = fp16(fp16(a.wt^T + residual) + bias), the
- *     two fp16-rounded adds of the LayerNorm kernel, plus per row the sums (sum x, sum x^2)
- *     of the rounded values in stats float2[rows_cap][n / 64]: a workgroup adds up its
- *     columns into one 64-column slot and zeroes the other slots it covers, so the sum over
- *     a row's slots is the row total (what consumers use).  residual_row_index (nullable,
- *     needs valid_rows): row r adds residual[residual_row_index[r]].  n % 64 == 0.
- * bt_fold_layernorm  once per weight set: scales the pre-packed wt[n][k] by gamma[k] in
- *     place and writes fold_g[n], fold_b[n] (fp32).
- * bt_gemm_layernorm_bias_gelu  the consumer: c = gelu(LN(a) . W + bias) from the raw a, the
- *     folded weights and the producer's stats (k / 64 slots per row).
- * bt_add_bias_lnresidual_layernorm[_restore]  the LayerNorm that follows, whose residual is
- *     that never-materialised LN(x): it is recomputed per element from residual_x, the
- *     stats and (residual_gamma, residual_beta), rounded to fp16, then used exactly as in
- *     bt_add_bias_residual_layernorm[_restore].  gamma_beta_fp32 applies to both pairs.
- */
-int bt_gemm_bias_residual_stats(const void *a, const void *wt, const void *bias,
-                                const void *residual, const int *residual_row_index, void *c,
-                                void *stats, const int *valid_rows, int rows_cap, int rows_hint,
-                                int n, int k, void *stream);
-int bt_fold_layernorm(void *wt, const void *gamma, const void *beta, int gamma_beta_fp32,
-                      const void *bias, float *fold_g, float *fold_b, int n, int k,
-                      void *stream);
-int bt_gemm_layernorm_bias_gelu(const void *a, const void *wt_folded, const void *stats,
-                                const float *fold_g, const float *fold_b, float eps, void *c,
-                                const int *valid_rows, int rows_cap, int rows_hint, int n, int k,
-                                void *stream);
-int bt_add_bias_lnresidual_layernorm(void *out, const void *residual_x,
-                                     const void *residual_stats, const void *residual_gamma,
-                                     const void *residual_beta, const void *bias,
-                                     const void *gamma, const void *beta, int gamma_beta_fp32,
-                                     const int *valid_rows, int rows_cap, int hidden_dim,
-                                     float eps, void *stream);
-int bt_add_bias_lnresidual_layernorm_restore(const void *out, const void *residual_x,
-                                             const void *residual_stats,
-                                             const void *residual_gamma,
-                                             const void *residual_beta, const void *bias,
-                                             const void *gamma, const void *beta,
-                                             int gamma_beta_fp32, void *out_padded,
-                                             const int *batch_idx, int batch_size, int seq_len,
-                                             int hidden_dim, float eps, void *stream);
-
-/*
  * Fused multi-head attention over the head-major Q/K/V written by
  * bt_gemm_qkv_bias_split; output is token-major [rows, H] with head g at
  * columns [g*d, g*d+d).  Per sequence b and head g:

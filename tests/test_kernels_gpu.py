@@ -259,136 +259,6 @@ def test_gather_fused_into_qkv_gemm_and_layernorm(device):
     assert torch.equal(a, b)
 
 
-# ---- LayerNorm folded into the GEMMs around it --------------------------------------
-@pytest.mark.parametrize("tile", [-1, 0, 1, 2, 3, 4])
-@pytest.mark.parametrize("gather", [False, True])
-def test_gemm_bias_residual_stats(device, tile, gather):
-    """x = fp16(fp16(a.w + residual) + bias) and the per-row sums of x, x^2 over the slots."""
-    _say("gemm residual stats", tile, gather)
-    rs = np.random.RandomState(31 + tile)
-    rows, M, N, K = 600, 531, 768, 768
-    a = rs.standard_normal((rows, K)).astype(np.float16)
-    w = (rs.standard_normal((K, N)) * 0.05).astype(np.float16)
-    bias = (rs.standard_normal(N) * 0.3).astype(np.float16)
-    res = rs.standard_normal((rows, N)).astype(np.float16)
-    idx = rs.permutation(rows)[:M].astype(np.int32) if gather else None
-    rrows = res[idx] if gather else res[:M]
-    c16 = O.gemm(a[:M], w).astype(np.float16)
-    exp = ((c16 + rrows).astype(np.float16) + bias).astype(np.float16)
-    ops.set_option("gemm_tile", tile)
-    try:
-        vr = torch.tensor([M], dtype=torch.int32, device=device)
-        pad_idx = None
-        if gather:
-            pad_idx = torch.full((rows,), -12345, dtype=torch.int32, device=device)   # dead rows are never indexed
-            pad_idx[:M] = _dev(idx, device)
-        x, stats = ops.gemm_bias_residual_stats(_dev(a, device), ops.transpose_weight(_dev(w, device)),
-                                                _dev(bias, device), _dev(res, device), valid_rows=vr,
-                                                residual_row_index=pad_idx)
-    finally:
-        ops.set_option("gemm_tile", -1)
-    x = x.cpu().numpy()
-    stats = stats.cpu().numpy().astype(np.float64)
-    # an fp16 GEMM result one ulp off moves x by one ulp: compare loosely, then check the
-    # sums against the x the kernel itself wrote (that is what the consumers pair them with)
-    err = np.abs(x[:M].astype(np.float64) - exp.astype(np.float64))
-    assert np.all(err <= 2.0 ** -9 * np.abs(exp.astype(np.float64)) + 2e-3), err.max()
-    xs = x[:M].astype(np.float64)
-    assert np.allclose(stats[:M, :, 0].sum(1), xs.sum(1), rtol=0, atol=2e-3)
-    assert np.allclose(stats[:M, :, 1].sum(1), (xs * xs).sum(1), rtol=2e-6, atol=2e-3)
-    assert np.all(x[M:] == 0)
-
-
-@pytest.mark.parametrize("gb32", [False, True])
-def test_fold_layernorm(device, gb32):
-    _say("fold layernorm", gb32)
-    rs = np.random.RandomState(5)
-    K, N = 768, 3072
-    w = (rs.standard_normal((K, N)) * 0.05).astype(np.float16)
-    gdt = np.float32 if gb32 else np.float16
-    gamma = (1 + 0.3 * rs.standard_normal(K)).astype(gdt)
-    beta = (0.2 * rs.standard_normal(K)).astype(gdt)
-    bias = (0.5 * rs.standard_normal(N)).astype(np.float16)
-    wt = ops.transpose_weight(_dev(w, device))
-    g, b = ops.fold_layernorm(wt, _dev(gamma, device), _dev(beta, device), _dev(bias, device))
-    wf = (w.astype(np.float32) * gamma.astype(np.float32)[:, None]).astype(np.float16)
-    assert np.array_equal(wt.cpu().numpy(), wf.T)
-    # 768 terms of |w'| <= 0.3 summed in fp32, in another order than NumPy's
-    assert np.allclose(g.cpu().numpy(), wf.astype(np.float64).sum(0), rtol=0, atol=3e-4)
-    bexp = (beta.astype(np.float64)[:, None] * w.astype(np.float64)).sum(0) + bias.astype(np.float64)
-    assert np.allclose(b.cpu().numpy(), bexp, rtol=0, atol=1e-4)
-
-
-@pytest.mark.parametrize("tile", [-1, 0, 1, 2, 3, 4])
-def test_gemm_layernorm_bias_gelu_matches_unfolded(device, tile):
-    """gelu(LN(x).W + bias) from raw x, folded weights and the producer's statistics."""
-    _say("gemm layernorm gelu", tile)
-    rs = np.random.RandomState(17 + tile)
-    rows, M, K, N = 700, 650, 768, 3072
-    x = (1.5 * rs.standard_normal((rows, K)) + 0.3).astype(np.float16)
-    w = (rs.standard_normal((K, N)) * 0.05).astype(np.float16)
-    gamma = (1 + 0.3 * rs.standard_normal(K)).astype(np.float16)
-    beta = (0.2 * rs.standard_normal(K)).astype(np.float16)
-    bias = (0.5 * rs.standard_normal(N)).astype(np.float16)
-    exp = O.gemm(O.layer_norm(x[:M], gamma, beta, 1e-6), w, bias, "gelu_tanh")
-    xs = x.astype(np.float64)
-    stats = np.zeros((rows, K // 64, 2), np.float32)
-    stats[:, :, 0] = xs.reshape(rows, K // 64, 64).sum(2)
-    stats[:, :, 1] = (xs * xs).reshape(rows, K // 64, 64).sum(2)
-    wt = ops.transpose_weight(_dev(w, device))
-    g, b = ops.fold_layernorm(wt, _dev(gamma, device), _dev(beta, device), _dev(bias, device))
-    ops.set_option("gemm_tile", tile)
-    try:
-        vr = torch.tensor([M], dtype=torch.int32, device=device)
-        got = ops.gemm_layernorm_bias_gelu(_dev(x, device), wt, _dev(stats, device), g, b,
-                                           valid_rows=vr).cpu().numpy()
-    finally:
-        ops.set_option("gemm_tile", -1)
-    err = np.abs(got[:M].astype(np.float64) - exp)
-    # the weights carry one more fp16 rounding (gamma folded in): ~2^-11 |w| per term
-    assert err.max() <= 6e-3 and err.mean() <= 4e-4, (err.max(), err.mean())
-    assert np.all(got[M:] == 0)
-
-
-@pytest.mark.parametrize("restore", [False, True])
-def test_layernorm_with_unmaterialised_residual(device, restore):
-    """residual = LN(x) recomputed from x and its slot sums, then the usual add + LN."""
-    _say("layernorm lnresidual", restore)
-    rs = np.random.RandomState(23)
-    lens = [40, 0, 17, 64] if restore else [121]
-    S, H = 64, 768
-    M = sum(lens)
-    out = rs.standard_normal((M, H)).astype(np.float16)
-    x = (1.3 * rs.standard_normal((M, H)) - 0.2).astype(np.float16)
-    g1 = (1 + 0.2 * rs.standard_normal(H)).astype(np.float16)
-    b1 = (0.1 * rs.standard_normal(H)).astype(np.float16)
-    g2 = (1 + 0.2 * rs.standard_normal(H)).astype(np.float16)
-    b2 = (0.1 * rs.standard_normal(H)).astype(np.float16)
-    bias = (0.3 * rs.standard_normal(H)).astype(np.float16)
-    xs = x.astype(np.float64)
-    stats = np.zeros((M, H // 64, 2), np.float32)
-    stats[:, :, 0] = xs.reshape(M, H // 64, 64).sum(2)
-    stats[:, :, 1] = (xs * xs).reshape(M, H // 64, 64).sum(2)
-    y1 = O.layer_norm(x, g1, b1, 1e-6).astype(np.float16)
-    exp = O.add_bias_residual_layernorm(out, y1, bias, g2, b2)
-    args = (_dev(x, device), _dev(stats, device), _dev(g1, device), _dev(b1, device),
-            _dev(bias, device), _dev(g2, device), _dev(b2, device))
-    if restore:
-        bi = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
-        got = ops.add_bias_lnresidual_layernorm_restore(_dev(out, device), *args, _dev(bi, device),
-                                                        len(lens), S).cpu().numpy()
-        for b, n in enumerate(lens):
-            t0 = int(bi[b])
-            err = np.abs(got[b, :n].astype(np.float64) - exp[t0:t0 + n])
-            assert n == 0 or err.max() <= 8e-3, err.max()
-            assert np.all(got[b, n:] == 0)
-    else:
-        got = ops.add_bias_lnresidual_layernorm(_dev(out, device), *args).cpu().numpy()
-        err = np.abs(got.astype(np.float64) - exp)
-        # y1 may round differently by one fp16 ulp (fp32 statistics from sums of squares)
-        assert err.max() <= 8e-3 and err.mean() <= 3e-4, (err.max(), err.mean())
-
-
 # ---- attention -----------------------------------------------------------------
 def _attention_case(rs, lens, S, heads, scale_q=1.0):
     B = len(lens)
