@@ -22,7 +22,7 @@ INC = os.path.join(ROOT, "include")
 ROCM = os.environ.get("ROCM_PATH", "/opt/rocm")
 HIPCC = os.path.join(ROCM, "bin", "hipcc")
 
-KERNEL_SOURCES = ["padding.hip", "layernorm.hip", "gemm.hip", "attention.hip"]
+KERNEL_SOURCES = ["padding.hip", "layernorm.hip", "gemm.hip", "attention.hip", "fp32_path.hip"]
 HOST_SOURCES = ["attention.cc", "bert_transformer.cc", "bert_encoder.cc", "c_api.cc"]
 TH_OP_SOURCES = ["ths_op_f.cc", "ths_op.cc"]
 

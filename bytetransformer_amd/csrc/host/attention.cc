@@ -10,8 +10,6 @@ namespace bytetransformer {
 
 template <OperationType OpType>
 void Attention<OpType>::infer(AttentionInferParam infer_param) {
-  if (OpType != OperationType::HALF)
-    throw std::runtime_error("[BT][ERROR] Attention: only OperationType::HALF is implemented");
   if (infer_param.et_param.batch_idx == nullptr)
     throw std::runtime_error("[BT][ERROR] Attention: et_param.batch_idx must be set");
   if (infer_param.batch_size > max_batch_size_ || infer_param.seq_len > max_seq_len_)
@@ -20,6 +18,17 @@ void Attention<OpType>::infer(AttentionInferParam infer_param) {
   const int rows_cap = infer_param.batch_size * infer_param.seq_len;
   const float scale = 1.0f / std::sqrt((float)size_per_head_) / param_.tao;
   const int padded_rows = is_remove_padding_ ? 0 : 1;
+  if constexpr (OpType == OperationType::FP32) {
+    // float: one streaming kernel over token-major [rows, 3H] projections; the mask tensor
+    // is applied on both row layouts, as the reference's float path does
+    // (attention_nofused.cu:85-94)
+    check_bt_error(bt_attention_f32(infer_param.qkv, infer_param.attention_output,
+                                    infer_param.et_param.batch_idx, infer_param.atten_mask,
+                                    infer_param.attention_bias, infer_param.batch_size,
+                                    infer_param.seq_len, rows_cap, head_num_, size_per_head_,
+                                    scale, padded_rows, infer_param.stream));
+    return;
+  }
   // on padded rows the mask tensor itself is applied (any 0/1 pattern), as in the
   // reference's non-remove-padding kernels; packed rows use the prefix lengths
   const void *mask = is_remove_padding_ ? nullptr : (const void *)infer_param.atten_mask;

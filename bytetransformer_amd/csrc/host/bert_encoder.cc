@@ -8,8 +8,7 @@ namespace bytetransformer {
 
 template <OperationType OpType>
 void BertEncoder<OpType>::prepack(void *prepacked, hipStream_t stream) const {
-  if (OpType != OperationType::HALF)
-    throw std::runtime_error("[BT][ERROR] BertEncoder: only OperationType::HALF is implemented");
+  if (OpType == OperationType::FP32) return;   // float weights are consumed as stored
   if (!prepacked) throw std::runtime_error("[BT][ERROR] BertEncoder::prepack: null destination");
   const int hidden = head_num_ * size_per_head_, inter = hidden * intermediate_size_;
   DataType_ *dst = (DataType_ *)prepacked;
@@ -27,8 +26,6 @@ void BertEncoder<OpType>::prepack(void *prepacked, hipStream_t stream) const {
 
 template <OperationType OpType>
 void BertEncoder<OpType>::infer(BertEncoderInferParam<DataType_> ip) {
-  if (OpType != OperationType::HALF)
-    throw std::runtime_error("[BT][ERROR] BertEncoder: only OperationType::HALF is implemented");
   if (layers_.empty()) throw std::runtime_error("[BT][ERROR] BertEncoder: initialize() first");
   if (!ip.input_tensor || !ip.atten_mask || !ip.transformer_output || !ip.buf)
     throw std::runtime_error("[BT][ERROR] BertEncoder: null input/mask/output/buf pointer");
@@ -73,6 +70,41 @@ void BertEncoder<OpType>::infer(BertEncoderInferParam<DataType_> ip) {
     const DataType_ *x = l == 0 ? ip.input_tensor : hidden_buf;
     const int *gather = (l == 0 && is_remove_padding_) ? et_param.word_idx : nullptr;
 
+    const bool last = l == L - 1;
+    // the last layer of the padded path writes straight into the caller's output
+    DataType_ *ffn2_out = (last && !is_remove_padding_) ? ip.transformer_output : hidden_buf;
+    attention_layer_->initialize(w.attention_param);
+
+    if constexpr (OpType == OperationType::FP32) {
+      check_bt_error(bt_gemm_f32(x, gather, w.attr_kernel_QKV, w.attention_param.attr_bias_QKV,
+                                 qkv_buf, 0, valid_rows, rows, 3 * hidden, hidden, stream));
+      struct AttentionInferParam<DataType_> att {
+        qkv_buf, ip.atten_mask, attr_out_buf, nullptr, batch_size, seq_len, nullptr, stream,
+            et_param
+      };
+      att.attention_bias = ip.attention_bias;
+      attention_layer_->infer(att);
+      check_bt_error(bt_gemm_f32(attr_out_buf, nullptr, w.attr_output_kernel, nullptr,
+                                 attr_matmul_buf, 0, valid_rows, rows, hidden, hidden, stream));
+      check_bt_error(bt_add_bias_residual_layernorm_f32(
+          attr_matmul_buf, x, gather, w.attr_output_bias, w.attr_output_layernorm_gamma,
+          w.attr_output_layernorm_beta, valid_rows, rows, hidden, layernorm_eps, stream));
+      check_bt_error(bt_gemm_f32(attr_matmul_buf, nullptr, w.inter_kernel, w.inter_bias,
+                                 inter_matmul_buf, 1, valid_rows, rows, inter, hidden, stream));
+      check_bt_error(bt_gemm_f32(inter_matmul_buf, nullptr, w.output_kernel, nullptr, ffn2_out, 0,
+                                 valid_rows, rows, hidden, inter, stream));
+      if (last && is_remove_padding_)
+        check_bt_error(bt_add_bias_residual_layernorm_restore_f32(
+            ffn2_out, attr_matmul_buf, w.output_bias, w.output_layernorm_gamma,
+            w.output_layernorm_beta, ip.transformer_output, et_param.batch_idx, batch_size,
+            seq_len, hidden, layernorm_eps, stream));
+      else
+        check_bt_error(bt_add_bias_residual_layernorm_f32(
+            ffn2_out, attr_matmul_buf, nullptr, w.output_bias, w.output_layernorm_gamma,
+            w.output_layernorm_beta, valid_rows, rows, hidden, layernorm_eps, stream));
+      continue;
+    }
+
     const DataType_ *wt_qkv;
     if (ip.prepacked) {
       wt_qkv = (const DataType_ *)ip.prepacked + (size_t)l * layer_weight_elems();
@@ -94,7 +126,6 @@ void BertEncoder<OpType>::infer(BertEncoderInferParam<DataType_> ip) {
                                           qkv_buf, valid_rows, rows, rows_hint, head_num_,
                                           size_per_head_, stream));
 
-    attention_layer_->initialize(w.attention_param);
     struct AttentionInferParam<DataType_> att {
       qkv_buf, ip.atten_mask, attr_out_buf, nullptr, batch_size, seq_len, nullptr, stream, et_param
     };
@@ -117,9 +148,6 @@ void BertEncoder<OpType>::infer(BertEncoderInferParam<DataType_> ip) {
     check_bt_error(bt_gemm_bias_gelu(attr_matmul_buf, wt_inter, w.inter_bias, inter_matmul_buf,
                                      valid_rows, rows, rows_hint, inter, hidden, stream));
 
-    const bool last = l == L - 1;
-    // the last layer of the padded path writes straight into the caller's output
-    DataType_ *ffn2_out = (last && !is_remove_padding_) ? ip.transformer_output : hidden_buf;
     check_bt_error(bt_gemm(inter_matmul_buf, wt_out, ffn2_out, valid_rows, rows, rows_hint, hidden,
                            inter, stream));
     if (last && is_remove_padding_)

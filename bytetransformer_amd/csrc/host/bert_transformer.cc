@@ -9,9 +9,6 @@ namespace bytetransformer {
 
 template <OperationType OpType>
 void BertTransformer<OpType>::bert_infer(BertTransformerInferParam infer_param) {
-  if (OpType != OperationType::HALF)
-    throw std::runtime_error(
-        "[BT][ERROR] BertTransformer: only OperationType::HALF is implemented");
   if (inner_buf_size_ == 0) cal_bufsize();
 
   const DataType_ *from_tensor = infer_param.input_tensor;
@@ -77,6 +74,41 @@ void BertTransformer<OpType>::bert_infer(BertTransformerInferParam infer_param) 
     restore_target = transformer_out;
     transformer_out = inner_buf;  // FFN2 output reuses the dead qkv region
     valid_rows = et_param.batch_idx + batch_size;
+  }
+
+  if constexpr (OpType == OperationType::FP32) {
+    // float: weights are consumed as stored, Q/K/V stay token-major [rows, 3H], gamma
+    // and beta are float by definition
+    check_bt_error(bt_gemm_f32(from_tensor, gather, param_.attr_kernel_QKV,
+                               param_.attention_param.attr_bias_QKV, qkv_buf, 0, valid_rows, rows,
+                               3 * hidden, hidden, stream));
+    struct AttentionInferParam<DataType_> attention_infer_param {
+      qkv_buf, atten_mask, attr_out_buf, base + inner_buf_size_, batch_size, seq_len,
+          infer_param.cublas_handle, stream, et_param
+    };
+    attention_infer_param.attention_bias = infer_param.attention_bias;
+    attention_layer_->infer(attention_infer_param);
+    check_bt_error(bt_gemm_f32(attr_out_buf, nullptr, param_.attr_output_kernel, nullptr,
+                               attr_matmul_buf, 0, valid_rows, rows, hidden, hidden, stream));
+    check_bt_error(bt_add_bias_residual_layernorm_f32(
+        attr_matmul_buf, from_tensor, gather, param_.attr_output_bias,
+        param_.attr_output_layernorm_gamma, param_.attr_output_layernorm_beta, valid_rows, rows,
+        hidden, layernorm_eps, stream));
+    check_bt_error(bt_gemm_f32(attr_matmul_buf, nullptr, param_.inter_kernel, param_.inter_bias,
+                               inter_matmul_buf, 1, valid_rows, rows, inter, hidden, stream));
+    check_bt_error(bt_gemm_f32(inter_matmul_buf, nullptr, param_.output_kernel, nullptr,
+                               transformer_out, 0, valid_rows, rows, hidden, inter, stream));
+    if (is_remove_padding_)
+      check_bt_error(bt_add_bias_residual_layernorm_restore_f32(
+          transformer_out, attr_matmul_buf, param_.output_bias, param_.output_layernorm_gamma,
+          param_.output_layernorm_beta, restore_target, et_param.batch_idx, batch_size, seq_len,
+          hidden, layernorm_eps, stream));
+    else
+      check_bt_error(bt_add_bias_residual_layernorm_f32(
+          transformer_out, attr_matmul_buf, nullptr, param_.output_bias,
+          param_.output_layernorm_gamma, param_.output_layernorm_beta, nullptr, rows, hidden,
+          layernorm_eps, stream));
+    return;
   }
 
   // k-contiguous weight pre-pack: all four matrices in one launch, unless the

@@ -21,8 +21,8 @@ int validate(const bt_encoder_config *cfg) {
     g_error = "[BT][ERROR] null config";
     return BT_ERR_INVALID_ARGUMENT;
   }
-  if (cfg->dtype != BT_F16) {
-    g_error = "[BT][ERROR] only BT_F16 is implemented";
+  if (cfg->dtype != BT_F16 && cfg->dtype != BT_F32) {
+    g_error = "[BT][ERROR] dtype must be BT_F16 or BT_F32";
     return BT_ERR_UNSUPPORTED;
   }
   if (cfg->max_batch_size <= 0 || cfg->max_seq_len <= 0 || cfg->head_num <= 0 ||
@@ -33,36 +33,61 @@ int validate(const bt_encoder_config *cfg) {
   return BT_OK;
 }
 
-BertTransformerParam<OperationType::HALF> make_param(const bt_encoder_config *cfg,
-                                                     const bt_layer_weights *w) {
-  BertTransformerParam<OperationType::HALF> p;
-  p.attr_kernel_QKV = (const __half *)w->qkv_kernel;
-  p.attention_param.attr_bias_QKV = (const __half *)w->qkv_bias;
+template <OperationType Op>
+BertTransformerParam<Op> make_param(const bt_encoder_config *cfg, const bt_layer_weights *w) {
+  using T = typename bytetransformer::Traits<Op>::DataType;
+  BertTransformerParam<Op> p;
+  p.attr_kernel_QKV = (const T *)w->qkv_kernel;
+  p.attention_param.attr_bias_QKV = (const T *)w->qkv_bias;
   p.attention_param.tao = cfg->tao > 0.f ? cfg->tao : 1.0f;
-  p.attr_output_kernel = (const __half *)w->attr_output_kernel;
-  p.attr_output_bias = (const __half *)w->attr_output_bias;
+  p.attr_output_kernel = (const T *)w->attr_output_kernel;
+  p.attr_output_bias = (const T *)w->attr_output_bias;
   p.attr_output_layernorm_gamma = w->attr_output_layernorm_gamma;
   p.attr_output_layernorm_beta = w->attr_output_layernorm_beta;
-  p.inter_kernel = (const __half *)w->inter_kernel;
-  p.inter_bias = (const __half *)w->inter_bias;
-  p.output_kernel = (const __half *)w->output_kernel;
-  p.output_bias = (const __half *)w->output_bias;
+  p.inter_kernel = (const T *)w->inter_kernel;
+  p.inter_bias = (const T *)w->inter_bias;
+  p.output_kernel = (const T *)w->output_kernel;
+  p.output_bias = (const T *)w->output_bias;
   p.output_layernorm_gamma = w->output_layernorm_gamma;
   p.output_layernorm_beta = w->output_layernorm_beta;
   p.intermediate_size = cfg->intermediate_size;
   return p;
 }
+
+template <OperationType Op>
+unsigned long long layer_bufsize(const bt_encoder_config *cfg) {
+  BertTransformer<Op> enc(cfg->max_batch_size, cfg->head_num, cfg->size_per_head,
+                          cfg->max_seq_len, cfg->use_fused_attention != 0,
+                          cfg->is_remove_padding != 0, cfg->gamma_beta_fp32 != 0);
+  BertTransformerParam<Op> p;
+  p.intermediate_size = cfg->intermediate_size;
+  enc.initialize(p);
+  return enc.cal_bufsize();
+}
+
+template <OperationType Op>
+void layer_forward(const bt_encoder_config *cfg, const bt_layer_weights *weights,
+                   const void *input, const void *atten_mask, const void *attention_bias,
+                   void *output, void *buf, int batch_size, int seq_len, void *stream) {
+  using T = typename bytetransformer::Traits<Op>::DataType;
+  BertTransformer<Op> enc(cfg->max_batch_size, cfg->head_num, cfg->size_per_head,
+                          cfg->max_seq_len, cfg->use_fused_attention != 0,
+                          cfg->is_remove_padding != 0, cfg->gamma_beta_fp32 != 0);
+  if (cfg->layernorm_eps > 0.f) enc.layernorm_eps = cfg->layernorm_eps;
+  enc.initialize(make_param<Op>(cfg, weights));
+  enc.cal_bufsize();
+  BertTransformerInferParam<T> ip{(const T *)input, (const T *)atten_mask, (T *)output, buf,
+                                  batch_size,       seq_len,               nullptr,
+                                  (hipStream_t)stream};
+  ip.attention_bias = (const T *)attention_bias;
+  enc.infer(ip);
+}
 }  // namespace
 
 extern "C" unsigned long long bt_encoder_bufsize(const bt_encoder_config *cfg) {
   if (validate(cfg) != BT_OK) return 0;
-  BertTransformer<OperationType::HALF> enc(cfg->max_batch_size, cfg->head_num, cfg->size_per_head,
-                                           cfg->max_seq_len, cfg->use_fused_attention != 0,
-                                           cfg->is_remove_padding != 0, cfg->gamma_beta_fp32 != 0);
-  BertTransformerParam<OperationType::HALF> p;
-  p.intermediate_size = cfg->intermediate_size;
-  enc.initialize(p);
-  return enc.cal_bufsize();
+  return cfg->dtype == BT_F32 ? layer_bufsize<OperationType::FP32>(cfg)
+                              : layer_bufsize<OperationType::HALF>(cfg);
 }
 
 extern "C" int bt_encoder_layer_forward(const bt_encoder_config *cfg,
@@ -91,22 +116,12 @@ extern "C" int bt_encoder_layer_forward_bias(const bt_encoder_config *cfg,
       return BT_ERR_INVALID_ARGUMENT;
     }
   try {
-    BertTransformer<OperationType::HALF> enc(
-        cfg->max_batch_size, cfg->head_num, cfg->size_per_head, cfg->max_seq_len,
-        cfg->use_fused_attention != 0, cfg->is_remove_padding != 0, cfg->gamma_beta_fp32 != 0);
-    if (cfg->layernorm_eps > 0.f) enc.layernorm_eps = cfg->layernorm_eps;
-    enc.initialize(make_param(cfg, weights));
-    enc.cal_bufsize();
-    BertTransformerInferParam<__half> ip{(const __half *)input,
-                                         (const __half *)atten_mask,
-                                         (__half *)output,
-                                         buf,
-                                         batch_size,
-                                         seq_len,
-                                         nullptr,
-                                         (hipStream_t)stream};
-    ip.attention_bias = (const __half *)attention_bias;
-    enc.infer(ip);
+    if (cfg->dtype == BT_F32)
+      layer_forward<OperationType::FP32>(cfg, weights, input, atten_mask, attention_bias, output,
+                                         buf, batch_size, seq_len, stream);
+    else
+      layer_forward<OperationType::HALF>(cfg, weights, input, atten_mask, attention_bias, output,
+                                         buf, batch_size, seq_len, stream);
   } catch (const std::exception &e) {
     g_error = e.what();
     return BT_ERR_INVALID_ARGUMENT;
@@ -119,19 +134,20 @@ namespace {
 using bytetransformer::BertEncoder;
 using bytetransformer::BertEncoderInferParam;
 
+template <OperationType Op>
 int make_encoder(const bt_encoder_config *cfg, int num_layers, const bt_layer_weights *weights,
-                 std::unique_ptr<BertEncoder<OperationType::HALF>> *out) {
+                 std::unique_ptr<BertEncoder<Op>> *out) {
   int rc = validate(cfg);
   if (rc != BT_OK) return rc;
   if (num_layers <= 0) {
     g_error = "[BT][ERROR] num_layers must be positive";
     return BT_ERR_INVALID_ARGUMENT;
   }
-  out->reset(new BertEncoder<OperationType::HALF>(
-      cfg->max_batch_size, cfg->head_num, cfg->size_per_head, cfg->max_seq_len,
-      cfg->use_fused_attention != 0, cfg->is_remove_padding != 0, cfg->gamma_beta_fp32 != 0));
+  out->reset(new BertEncoder<Op>(cfg->max_batch_size, cfg->head_num, cfg->size_per_head,
+                                 cfg->max_seq_len, cfg->use_fused_attention != 0,
+                                 cfg->is_remove_padding != 0, cfg->gamma_beta_fp32 != 0));
   if (cfg->layernorm_eps > 0.f) (*out)->layernorm_eps = cfg->layernorm_eps;
-  std::vector<BertTransformerParam<OperationType::HALF>> layers((size_t)num_layers);
+  std::vector<BertTransformerParam<Op>> layers((size_t)num_layers);
   for (int l = 0; l < num_layers; ++l) {
     if (weights) {
       const void *const *wp = (const void *const *)(weights + l);
@@ -141,7 +157,7 @@ int make_encoder(const bt_encoder_config *cfg, int num_layers, const bt_layer_we
                     std::to_string(l);
           return BT_ERR_INVALID_ARGUMENT;
         }
-      layers[(size_t)l] = make_param(cfg, weights + l);
+      layers[(size_t)l] = make_param<Op>(cfg, weights + l);
     } else {
       layers[(size_t)l].intermediate_size = cfg->intermediate_size;
     }
@@ -149,19 +165,54 @@ int make_encoder(const bt_encoder_config *cfg, int num_layers, const bt_layer_we
   (*out)->initialize(layers);
   return BT_OK;
 }
+
+template <OperationType Op>
+unsigned long long encoder_sizes(const bt_encoder_config *cfg, int num_layers, bool prepack) {
+  std::unique_ptr<BertEncoder<Op>> enc;
+  if (make_encoder<Op>(cfg, num_layers, nullptr, &enc) != BT_OK) return 0;
+  return prepack ? enc->prepack_bytes() : enc->cal_bufsize();
+}
+
+template <OperationType Op>
+int encoder_prepack(const bt_encoder_config *cfg, int num_layers, const bt_layer_weights *weights,
+                    void *prepacked, void *stream) {
+  std::unique_ptr<BertEncoder<Op>> enc;
+  int rc = make_encoder<Op>(cfg, num_layers, weights, &enc);
+  if (rc != BT_OK) return rc;
+  enc->prepack(prepacked, (hipStream_t)stream);
+  return BT_OK;
+}
+
+template <OperationType Op>
+int encoder_forward(const bt_encoder_config *cfg, int num_layers, const bt_layer_weights *weights,
+                    const void *prepacked, const void *input, const void *atten_mask,
+                    const void *attention_bias, void *output, void *buf, int batch_size,
+                    int seq_len, int valid_rows_hint, void *stream) {
+  using T = typename bytetransformer::Traits<Op>::DataType;
+  std::unique_ptr<BertEncoder<Op>> enc;
+  int rc = make_encoder<Op>(cfg, num_layers, weights, &enc);
+  if (rc != BT_OK) return rc;
+  BertEncoderInferParam<T> ip{(const T *)input, (const T *)atten_mask, (T *)output, buf,
+                              batch_size,       seq_len,               (hipStream_t)stream};
+  ip.attention_bias = (const T *)attention_bias;
+  ip.prepacked = prepacked;
+  ip.valid_rows_hint = valid_rows_hint;
+  enc->infer(ip);
+  return BT_OK;
+}
+
+bool is_f32(const bt_encoder_config *cfg) { return cfg && cfg->dtype == BT_F32; }
 }  // namespace
 
 extern "C" unsigned long long bt_encoder_forward_bufsize(const bt_encoder_config *cfg) {
-  std::unique_ptr<BertEncoder<OperationType::HALF>> enc;
-  if (make_encoder(cfg, 1, nullptr, &enc) != BT_OK) return 0;
-  return enc->cal_bufsize();
+  return is_f32(cfg) ? encoder_sizes<OperationType::FP32>(cfg, 1, false)
+                     : encoder_sizes<OperationType::HALF>(cfg, 1, false);
 }
 
 extern "C" unsigned long long bt_encoder_prepack_bytes(const bt_encoder_config *cfg,
                                                        int num_layers) {
-  std::unique_ptr<BertEncoder<OperationType::HALF>> enc;
-  if (make_encoder(cfg, num_layers, nullptr, &enc) != BT_OK) return 0;
-  return enc->prepack_bytes();
+  return is_f32(cfg) ? encoder_sizes<OperationType::FP32>(cfg, num_layers, true)
+                     : encoder_sizes<OperationType::HALF>(cfg, num_layers, true);
 }
 
 extern "C" int bt_encoder_prepack(const bt_encoder_config *cfg, int num_layers,
@@ -171,16 +222,14 @@ extern "C" int bt_encoder_prepack(const bt_encoder_config *cfg, int num_layers,
     g_error = "[BT][ERROR] null weights";
     return BT_ERR_INVALID_ARGUMENT;
   }
-  std::unique_ptr<BertEncoder<OperationType::HALF>> enc;
-  int rc = make_encoder(cfg, num_layers, weights, &enc);
-  if (rc != BT_OK) return rc;
   try {
-    enc->prepack(prepacked, (hipStream_t)stream);
+    return is_f32(cfg)
+               ? encoder_prepack<OperationType::FP32>(cfg, num_layers, weights, prepacked, stream)
+               : encoder_prepack<OperationType::HALF>(cfg, num_layers, weights, prepacked, stream);
   } catch (const std::exception &e) {
     g_error = e.what();
     return BT_ERR_INVALID_ARGUMENT;
   }
-  return BT_OK;
 }
 
 extern "C" int bt_encoder_forward(const bt_encoder_config *cfg, int num_layers,
@@ -193,23 +242,18 @@ extern "C" int bt_encoder_forward(const bt_encoder_config *cfg, int num_layers,
     g_error = "[BT][ERROR] null weights";
     return BT_ERR_INVALID_ARGUMENT;
   }
-  std::unique_ptr<BertEncoder<OperationType::HALF>> enc;
-  int rc = make_encoder(cfg, num_layers, weights, &enc);
-  if (rc != BT_OK) return rc;
   try {
-    BertEncoderInferParam<__half> ip{(const __half *)input, (const __half *)atten_mask,
-                                     (__half *)output,      buf,
-                                     batch_size,            seq_len,
-                                     (hipStream_t)stream};
-    ip.attention_bias = (const __half *)attention_bias;
-    ip.prepacked = prepacked;
-    ip.valid_rows_hint = valid_rows_hint;
-    enc->infer(ip);
+    return is_f32(cfg)
+               ? encoder_forward<OperationType::FP32>(cfg, num_layers, weights, prepacked, input,
+                                                      atten_mask, attention_bias, output, buf,
+                                                      batch_size, seq_len, valid_rows_hint, stream)
+               : encoder_forward<OperationType::HALF>(cfg, num_layers, weights, prepacked, input,
+                                                      atten_mask, attention_bias, output, buf,
+                                                      batch_size, seq_len, valid_rows_hint, stream);
   } catch (const std::exception &e) {
     g_error = e.what();
     return BT_ERR_INVALID_ARGUMENT;
   }
-  return BT_OK;
 }
 
 extern "C" const char *bt_encoder_last_error(void) { return g_error.c_str(); }

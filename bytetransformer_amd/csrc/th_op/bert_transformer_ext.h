@@ -108,7 +108,7 @@ class BTEncoder : public IBTEncoder {
  private:
   // The four [N, K] weight copies, from the process-wide cache when the same
   // tensors were seen before, else packed now (one launch) and remembered.
-  // Empty for dtypes the kernels do not run (infer() raises for those).
+  // Empty for float, whose kernels read the weights as stored.
   std::vector<Tensor> prepacked_weights(hipStream_t stream) {
     std::vector<Tensor> out;
     if (kOp != OperationType::HALF) return out;
@@ -146,8 +146,7 @@ class BTEncoder : public IBTEncoder {
 
   bool mask_plan(const Tensor &mask, int batch_size, int seq_len, hipStream_t stream,
                  MaskPlanCache::Plan *plan) {
-    if (kOp != OperationType::HALF || !PrepackCache::instance().enabled() || mask.is_inference())
-      return false;
+    if (!PrepackCache::instance().enabled() || mask.is_inference()) return false;
     hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
     if (hipStreamIsCapturing(stream, &capturing) != hipSuccess ||
         capturing != hipStreamCaptureStatusNone)
@@ -158,7 +157,7 @@ class BTEncoder : public IBTEncoder {
     plan->batch_idx = torch::empty({(int64_t)batch_size + 1}, opts);
     plan->word_idx = torch::empty({(int64_t)batch_size * seq_len}, opts);
     plan->seq_order = torch::empty({(int64_t)batch_size}, opts);
-    check_bt_error(bt_build_offsets(mask.data_ptr(), BT_F16, batch_size, seq_len,
+    check_bt_error(bt_build_offsets(mask.data_ptr(), Traits<kOp>::dtype, batch_size, seq_len,
                                     plan->batch_idx.data_ptr<int>(), plan->word_idx.data_ptr<int>(),
                                     plan->seq_order.data_ptr<int>(), &plan->valid_word_num,
                                     stream));

@@ -1,7 +1,7 @@
 """Host-side mirror of the reference's per-layer interface for Python callers
 that do not go through torch.ops: BertEncoderLayer wraps
 bt_encoder_layer_forward (include/bt_encoder.h), i.e. the C++
-BertTransformer<HALF>::infer, with torch tensors providing device memory and
+BertTransformer<HALF or FP32>::infer, with torch tensors providing device memory and
 the current stream."""
 import ctypes
 
@@ -9,6 +9,28 @@ import torch
 
 from ._lib import EncoderConfig, LayerWeights, host_lib
 from .workload import WEIGHT_NAMES
+
+
+_DTYPE_CODE = {torch.float32: 0, torch.float16: 1}   # BT_F32, BT_F16
+
+
+def _activation_dtype(weights):
+    """The layer's OperationType follows the QKV weight, as in the PyTorch operator."""
+    dt = weights[0].dtype
+    if dt not in _DTYPE_CODE:
+        raise ValueError("weights must be float16 or float32, got %s" % dt)
+    for i, w in enumerate(weights):
+        loose = i in (4, 5, 10, 11)      # gamma / beta of fp16 layers may be float
+        if w.dtype != dt and not (loose and dt == torch.float16 and w.dtype == torch.float32):
+            raise ValueError("weight #%d has dtype %s, expected %s" % (i, w.dtype, dt))
+    return dt
+
+
+def _check_io(dtype, x, mask):
+    if x.dtype != dtype or mask.dtype != dtype:
+        raise RuntimeError("input and mask must have the weights' dtype %s" % dtype)
+    if not (x.is_cuda and x.is_contiguous() and mask.is_cuda and mask.is_contiguous()):
+        raise RuntimeError("input and mask must be contiguous GPU tensors")
 
 
 class BertEncoderLayer:
@@ -32,9 +54,10 @@ class BertEncoderLayer:
         self.layernorm_eps, self.tao = layernorm_eps, tao
         self._w = LayerWeights(*[ctypes.c_void_p(w.data_ptr()) for w in self.weights])
         self._buf = None
+        self.dtype = _activation_dtype(self.weights)
 
     def _config(self, B, S):
-        return EncoderConfig(1, B, S, self.head_num, self.head_size,
+        return EncoderConfig(_DTYPE_CODE[self.dtype], B, S, self.head_num, self.head_size,
                              self.weights[6].shape[1] // self.hidden,
                              int(self.use_fused_attention), int(self.is_remove_padding),
                              int(self.weights[10].dtype == torch.float32), self.tao,
@@ -42,8 +65,7 @@ class BertEncoderLayer:
 
     def __call__(self, x, mask, out=None, attention_bias=None):
         lib = host_lib()
-        if x.dtype != torch.float16:
-            raise RuntimeError("only fp16 activations are implemented")
+        _check_io(self.dtype, x, mask)
         B, S, H = x.shape
         cfg = self._config(B, S)
         need = lib.bt_encoder_bufsize(ctypes.byref(cfg))
@@ -112,10 +134,14 @@ class BertEncoder:
             *[LayerWeights(*[ctypes.c_void_p(t.data_ptr()) for t in w]) for w in sets])
         self._prepacked = None
         self._buf = None
+        self.dtype = _activation_dtype(sets[0])
+        for w in sets[1:]:
+            if _activation_dtype(w) != self.dtype:
+                raise ValueError("all layers must share one weight dtype")
 
     def _config(self, B, S):
         w0 = self.weights[0]
-        return EncoderConfig(1, B, S, self.head_num, self.head_size,
+        return EncoderConfig(_DTYPE_CODE[self.dtype], B, S, self.head_num, self.head_size,
                              w0[6].shape[1] // self.hidden, int(self.use_fused_attention),
                              int(self.is_remove_padding), int(w0[10].dtype == torch.float32),
                              self.tao, self.layernorm_eps)
@@ -137,8 +163,7 @@ class BertEncoder:
 
     def __call__(self, x, mask, out=None, attention_bias=None, valid_rows_hint=0):
         lib = host_lib()
-        if x.dtype != torch.float16:
-            raise RuntimeError("only fp16 activations are implemented")
+        _check_io(self.dtype, x, mask)
         B, S, H = x.shape
         if attention_bias is not None and (
                 attention_bias.dtype != x.dtype or not attention_bias.is_contiguous()
@@ -181,9 +206,9 @@ class GraphedBertEncoder:
         dev = encoder.weights[0][0].device
         self.encoder = encoder
         with torch.cuda.device(dev):
-            self.input = torch.zeros(batch_size, seq_len, encoder.hidden, dtype=torch.float16,
+            self.input = torch.zeros(batch_size, seq_len, encoder.hidden, dtype=encoder.dtype,
                                      device=dev)
-            self.mask = torch.ones(batch_size, seq_len, seq_len, dtype=torch.float16, device=dev)
+            self.mask = torch.ones(batch_size, seq_len, seq_len, dtype=encoder.dtype, device=dev)
             self.output = torch.empty_like(self.input)
             # first call outside the capture: one-time kernel attribute set-up, pre-pack, scratch
             side = torch.cuda.Stream(device=dev)

@@ -170,3 +170,62 @@ def add_bias_residual_layernorm_restore(out, residual, bias, gamma, beta, batch_
         int(gamma.dtype == torch.float32), _ptr(out_padded), _ptr(batch_idx), batch_size, seq_len,
         H, float(eps), _stream()))
     return out_padded
+
+
+# ---- float (OperationType::FP32) entry points ---------------------------------
+def _need_f32(*ts):
+    for t in ts:
+        if t is not None and t.dtype != torch.float32:
+            raise BtError("the *_f32 entry points take float tensors only")
+
+
+def gemm_f32(a, w, bias=None, gelu=False, valid_rows=None, a_row_index=None, rows_cap=None,
+             out=None):
+    """c = a . w (+ bias) (+ tanh-GELU); w is [K, N] as stored."""
+    _need_f32(a, w, bias, out)
+    rows = a.shape[0] if rows_cap is None else rows_cap
+    K, N = w.shape
+    if out is None:
+        out = torch.zeros(rows, N, dtype=a.dtype, device=a.device)
+    _check(kernel_lib().bt_gemm_f32(_ptr(a), _ptr(a_row_index), _ptr(w), _ptr(bias), _ptr(out),
+                                    int(gelu), _ptr(valid_rows), rows, N, K, _stream()))
+    return out
+
+
+def attention_f32(qkv, batch_idx, batch_size, seq_len, head_num, scale, padded_rows=False,
+                  mask=None, bias=None, out=None):
+    """qkv [rows, 3 * hidden] (bias added) -> [rows, hidden]."""
+    _need_f32(qkv, mask, bias, out)
+    rows_cap, three_h = qkv.shape
+    hidden = three_h // 3
+    if out is None:
+        out = torch.zeros(rows_cap, hidden, dtype=qkv.dtype, device=qkv.device)
+    if bias is not None and tuple(bias.shape) != (head_num, seq_len, seq_len):
+        raise ValueError("attention bias must be [head_num, seq_len, seq_len]")
+    _check(kernel_lib().bt_attention_f32(_ptr(qkv), _ptr(out), _ptr(batch_idx), _ptr(mask),
+                                         _ptr(bias), batch_size, seq_len, rows_cap, head_num,
+                                         hidden // head_num, float(scale), int(padded_rows),
+                                         _stream()))
+    return out
+
+
+def add_bias_residual_layernorm_f32(out, residual, bias, gamma, beta, eps=1e-6, valid_rows=None,
+                                    residual_row_index=None):
+    _need_f32(out, residual, bias, gamma, beta)
+    rows, H = out.shape
+    _check(kernel_lib().bt_add_bias_residual_layernorm_f32(
+        _ptr(out), _ptr(residual), _ptr(residual_row_index), _ptr(bias), _ptr(gamma), _ptr(beta),
+        _ptr(valid_rows), rows, H, float(eps), _stream()))
+    return out
+
+
+def add_bias_residual_layernorm_restore_f32(out, residual, bias, gamma, beta, batch_idx,
+                                            batch_size, seq_len, eps=1e-6, out_padded=None):
+    _need_f32(out, residual, bias, gamma, beta, out_padded)
+    H = out.shape[-1]
+    if out_padded is None:
+        out_padded = torch.empty(batch_size, seq_len, H, dtype=out.dtype, device=out.device)
+    _check(kernel_lib().bt_add_bias_residual_layernorm_restore_f32(
+        _ptr(out), _ptr(residual), _ptr(bias), _ptr(gamma), _ptr(beta), _ptr(out_padded),
+        _ptr(batch_idx), batch_size, seq_len, H, float(eps), _stream()))
+    return out_padded

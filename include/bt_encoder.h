@@ -34,7 +34,7 @@ typedef struct bt_layer_weights {
 } bt_layer_weights;
 
 typedef struct bt_encoder_config {
-  int dtype;               /* BT_F16 (BT_F32 is rejected: not implemented) */
+  int dtype;               /* BT_F16 or BT_F32: element type of every tensor (OperationType) */
   int max_batch_size;
   int max_seq_len;
   int head_num;
@@ -59,7 +59,7 @@ int bt_encoder_layer_forward(const bt_encoder_config *cfg, const bt_layer_weight
                              int batch_size, int seq_len, void *stream);
 
 /* The same with the optional attention bias of the reference's infer parameters
- * (bert_transformer.h:93, attention.h:56): fp16 [head_num, seq_len, seq_len],
+ * (bert_transformer.h:93, attention.h:56): [head_num, seq_len, seq_len] of cfg->dtype,
  * added to the scaled logits before the mask term (softmax.h:41-46).  NULL = none. */
 int bt_encoder_layer_forward_bias(const bt_encoder_config *cfg, const bt_layer_weights *weights,
                                   const void *input, const void *atten_mask,

@@ -209,6 +209,56 @@ int bt_add_bias_residual_layernorm_restore(const void *out, const void *residual
                                            int batch_size, int seq_len, int hidden_dim,
                                            float eps, void *stream);
 
+/*
+ * ---- OperationType::FP32 ------------------------------------------------------
+ * The float flavour of the layer: every tensor (activations, weights, biases, gamma,
+ * beta, mask, attention bias) is float, products run on the fp32 MFMA with fp32
+ * operands and accumulators.  Weights are read as the caller stores them ([K, N]
+ * row-major): there is no pre-pack.
+ *
+ * bt_gemm_f32: c[M, n] = a[M, k] . w[k, n] (+ bias[n]) (then tanh-GELU when gelu != 0,
+ * which needs a bias).  a_row_index (nullable, needs valid_rows): row r of A is
+ * a[a_row_index[r], :].  n % 4 == 0, k % 4 == 0.  Replaces the cuBLAS calls of
+ * dense_layer_kernel_launcher<float> (bytetransformer/src/gemm.cu:32-39), the QKV bias
+ * add of add_QKV_bias (attention_nofused_utils.cu:143-184) and
+ * gemm_bias_gelu<float> (gemm_bias_act.cu:24-75).
+ */
+int bt_gemm_f32(const void *a, const int *a_row_index, const void *w, const void *bias, void *c,
+                int gelu, const int *valid_rows, int rows_cap, int n, int k, void *stream);
+
+/*
+ * Fused multi-head attention on float, token-major projections qkv [rows, 3 * hidden]
+ * (Q | K | V per row, QKV bias already added) -> attention_output [rows, hidden].
+ * P = exp(x - max) / (sum + 1e-6) with x = scale q.k + attention_bias[head, q, key]
+ * + (atten_mask[b, q, key] - 1) * 10000, the arithmetic of softmax_kernel_warp[_et]
+ * (bytetransformer/include/softmax.h:25-60,103-140); replaces the whole unfused path
+ * Attention<FP32>::nofused_infer (attention_nofused.cu:27-114) without its logits
+ * buffer.  atten_mask (nullable, float [B,S,S]) is applied on both row layouts; keys at
+ * or past the sequence length are excluded by index on packed rows (they do not exist
+ * there) and, without a mask, on padded rows.  size_per_head in {32, 64, 128}.
+ */
+int bt_attention_f32(const void *qkv, void *attention_output, const int *batch_idx,
+                     const void *atten_mask, const void *attention_bias, int batch_size,
+                     int seq_len, int rows_cap, int head_num, int size_per_head, float scale,
+                     int padded_rows, void *stream);
+
+/*
+ * The two LayerNorm entry points on float: x = out + residual + bias in fp32, two-pass
+ * statistics, hidden_dim % 4 == 0 (layernorm.h:20-40, layernorm.cu:89-148 for float).
+ */
+int bt_add_bias_residual_layernorm_f32(void *out, const void *residual,
+                                       const int *residual_row_index, const void *bias,
+                                       const void *gamma, const void *beta,
+                                       const int *valid_rows, int rows_cap, int hidden_dim,
+                                       float eps, void *stream);
+
+int bt_add_bias_residual_layernorm_restore_f32(const void *out, const void *residual,
+                                               const void *bias, const void *gamma,
+                                               const void *beta, void *out_padded,
+                                               const int *batch_idx, int batch_size,
+                                               int seq_len, int hidden_dim, float eps,
+                                               void *stream);
+
 #ifdef __cplusplus
 }
 #endif

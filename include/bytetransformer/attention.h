@@ -21,8 +21,9 @@ class AttentionParam {
 
 template <typename T>
 struct AttentionInferParam {
-  // Head-major projections with the QKV bias already added:
-  // [3][head_num][batch_size * seq_len][size_per_head] (written by the QKV GEMM).
+  // Projections with the QKV bias already added, as the QKV GEMM writes them:
+  // fp16 head-major [3][head_num][batch_size * seq_len][size_per_head],
+  // float token-major [batch_size * seq_len][3 * hidden_dim].
   const T *qkv;
   const T *atten_mask;  // [batch_size, seq_len, seq_len]; lengths come from et_param.batch_idx
   T *attention_output;  // token-major [rows, hidden_dim]

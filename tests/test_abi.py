@@ -63,6 +63,15 @@ def test_argument_validation_returns_codes_without_gpu():
     assert lib.bt_add_bias_residual_layernorm_restore(p, p, p, p, p, 0, None, p, 2, 4, 64, 1e-6,
                                                       None) == 1
     assert lib.bt_transpose_weight(None, p, 8, 8, None) == 1
+    # float entry points
+    assert lib.bt_gemm_f32(p, None, p, None, p, 0, None, 4, 6, 8, None) == 2 and "multiples of 4" in err()
+    assert lib.bt_gemm_f32(p, None, p, None, p, 1, None, 4, 8, 8, None) == 1 and "gelu needs a bias" in err()
+    assert lib.bt_gemm_f32(p, p, p, None, p, 0, None, 4, 8, 8, None) == 1 and "needs valid_rows" in err()
+    assert lib.bt_attention_f32(p, p, p, None, None, 1, 16, 16, 12, 48, 0.125, 0, None) == 2
+    assert lib.bt_attention_f32(p, p, p, None, None, 2, 16, 16, 12, 64, 0.125, 1, None) == 1
+    assert lib.bt_add_bias_residual_layernorm_f32(p, p, None, p, p, p, None, 4, 6, 1e-6, None) == 2
+    assert lib.bt_add_bias_residual_layernorm_restore_f32(p, p, p, p, p, None, p, 2, 4, 64, 1e-6,
+                                                          None) == 1
 
 
 def test_encoder_c_api_validation_and_bufsize():
@@ -73,9 +82,12 @@ def test_encoder_c_api_validation_and_bufsize():
     # nine activation tensors + two index arrays + the pre-packed weights
     assert need >= 9 * T * 2 + 2 * 16 * 512 * 4 + 12 * 768 * 768 * 2
     assert need < 9 * T * 2 + 2 * 16 * 512 * 4 + 12 * 768 * 768 * 2 + 8192
-    bad = _lib.EncoderConfig(0, 16, 512, 12, 64, 4, 1, 1, 0, 1.0, 1e-6)   # fp32: not implemented
+    f32 = _lib.EncoderConfig(0, 16, 512, 12, 64, 4, 1, 1, 0, 1.0, 1e-6)   # float: twice the bytes
+    need32 = lib.bt_encoder_bufsize(ctypes.byref(f32))
+    assert 2 * need - 4 * 16 * 512 * 4 - 8192 < need32 < 2 * need
+    bad = _lib.EncoderConfig(7, 16, 512, 12, 64, 4, 1, 1, 0, 1.0, 1e-6)
     assert lib.bt_encoder_bufsize(ctypes.byref(bad)) == 0
-    assert b"BT_F16" in lib.bt_encoder_last_error()
+    assert b"BT_F16 or BT_F32" in lib.bt_encoder_last_error()
     w = _lib.LayerWeights()
     rc = lib.bt_encoder_layer_forward(ctypes.byref(cfg), ctypes.byref(w), None, None, None, None,
                                       1, 1, None)
