@@ -77,22 +77,23 @@ void BertEncoder<OpType>::infer(BertEncoderInferParam<DataType_> ip) {
 
     if constexpr (OpType == OperationType::FP32) {
       check_bt_error(bt_gemm_f32(x, gather, w.attr_kernel_QKV, w.attention_param.attr_bias_QKV,
-                                 qkv_buf, 0, valid_rows, rows, 3 * hidden, hidden, stream));
+                                 qkv_buf, 0, valid_rows, rows, rows_hint, 3 * hidden, hidden, stream));
       struct AttentionInferParam<DataType_> att {
         qkv_buf, ip.atten_mask, attr_out_buf, nullptr, batch_size, seq_len, nullptr, stream,
             et_param
       };
       att.attention_bias = ip.attention_bias;
+      att.seq_order = seq_order;
       attention_layer_->infer(att);
       check_bt_error(bt_gemm_f32(attr_out_buf, nullptr, w.attr_output_kernel, nullptr,
-                                 attr_matmul_buf, 0, valid_rows, rows, hidden, hidden, stream));
+                                 attr_matmul_buf, 0, valid_rows, rows, rows_hint, hidden, hidden, stream));
       check_bt_error(bt_add_bias_residual_layernorm_f32(
           attr_matmul_buf, x, gather, w.attr_output_bias, w.attr_output_layernorm_gamma,
           w.attr_output_layernorm_beta, valid_rows, rows, hidden, layernorm_eps, stream));
       check_bt_error(bt_gemm_f32(attr_matmul_buf, nullptr, w.inter_kernel, w.inter_bias,
-                                 inter_matmul_buf, 1, valid_rows, rows, inter, hidden, stream));
+                                 inter_matmul_buf, 1, valid_rows, rows, rows_hint, inter, hidden, stream));
       check_bt_error(bt_gemm_f32(inter_matmul_buf, nullptr, w.output_kernel, nullptr, ffn2_out, 0,
-                                 valid_rows, rows, hidden, inter, stream));
+                                 valid_rows, rows, rows_hint, hidden, inter, stream));
       if (last && is_remove_padding_)
         check_bt_error(bt_add_bias_residual_layernorm_restore_f32(
             ffn2_out, attr_matmul_buf, w.output_bias, w.output_layernorm_gamma,

@@ -80,24 +80,25 @@ void BertTransformer<OpType>::bert_infer(BertTransformerInferParam infer_param) 
     // float: weights are consumed as stored, Q/K/V stay token-major [rows, 3H], gamma
     // and beta are float by definition
     check_bt_error(bt_gemm_f32(from_tensor, gather, param_.attr_kernel_QKV,
-                               param_.attention_param.attr_bias_QKV, qkv_buf, 0, valid_rows, rows,
+                               param_.attention_param.attr_bias_QKV, qkv_buf, 0, valid_rows, rows, rows_hint,
                                3 * hidden, hidden, stream));
     struct AttentionInferParam<DataType_> attention_infer_param {
       qkv_buf, atten_mask, attr_out_buf, base + inner_buf_size_, batch_size, seq_len,
           infer_param.cublas_handle, stream, et_param
     };
     attention_infer_param.attention_bias = infer_param.attention_bias;
+    attention_infer_param.seq_order = seq_order;
     attention_layer_->infer(attention_infer_param);
     check_bt_error(bt_gemm_f32(attr_out_buf, nullptr, param_.attr_output_kernel, nullptr,
-                               attr_matmul_buf, 0, valid_rows, rows, hidden, hidden, stream));
+                               attr_matmul_buf, 0, valid_rows, rows, rows_hint, hidden, hidden, stream));
     check_bt_error(bt_add_bias_residual_layernorm_f32(
         attr_matmul_buf, from_tensor, gather, param_.attr_output_bias,
         param_.attr_output_layernorm_gamma, param_.attr_output_layernorm_beta, valid_rows, rows,
         hidden, layernorm_eps, stream));
     check_bt_error(bt_gemm_f32(attr_matmul_buf, nullptr, param_.inter_kernel, param_.inter_bias,
-                               inter_matmul_buf, 1, valid_rows, rows, inter, hidden, stream));
+                               inter_matmul_buf, 1, valid_rows, rows, rows_hint, inter, hidden, stream));
     check_bt_error(bt_gemm_f32(inter_matmul_buf, nullptr, param_.output_kernel, nullptr,
-                               transformer_out, 0, valid_rows, rows, hidden, inter, stream));
+                               transformer_out, 0, valid_rows, rows, rows_hint, hidden, inter, stream));
     if (is_remove_padding_)
       check_bt_error(bt_add_bias_residual_layernorm_restore_f32(
           transformer_out, attr_matmul_buf, param_.output_bias, param_.output_layernorm_gamma,

@@ -52,7 +52,40 @@ struct AttArgs {
   int B, S, rows_cap, heads;
   float scale_log2e;   // scale * log2(e)
   int padded_rows;
+  int nqb;             // query tiles per sequence (set by the launcher)
+  unsigned nqb_grid;   // host only: workgroups of the launch
+  int xcd_map;         // 1: XCD-aware workgroup order, 0: plain (tile, head, sequence) order
 };
+
+// Which (sequence rank, head, query tile) a workgroup of the 1-D grid works on.  The
+// hardware deals consecutive workgroup ids round-robin to the 8 XCDs.  In a plain
+// (tile fastest) order the XCD of a workgroup is a function of its query-tile index, and
+// with ragged lengths the high tiles are mostly dead: some XCDs get a fraction of the
+// work of others.  The XCD-aware order gives XCD x the (sequence, head) pairs
+// p = x (mod 8) - pairs counted sequence-major over the longest-first order, so every
+// XCD sees the same mix of lengths - and runs the query tiles of one pair back to back
+// on that XCD, whose L2 then serves the pair's K / V to all of them.
+struct AttItem {
+  int rank, head, qb;
+  bool exists;
+};
+__device__ __forceinline__ AttItem att_item(const AttArgs &p) {
+  AttItem it;
+  const unsigned lin = blockIdx.x;
+  if (p.xcd_map) {
+    const unsigned slot = lin >> 3, pair = (slot / p.nqb) * 8 + (lin & 7);
+    it.qb = slot % p.nqb;
+    it.exists = pair < (unsigned)(p.B * p.heads);
+    it.rank = pair / p.heads;
+    it.head = pair % p.heads;
+  } else {
+    it.qb = lin % p.nqb;
+    it.head = (lin / p.nqb) % p.heads;
+    it.rank = lin / (p.nqb * p.heads);
+    it.exists = true;
+  }
+  return it;
+}
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
@@ -97,11 +130,10 @@ __device__ __forceinline__ float rows_sum(float x) {
 // are the wave's last instructions; nothing reads their results.
 __device__ __forceinline__ void prefetch_slice(const AttArgs &p) {
   if (!p.prefetch) return;
-  const unsigned z0 = gridDim.z / 2;
-  if (blockIdx.z < z0) return;
-  const unsigned long long duty = (unsigned long long)gridDim.x * gridDim.y * (gridDim.z - z0);
-  const unsigned long long me =
-      ((unsigned long long)(blockIdx.z - z0) * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x;
+  const unsigned z0 = gridDim.x / 2;
+  if (blockIdx.x < z0) return;
+  const unsigned long long duty = gridDim.x - z0;
+  const unsigned long long me = blockIdx.x - z0;
   const unsigned long long lines = (p.prefetch_bytes + 127) / 128;
   const unsigned long long per = (lines + duty - 1) / duty;
   const unsigned long long first = me * per;
@@ -199,13 +231,18 @@ __global__ __launch_bounds__(kAttThreads, 2) void attention_grouped_kernel(AttAr
   constexpr int BQ = 4 * QB * 16;
   __shared__ __attribute__((aligned(1024))) half_t ring[kAttStages * 2 * kTileHalfs];
 
-  const int b = p.seq_order ? p.seq_order[blockIdx.z] : blockIdx.z, head = blockIdx.y;
+  const AttItem item = att_item(p);
+  if (!item.exists) {
+    prefetch_slice(p);
+    return;
+  }
+  const int b = p.seq_order ? p.seq_order[item.rank] : item.rank, head = item.head;
   const int seq_start = p.batch_idx[b];
   // with a mask tensor every one of the S key rows takes part
   const int klen = ADD && p.mask ? p.S : p.batch_idx[b + 1] - seq_start;
   const int row_start = p.padded_rows ? b * p.S : seq_start;
   const int nq = p.padded_rows ? p.S : klen;
-  const int q0 = blockIdx.x * BQ;
+  const int q0 = item.qb * BQ;
   if (q0 >= nq) {
     prefetch_slice(p);
     return;
@@ -421,12 +458,17 @@ __global__ __launch_bounds__(kAttThreads) void attention_short_kernel(AttArgs p)
   half_t *sK = att_smem;                      // [KEYS][64] swizzled
   half_t *sV = att_smem + KEYS * kHeadDim;    // [KEYS][64] swizzled
 
-  const int b = p.seq_order ? p.seq_order[blockIdx.z] : blockIdx.z, head = blockIdx.y;
+  const AttItem item = att_item(p);
+  if (!item.exists) {
+    prefetch_slice(p);
+    return;
+  }
+  const int b = p.seq_order ? p.seq_order[item.rank] : item.rank, head = item.head;
   const int seq_start = p.batch_idx[b];
   const int klen = ADD && p.mask ? p.S : p.batch_idx[b + 1] - seq_start;
   const int row_start = p.padded_rows ? b * p.S : seq_start;
   const int nq = p.padded_rows ? p.S : klen;
-  const int q0 = blockIdx.x * BQ;
+  const int q0 = item.qb * BQ;
   if (q0 >= nq) {
     prefetch_slice(p);
     return;
@@ -549,15 +591,23 @@ __global__ __launch_bounds__(kAttThreads) void attention_short_kernel(AttArgs p)
 // and up) and a loss of 2-3 % with smaller grids, which therefore skip it.  Each
 // duty workgroup (second half of the issue order) touches at most a couple of
 // lines per thread; the range is cut to that.
-static void set_prefetch(AttArgs &a, dim3 grid, const void *prefetch, unsigned long long bytes) {
+static void set_prefetch(AttArgs &a, unsigned grid, const void *prefetch, unsigned long long bytes) {
   a.prefetch = nullptr;
   a.prefetch_bytes = 0;
   if (!prefetch || !bytes || !option_prefetch()) return;
-  const unsigned long long duty = (unsigned long long)grid.x * grid.y * (grid.z - grid.z / 2);
-  if ((unsigned long long)grid.x * grid.y * grid.z < 512) return;
+  const unsigned long long duty = grid - grid / 2;
+  if (grid < 512) return;
   const unsigned long long cap = duty * 2 * kAttThreads * 128;
   a.prefetch = (const char *)prefetch;
   a.prefetch_bytes = bytes < cap ? bytes : cap;
+}
+
+// Size of the 1-D grid for `nqb` query tiles per sequence; fills the mapping fields.
+static unsigned att_grid(AttArgs &a, int nqb) {
+  a.nqb = nqb;
+  a.xcd_map = option_attention_xcd_map();
+  const unsigned pairs = (unsigned)a.B * a.heads;
+  return a.xcd_map ? (pairs + 7) / 8 * 8 * nqb : pairs * nqb;
 }
 
 static int check_att_args(const char *who, const void *qkv, const void *out, const int *batch_idx,
@@ -583,8 +633,7 @@ static int launch_short_impl(const AttArgs &a, hipStream_t s) {
   const int rc = allow_dynamic_lds(attention_short_kernel<NKB, ADD>, smem, configured,
                                    "hipFuncSetAttribute(attention_short_kernel)");
   if (rc != BT_OK) return rc;
-  dim3 grid((a.S + 63) / 64, a.heads, a.B);
-  attention_short_kernel<NKB, ADD><<<grid, kAttThreads, smem, s>>>(a);
+  attention_short_kernel<NKB, ADD><<<a.nqb_grid, kAttThreads, smem, s>>>(a);
   BT_CHECK_LAUNCH("attention_short_kernel");
   return BT_OK;
 }
@@ -615,7 +664,8 @@ extern "C" int bt_attention_short(const void *qkv_heads, void *attention_output,
             nullptr, 0, batch_size, seq_len,
             rows_cap, head_num, scale * kLog2e, padded_rows};
   hipStream_t s = as_stream(stream);
-  set_prefetch(a, dim3((seq_len + 63) / 64, head_num, batch_size), prefetch, prefetch_bytes);
+  a.nqb_grid = att_grid(a, (seq_len + 63) / 64);
+  set_prefetch(a, a.nqb_grid, prefetch, prefetch_bytes);
   if (seq_len <= 64) return launch_short<4>(a, s);
   if (seq_len <= 128) return launch_short<8>(a, s);
   if (seq_len <= 256) return launch_short<16>(a, s);
@@ -643,14 +693,14 @@ extern "C" int bt_attention_grouped(const void *qkv_heads, void *attention_outpu
   const long long blocks128 = (long long)((seq_len + 127) / 128) * head_num * batch_size;
   const int qb = option_attention_qb();
   if (qb == 2 || (qb < 0 && blocks128 >= 512)) {
-    dim3 grid((seq_len + 127) / 128, head_num, batch_size);
+    const unsigned grid = att_grid(a, (seq_len + 127) / 128);
     set_prefetch(a, grid, prefetch, prefetch_bytes);
     if (a.mask || a.bias)
       attention_grouped_kernel<2, true><<<grid, kAttThreads, 0, s>>>(a);
     else
       attention_grouped_kernel<2, false><<<grid, kAttThreads, 0, s>>>(a);
   } else {
-    dim3 grid((seq_len + 63) / 64, head_num, batch_size);
+    const unsigned grid = att_grid(a, (seq_len + 63) / 64);
     set_prefetch(a, grid, prefetch, prefetch_bytes);
     if (a.mask || a.bias)
       attention_grouped_kernel<1, true><<<grid, kAttThreads, 0, s>>>(a);

@@ -31,10 +31,13 @@ namespace {
 constexpr float kLog2eF = 1.4426950408889634f;
 constexpr float kDeadLogit = -1.0e30f;
 
-__device__ __forceinline__ float gelu_tanh_exact(float x) {
+__device__ __forceinline__ float gelu_tanh(float x) {
   // 0.5 x (1 + tanh(u)) == x / (1 + exp(-2u)),  u = 0.79788456 (x + 0.044715 x^3)
-  const float u = 0.7978845608028654f * (x + 0.044715f * x * x * x);
-  return x / (1.0f + __expf(-2.0f * u));
+  // exponent folded into one polynomial: -2 u log2(e) = x (c1 + c3 x^2)
+  constexpr float c1 = -2.0f * 0.7978845608028654f * 1.4426950408889634f;
+  constexpr float c3 = c1 * 0.044715f;
+  const float e = __builtin_amdgcn_exp2f(x * (c1 + c3 * x * x));
+  return x * __builtin_amdgcn_rcpf(1.0f + e);
 }
 
 // ---------------------------------------------------------------------------
@@ -52,16 +55,19 @@ struct F32GemmArgs {
 };
 
 constexpr int kF32BK = 16;
+constexpr int kF32CUs = 256;
 
-// 256 threads = 2 x 2 waves, each wave a (BM/2) x (BN/2) block of 32x32 MFMA tiles.
+// WGM x WGN waves, each a (BM/WGM) x (BN/WGN) block of 32x32 MFMA tiles.
 // LDS: A tile k-major [16][BM+4] (the gather / transposition happens in the store),
 // W tile [16][BN+32]; both strides make the operand reads of one wave conflict free.
-template <int BM, int BN>
-__global__ __launch_bounds__(256) void f32_gemm_kernel(F32GemmArgs p) {
+template <int BM, int BN, int WGM, int WGN>
+__global__ __launch_bounds__(64 * WGM *WGN) void f32_gemm_kernel(F32GemmArgs p) {
+  constexpr int THREADS = 64 * WGM * WGN;
   constexpr int SA = BM + 4, SW = BN + 32;
-  constexpr int WM = BM / 2, WN = BN / 2, MT = WM / 32, NT = WN / 32;
-  constexpr int AV = BM / 64;          // float4 of A per thread and k-tile
-  constexpr int WV = BN / 64;          // float4 of W per thread and k-tile
+  constexpr int WM = BM / WGM, WN = BN / WGN, MT = WM / 32, NT = WN / 32;
+  constexpr int AV = BM * 4 / THREADS;     // float4 of A per thread and k-tile
+  constexpr int WV = BN * 4 / THREADS;     // float4 of W per thread and k-tile
+  static_assert(MT >= 1 && NT >= 1 && AV >= 1 && WV >= 1, "tile too small for the wave grid");
   __shared__ float sA[2][kF32BK * SA];
   __shared__ __attribute__((aligned(16))) float sW[2][kF32BK * SW];
 
@@ -71,22 +77,23 @@ __global__ __launch_bounds__(256) void f32_gemm_kernel(F32GemmArgs p) {
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int l32 = lane & 31, half = lane >> 5;
-  const int wm = wave >> 1, wn = wave & 1;
+  const int wm = wave / WGN, wn = wave % WGN;
 
   // global -> register staging
   const int a_kq = tid & 3;            // which float4 of the 16 k
+  constexpr int AROWS = THREADS / 4;   // tile rows covered by one pass of the workgroup
   const float *a_src[AV];
 #pragma unroll
   for (int i = 0; i < AV; ++i) {
-    const int r = m0 + (tid >> 2) + i * 64;
+    const int r = m0 + (tid >> 2) + i * AROWS;
     a_src[i] = nullptr;
     if (r < M) {
       const size_t row = p.a_row_index ? (size_t)p.a_row_index[r] : (size_t)r;
       a_src[i] = p.a + row * p.K + 4 * a_kq;
     }
   }
-  constexpr int WPR = BN / 4;          // float4 per W tile row
-  constexpr int WROWS = 256 / WPR;     // tile rows covered by one pass of the workgroup
+  constexpr int WPR = BN / 4;            // float4 per W tile row
+  constexpr int WROWS = THREADS / WPR;   // tile rows covered by one pass of the workgroup
   const int w_k = tid / WPR, w_n = n0 + 4 * (tid % WPR);
   const bool w_ok = w_n < p.N;
 
@@ -107,7 +114,7 @@ __global__ __launch_bounds__(256) void f32_gemm_kernel(F32GemmArgs p) {
   auto stash = [&](int buf) {
 #pragma unroll
     for (int i = 0; i < AV; ++i) {
-      float *d = &sA[buf][(4 * a_kq) * SA + (tid >> 2) + i * 64];
+      float *d = &sA[buf][(4 * a_kq) * SA + (tid >> 2) + i * AROWS];
 #pragma unroll
       for (int j = 0; j < 4; ++j) d[j * SA] = ra[i][j];
     }
@@ -133,19 +140,26 @@ __global__ __launch_bounds__(256) void f32_gemm_kernel(F32GemmArgs p) {
     if (kt + 1 < nk) fetch((kt + 1) * kF32BK);
     const float *a_base = &sA[cur][half * SA + wm * WM + l32];
     const float *w_base = &sW[cur][half * SW + wn * WN + l32];
+    // all operand fetches of the k-tile first, the MFMA chain after them: the fence keeps
+    // the compiler from sinking each ds_read next to its MFMA (which exposes the LDS
+    // latency once per MFMA pair instead of once per k-tile)
+    float af[kF32BK / 2][MT], bf[kF32BK / 2][NT];
 #pragma unroll
     for (int kk = 0; kk < kF32BK / 2; ++kk) {
-      float af[MT], bf[NT];
 #pragma unroll
-      for (int mt = 0; mt < MT; ++mt) af[mt] = a_base[2 * kk * SA + mt * 32];
+      for (int mt = 0; mt < MT; ++mt) af[kk][mt] = a_base[2 * kk * SA + mt * 32];
 #pragma unroll
-      for (int nt = 0; nt < NT; ++nt) bf[nt] = w_base[2 * kk * SW + nt * 32];
+      for (int nt = 0; nt < NT; ++nt) bf[kk][nt] = w_base[2 * kk * SW + nt * 32];
+    }
+    asm volatile("" ::: "memory");
+#pragma unroll
+    for (int kk = 0; kk < kF32BK / 2; ++kk)
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt)
-          acc[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[mt], bf[nt], acc[mt][nt], 0, 0, 0);
-    }
+          acc[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[kk][mt], bf[kk][nt], acc[mt][nt],
+                                                             0, 0, 0);
     if (kt + 1 < nk) stash(cur ^ 1);
     __syncthreads();
     cur ^= 1;
@@ -164,7 +178,7 @@ __global__ __launch_bounds__(256) void f32_gemm_kernel(F32GemmArgs p) {
         const int row = m0 + wm * WM + mt * 32 + 8 * (i >> 2) + 4 * half + (i & 3);
         if (row >= M) continue;
         float v = acc[mt][nt][i] + bv;
-        if (p.gelu) v = gelu_tanh_exact(v);
+        if (p.gelu) v = gelu_tanh(v);
         p.c[(size_t)row * p.N + col] = v;
       }
   }
@@ -177,42 +191,52 @@ struct F32AttArgs {
   const float *qkv;    // [rows, 3H], QKV bias already added
   float *out;          // [rows, H]
   const int *batch_idx;
+  const int *seq_order;   // optional: rank -> sequence, longest first
   const float *mask;   // optional [B,S,S]
   const float *bias;   // optional [heads,S,S]
   int B, S, rows_cap, heads;
   float scale;
   int padded_rows;
+  int nqb;             // query tiles per sequence
 };
 
 constexpr int kF32KT = 32;   // keys per tile
-constexpr int kF32BQ = 128;  // queries per workgroup (32 per wave)
 
-// One workgroup = 128 queries of one (sequence, head).  The logits are computed
+// One workgroup = NW waves x 32 queries of one (sequence, head).  The logits are computed
 // transposed, S^T = K.Q^T (lane = query, 16 keys per lane), so their accumulator is
 // directly the "B" operand of O^T = V^T.P^T and the softmax statistics of a query are
 // lane-local up to one exchange between the two halves of the wave.  The MFMA's k index
 // may be any bijection as long as both operands agree; it is chosen so that Q and K are
 // read as float4 (k = half*D/2 + step) and P needs no shuffle (key of step j in half h
 // = 8*(j/4) + 4*h + j%4, the accumulator's own row order).
-template <int ND>
-__global__ __launch_bounds__(256) void f32_attention_kernel(F32AttArgs p) {
+template <int ND, int NW>
+__global__ __launch_bounds__(64 * NW) void f32_attention_kernel(F32AttArgs p) {
   constexpr int D = 32 * ND;
+  constexpr int THREADS = 64 * NW, BQ = 32 * NW;   // 32 queries per wave
   constexpr int SK = D + 4, SV = D + 8;
   __shared__ __attribute__((aligned(16))) float sK[kF32KT * SK];
   __shared__ __attribute__((aligned(16))) float sV[kF32KT * SV];
 
-  const int b = blockIdx.z, head = blockIdx.y;
+  // 1-D grid, XCD-aware: the hardware deals consecutive workgroup ids round-robin to the
+  // 8 XCDs; XCD x works on the (sequence, head) pairs p = x (mod 8), the query tiles of
+  // one pair back to back (its K / V then come from that XCD's L2), so every XCD sees the
+  // same mix of sequence lengths however ragged the batch is.
+  const unsigned lin = blockIdx.x, slot = lin >> 3;
+  const unsigned pair = (slot / p.nqb) * 8 + (lin & 7);
+  if (pair >= (unsigned)(p.B * p.heads)) return;
+  const int rank = pair / p.heads, head = pair % p.heads;
+  const int b = p.seq_order ? p.seq_order[rank] : rank;
   const int seq_start = p.batch_idx[b];
   const int len = p.batch_idx[b + 1] - seq_start;
   const int klen = (p.mask && p.padded_rows) ? p.S : len;
   const int row_start = p.padded_rows ? b * p.S : seq_start;
   const int nq = p.padded_rows ? p.S : len;
-  const int q0 = blockIdx.x * kF32BQ;
+  const int q0 = (int)(slot % p.nqb) * BQ;
   if (q0 >= nq || klen <= 0) {
     // padded rows of an empty sequence still get defined output: zeros
     if (q0 < nq) {
       const int H = p.heads * D;
-      for (int i = threadIdx.x; i < kF32BQ * D; i += 256) {
+      for (int i = threadIdx.x; i < BQ * D; i += THREADS) {
         const int q = q0 + i / D;
         if (q < nq) p.out[(size_t)(row_start + q) * H + head * D + i % D] = 0.f;
       }
@@ -241,13 +265,14 @@ __global__ __launch_bounds__(256) void f32_attention_kernel(F32AttArgs p) {
     for (int j = 0; j < 4; ++j) qf[4 * i + j] = v[j];
   }
 
-  // tile staging: 32 keys x D floats of K and of V, ND float4 each per thread
+  // tile staging: 32 keys x D floats of K and of V, NV float4 each per thread
   constexpr int CPR = D / 4;   // float4 per row
-  float4_t rk[ND], rv[ND];
+  constexpr int NV = kF32KT * CPR / THREADS;
+  float4_t rk[NV], rv[NV];
   auto fetch = [&](int k0) {
 #pragma unroll
-    for (int i = 0; i < ND; ++i) {
-      const int idx = tid + 256 * i;
+    for (int i = 0; i < NV; ++i) {
+      const int idx = tid + THREADS * i;
       const int key = min(k0 + idx / CPR, klen - 1);
       const size_t off = (size_t)key * ld + 4 * (idx % CPR);
       rk[i] = *(const float4_t *)(K + off);
@@ -256,8 +281,8 @@ __global__ __launch_bounds__(256) void f32_attention_kernel(F32AttArgs p) {
   };
   auto stash = [&]() {
 #pragma unroll
-    for (int i = 0; i < ND; ++i) {
-      const int idx = tid + 256 * i;
+    for (int i = 0; i < NV; ++i) {
+      const int idx = tid + THREADS * i;
       *(float4_t *)&sK[(idx / CPR) * SK + 4 * (idx % CPR)] = rk[i];
       *(float4_t *)&sV[(idx / CPR) * SV + 4 * (idx % CPR)] = rv[i];
     }
@@ -278,10 +303,35 @@ __global__ __launch_bounds__(256) void f32_attention_kernel(F32AttArgs p) {
   fetch(0);
   stash();
   __syncthreads();
+  const bool has_add = mrow || brow;
+  const bool add_vec = (p.S & 3) == 0;
   for (int t = 0; t < ntiles; ++t) {
+    const int k0 = t * kF32KT;
+    // additive terms of this tile's 16 keys per lane (4 groups of 4 consecutive keys),
+    // in the exp2 domain; issued ahead of the next tile's K / V so that the wait for
+    // them does not include those
+    float4_t add[4];
+    if (has_add && wave_live) {
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const int key = k0 + 8 * g + 4 * half;
+        float4_t mv = {1.f, 1.f, 1.f, 1.f}, bv = {0.f, 0.f, 0.f, 0.f};
+        if (add_vec && key + 3 < p.S) {
+          if (mrow) mv = *(const float4_t *)(mrow + key);
+          if (brow) bv = *(const float4_t *)(brow + key);
+        } else {
+#pragma unroll
+          for (int r = 0; r < 4; ++r)
+            if (key + r < p.S) {
+              if (mrow) mv[r] = mrow[key + r];
+              if (brow) bv[r] = brow[key + r];
+            }
+        }
+        add[g] = (mv - 1.0f) * (10000.0f * kLog2eF) + bv * kLog2eF;
+      }
+    }
     if (t + 1 < ntiles) fetch((t + 1) * kF32KT);
     if (wave_live) {
-      const int k0 = t * kF32KT;
       // S^T = K . Q^T : A operand K[key = l32][k = half*D/2 + i]
       float16_t s;
 #pragma unroll
@@ -301,12 +351,8 @@ __global__ __launch_bounds__(256) void f32_attention_kernel(F32AttArgs p) {
       for (int i = 0; i < 16; ++i) {
         const int key = k0 + 8 * (i >> 2) + 4 * half + (i & 3);
         float v = s[i] * c;
-        if (key < klen) {
-          if (brow) v += brow[key] * kLog2eF;
-          if (mrow) v += (mrow[key] - 1.0f) * (10000.0f * kLog2eF);
-        } else {
-          v = kDeadLogit;
-        }
+        if (has_add) v += add[i >> 2][i & 3];
+        if (key >= klen) v = kDeadLogit;
         x[i] = v;
         tmax = fmaxf(tmax, v);
       }
@@ -323,10 +369,14 @@ __global__ __launch_bounds__(256) void f32_attention_kernel(F32AttArgs p) {
         psum += pv;
       }
       l_run = l_run * alpha + psum;
+      // the running maximum of most queries settles after a few tiles: skip the rescale
+      // of the accumulators when it moved for no query of the wave
+      if (__any(alpha != 1.0f)) {
 #pragma unroll
-      for (int dt = 0; dt < ND; ++dt)
+        for (int dt = 0; dt < ND; ++dt)
 #pragma unroll
-        for (int i = 0; i < 16; ++i) o[dt][i] *= alpha;
+          for (int i = 0; i < 16; ++i) o[dt][i] *= alpha;
+      }
       // O^T += V^T . P^T : A operand V[key(j, half)][d = 32*dt + l32], B operand P^T = x[j]
 #pragma unroll
       for (int j = 0; j < 16; ++j) {
@@ -458,8 +508,8 @@ int launch_f32_ln(const void *src, const void *residual, const void *bias, const
 using namespace bt;
 
 extern "C" int bt_gemm_f32(const void *a, const int *a_row_index, const void *w, const void *bias,
-                           void *c, int gelu, const int *valid_rows, int rows_cap, int n, int k,
-                           void *stream) {
+                           void *c, int gelu, const int *valid_rows, int rows_cap, int rows_hint,
+                           int n, int k, void *stream) {
   BT_REQUIRE(a && w && c, BT_ERR_INVALID_ARGUMENT, "bt_gemm_f32: null pointer argument");
   BT_REQUIRE(rows_cap >= 0 && n > 0 && k > 0, BT_ERR_INVALID_ARGUMENT,
              "bt_gemm_f32: sizes must be positive");
@@ -472,23 +522,43 @@ extern "C" int bt_gemm_f32(const void *a, const int *a_row_index, const void *w,
   if (rows_cap == 0) return BT_OK;
   F32GemmArgs p{(const float *)a, (const float *)w, (const float *)bias, (float *)c, valid_rows,
                 a_row_index, rows_cap, n, k, gelu ? 1 : 0};
-  // 128x128 tiles once they fill the chip; 64x64 below that
-  const long long big = (long long)((rows_cap + 127) / 128) * ((n + 127) / 128);
-  if (big >= 192) {
-    dim3 grid((n + 127) / 128, (rows_cap + 127) / 128);
-    BT_REQUIRE(grid.y <= 65535, BT_ERR_UNSUPPORTED, "bt_gemm_f32: too many rows");
-    f32_gemm_kernel<128, 128><<<grid, 256, 0, as_stream(stream)>>>(p);
-  } else {
-    dim3 grid((n + 63) / 64, (rows_cap + 63) / 64);
-    BT_REQUIRE(grid.y <= 65535, BT_ERR_UNSUPPORTED, "bt_gemm_f32: too many rows");
-    f32_gemm_kernel<64, 64><<<grid, 256, 0, as_stream(stream)>>>(p);
+  // Tile table: 0: 128x128, 8 waves | 1: 128x64, 4 waves | 2: 64x64, 4 waves.
+  // Choice by a two-term model per k-tile of 16: a workgroup alone on its CU needs
+  // `alone` us (latency bound), a CU shared by b workgroups needs b * `shared` us (MFMA
+  // bound); b = ceil(workgroups / CUs).  Constants measured on MI355X.
+  struct Cand { int id, bm, bn; float alone, shared; };
+  static const Cand cands[3] = {{0, 128, 128, 1.20f, 1.15f}, {1, 128, 64, 0.76f, 0.60f},
+                                {2, 64, 64, 0.49f, 0.31f}};
+  int tile = option_f32_gemm_tile();
+  if (tile < 0) {
+    // the row count that matters is the live one; the hint is the caller's estimate of it
+    const int rows = (valid_rows && rows_hint > 0 && rows_hint < rows_cap) ? rows_hint : rows_cap;
+    float best = 0.f;
+    for (const Cand &cd : cands) {
+      const long long wgs = (long long)((rows + cd.bm - 1) / cd.bm) * ((n + cd.bn - 1) / cd.bn);
+      const float b = (float)((wgs + kF32CUs - 1) / kF32CUs);
+      const float cost = fmaxf(cd.alone, b * cd.shared);
+      if (tile < 0 || cost < best) {
+        best = cost;
+        tile = cd.id;
+      }
+    }
+  }
+  const int bm = cands[tile].bm, bn = cands[tile].bn;
+  dim3 grid((n + bn - 1) / bn, (rows_cap + bm - 1) / bm);
+  BT_REQUIRE(grid.y <= 65535, BT_ERR_UNSUPPORTED, "bt_gemm_f32: too many rows");
+  hipStream_t s = as_stream(stream);
+  switch (tile) {
+    case 0: f32_gemm_kernel<128, 128, 4, 2><<<grid, 512, 0, s>>>(p); break;
+    case 1: f32_gemm_kernel<128, 64, 2, 2><<<grid, 256, 0, s>>>(p); break;
+    default: f32_gemm_kernel<64, 64, 2, 2><<<grid, 256, 0, s>>>(p); break;
   }
   BT_CHECK_LAUNCH("bt_gemm_f32");
   return BT_OK;
 }
 
 extern "C" int bt_attention_f32(const void *qkv, void *out, const int *batch_idx,
-                                const void *atten_mask, const void *attention_bias,
+                                const int *seq_order, const void *atten_mask, const void *attention_bias,
                                 int batch_size, int seq_len, int rows_cap, int head_num,
                                 int size_per_head, float scale, int padded_rows, void *stream) {
   BT_REQUIRE(qkv && out && batch_idx, BT_ERR_INVALID_ARGUMENT,
@@ -502,17 +572,21 @@ extern "C" int bt_attention_f32(const void *qkv, void *out, const int *batch_idx
              "bt_attention_f32: batch_size / head_num exceed the grid limit");
   BT_REQUIRE(!padded_rows || (long long)batch_size * seq_len <= rows_cap, BT_ERR_INVALID_ARGUMENT,
              "bt_attention_f32: padded rows need rows_cap >= batch_size * seq_len");
-  F32AttArgs p{(const float *)qkv, (float *)out, batch_idx, (const float *)atten_mask,
+  F32AttArgs p{(const float *)qkv, (float *)out, batch_idx, seq_order, (const float *)atten_mask,
                (const float *)attention_bias, batch_size, seq_len, rows_cap, head_num, scale,
                padded_rows ? 1 : 0};
-  dim3 grid((seq_len + kF32BQ - 1) / kF32BQ, head_num, batch_size);
   hipStream_t s = as_stream(stream);
+  constexpr int kWaves = 4;    // 128 queries per workgroup (two-wave workgroups measured slower)
+  p.nqb = (seq_len + 32 * kWaves - 1) / (32 * kWaves);
+  const unsigned grid = ((unsigned)batch_size * head_num + 7) / 8 * 8 * p.nqb;
+#define BT_F32_ATT(ND_) f32_attention_kernel<ND_, kWaves><<<grid, 64 * kWaves, 0, s>>>(p)
   if (size_per_head == 32)
-    f32_attention_kernel<1><<<grid, 256, 0, s>>>(p);
+    BT_F32_ATT(1);
   else if (size_per_head == 64)
-    f32_attention_kernel<2><<<grid, 256, 0, s>>>(p);
+    BT_F32_ATT(2);
   else
-    f32_attention_kernel<4><<<grid, 256, 0, s>>>(p);
+    BT_F32_ATT(4);
+#undef BT_F32_ATT
   BT_CHECK_LAUNCH("bt_attention_f32");
   return BT_OK;
 }

@@ -30,6 +30,10 @@ int hip_fail(hipError_t e, const char *what) {
 static std::atomic<int> g_gemm_tile{-1};
 static std::atomic<int> g_attention_qb{-1};
 static std::atomic<int> g_prefetch{1};
+static std::atomic<int> g_f32_gemm_tile{-1};
+static std::atomic<int> g_attention_xcd_map{1};
+int option_attention_xcd_map() { return g_attention_xcd_map.load(std::memory_order_relaxed); }
+int option_f32_gemm_tile() { return g_f32_gemm_tile.load(std::memory_order_relaxed); }
 int option_gemm_tile() { return g_gemm_tile.load(std::memory_order_relaxed); }
 int option_attention_qb() { return g_attention_qb.load(std::memory_order_relaxed); }
 int option_prefetch() { return g_prefetch.load(std::memory_order_relaxed); }
@@ -136,6 +140,14 @@ extern "C" int bt_set_option(const char *name, int value) {
     BT_REQUIRE(value == -1 || value == 1 || value == 2, BT_ERR_INVALID_ARGUMENT,
                "bt_set_option: attention_qb=%d must be -1, 1 or 2", value);
     g_attention_qb.store(value);
+  } else if (!strcmp(name, "f32_gemm_tile")) {
+    BT_REQUIRE(value >= -1 && value <= 2, BT_ERR_INVALID_ARGUMENT,
+               "bt_set_option: f32_gemm_tile=%d outside [-1, 2]", value);
+    g_f32_gemm_tile.store(value);
+  } else if (!strcmp(name, "attention_xcd_map")) {
+    BT_REQUIRE(value == 0 || value == 1, BT_ERR_INVALID_ARGUMENT,
+               "bt_set_option: attention_xcd_map=%d must be 0 or 1", value);
+    g_attention_xcd_map.store(value);
   } else if (!strcmp(name, "prefetch")) {
     BT_REQUIRE(value == 0 || value == 1, BT_ERR_INVALID_ARGUMENT,
                "bt_set_option: prefetch=%d must be 0 or 1", value);

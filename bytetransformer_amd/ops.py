@@ -180,7 +180,7 @@ def _need_f32(*ts):
 
 
 def gemm_f32(a, w, bias=None, gelu=False, valid_rows=None, a_row_index=None, rows_cap=None,
-             out=None):
+             out=None, rows_hint=0):
     """c = a . w (+ bias) (+ tanh-GELU); w is [K, N] as stored."""
     _need_f32(a, w, bias, out)
     rows = a.shape[0] if rows_cap is None else rows_cap
@@ -188,12 +188,13 @@ def gemm_f32(a, w, bias=None, gelu=False, valid_rows=None, a_row_index=None, row
     if out is None:
         out = torch.zeros(rows, N, dtype=a.dtype, device=a.device)
     _check(kernel_lib().bt_gemm_f32(_ptr(a), _ptr(a_row_index), _ptr(w), _ptr(bias), _ptr(out),
-                                    int(gelu), _ptr(valid_rows), rows, N, K, _stream()))
+                                    int(gelu), _ptr(valid_rows), rows, int(rows_hint), N, K,
+                                    _stream()))
     return out
 
 
 def attention_f32(qkv, batch_idx, batch_size, seq_len, head_num, scale, padded_rows=False,
-                  mask=None, bias=None, out=None):
+                  mask=None, bias=None, out=None, seq_order=None):
     """qkv [rows, 3 * hidden] (bias added) -> [rows, hidden]."""
     _need_f32(qkv, mask, bias, out)
     rows_cap, three_h = qkv.shape
@@ -202,7 +203,8 @@ def attention_f32(qkv, batch_idx, batch_size, seq_len, head_num, scale, padded_r
         out = torch.zeros(rows_cap, hidden, dtype=qkv.dtype, device=qkv.device)
     if bias is not None and tuple(bias.shape) != (head_num, seq_len, seq_len):
         raise ValueError("attention bias must be [head_num, seq_len, seq_len]")
-    _check(kernel_lib().bt_attention_f32(_ptr(qkv), _ptr(out), _ptr(batch_idx), _ptr(mask),
+    _check(kernel_lib().bt_attention_f32(_ptr(qkv), _ptr(out), _ptr(batch_idx), _ptr(seq_order),
+                                         _ptr(mask),
                                          _ptr(bias), batch_size, seq_len, rows_cap, head_num,
                                          hidden // head_num, float(scale), int(padded_rows),
                                          _stream()))

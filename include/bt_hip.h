@@ -50,6 +50,8 @@ const char *bt_last_error_string(void);
  *                   waves | 2: 256x128, 8 + 4 waves | 3: 256x192, 8 waves | 4: 32x64, 2 + 2 waves
  *   "attention_qb"  -1 heuristic | 1 | 2: 16-query blocks per wave in the grouped kernel
  *   "prefetch"      1 (default) | 0: honour / ignore the prefetch hint of the attention entries
+ *   "f32_gemm_tile" -1 heuristic | 0: 128x128 tile, 8 waves | 1: 128x64, 4 waves | 2: 64x64, 4 waves
+ *                   (bt_gemm_f32 only)
  * Process-wide; results do not depend on it beyond fp32 summation order.
  */
 int bt_set_option(const char *name, int value);
@@ -218,13 +220,15 @@ int bt_add_bias_residual_layernorm_restore(const void *out, const void *residual
  *
  * bt_gemm_f32: c[M, n] = a[M, k] . w[k, n] (+ bias[n]) (then tanh-GELU when gelu != 0,
  * which needs a bias).  a_row_index (nullable, needs valid_rows): row r of A is
- * a[a_row_index[r], :].  n % 4 == 0, k % 4 == 0.  Replaces the cuBLAS calls of
+ * a[a_row_index[r], :].  rows_hint: expected live rows or 0, steers the tile shape only.
+ * n % 4 == 0, k % 4 == 0.  Replaces the cuBLAS calls of
  * dense_layer_kernel_launcher<float> (bytetransformer/src/gemm.cu:32-39), the QKV bias
  * add of add_QKV_bias (attention_nofused_utils.cu:143-184) and
  * gemm_bias_gelu<float> (gemm_bias_act.cu:24-75).
  */
 int bt_gemm_f32(const void *a, const int *a_row_index, const void *w, const void *bias, void *c,
-                int gelu, const int *valid_rows, int rows_cap, int n, int k, void *stream);
+                int gelu, const int *valid_rows, int rows_cap, int rows_hint, int n, int k,
+                void *stream);
 
 /*
  * Fused multi-head attention on float, token-major projections qkv [rows, 3 * hidden]
@@ -235,10 +239,11 @@ int bt_gemm_f32(const void *a, const int *a_row_index, const void *w, const void
  * Attention<FP32>::nofused_infer (attention_nofused.cu:27-114) without its logits
  * buffer.  atten_mask (nullable, float [B,S,S]) is applied on both row layouts; keys at
  * or past the sequence length are excluded by index on packed rows (they do not exist
- * there) and, without a mask, on padded rows.  size_per_head in {32, 64, 128}.
+ * there) and, without a mask, on padded rows.  seq_order (nullable) as in the fp16
+ * entries: issue order only.  size_per_head in {32, 64, 128}.
  */
 int bt_attention_f32(const void *qkv, void *attention_output, const int *batch_idx,
-                     const void *atten_mask, const void *attention_bias, int batch_size,
+                     const int *seq_order, const void *atten_mask, const void *attention_bias, int batch_size,
                      int seq_len, int rows_cap, int head_num, int size_per_head, float scale,
                      int padded_rows, void *stream);
 

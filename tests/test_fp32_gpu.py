@@ -192,8 +192,14 @@ def test_attention_f32(device, lens, S, heads, d, padded):
     qkv[:, :H] *= 2.0
     scale = 1 / math.sqrt(d)
     exp = _naive_attention(qkv, lens, S, heads, d, scale, padded)
+    # the issue order (longest first) must not change anything
+    order = np.argsort(-np.asarray(lens), kind="stable").astype(np.int32)
     g = ops.attention_f32(_dev(qkv, device), _dev(bi, device), B, S, heads, scale,
-                          padded_rows=padded).cpu().numpy()
+                          padded_rows=padded, seq_order=_dev(order, device)).cpu().numpy()
+    g0 = ops.attention_f32(_dev(qkv, device), _dev(bi, device), B, S, heads, scale,
+                           padded_rows=padded).cpu().numpy()
+    live = ~np.isnan(g0)
+    assert np.array_equal(np.isnan(g), ~live) and np.array_equal(g[live], g0[live])
     for b, n in enumerate(lens):
         r0 = b * S if padded else bi[b]
         # padded rows: queries past the length attend the valid keys too (defined output)
