@@ -264,6 +264,27 @@ def main():
         "whole_encoder_graph_ms": timed(graphed.replay),
     }
 
+    # OperationType::FP32: the same batch and weights as float tensors (float kernels
+    # throughout), a few steps only - reported beside the headline, never as `value`
+    layers32 = [[w.float() for w in ws] for ws in layers]
+    x32, mask32 = x.float(), mask.float()
+
+    def forward32():
+        h = x32
+        for w in layers32:
+            h = op(cfg.head_num, cfg.head_size, *w, h, mask32, True, True)
+        return h
+
+    forward32()
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    n32 = max(1, min(args.steps, 10))
+    for _ in range(n32):
+        forward32()
+    torch.cuda.synchronize()
+    other["float_th_op_ms"] = round((time.perf_counter() - t1) * 1e3 / n32, 4)
+    del layers32, x32, mask32
+
     gemm_f, attn_f = workload.layer_flops(cfg, wl.lens)
     kernels = kernel_table(wl, dev, args.kernel_iters)
     dominant = max((k for k in kernels if kernels[k]["bound"] == "mfma"),

@@ -303,6 +303,7 @@ __global__ __launch_bounds__(kAttThreads, 2) void attention_grouped_kernel(AttAr
   }
   const half8_t ones = {1, 1, 1, 1, 1, 1, 1, 1};
 
+  const bool wave_live = q0 + wave * QB * 16 < nq;
   const int ntiles = (klen + kKT - 1) / kKT;
   if (ntiles > 0) issue_tile(0, 0);
   if (ntiles > 1) issue_tile(1, 1);
@@ -327,6 +328,11 @@ __global__ __launch_bounds__(kAttThreads, 2) void attention_grouped_kernel(AttAr
       int ps = stage + 2;
       if (ps >= kAttStages) ps -= kAttStages;
       issue_tile(t + 2, ps);
+    }
+    // a wave whose queries all lie past the sequence only copies and keeps the barriers
+    if (!wave_live) {
+      if (++stage == kAttStages) stage = 0;
+      return;
     }
     const half_t *sK = ring + stage * 2 * kTileHalfs;
     const half_t *sV = sK + kTileHalfs;
@@ -507,6 +513,11 @@ __global__ __launch_bounds__(kAttThreads) void attention_short_kernel(AttArgs p)
   att_wait_vmcnt<0>();
   asm volatile("" ::: "memory");
   __syncthreads();
+  // no barrier follows: a wave whose 16 queries all lie past the sequence is done
+  if (q0 + wave * 16 >= nq) {
+    prefetch_slice(p);
+    return;
+  }
 
   const int nkb = keys32 >> 4;  // even
   float4_t s[NKB];
