@@ -147,6 +147,13 @@ def kernel_table(wl, dev, iters):
     rows.append(("copy_calibration_64MiB",
                  lambda: ops.compress(calib_src, c_bi, c_wi, out=calib_dst), "hbm",
                  2 * calib_src.numel() * 2))
+    # The memory-bound kernels at a size where the launch cost (a few us, the same for
+    # a plain copy) no longer dominates: 16x the rows of the workload.
+    big = 16 * T
+    big_out = torch.empty(big, H, dtype=torch.float16, device=dev).normal_()
+    big_res = torch.empty(big, H, dtype=torch.float16, device=dev).normal_()
+    rows.append(("layernorm_16x_rows", lambda: ops.add_bias_residual_layernorm(
+        big_out, big_res, w["attr_output_bias"], g1, b1), "hbm", 3 * big * H * 2))
     table = {}
     for name, fn, bound, work in rows:
         ms = time_kernel(fn, iters)

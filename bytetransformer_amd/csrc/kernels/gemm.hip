@@ -384,6 +384,68 @@ static int launch_gemm_tile(GemmArgs p, hipStream_t s) {
   return BT_OK;
 }
 
+static int cu_count() {
+  static const int cus = [] {
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
+        n <= 0)
+      n = 256;
+    return n;
+  }();
+  return cus;
+}
+
+// Live rows the tile choice is made for: the exact count when every row is live, the
+// caller's hint when it has one, else 60 % of the capacity (the fill the padding-free
+// path is built for).
+static long long estimated_rows(const GemmArgs &p) {
+  if (!p.valid_rows) return p.rows_cap;
+  if (p.rows_hint > 0) return p.rows_hint < p.rows_cap ? p.rows_hint : p.rows_cap;
+  return (p.rows_cap * 3LL + 4) / 5;
+}
+
+#include "gemm_tuned.inc"
+
+// Measured time of tile t between two table rows (0 = not measured at one of them).
+static float tuned_time(const float *lo, const float *hi, float w, int t) {
+  if (t < 0 || t >= kTunedTiles || lo[t] <= 0.f || hi[t] <= 0.f) return 0.f;
+  return lo[t] + (hi[t] - lo[t]) * w;
+}
+
+// Tile with the smallest measured time for this weight shape at m rows, times
+// interpolated linearly between the measured row counts; -1 when the shape is not in
+// the table or m lies beyond it (the analytic model then decides).
+static int tuned_choice(long long m, int n, int k, int epi, const float **row_lo,
+                        const float **row_hi, float *weight) {
+  if (cu_count() != 256) return -1;     // the table was measured on a 256-CU part
+  for (const TunedShape &ts : kTunedShapes) {
+    if (ts.n != n || ts.k != k || ts.epi != epi) continue;
+    // below about a thousand rows a launch is latency bound and a loop of identical
+    // launches says little about the layer sequence: the model decides there
+    if (m > kTunedRows[kTunedPoints - 1] || m < 1024) return -1;
+    int hi = 0;
+    while (hi < kTunedPoints - 1 && kTunedRows[hi] < m) ++hi;
+    const int lo = hi > 0 && kTunedRows[hi] > m ? hi - 1 : hi;
+    const float w = hi == lo ? 0.f
+                             : (float)(m - kTunedRows[lo]) / (float)(kTunedRows[hi] - kTunedRows[lo]);
+    *row_lo = ts.us[lo];
+    *row_hi = ts.us[hi];
+    *weight = w;
+    int best = -1;
+    float best_us = 0.f;
+    for (int t = 0; t < kTunedTiles; ++t) {
+      const float us = tuned_time(ts.us[lo], ts.us[hi], w, t);
+      if (us > 0.f && (best < 0 || us < best_us)) {
+        best = t;
+        best_us = us;
+      }
+    }
+    return best;
+  }
+  return -1;
+}
+
 template <int EPI>
 static int launch_gemm(GemmArgs p, hipStream_t s) {
   // Tile table (rows x cols, ring depth, computing wave grid, loader waves):
@@ -394,23 +456,18 @@ static int launch_gemm(GemmArgs p, hipStream_t s) {
   //                           full wave of 256-wide ones (QKV at hidden 768)
   //   4:  32x64,  4, 1x2, 2   a few hundred rows or fewer: the k loop of one tile is the
   //                           whole run time, and a small tile has the shortest k-step
-  // The choice minimises rounds x (k-steps x time of one k-step + fill and epilogue)
-  // with the measured per-shape times below, for the estimated live rows: the exact
-  // count when every row is live, the caller's hint when it has one, else 60 % of
-  // the capacity (the fill the padding-free path is built for).
-  int choice = option_gemm_tile();
+  //   5: 128x128, 2, 2x2, 4   tile 1 with a two-deep ring: 64 KB of LDS, so two workgroups
+  //                           share a CU and one's fill and epilogue hide under the other's
+  //                           k loop; pays when tile 1 would need several rounds
+  // The choice minimises rounds x (k-steps x time of one k-step + fill and epilogue) with
+  // the per-tile constants below, for the estimated live rows; for the weight shapes of
+  // BERT-base and BERT-large a table of measured times (gemm_tuned.inc) then overrides it
+  // where another tile is clearly faster.
+  const int forced = option_gemm_tile();
+  int choice = forced;
   if (choice < 0) {
-    static const int cus = [] {
-      int dev = 0, n = 0;
-      if (hipGetDevice(&dev) != hipSuccess ||
-          hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
-          n <= 0)
-        n = 256;
-      return n;
-    }();
-    const long long m_est = !p.valid_rows ? p.rows_cap
-                            : p.rows_hint > 0 ? (p.rows_hint < p.rows_cap ? p.rows_hint : p.rows_cap)
-                                              : (p.rows_cap * 3LL + 4) / 5;
+    const int cus = cu_count();
+    const long long m_est = estimated_rows(p);
     struct Cand {
       int id, bm, bn;
       float step_us, fixed_us;   // one k-step of one tile; fill + epilogue of one tile
@@ -438,6 +495,18 @@ static int launch_gemm(GemmArgs p, hipStream_t s) {
       }
     }
   }
+  if (forced < 0) {
+    // the table overrides the model only for a clear win: the timings come from a loop
+    // of identical launches, and differences of a few per cent do not carry over to the
+    // layer sequence
+    const float *lo = nullptr, *hi = nullptr;
+    float w = 0.f;
+    const int tuned = tuned_choice(estimated_rows(p), p.N, p.K, EPI, &lo, &hi, &w);
+    if (tuned >= 0 && tuned != choice) {
+      const float t_model = tuned_time(lo, hi, w, choice), t_tuned = tuned_time(lo, hi, w, tuned);
+      if (t_model <= 0.f || t_tuned < 0.96f * t_model) choice = tuned;
+    }
+  }
   switch (choice) {
     case 0:
       return launch_gemm_tile<256, 256, 2, 2, 4, 0, 1, EPI>(p, s);
@@ -447,6 +516,8 @@ static int launch_gemm(GemmArgs p, hipStream_t s) {
       return launch_gemm_tile<256, 192, 2, 4, 2, 0, 1, EPI>(p, s);
     case 4:
       return launch_gemm_tile<32, 64, 4, 1, 2, 2, 0, EPI>(p, s);
+    case 5:
+      return launch_gemm_tile<128, 128, 2, 2, 2, 4, 0, EPI>(p, s);
     default:
       return launch_gemm_tile<128, 128, 3, 2, 2, 4, 0, EPI>(p, s);
   }

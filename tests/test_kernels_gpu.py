@@ -153,7 +153,7 @@ def _gemm_tol(exp, K, amax, wmax):
     return 2.0 ** -10 * np.abs(exp) + 4 * K * 2.0 ** -24 * amax * wmax + 1e-6
 
 
-@pytest.mark.parametrize("tile", [0, 1, 2, 3, 4])
+@pytest.mark.parametrize("tile", [0, 1, 2, 3, 4, 5])
 @pytest.mark.parametrize("rows,M,N,K", [(300, 300, 768, 768), (1000, 777, 2304, 768),
                                         (520, 513, 768, 3072), (64, 1, 136, 64),
                                         (257, 257, 3072, 768)])
@@ -177,7 +177,7 @@ def test_gemm_plain(device, tile, rows, M, N, K):
     assert np.all(g[M:] == 3.0)
 
 
-@pytest.mark.parametrize("tile", [0, 1, 2, 3, 4])
+@pytest.mark.parametrize("tile", [0, 1, 2, 3, 4, 5])
 def test_gemm_bias_gelu(device, tile):
     _say("gemm_bias_gelu", tile)
     rs = np.random.RandomState(tile)
@@ -199,7 +199,7 @@ def test_gemm_bias_gelu(device, tile):
     assert np.all(g[M:] == 0)
 
 
-@pytest.mark.parametrize("tile", [0, 1, 2, 3, 4])
+@pytest.mark.parametrize("tile", [0, 1, 2, 3, 4, 5])
 @pytest.mark.parametrize("heads", [12, 16])
 def test_gemm_qkv_bias_split(device, tile, heads):
     _say("gemm_qkv", tile, heads)
