@@ -52,7 +52,7 @@ void BertEncoder<OpType>::infer(BertEncoderInferParam<DataType_> ip) {
   et_param.word_idx = (int *)(base + off);
   et_param.batch_idx = et_param.word_idx + max_rows;
   et_param.valid_word_num = rows;
-  int *seq_order = et_param.batch_idx + max_rows;
+  int *seq_order = et_param.batch_idx + max_batch_size_ + 1;
   off += align_up((max_rows * 2 + 2 * (unsigned long long)max_batch_size_ + 2) * sizeof(int), 256);
   DataType_ *staging = (DataType_ *)(base + off);      // one layer's weights when none were passed
 

@@ -44,7 +44,7 @@ void BertTransformer<OpType>::bert_infer(BertTransformerInferParam infer_param) 
   et_param.word_idx = (int *)(base + off);
   et_param.batch_idx = et_param.word_idx + max_rows;
   et_param.valid_word_num = rows;
-  int *seq_order = et_param.batch_idx + max_rows;   // int[max_batch_size]
+  int *seq_order = et_param.batch_idx + max_batch_size_ + 1;   // int[max_batch_size]
   off += align_up((max_rows * 2 + 2 * (unsigned long long)max_batch_size_ + 2) * sizeof(int), 256);
   DataType_ *wt_qkv = (DataType_ *)(base + off);
   DataType_ *wt_proj = wt_qkv + (size_t)3 * hidden * hidden;

@@ -88,7 +88,7 @@ class BertEncoder {
 
   // Scratch (elements of DataType_, T = max_batch*max_seq*hidden): [0,3T) qkv heads |
   // [3T,4T) attention out | [4T,5T) projection / LN1 | [5T,6T) packed hidden state |
-  // [6T,(6+mult)T) FFN1 | word_idx int[B*S] | batch_idx int[B*S] | seq order int[B] |
+  // [6T,(6+mult)T) FFN1 | word_idx int[B*S] | batch_idx int[B+1] | seq order int[B] |
   // one layer's pre-packed weights (used only when the caller passes none)
   unsigned long long cal_bufsize() const {
     const unsigned long long rows = (unsigned long long)max_batch_size_ * max_seq_len_;

@@ -308,6 +308,55 @@ def test_ragged_edge_cases(device):
     _check(_run_th_op(wl, device), _oracle(wl), wl.lens, tag="ragged/th_op")
 
 
+@pytest.mark.parametrize("seed", range(48))
+def test_random_small_configurations(device, seed):
+    """Seeded random shapes - batch, sequence length, head count, lengths with zeros and
+    full ones, both dtypes, both row layouts, both attention kernels - one layer each
+    through the C API against the oracle."""
+    rs = np.random.RandomState(1000 + seed)
+    B = int(rs.randint(1, 10))
+    S = int(rs.choice([1, 2, 7, 16, 31, 64, 65, 100, 129, 200, 257, 300]))
+    heads = int(rs.choice([1, 2, 3, 5, 12]))
+    lens = rs.randint(0, S + 1, size=B)
+    lens[rs.randint(B)] = S
+    rm = bool(rs.randint(2))
+    fused = bool(rs.randint(2))
+    dtype = "fp32" if seed % 4 == 3 else "fp16"
+    _say("random", seed, B, S, heads, lens.tolist(), rm, fused, dtype)
+    cfg = workload.EncoderConfig("rnd%d" % seed, B, S, heads, layers=1, dtype=dtype,
+                                 lens=tuple(int(v) for v in lens), seed=seed)
+    wl = workload.make_workload(cfg, bias_std=0.05, random_affine=True)
+    if dtype == "fp32":
+        exp = O.masked_output(O.encoder(wl.x, wl.mask, wl.layers, heads).numpy(), wl.lens)
+    else:
+        exp = _oracle(wl)
+    got = _run_c_api(wl, device, is_remove_padding=rm, use_fused_attention=fused)
+    packed = rm and B > 2          # batches of one or two run on the padded rows
+    if not packed:
+        got = O.masked_output(got, wl.lens)
+    mx, mean, pads_zero = O.parity_metrics(got, exp, wl.lens)
+    _say("parity random/%d: max-abs %.3e mean-abs %.3e" % (seed, mx, mean))
+    assert np.isfinite(np.asarray(got, np.float32)).all()
+    if dtype == "fp32":
+        assert mx <= 2e-4 and mean <= 2e-5, (mx, mean)
+    else:
+        assert mx <= MAX_ABS and mean <= MEAN_ABS, (mx, mean)
+    assert pads_zero
+
+
+@pytest.mark.parametrize("dtype", ["fp16", "fp32"])
+def test_seq_len_one(device, dtype):
+    """seq_len 1: batch_idx has one entry more than there are rows (the scratch carve once
+    let the sequence order overwrite its last entry, the live-row count)."""
+    cfg = workload.EncoderConfig("s1", 6, 1, 12, layers=1, dtype=dtype, lens=(0, 1, 0, 0, 1, 0))
+    wl = workload.make_workload(cfg, bias_std=0.05, random_affine=True)
+    exp = O.masked_output(O.encoder(wl.x.astype(np.float32), wl.mask.astype(np.float32),
+                                    [{k: np.asarray(v, np.float32) for k, v in wl.layers[0].items()}],
+                                    12).numpy(), wl.lens)
+    _check(_run_c_api(wl, device), exp, wl.lens, tag="seq_len 1/" + dtype)
+    _check(_run_th_op(wl, device), exp, wl.lens, tag="seq_len 1/th_op/" + dtype)
+
+
 def test_th_op_prepack_cache_tracks_weight_updates(device):
     """The operator caches the k-contiguous weight copies per tensor object; an
     in-place update of a weight (version counter bump) must be picked up, and a
