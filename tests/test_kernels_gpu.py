@@ -177,6 +177,35 @@ def test_gemm_plain(device, tile, rows, M, N, K):
     assert np.all(g[M:] == 3.0)
 
 
+@pytest.mark.parametrize("seed", range(12))
+def test_gemm_random_shapes_all_tiles_and_auto(device, seed):
+    """Random row counts and n / k at the granularity the entry point accepts (8 and 64),
+    every tile shape and the automatic choice."""
+    rs = np.random.RandomState(300 + seed)
+    rows = int(rs.randint(1, 700))
+    M = int(rs.randint(0, rows + 1))
+    N = 8 * int(rs.randint(1, 130))
+    K = 64 * int(rs.randint(1, 17))
+    _say("gemm random", seed, rows, M, N, K)
+    a = rs.standard_normal((rows, K)).astype(np.float16)
+    a[M:] = np.float16("nan")                       # rows past the live count are never used
+    w = (rs.standard_normal((K, N)) * 0.05).astype(np.float16)
+    exp = O.gemm(a[:M], w)
+    tol = _gemm_tol(exp, K, np.abs(a[:M]).max() if M else 0.0, np.abs(w).max())
+    wt = ops.transpose_weight(_dev(w, device))
+    vr = torch.tensor([M], dtype=torch.int32, device=device)
+    try:
+        for tile in (-1, 0, 1, 2, 3, 4, 5):
+            ops.set_option("gemm_tile", tile)
+            out = torch.full((rows, N), 3.0, dtype=torch.float16, device=device)
+            g = ops.gemm(_dev(a, device), wt, valid_rows=vr, out=out, rows_hint=M).cpu().numpy()
+            err = np.abs(g[:M].astype(np.float64) - exp)
+            assert np.all(err <= tol), (tile, err.max())
+            assert np.all(g[M:] == 3.0), tile
+    finally:
+        ops.set_option("gemm_tile", -1)
+
+
 @pytest.mark.parametrize("tile", [0, 1, 2, 3, 4, 5])
 def test_gemm_bias_gelu(device, tile):
     _say("gemm_bias_gelu", tile)

@@ -344,6 +344,66 @@ def test_random_small_configurations(device, seed):
     assert pads_zero
 
 
+@pytest.mark.parametrize("seed", range(24))
+def test_random_whole_encoder_bias_masks_and_operator(device, seed):
+    """Seeded random stacks of 1-3 layers through the whole-encoder entry and the PyTorch
+    operator: FFN widths 1-4x, optional attention bias, arbitrary 0/1 masks on the padded
+    rows, both dtypes."""
+    rs = np.random.RandomState(5000 + seed)
+    B = int(rs.randint(1, 8))
+    S = int(rs.choice([3, 8, 33, 64, 72, 130, 260]))
+    heads = int(rs.choice([1, 2, 4]))
+    layers = int(rs.randint(1, 4))
+    mult = int(rs.choice([1, 2, 4]))
+    rm = bool(rs.randint(2))
+    fused = bool(rs.randint(2))
+    with_bias = bool(rs.randint(2))
+    dtype = "fp32" if seed % 3 == 2 else "fp16"
+    npdt = np.float32 if dtype == "fp32" else np.float16
+    packed = rm and B > 2
+    lens = rs.randint(0, S + 1, size=B)
+    lens[rs.randint(B)] = S
+    if not packed:
+        lens[:] = S                      # arbitrary masks below: every row is a valid row
+    _say("random stack", seed, B, S, heads, layers, mult, rm, fused, with_bias, dtype, lens.tolist())
+    cfg = workload.EncoderConfig("rs%d" % seed, B, S, heads, layers=layers, ffn_mult=mult,
+                                 dtype=dtype, lens=tuple(int(v) for v in lens), seed=seed)
+    wl = workload.make_workload(cfg, bias_std=0.05, random_affine=True)
+    mask = wl.mask
+    if not packed:
+        mask = (rs.rand(B, S, S) < 0.7).astype(npdt)
+        mask[:, :, 0] = 1                # every query keeps a key
+    bias = (0.5 * rs.standard_normal((heads, S, S))).astype(npdt) if with_bias else None
+    h = torch.from_numpy(wl.x.astype(np.float32))
+    for w in wl.layers:
+        h = O.encoder_layer(h, mask.astype(np.float32),
+                            {k: np.asarray(v, np.float32) for k, v in w.items()}, heads,
+                            attention_bias=None if bias is None else bias.astype(np.float32))
+    exp = O.masked_output(h.numpy(), wl.lens)
+    x, m = _dev(wl.x, device), _dev(mask, device)
+    bd = None if bias is None else _dev(bias, device)
+    enc = bt.BertEncoder(heads, 64, [{k: _dev(v, device) for k, v in w.items()} for w in wl.layers],
+                         is_remove_padding=rm, use_fused_attention=fused)
+    got = enc(x, m, attention_bias=bd).cpu().numpy()
+    tol = (2e-4, 2e-5) if dtype == "fp32" else (MAX_ABS, MEAN_ABS)
+    for tag, g in (("whole", got),):
+        mx, mean, pads_zero = O.parity_metrics(g if packed else O.masked_output(g, wl.lens), exp, wl.lens)
+        _say("parity random stack/%d/%s: max-abs %.3e mean-abs %.3e" % (seed, tag, mx, mean))
+        assert np.isfinite(np.asarray(g, np.float32)).all()
+        assert mx <= tol[0] and mean <= tol[1], (tag, mx, mean)
+        assert pads_zero
+    if bias is None:                     # the operator's schema has no attention_bias argument
+        bt.load_th_op()
+        g = x
+        for w in wl.layers:
+            g = torch.ops.ByteTransformer.BertTransformer(
+                heads, 64, *[_dev(w[n], device) for n in workload.WEIGHT_NAMES], g, m, rm, fused)
+        g = g.cpu().numpy()
+        mx, mean, _ = O.parity_metrics(g if packed else O.masked_output(g, wl.lens), exp, wl.lens)
+        _say("parity random stack/%d/th_op: max-abs %.3e mean-abs %.3e" % (seed, mx, mean))
+        assert mx <= tol[0] and mean <= tol[1], ("th_op", mx, mean)
+
+
 @pytest.mark.parametrize("dtype", ["fp16", "fp32"])
 def test_seq_len_one(device, dtype):
     """seq_len 1: batch_idx has one entry more than there are rows (the scratch carve once
