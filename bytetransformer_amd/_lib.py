@@ -50,6 +50,9 @@ KERNEL_ABI = {
                                                c_float, _P]),
     "bt_add_bias_residual_layernorm_restore": (c_int, [_P, _P, _P, _P, _P, c_int, _P, _IP, c_int,
                                                        c_int, c_int, c_float, _P]),
+    "bt_gemm_splitk": (c_int, [_P, _P, _P, c_int, _IP, c_int, c_int, c_int, _P]),
+    "bt_splitk_layernorm": (c_int, [_P, c_int, _P, _IP, _P, _P, _P, c_int, _P, _IP, _IP, c_int,
+                                    c_int, c_int, c_int, c_float, _P]),
     "bt_gemm_f32": (c_int, [_P, _IP, _P, _P, _P, c_int, _IP, c_int, c_int, c_int, c_int, _P]),
     "bt_attention_f32": (c_int, [_P, _P, _IP, _IP, _P, _P, c_int, c_int, c_int, c_int, c_int, c_float,
                                  c_int, _P]),

@@ -55,6 +55,8 @@ void BertEncoder<OpType>::infer(BertEncoderInferParam<DataType_> ip) {
   int *seq_order = et_param.batch_idx + max_batch_size_ + 1;
   off += align_up((max_rows * 2 + 2 * (unsigned long long)max_batch_size_ + 2) * sizeof(int), 256);
   DataType_ *staging = (DataType_ *)(base + off);      // one layer's weights when none were passed
+  off += align_up(layer_weight_elems() * sizeof(DataType_), 256);
+  float *splitk_buf = (float *)(base + off);
 
   check_bt_error(bt_build_offsets(ip.atten_mask, Traits_::dtype, batch_size, seq_len,
                                   et_param.batch_idx, et_param.word_idx, seq_order, nullptr,
@@ -149,6 +151,22 @@ void BertEncoder<OpType>::infer(BertEncoderInferParam<DataType_> ip) {
     check_bt_error(bt_gemm_bias_gelu(attr_matmul_buf, wt_inter, w.inter_bias, inter_matmul_buf,
                                      valid_rows, rows, rows_hint, inter, hidden, stream));
 
+    // few rows, long k: FFN2 as split-k partial sums that the last LayerNorm folds in
+    const long long rows_expected =
+        !valid_rows ? rows : (rows_hint > 0 ? rows_hint : (rows * 3LL + 4) / 5);
+    const int splits = splitk_splits(rows, rows_expected, inter);
+    if (splits > 1) {
+      const bool restore = last && is_remove_padding_;
+      check_bt_error(bt_gemm_splitk(inter_matmul_buf, wt_out, splitk_buf, splits, valid_rows, rows,
+                                    hidden, inter, stream));
+      check_bt_error(bt_splitk_layernorm(
+          splitk_buf, splits, attr_matmul_buf, nullptr, w.output_bias, w.output_layernorm_gamma,
+          w.output_layernorm_beta, use_fp32_ ? 1 : 0,
+          restore ? (void *)ip.transformer_output : (void *)ffn2_out,
+          restore ? et_param.batch_idx : nullptr, restore ? nullptr : valid_rows, batch_size,
+          seq_len, rows, hidden, layernorm_eps, stream));
+      continue;
+    }
     check_bt_error(bt_gemm(inter_matmul_buf, wt_out, ffn2_out, valid_rows, rows, rows_hint, hidden,
                            inter, stream));
     if (last && is_remove_padding_)

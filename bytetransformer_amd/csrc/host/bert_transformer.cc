@@ -50,6 +50,10 @@ void BertTransformer<OpType>::bert_infer(BertTransformerInferParam infer_param) 
   DataType_ *wt_proj = wt_qkv + (size_t)3 * hidden * hidden;
   DataType_ *wt_inter = wt_proj + (size_t)hidden * hidden;
   DataType_ *wt_out = wt_inter + (size_t)hidden * inter;
+  off += align_up((4 + 2 * (unsigned long long)param_.intermediate_size) * hidden * hidden *
+                      sizeof(DataType_),
+                  256);
+  float *splitk_buf = (float *)(base + off);
 
   // lengths from the mask (needed on both paths: keys past len_b are excluded),
   // unless the caller already holds the offsets of this mask
@@ -160,6 +164,22 @@ void BertTransformer<OpType>::bert_infer(BertTransformerInferParam infer_param) 
 
   check_bt_error(bt_gemm_bias_gelu(attr_matmul_buf, wt_inter, param_.inter_bias, inter_matmul_buf,
                                    valid_rows, rows, rows_hint, inter, hidden, stream));
+
+  // few rows, long k: FFN2 as split-k partial sums that the last LayerNorm folds in
+  const long long rows_expected =
+      !valid_rows ? rows : (rows_hint > 0 ? rows_hint : (rows * 3LL + 4) / 5);
+  const int splits = splitk_splits(rows, rows_expected, inter);
+  if (splits > 1) {
+    check_bt_error(bt_gemm_splitk(inter_matmul_buf, wt_out, splitk_buf, splits, valid_rows, rows,
+                                  hidden, inter, stream));
+    check_bt_error(bt_splitk_layernorm(
+        splitk_buf, splits, attr_matmul_buf, nullptr, param_.output_bias,
+        param_.output_layernorm_gamma, param_.output_layernorm_beta, use_fp32_ ? 1 : 0,
+        is_remove_padding_ ? restore_target : transformer_out,
+        is_remove_padding_ ? et_param.batch_idx : nullptr, nullptr, batch_size, seq_len, rows,
+        hidden, layernorm_eps, stream));
+    return;
+  }
 
   check_bt_error(
       bt_gemm(inter_matmul_buf, wt_out, transformer_out, valid_rows, rows, rows_hint, hidden, inter,

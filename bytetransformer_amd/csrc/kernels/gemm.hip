@@ -33,7 +33,8 @@
 namespace bt {
 
 
-enum Epilogue { kEpiPlain = 0, kEpiBiasGelu = 1, kEpiQkvSplit = 2 };
+// kEpiPartial: split-k launch (grid y = split): fp32 partial sums to c32[split][rows_cap][N]
+enum Epilogue { kEpiPlain = 0, kEpiBiasGelu = 1, kEpiQkvSplit = 2, kEpiPartial = 3 };
 
 struct GemmArgs {
   const half_t *a;      // [rows_cap, K]
@@ -45,6 +46,7 @@ struct GemmArgs {
   int rows_cap, N, K;
   int tiles_n;
   int rows_hint;        // host-side estimate of the live rows (0 = unknown); tile choice only
+  float *c32;           // kEpiPartial only: [splits][rows_cap][N]
 };
 
 __device__ __forceinline__ float gelu_tanh_f32(float x) {
@@ -139,7 +141,9 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs &p) {
     tile_n = L - tile_m * p.tiles_n;
   }
   const int m0 = tile_m * BM, n0 = tile_n * BN;
-  const int nk = p.K / BK;
+  // a split-k launch gives grid row y the k range [y, y+1) * K / gridDim.y
+  const int nk = EPI == kEpiPartial ? p.K / BK / (int)gridDim.y : p.K / BK;
+  const int k_first = EPI == kEpiPartial ? (int)blockIdx.y * nk * BK : 0;
 
   // ---- loading side ---------------------------------------------------------
   // Global -> LDS copies are buffer loads with the LDS destination: descriptor and
@@ -159,10 +163,11 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs &p) {
   const int lw = NP == 0 ? wave : wave - NW;    // index among the loading waves
   const bool gather = p.a_row_index != nullptr;
   const rsrc_t rs_a =
-      gather ? make_rsrc(p.a, (size_t)p.rows_cap * p.K * sizeof(half_t))
-             : make_rsrc(p.a + (size_t)m0 * p.K, (size_t)(p.rows_cap - m0) * p.K * sizeof(half_t));
-  const rsrc_t rs_w =
-      make_rsrc(p.wt + (size_t)n0 * p.K, (size_t)(p.N - n0) * p.K * sizeof(half_t));
+      gather ? make_rsrc(p.a + k_first, ((size_t)p.rows_cap * p.K - k_first) * sizeof(half_t))
+             : make_rsrc(p.a + (size_t)m0 * p.K + k_first,
+                         ((size_t)(p.rows_cap - m0) * p.K - k_first) * sizeof(half_t));
+  const rsrc_t rs_w = make_rsrc(p.wt + (size_t)n0 * p.K + k_first,
+                                ((size_t)(p.N - n0) * p.K - k_first) * sizeof(half_t));
   int voff[NI];
   if (loader) {
 #pragma unroll
@@ -267,6 +272,25 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs &p) {
   __builtin_amdgcn_s_barrier();   // all waves are done with the last stage
   half_t *st = smem + wave * 32 * EP;
   const int row_in = lane & 31, col_in = (lane >> 5) * 4;
+  if (EPI == kEpiPartial) {
+    // fp32 partial sums straight from the accumulators: 16 bytes per lane and quad
+    float *dst = p.c32 + (size_t)blockIdx.y * p.rows_cap * p.N;
+#pragma unroll
+    for (int j = 0; j < TM; ++j) {
+      const int m = m0 + wm * WTM + j * 32 + row_in;
+#pragma unroll
+      for (int i = 0; i < TN; ++i)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const int n = n0 + wn * WTN + i * 32 + q * 8 + col_in;
+          if (m < M && n < p.N)
+            *(float4_t *)(dst + (size_t)m * p.N + n) =
+                float4_t{acc[i][j][4 * q + 0], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2],
+                         acc[i][j][4 * q + 3]};
+        }
+    }
+    return;
+  }
   constexpr int CPRW = WTN / 8;   // 16-byte chunks per staged row
   constexpr int RPS = 64 / CPRW;  // rows per store instruction
   const int sr = lane / CPRW, sc = (lane % CPRW) * 8;
@@ -278,7 +302,7 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs &p) {
       for (int q = 0; q < 4; ++q) {
         float v0 = acc[i][j][4 * q + 0], v1 = acc[i][j][4 * q + 1];
         float v2 = acc[i][j][4 * q + 2], v3 = acc[i][j][4 * q + 3];
-        if (EPI != kEpiPlain) {
+        if (EPI == kEpiBiasGelu || EPI == kEpiQkvSplit) {
           const int n = min(n0 + wn * WTN + i * 32 + q * 8 + col_in, p.N - 4);
           const half4_t b = *(const half4_t *)(p.bias + n);
           v0 += (float)b[0];
@@ -369,7 +393,7 @@ __global__ __launch_bounds__(256) void transpose_kernel(TransposeArgs a) {
 }
 
 template <int BM, int BN, int STAGES, int WM, int WN, int NP, int SCHED, int EPI>
-static int launch_gemm_tile(GemmArgs p, hipStream_t s) {
+static int launch_gemm_tile(GemmArgs p, hipStream_t s, int splits = 1) {
   constexpr size_t smem = (size_t)STAGES * (BM + BN) * kBK * sizeof(half_t);
   static_assert(smem <= 160 * 1024, "LDS budget");
   static std::atomic<bool> configured[kMaxDevices];
@@ -378,7 +402,7 @@ static int launch_gemm_tile(GemmArgs p, hipStream_t s) {
   if (rc != BT_OK) return rc;
   const int tiles_m = (p.rows_cap + BM - 1) / BM;
   p.tiles_n = (p.N + BN - 1) / BN;
-  const int grid = (tiles_m * p.tiles_n + 7) / 8 * 8;
+  const dim3 grid((tiles_m * p.tiles_n + 7) / 8 * 8, splits);
   gemm_kernel<BM, BN, STAGES, WM, WN, NP, SCHED, EPI><<<grid, (WM * WN + NP) * 64, smem, s>>>(p);
   BT_CHECK_LAUNCH("gemm_kernel");
   return BT_OK;
@@ -577,6 +601,20 @@ extern "C" int bt_gemm(const void *a, const void *wt, void *c, const int *valid_
   GemmArgs p{(const half_t *)a, (const half_t *)wt, nullptr, (half_t *)c, valid_rows, nullptr,
              rows_cap,          n,                  k,       0,           rows_hint};
   return launch_gemm<kEpiPlain>(p, as_stream(stream));
+}
+
+extern "C" int bt_gemm_splitk(const void *a, const void *wt, void *partials, int splits,
+                              const int *valid_rows, int rows_cap, int n, int k, void *stream) {
+  int rc = check_gemm_args("bt_gemm_splitk", a, wt, partials, rows_cap, n, k);
+  if (rc) return rc;
+  BT_REQUIRE(splits >= 1 && splits <= 16 && k % (splits * kBK) == 0, BT_ERR_INVALID_ARGUMENT,
+             "bt_gemm_splitk: splits=%d must lie in [1, 16] and divide k / 64 = %d", splits,
+             k / kBK);
+  if (rows_cap == 0) return BT_OK;
+  GemmArgs p{(const half_t *)a, (const half_t *)wt, nullptr, nullptr, valid_rows, nullptr,
+             rows_cap,          n,                  k,       0,       0,          (float *)partials};
+  // the small tile only: splitting k is for launches whose k loop is the whole run time
+  return launch_gemm_tile<32, 64, 4, 1, 2, 2, 0, kEpiPartial>(p, as_stream(stream), splits);
 }
 
 extern "C" int bt_gemm_bias_gelu(const void *a, const void *wt, const void *bias, void *c,

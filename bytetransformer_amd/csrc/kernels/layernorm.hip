@@ -12,7 +12,9 @@ namespace bt {
 
 constexpr int kLnRowsPerBlock = 4;
 
-template <int NC, bool RESTORE, bool GB32>
+// SPLITS > 0: `src` holds SPLITS fp32 partial sums of the row ([SPLITS][rows_cap][H], the
+// output of a split-k GEMM); their sum, rounded to fp16 once, takes the place of `out`.
+template <int NC, bool RESTORE, bool GB32, int SPLITS>
 __global__ __launch_bounds__(kLnRowsPerBlock *kWave) void layernorm_kernel(
     const half8_t *src, const half8_t *__restrict__ residual,
     const half8_t *__restrict__ bias, const void *__restrict__ gamma,
@@ -50,7 +52,24 @@ __global__ __launch_bounds__(kLnRowsPerBlock *kWave) void layernorm_kernel(
   for (int i = 0; i < NC; ++i) {
     const int c = lane + i * kWave;
     if (c < chunks) {
-      half8_t x = (a[c] + b[c]) + bias[c];  // two fp16-rounded adds
+      half8_t av;
+      if (SPLITS > 0) {
+        const float4_t *pp = (const float4_t *)src + (src_row * chunks + c) * 2;
+        float4_t lo = pp[0], hi = pp[1];
+#pragma unroll
+        for (int sp = 1; sp < SPLITS; ++sp) {
+          lo += pp[(size_t)sp * rows_cap * chunks * 2];
+          hi += pp[(size_t)sp * rows_cap * chunks * 2 + 1];
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          av[j] = (half_t)lo[j];
+          av[4 + j] = (half_t)hi[j];
+        }
+      } else {
+        av = a[c];
+      }
+      half8_t x = (av + b[c]) + bias[c];  // two fp16-rounded adds
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
         v[i][j] = (float)x[j];
@@ -109,7 +128,7 @@ __global__ __launch_bounds__(kLnRowsPerBlock *kWave) void layernorm_kernel(
   }
 }
 
-template <bool RESTORE>
+template <bool RESTORE, int SPLITS = 0>
 static int launch_ln(const void *src, const void *residual, const void *bias, const void *gamma,
                      const void *beta, int gb32, void *dst, const int *idx,
                      const int *residual_row_index, int B, int S, int rows_cap, int H, float eps,
@@ -123,7 +142,7 @@ static int launch_ln(const void *src, const void *residual, const void *bias, co
   const int grid = (rows_cap + kLnRowsPerBlock - 1) / kLnRowsPerBlock;
   const float inv_n = 1.0f / (float)H;
 #define BT_LN_LAUNCH(NC_, GB_)                                                                  \
-  layernorm_kernel<NC_, RESTORE, GB_><<<grid, kLnRowsPerBlock * kWave, 0, s>>>(                 \
+  layernorm_kernel<NC_, RESTORE, GB_, SPLITS><<<grid, kLnRowsPerBlock * kWave, 0, s>>>(         \
       (const half8_t *)src, (const half8_t *)residual, (const half8_t *)bias, gamma, beta,      \
       (half8_t *)dst, idx, residual_row_index, B, S, rows_cap, chunks, inv_n, eps)
 #define BT_LN_NC(NC_)              \
@@ -182,4 +201,42 @@ extern "C" int bt_add_bias_residual_layernorm_restore(
   return launch_ln<true>(out, residual, bias, gamma, beta, gamma_beta_fp32, out_padded, batch_idx,
                          nullptr, batch_size, seq_len, batch_size * seq_len, hidden_dim, eps,
                          as_stream(stream), "bt_add_bias_residual_layernorm_restore");
+}
+
+extern "C" int bt_splitk_layernorm(const void *partials, int splits, const void *residual,
+                                   const int *residual_row_index, const void *bias,
+                                   const void *gamma, const void *beta, int gamma_beta_fp32,
+                                   void *dst, const int *batch_idx, const int *valid_rows,
+                                   int batch_size, int seq_len, int rows_cap, int hidden_dim,
+                                   float eps, void *stream) {
+  BT_REQUIRE(partials && residual && bias && gamma && beta && dst, BT_ERR_INVALID_ARGUMENT,
+             "bt_splitk_layernorm: null pointer argument");
+  BT_REQUIRE(splits == 2 || splits == 4, BT_ERR_UNSUPPORTED,
+             "bt_splitk_layernorm: splits=%d (supported: 2, 4)", splits);
+  BT_REQUIRE(rows_cap >= 0, BT_ERR_INVALID_ARGUMENT, "bt_splitk_layernorm: negative rows_cap");
+  hipStream_t s = as_stream(stream);
+  if (batch_idx) {
+    // restore mode: dst is the padded [batch_size, seq_len, hidden] output
+    BT_REQUIRE(batch_size > 0 && seq_len > 0 && (long long)batch_size * seq_len == rows_cap,
+               BT_ERR_INVALID_ARGUMENT,
+               "bt_splitk_layernorm: restore needs rows_cap == batch_size * seq_len");
+    BT_REQUIRE(!residual_row_index, BT_ERR_INVALID_ARGUMENT,
+               "bt_splitk_layernorm: no residual gather in restore mode");
+    return splits == 2
+               ? launch_ln<true, 2>(partials, residual, bias, gamma, beta, gamma_beta_fp32, dst,
+                                    batch_idx, nullptr, batch_size, seq_len, rows_cap, hidden_dim,
+                                    eps, s, "bt_splitk_layernorm")
+               : launch_ln<true, 4>(partials, residual, bias, gamma, beta, gamma_beta_fp32, dst,
+                                    batch_idx, nullptr, batch_size, seq_len, rows_cap, hidden_dim,
+                                    eps, s, "bt_splitk_layernorm");
+  }
+  BT_REQUIRE(!residual_row_index || valid_rows, BT_ERR_INVALID_ARGUMENT,
+             "bt_splitk_layernorm: residual_row_index needs valid_rows");
+  return splits == 2
+             ? launch_ln<false, 2>(partials, residual, bias, gamma, beta, gamma_beta_fp32, dst,
+                                   valid_rows, residual_row_index, 0, 1, rows_cap, hidden_dim, eps,
+                                   s, "bt_splitk_layernorm")
+             : launch_ln<false, 4>(partials, residual, bias, gamma, beta, gamma_beta_fp32, dst,
+                                   valid_rows, residual_row_index, 0, 1, rows_cap, hidden_dim, eps,
+                                   s, "bt_splitk_layernorm");
 }

@@ -172,6 +172,27 @@ def add_bias_residual_layernorm_restore(out, residual, bias, gamma, beta, batch_
     return out_padded
 
 
+def gemm_splitk(a, wt, splits, valid_rows=None, out=None):
+    """fp32 partial sums [splits, rows, N] of a . wt^T over `splits` k ranges."""
+    rows, K = a.shape
+    N = wt.shape[0]
+    if out is None:
+        out = torch.zeros(splits, rows, N, dtype=torch.float32, device=a.device)
+    _check(kernel_lib().bt_gemm_splitk(_ptr(a), _ptr(wt), _ptr(out), int(splits), _ptr(valid_rows),
+                                       rows, N, K, _stream()))
+    return out
+
+
+def splitk_layernorm(partials, residual, bias, gamma, beta, dst, eps=1e-6, valid_rows=None,
+                     residual_row_index=None, batch_idx=None, batch_size=0, seq_len=1):
+    splits, rows, H = partials.shape
+    _check(kernel_lib().bt_splitk_layernorm(
+        _ptr(partials), splits, _ptr(residual), _ptr(residual_row_index), _ptr(bias), _ptr(gamma),
+        _ptr(beta), int(gamma.dtype == torch.float32), _ptr(dst), _ptr(batch_idx),
+        _ptr(valid_rows), batch_size, seq_len, rows, H, float(eps), _stream()))
+    return dst
+
+
 # ---- float (OperationType::FP32) entry points ---------------------------------
 def _need_f32(*ts):
     for t in ts:

@@ -213,6 +213,29 @@ int bt_add_bias_residual_layernorm_restore(const void *out, const void *residual
                                            float eps, void *stream);
 
 /*
+ * Split-k pair for launches with few rows and a long k (FFN2 at a few hundred tokens),
+ * where one tile's k loop is the whole run time.  No counterpart in the reference.
+ *
+ * bt_gemm_splitk: partials[s][m][:] = a[m, ks:ke] . wt[:, ks:ke]^T as fp32, split s covering
+ * k range [s, s+1) * k / splits; partials is float [splits][rows_cap][n]; splits in [1, 16]
+ * dividing k / 64.
+ *
+ * bt_splitk_layernorm: the add-bias + residual + LayerNorm entry points with the fp32
+ * partials (summed, rounded to fp16 once) in the place of `out`; splits 2 or 4.
+ * batch_idx == NULL: packed rows, dst [rows_cap, hidden] (valid_rows / residual_row_index as
+ * in bt_add_bias_residual_layernorm); batch_idx != NULL: dst is the padded
+ * [batch_size, seq_len, hidden] output with zero fill, rows_cap == batch_size * seq_len.
+ */
+int bt_gemm_splitk(const void *a, const void *wt, void *partials, int splits,
+                   const int *valid_rows, int rows_cap, int n, int k, void *stream);
+
+int bt_splitk_layernorm(const void *partials, int splits, const void *residual,
+                        const int *residual_row_index, const void *bias, const void *gamma,
+                        const void *beta, int gamma_beta_fp32, void *dst, const int *batch_idx,
+                        const int *valid_rows, int batch_size, int seq_len, int rows_cap,
+                        int hidden_dim, float eps, void *stream);
+
+/*
  * ---- OperationType::FP32 ------------------------------------------------------
  * The float flavour of the layer: every tensor (activations, weights, biases, gamma,
  * beta, mask, attention bias) is float, products run on the fp32 MFMA with fp32

@@ -130,7 +130,7 @@ class BertTransformer {
   // Scratch layout (elements of DataType_, T = max_batch*max_seq*hidden):
   //   [0,3T) qkv heads | [3T,4T) attention out | [4T,5T) projection / LN1 |
   //   [5T,(5+mult)T) FFN1 | word_idx int[B*S] | batch_idx int[B+1] | seq order int[B] |
-  //   pre-packed weights (3+1+2*mult)*H*H | attention scratch (none)
+  //   pre-packed weights (3+1+2*mult)*H*H | split-k partial sums | attention scratch (none)
   unsigned long long cal_bufsize() {
     const unsigned long long rows = (unsigned long long)max_batch_size_ * max_seq_len_;
     const unsigned long long hidden = (unsigned long long)head_num_ * size_per_head_;
@@ -142,6 +142,7 @@ class BertTransformer {
         (4 + 2 * (unsigned long long)param_.intermediate_size) * hidden * hidden *
             sizeof(DataType_),
         256);
+    inner_buf_size_ += align_up(splitk_scratch_bytes(rows, hidden), 256);
     return inner_buf_size_ + attention_layer_->cal_bufsize();
   }
 

@@ -11,6 +11,7 @@
 #include <hip/hip_runtime_api.h>
 
 #include <cstdint>
+#include <cstdlib>
 #include <stdexcept>
 #include <string>
 
@@ -50,6 +51,29 @@ typedef struct {
   int *word_idx;
   int valid_word_num;
 } ET_Param;
+
+// FFN2 with few rows and a long k runs as a split-k GEMM whose fp32 partial sums the last
+// LayerNorm folds in (bt_gemm_splitk / bt_splitk_layernorm): 4 splits up to 192 expected
+// rows, 2 up to 272, none beyond or when the batch has more than kSplitKMaxRows padded rows
+// (the partials live in a scratch area sized for that).
+constexpr int kSplitKMaxRows = 512;
+inline int splitk_splits(long long rows_cap, long long rows_expected, int k) {
+  static const bool enabled = [] {
+    const char *e = std::getenv("BT_SPLITK");     // BT_SPLITK=0 turns the split-k path off
+    return !(e && e[0] == '0');
+  }();
+  if (!enabled || rows_cap > kSplitKMaxRows || k < 2048) return 1;
+  if (rows_expected <= 192 && k % (4 * 64) == 0) return 4;
+  if (rows_expected <= 272 && k % (2 * 64) == 0) return 2;
+  return 1;
+}
+inline unsigned long long splitk_scratch_bytes(unsigned long long max_rows,
+                                               unsigned long long hidden) {
+  const unsigned long long rows = max_rows < (unsigned long long)kSplitKMaxRows
+                                      ? max_rows
+                                      : (unsigned long long)kSplitKMaxRows;
+  return 4ull * rows * hidden * sizeof(float);
+}
 
 enum ModelType { Bert };
 

@@ -79,12 +79,13 @@ def test_encoder_c_api_validation_and_bufsize():
     cfg = _lib.EncoderConfig(1, 16, 512, 12, 64, 4, 1, 1, 0, 1.0, 1e-6)
     need = lib.bt_encoder_bufsize(ctypes.byref(cfg))
     T = 16 * 512 * 768
-    # nine activation tensors + two index arrays + the pre-packed weights
-    assert need >= 9 * T * 2 + 2 * 16 * 512 * 4 + 12 * 768 * 768 * 2
-    assert need < 9 * T * 2 + 2 * 16 * 512 * 4 + 12 * 768 * 768 * 2 + 8192
+    # nine activation tensors + two index arrays + the pre-packed weights + the split-k area
+    splitk = 4 * 512 * 768 * 4
+    assert need >= 9 * T * 2 + 2 * 16 * 512 * 4 + 12 * 768 * 768 * 2 + splitk
+    assert need < 9 * T * 2 + 2 * 16 * 512 * 4 + 12 * 768 * 768 * 2 + splitk + 8192
     f32 = _lib.EncoderConfig(0, 16, 512, 12, 64, 4, 1, 1, 0, 1.0, 1e-6)   # float: twice the bytes
     need32 = lib.bt_encoder_bufsize(ctypes.byref(f32))
-    assert 2 * need - 4 * 16 * 512 * 4 - 8192 < need32 < 2 * need
+    assert 2 * need - 4 * 16 * 512 * 4 - splitk - 8192 < need32 < 2 * need
     bad = _lib.EncoderConfig(7, 16, 512, 12, 64, 4, 1, 1, 0, 1.0, 1e-6)
     assert lib.bt_encoder_bufsize(ctypes.byref(bad)) == 0
     assert b"BT_F16 or BT_F32" in lib.bt_encoder_last_error()

@@ -206,6 +206,60 @@ def test_gemm_random_shapes_all_tiles_and_auto(device, seed):
         ops.set_option("gemm_tile", -1)
 
 
+@pytest.mark.parametrize("splits,restore", [(2, False), (4, False), (4, True), (2, True)])
+def test_splitk_gemm_and_layernorm(device, splits, restore):
+    """FFN2 as split-k partial sums + the LayerNorm that folds them: same result as the
+    plain GEMM followed by the plain LayerNorm (one fp16 rounding of the product, then the
+    fp16 adds), against the oracle and bit-for-bit against the unsplit pair up to the
+    summation order of the fp32 partials."""
+    _say("splitk", splits, restore)
+    rs = np.random.RandomState(40 + splits)
+    B, S, H, F = 3, 50, 128, 1024
+    lens = np.array([50, 7, 31])
+    mask = workload.make_mask(lens, S, np.float16)
+    bi, wi, M = O.build_offsets(mask)
+    rows = B * S
+    a = np.zeros((rows, F), np.float16)
+    a[:M] = rs.standard_normal((M, F)).astype(np.float16)
+    a[M:] = np.float16("nan")
+    w = (rs.standard_normal((F, H)) * 0.05).astype(np.float16)
+    res = rs.standard_normal((rows, H)).astype(np.float16)
+    bias = (rs.standard_normal(H) * 0.5).astype(np.float16)
+    gamma = (1 + 0.2 * rs.standard_normal(H)).astype(np.float16)
+    beta = (0.3 * rs.standard_normal(H)).astype(np.float16)
+    prod = O.f16(O.gemm(a[:M], w))
+    exp = O.add_bias_residual_layernorm(prod, res[:M], bias, gamma, beta, 1e-6)
+    g_bi, _, _ = ops.build_offsets(_dev(mask, device))
+    vr = g_bi[B:]
+    wt = ops.transpose_weight(_dev(w, device))
+    parts = ops.gemm_splitk(_dev(a, device), wt, splits, valid_rows=vr)
+    # the partial sums add up to the product
+    total = parts.sum(0).cpu().numpy()[:M]
+    assert np.all(np.abs(total - O.gemm(a[:M], w)) <= 1e-3 + 1e-4 * np.abs(total))
+    args = (_dev(res, device), _dev(bias, device), _dev(gamma, device), _dev(beta, device))
+    if restore:
+        dst = torch.full((B, S, H), float("nan"), dtype=torch.float16, device=device)
+        g = ops.splitk_layernorm(parts, *args, dst, batch_idx=g_bi, batch_size=B, seq_len=S)
+        g = g.cpu().numpy()
+        exp_pad = O.restore(exp, bi, B, S)
+        for b in range(B):
+            assert np.all(g[b, lens[b]:].view(np.uint16) == 0)
+        err = np.abs(g.astype(np.float64) - exp_pad)
+        assert np.all(err <= 2.0 ** -9 * np.abs(exp_pad) + 4e-3), err.max()
+    else:
+        dst = torch.full((rows, H), 5.0, dtype=torch.float16, device=device)
+        g = ops.splitk_layernorm(parts, *args, dst, valid_rows=vr).cpu().numpy()
+        err = np.abs(g[:M].astype(np.float64) - exp)
+        assert np.all(err <= 2.0 ** -9 * np.abs(exp) + 4e-3), err.max()
+        assert np.all(g[M:] == 5.0)
+        # and the unsplit pair gives the same numbers except where the fp16 rounding of the
+        # product flips on the last bit of the fp32 sum
+        plain = ops.gemm(_dev(a, device), wt, valid_rows=vr)
+        ref = ops.add_bias_residual_layernorm(plain, *args, valid_rows=vr).cpu().numpy()
+        assert np.mean(ref[:M] == g[:M]) > 0.97
+        assert np.abs(ref[:M].astype(np.float32) - g[:M].astype(np.float32)).max() <= 2e-2
+
+
 @pytest.mark.parametrize("tile", [0, 1, 2, 3, 4, 5])
 def test_gemm_bias_gelu(device, tile):
     _say("gemm_bias_gelu", tile)
