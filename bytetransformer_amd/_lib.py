@@ -54,6 +54,8 @@ KERNEL_ABI = {
     "bt_splitk_layernorm": (c_int, [_P, c_int, _P, _IP, _P, _P, _P, c_int, _P, _IP, _IP, c_int,
                                     c_int, c_int, c_int, c_float, _P]),
     "bt_gemm_f32": (c_int, [_P, _IP, _P, _P, _P, c_int, _IP, c_int, c_int, c_int, c_int, _P]),
+    "bt_attention_generic_f16": (c_int, [_P, _P, _IP, _IP, _P, _P, c_int, c_int, c_int, c_int, c_int,
+                                         c_float, c_int, _P]),
     "bt_attention_f32": (c_int, [_P, _P, _IP, _IP, _P, _P, c_int, c_int, c_int, c_int, c_int, c_float,
                                  c_int, _P]),
     "bt_add_bias_residual_layernorm_f32": (c_int, [_P, _P, _IP, _P, _P, _P, _IP, c_int, c_int,

@@ -33,6 +33,16 @@ void Attention<OpType>::infer(AttentionInferParam infer_param) {
   // on padded rows the mask tensor itself is applied (any 0/1 pattern), as in the
   // reference's non-remove-padding kernels; packed rows use the prefix lengths
   const void *mask = is_remove_padding_ ? nullptr : (const void *)infer_param.atten_mask;
+  if (size_per_head_ != 64) {
+    // the fp16 kernels are built for 64-wide heads; other head sizes (32, 96, 128) take the
+    // generic kernel over token-major projections (the reference's unfused path for them)
+    check_bt_error(bt_attention_generic_f16(
+        infer_param.qkv, infer_param.attention_output, infer_param.et_param.batch_idx,
+        infer_param.seq_order, mask, infer_param.attention_bias, infer_param.batch_size,
+        infer_param.seq_len, rows_cap, head_num_, size_per_head_, scale, padded_rows,
+        infer_param.stream));
+    return;
+  }
   if (uses_short_kernel(infer_param.seq_len))
     check_bt_error(bt_attention_short(infer_param.qkv, infer_param.attention_output,
                                       infer_param.et_param.batch_idx, infer_param.seq_order, mask,

@@ -187,13 +187,28 @@ __global__ __launch_bounds__(64 * WGM *WGN) void f32_gemm_kernel(F32GemmArgs p) 
 // ---------------------------------------------------------------------------
 // attention
 // ---------------------------------------------------------------------------
+// Four consecutive elements of a float or fp16 tensor as floats, and back.
+__device__ __forceinline__ float4_t load4(const float *p) { return *(const float4_t *)p; }
+__device__ __forceinline__ float4_t load4(const half_t *p) {
+  const half4_t h = *(const half4_t *)p;
+  return float4_t{(float)h[0], (float)h[1], (float)h[2], (float)h[3]};
+}
+__device__ __forceinline__ void store4(float *p, float4_t v) { *(float4_t *)p = v; }
+__device__ __forceinline__ void store4(half_t *p, float4_t v) {
+  *(half4_t *)p = half4_t{(half_t)v[0], (half_t)v[1], (half_t)v[2], (half_t)v[3]};
+}
+
+// T = float for OperationType::FP32; T = half_t serves fp16 layers whose head size the fp16
+// attention kernels do not cover (they are built for 64): same kernel, operands widened to
+// float on the way into LDS and registers.
+template <typename T>
 struct F32AttArgs {
-  const float *qkv;    // [rows, 3H], QKV bias already added
-  float *out;          // [rows, H]
+  const T *qkv;        // [rows, 3H], QKV bias already added
+  T *out;              // [rows, H]
   const int *batch_idx;
   const int *seq_order;   // optional: rank -> sequence, longest first
-  const float *mask;   // optional [B,S,S]
-  const float *bias;   // optional [heads,S,S]
+  const T *mask;       // optional [B,S,S]
+  const T *bias;       // optional [heads,S,S]
   int B, S, rows_cap, heads;
   float scale;
   int padded_rows;
@@ -209,8 +224,8 @@ constexpr int kF32KT = 32;   // keys per tile
 // may be any bijection as long as both operands agree; it is chosen so that Q and K are
 // read as float4 (k = half*D/2 + step) and P needs no shuffle (key of step j in half h
 // = 8*(j/4) + 4*h + j%4, the accumulator's own row order).
-template <int ND, int NW>
-__global__ __launch_bounds__(64 * NW) void f32_attention_kernel(F32AttArgs p) {
+template <typename T, int ND, int NW>
+__global__ __launch_bounds__(64 * NW) void f32_attention_kernel(F32AttArgs<T> p) {
   constexpr int D = 32 * ND;
   constexpr int THREADS = 64 * NW, BQ = 32 * NW;   // 32 queries per wave
   constexpr int SK = D + 4, SV = D + 8;
@@ -238,7 +253,7 @@ __global__ __launch_bounds__(64 * NW) void f32_attention_kernel(F32AttArgs p) {
       const int H = p.heads * D;
       for (int i = threadIdx.x; i < BQ * D; i += THREADS) {
         const int q = q0 + i / D;
-        if (q < nq) p.out[(size_t)(row_start + q) * H + head * D + i % D] = 0.f;
+        if (q < nq) p.out[(size_t)(row_start + q) * H + head * D + i % D] = (T)0.f;
       }
     }
     return;
@@ -248,9 +263,9 @@ __global__ __launch_bounds__(64 * NW) void f32_attention_kernel(F32AttArgs p) {
   const int l32 = lane & 31, half = lane >> 5;
   const int H = p.heads * D;
   const size_t ld = (size_t)3 * H;
-  const float *Q = p.qkv + (size_t)row_start * ld + head * D;
-  const float *K = Q + H;
-  const float *V = K + H;
+  const T *Q = p.qkv + (size_t)row_start * ld + head * D;
+  const T *K = Q + H;
+  const T *V = K + H;
 
   const int q = q0 + wave * 32 + l32;       // this lane's query
   const bool wave_live = q0 + wave * 32 < nq;
@@ -260,7 +275,7 @@ __global__ __launch_bounds__(64 * NW) void f32_attention_kernel(F32AttArgs p) {
   float qf[D / 2];
 #pragma unroll
   for (int i = 0; i < D / 8; ++i) {
-    const float4_t v = *(const float4_t *)(Q + (size_t)qc * ld + half * (D / 2) + 4 * i);
+    const float4_t v = load4(Q + (size_t)qc * ld + half * (D / 2) + 4 * i);
 #pragma unroll
     for (int j = 0; j < 4; ++j) qf[4 * i + j] = v[j];
   }
@@ -275,8 +290,8 @@ __global__ __launch_bounds__(64 * NW) void f32_attention_kernel(F32AttArgs p) {
       const int idx = tid + THREADS * i;
       const int key = min(k0 + idx / CPR, klen - 1);
       const size_t off = (size_t)key * ld + 4 * (idx % CPR);
-      rk[i] = *(const float4_t *)(K + off);
-      rv[i] = *(const float4_t *)(V + off);
+      rk[i] = load4(K + off);
+      rv[i] = load4(V + off);
     }
   };
   auto stash = [&]() {
@@ -296,8 +311,8 @@ __global__ __launch_bounds__(64 * NW) void f32_attention_kernel(F32AttArgs p) {
   float m_run = kDeadLogit, l_run = 0.f;
 
   const float c = p.scale * kLog2eF;
-  const float *mrow = p.mask ? p.mask + ((size_t)b * p.S + min(q, p.S - 1)) * p.S : nullptr;
-  const float *brow = p.bias ? p.bias + ((size_t)head * p.S + min(q, p.S - 1)) * p.S : nullptr;
+  const T *mrow = p.mask ? p.mask + ((size_t)b * p.S + min(q, p.S - 1)) * p.S : nullptr;
+  const T *brow = p.bias ? p.bias + ((size_t)head * p.S + min(q, p.S - 1)) * p.S : nullptr;
 
   const int ntiles = (klen + kF32KT - 1) / kF32KT;
   fetch(0);
@@ -317,14 +332,14 @@ __global__ __launch_bounds__(64 * NW) void f32_attention_kernel(F32AttArgs p) {
         const int key = k0 + 8 * g + 4 * half;
         float4_t mv = {1.f, 1.f, 1.f, 1.f}, bv = {0.f, 0.f, 0.f, 0.f};
         if (add_vec && key + 3 < p.S) {
-          if (mrow) mv = *(const float4_t *)(mrow + key);
-          if (brow) bv = *(const float4_t *)(brow + key);
+          if (mrow) mv = load4(mrow + key);
+          if (brow) bv = load4(brow + key);
         } else {
 #pragma unroll
           for (int r = 0; r < 4; ++r)
             if (key + r < p.S) {
-              if (mrow) mv[r] = mrow[key + r];
-              if (brow) bv[r] = brow[key + r];
+              if (mrow) mv[r] = (float)mrow[key + r];
+              if (brow) bv[r] = (float)brow[key + r];
             }
         }
         add[g] = (mv - 1.0f) * (10000.0f * kLog2eF) + bv * kLog2eF;
@@ -397,7 +412,7 @@ __global__ __launch_bounds__(64 * NW) void f32_attention_kernel(F32AttArgs p) {
   const float l_all = l_run + __shfl_xor(l_run, 32, 64);
   const float inv = 1.0f / (l_all + 1e-6f);
   // accumulator element i of d-tile dt: d = 32*dt + 8*(i/4) + 4*half + i%4, query = l32
-  float *orow = p.out + (size_t)(row_start + q) * H + head * D;
+  T *orow = p.out + (size_t)(row_start + q) * H + head * D;
 #pragma unroll
   for (int dt = 0; dt < ND; ++dt)
 #pragma unroll
@@ -405,7 +420,7 @@ __global__ __launch_bounds__(64 * NW) void f32_attention_kernel(F32AttArgs p) {
       float4_t v;
 #pragma unroll
       for (int r = 0; r < 4; ++r) v[r] = o[dt][4 * g + r] * inv;
-      *(float4_t *)(orow + 32 * dt + 8 * g + 4 * half) = v;
+      store4(orow + 32 * dt + 8 * g + 4 * half, v);
     }
 }
 
@@ -502,6 +517,41 @@ int launch_f32_ln(const void *src, const void *residual, const void *bias, const
   return BT_OK;
 }
 
+template <typename T>
+static int launch_generic_attention(const char *who, const void *qkv, void *out,
+                                    const int *batch_idx, const int *seq_order,
+                                    const void *atten_mask, const void *attention_bias,
+                                    int batch_size, int seq_len, int rows_cap, int head_num,
+                                    int size_per_head, float scale, int padded_rows,
+                                    hipStream_t s) {
+  BT_REQUIRE(qkv && out && batch_idx, BT_ERR_INVALID_ARGUMENT, "%s: null pointer argument", who);
+  BT_REQUIRE(batch_size > 0 && seq_len > 0 && head_num > 0 && rows_cap >= 0,
+             BT_ERR_INVALID_ARGUMENT, "%s: sizes must be positive", who);
+  BT_REQUIRE(size_per_head > 0 && size_per_head % 32 == 0 && size_per_head <= 128,
+             BT_ERR_UNSUPPORTED, "%s: size_per_head %d (supported: 32, 64, 96, 128)", who,
+             size_per_head);
+  BT_REQUIRE(batch_size <= 65535 && head_num <= 65535, BT_ERR_UNSUPPORTED,
+             "%s: batch_size / head_num exceed the grid limit", who);
+  BT_REQUIRE(!padded_rows || (long long)batch_size * seq_len <= rows_cap, BT_ERR_INVALID_ARGUMENT,
+             "%s: padded rows need rows_cap >= batch_size * seq_len", who);
+  F32AttArgs<T> p{(const T *)qkv, (T *)out, batch_idx, seq_order, (const T *)atten_mask,
+                  (const T *)attention_bias, batch_size, seq_len, rows_cap, head_num, scale,
+                  padded_rows ? 1 : 0};
+  constexpr int kWaves = 4;    // 128 queries per workgroup (two-wave workgroups measured slower)
+  p.nqb = (seq_len + 32 * kWaves - 1) / (32 * kWaves);
+  const unsigned grid = ((unsigned)batch_size * head_num + 7) / 8 * 8 * p.nqb;
+#define BT_F32_ATT(ND_) f32_attention_kernel<T, ND_, kWaves><<<grid, 64 * kWaves, 0, s>>>(p)
+  switch (size_per_head / 32) {
+    case 1: BT_F32_ATT(1); break;
+    case 2: BT_F32_ATT(2); break;
+    case 3: BT_F32_ATT(3); break;
+    default: BT_F32_ATT(4); break;
+  }
+#undef BT_F32_ATT
+  BT_CHECK_LAUNCH(who);
+  return BT_OK;
+}
+
 }  // namespace
 }  // namespace bt
 
@@ -558,37 +608,25 @@ extern "C" int bt_gemm_f32(const void *a, const int *a_row_index, const void *w,
 }
 
 extern "C" int bt_attention_f32(const void *qkv, void *out, const int *batch_idx,
-                                const int *seq_order, const void *atten_mask, const void *attention_bias,
-                                int batch_size, int seq_len, int rows_cap, int head_num,
-                                int size_per_head, float scale, int padded_rows, void *stream) {
-  BT_REQUIRE(qkv && out && batch_idx, BT_ERR_INVALID_ARGUMENT,
-             "bt_attention_f32: null pointer argument");
-  BT_REQUIRE(batch_size > 0 && seq_len > 0 && head_num > 0 && rows_cap >= 0,
-             BT_ERR_INVALID_ARGUMENT, "bt_attention_f32: sizes must be positive");
-  BT_REQUIRE(size_per_head == 32 || size_per_head == 64 || size_per_head == 128,
-             BT_ERR_UNSUPPORTED, "bt_attention_f32: size_per_head %d (supported: 32, 64, 128)",
-             size_per_head);
-  BT_REQUIRE(batch_size <= 65535 && head_num <= 65535, BT_ERR_UNSUPPORTED,
-             "bt_attention_f32: batch_size / head_num exceed the grid limit");
-  BT_REQUIRE(!padded_rows || (long long)batch_size * seq_len <= rows_cap, BT_ERR_INVALID_ARGUMENT,
-             "bt_attention_f32: padded rows need rows_cap >= batch_size * seq_len");
-  F32AttArgs p{(const float *)qkv, (float *)out, batch_idx, seq_order, (const float *)atten_mask,
-               (const float *)attention_bias, batch_size, seq_len, rows_cap, head_num, scale,
-               padded_rows ? 1 : 0};
-  hipStream_t s = as_stream(stream);
-  constexpr int kWaves = 4;    // 128 queries per workgroup (two-wave workgroups measured slower)
-  p.nqb = (seq_len + 32 * kWaves - 1) / (32 * kWaves);
-  const unsigned grid = ((unsigned)batch_size * head_num + 7) / 8 * 8 * p.nqb;
-#define BT_F32_ATT(ND_) f32_attention_kernel<ND_, kWaves><<<grid, 64 * kWaves, 0, s>>>(p)
-  if (size_per_head == 32)
-    BT_F32_ATT(1);
-  else if (size_per_head == 64)
-    BT_F32_ATT(2);
-  else
-    BT_F32_ATT(4);
-#undef BT_F32_ATT
-  BT_CHECK_LAUNCH("bt_attention_f32");
-  return BT_OK;
+                                const int *seq_order, const void *atten_mask,
+                                const void *attention_bias, int batch_size, int seq_len,
+                                int rows_cap, int head_num, int size_per_head, float scale,
+                                int padded_rows, void *stream) {
+  return launch_generic_attention<float>("bt_attention_f32", qkv, out, batch_idx, seq_order,
+                                         atten_mask, attention_bias, batch_size, seq_len,
+                                         rows_cap, head_num, size_per_head, scale, padded_rows,
+                                         as_stream(stream));
+}
+
+extern "C" int bt_attention_generic_f16(const void *qkv, void *out, const int *batch_idx,
+                                        const int *seq_order, const void *atten_mask,
+                                        const void *attention_bias, int batch_size, int seq_len,
+                                        int rows_cap, int head_num, int size_per_head,
+                                        float scale, int padded_rows, void *stream) {
+  return launch_generic_attention<half_t>("bt_attention_generic_f16", qkv, out, batch_idx,
+                                          seq_order, atten_mask, attention_bias, batch_size,
+                                          seq_len, rows_cap, head_num, size_per_head, scale,
+                                          padded_rows, as_stream(stream));
 }
 
 extern "C" int bt_add_bias_residual_layernorm_f32(void *out, const void *residual,

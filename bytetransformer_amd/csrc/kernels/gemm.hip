@@ -34,7 +34,8 @@ namespace bt {
 
 
 // kEpiPartial: split-k launch (grid y = split): fp32 partial sums to c32[split][rows_cap][N]
-enum Epilogue { kEpiPlain = 0, kEpiBiasGelu = 1, kEpiQkvSplit = 2, kEpiPartial = 3 };
+// kEpiBias: + bias, row-major store (the QKV projection of layers whose head size is not 64)
+enum Epilogue { kEpiPlain = 0, kEpiBiasGelu = 1, kEpiQkvSplit = 2, kEpiPartial = 3, kEpiBias = 4 };
 
 struct GemmArgs {
   const half_t *a;      // [rows_cap, K]
@@ -302,7 +303,7 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs &p) {
       for (int q = 0; q < 4; ++q) {
         float v0 = acc[i][j][4 * q + 0], v1 = acc[i][j][4 * q + 1];
         float v2 = acc[i][j][4 * q + 2], v3 = acc[i][j][4 * q + 3];
-        if (EPI == kEpiBiasGelu || EPI == kEpiQkvSplit) {
+        if (EPI == kEpiBiasGelu || EPI == kEpiQkvSplit || EPI == kEpiBias) {
           const int n = min(n0 + wn * WTN + i * 32 + q * 8 + col_in, p.N - 4);
           const half4_t b = *(const half4_t *)(p.bias + n);
           v0 += (float)b[0];
@@ -636,8 +637,8 @@ extern "C" int bt_gemm_qkv_bias_split(const void *a, const int *a_row_index, con
                                       int head_num, int size_per_head, void *stream) {
   BT_REQUIRE(head_num > 0, BT_ERR_INVALID_ARGUMENT, "bt_gemm_qkv_bias_split: head_num=%d",
              head_num);
-  BT_REQUIRE(size_per_head == 64, BT_ERR_UNSUPPORTED,
-             "bt_gemm_qkv_bias_split: size_per_head=%d, only 64 is supported", size_per_head);
+  BT_REQUIRE(size_per_head > 0, BT_ERR_INVALID_ARGUMENT,
+             "bt_gemm_qkv_bias_split: size_per_head=%d", size_per_head);
   const int H = head_num * size_per_head;
   int rc = check_gemm_args("bt_gemm_qkv_bias_split", a, wt_qkv, qkv_heads, rows_cap, 3 * H, H);
   if (rc) return rc;
@@ -650,5 +651,9 @@ extern "C" int bt_gemm_qkv_bias_split(const void *a, const int *a_row_index, con
              "bt_gemm_qkv_bias_split: a gathered input of %d x %d halfs is beyond 2 GiB", rows_cap, H);
   GemmArgs p{(const half_t *)a, (const half_t *)wt_qkv, (const half_t *)bias_qkv,
              (half_t *)qkv_heads, valid_rows, a_row_index, rows_cap, 3 * H, H, 0, rows_hint};
+  // the head-major split is the layout of the fp16 attention kernels, which are built for
+  // 64-wide heads; any other head size keeps the projections token-major [rows_cap, 3H]
+  // for bt_attention_generic_f16
+  if (size_per_head != 64) return launch_gemm<kEpiBias>(p, as_stream(stream));
   return launch_gemm<kEpiQkvSplit>(p, as_stream(stream));
 }

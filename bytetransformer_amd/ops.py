@@ -232,6 +232,20 @@ def attention_f32(qkv, batch_idx, batch_size, seq_len, head_num, scale, padded_r
     return out
 
 
+def attention_generic_f16(qkv, batch_idx, batch_size, seq_len, head_num, scale, padded_rows=False,
+                          mask=None, bias=None, out=None, seq_order=None):
+    """fp16 qkv [rows, 3 * hidden] (bias added) -> [rows, hidden]; head sizes 32, 64, 96, 128."""
+    rows_cap, three_h = qkv.shape
+    hidden = three_h // 3
+    if out is None:
+        out = torch.zeros(rows_cap, hidden, dtype=qkv.dtype, device=qkv.device)
+    _check(kernel_lib().bt_attention_generic_f16(
+        _ptr(qkv), _ptr(out), _ptr(batch_idx), _ptr(seq_order), _ptr(mask), _ptr(bias), batch_size,
+        seq_len, rows_cap, head_num, hidden // head_num, float(scale), int(padded_rows),
+        _stream()))
+    return out
+
+
 def add_bias_residual_layernorm_f32(out, residual, bias, gamma, beta, eps=1e-6, valid_rows=None,
                                     residual_row_index=None):
     _need_f32(out, residual, bias, gamma, beta)

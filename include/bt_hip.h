@@ -121,10 +121,12 @@ int bt_gemm_bias_gelu(const void *a, const void *wt, const void *bias, void *c,
  * [3][head_num][rows_cap][size_per_head].  Replaces the bias-free QKV
  * dense_layer_kernel_launcher call (bert_transformer.cu:85-87) plus
  * add_QKV_bias_padding (attention_nofused_utils.cu:143-184) / the in-kernel
- * bias add of attention_fused.cu:318-325.  size_per_head must be 64.
+ * bias add of attention_fused.cu:318-325.  The head split needs size_per_head == 64.
  * a_row_index (nullable, needs valid_rows): live row t of A is a[a_row_index[t], :] -
  * passing word_idx reads the valid tokens straight out of the padded input, which
  * folds compressBertInput (remove_padding.h:104-121) into this GEMM's operand fetch.
+ * size_per_head != 64: the projections stay token-major, qkv_heads = [rows_cap, 3 * hidden]
+ * (Q | K | V per row), the layout bt_attention_generic_f16 reads.
  */
 int bt_gemm_qkv_bias_split(const void *a, const int *a_row_index, const void *wt_qkv,
                            const void *bias_qkv, void *qkv_heads, const int *valid_rows,
@@ -264,8 +266,18 @@ int bt_gemm_f32(const void *a, const int *a_row_index, const void *w, const void
  * buffer.  atten_mask (nullable, float [B,S,S]) is applied on both row layouts; keys at
  * or past the sequence length are excluded by index on packed rows (they do not exist
  * there) and, without a mask, on padded rows.  seq_order (nullable) as in the fp16
- * entries: issue order only.  size_per_head in {32, 64, 128}.
+ * entries: issue order only.  size_per_head in {32, 64, 96, 128}.
  */
+/* The same kernel on fp16 tensors (operands widened to float on chip), for fp16 layers whose
+ * head size the fp16 attention entries do not cover: size_per_head in {32, 64, 96, 128}.
+ * Role of the reference's unfused path for size_per_head != 64 (bert_transformer.h:132-133,
+ * attention_nofused.cu:27-114). */
+int bt_attention_generic_f16(const void *qkv, void *attention_output, const int *batch_idx,
+                             const int *seq_order, const void *atten_mask,
+                             const void *attention_bias, int batch_size, int seq_len,
+                             int rows_cap, int head_num, int size_per_head, float scale,
+                             int padded_rows, void *stream);
+
 int bt_attention_f32(const void *qkv, void *attention_output, const int *batch_idx,
                      const int *seq_order, const void *atten_mask, const void *attention_bias, int batch_size,
                      int seq_len, int rows_cap, int head_num, int size_per_head, float scale,

@@ -46,8 +46,8 @@ def test_argument_validation_returns_codes_without_gpu():
     p = ctypes.c_void_p(256)   # never dereferenced: validation fails first
     assert lib.bt_gemm(p, p, p, None, 4, 0, 8, 100, None) == 2 and "multiple of 64" in err()
     assert lib.bt_gemm(p, p, p, None, 4, 0, 12, 64, None) == 2 and "multiple of 8" in err()
-    assert lib.bt_gemm_qkv_bias_split(p, None, p, p, p, None, 4, 0, 12, 32, None) == 2
-    assert "size_per_head=32" in err()
+    assert lib.bt_gemm_qkv_bias_split(p, None, p, p, p, None, 4, 0, 1, 32, None) == 2
+    assert "multiple of 64" in err()        # hidden = 1 * 32
     assert lib.bt_gemm_qkv_bias_split(p, p, p, p, p, None, 4, 0, 12, 64, None) == 1
     assert "needs valid_rows" in err()
     assert lib.bt_attention_short(p, p, p, None, None, None, 1, 1024, 1024, 12, 64, 0.125, 0, None, 0, None) == 2

@@ -237,6 +237,39 @@ def test_attention_f32_mask_and_bias(device, padded):
         assert err.max() <= 2e-5, (b, err.max())
 
 
+@pytest.mark.parametrize("padded", [False, True])
+@pytest.mark.parametrize("lens,S,heads,d", [([70, 9, 33], 72, 2, 128), ([40, 33], 40, 4, 32),
+                                            ([150, 64, 1], 160, 2, 96), ([64, 38], 64, 3, 64)])
+def test_attention_generic_f16(device, lens, S, heads, d, padded):
+    """The same kernel on fp16 tensors (head sizes the fp16 attention kernels do not take):
+    inputs rounded to fp16, arithmetic in float, one fp16 rounding of the output."""
+    _say("attention_generic_f16", lens, S, heads, d, padded)
+    rs = np.random.RandomState(S + heads + d)
+    B, H = len(lens), heads * d
+    bi = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    qkv = rs.standard_normal((B * S, 3 * H)).astype(np.float16)
+    if not padded:
+        qkv[bi[-1]:] = np.float16("nan")
+    mask = None
+    bias = (0.5 * rs.standard_normal((heads, S, S))).astype(np.float16)
+    if padded:
+        mask = (rs.rand(B, S, S) < 0.7).astype(np.float16)
+        mask[:, :, 0] = 1
+    scale = 1 / math.sqrt(d)
+    exp = _naive_attention(qkv.astype(np.float32), lens, S, heads, d, scale, padded,
+                           None if mask is None else mask.astype(np.float32),
+                           bias.astype(np.float32))
+    g = ops.attention_generic_f16(_dev(qkv, device), _dev(bi, device), B, S, heads, scale,
+                                  padded_rows=padded,
+                                  mask=None if mask is None else _dev(mask, device),
+                                  bias=_dev(bias, device)).cpu().numpy()
+    assert g.dtype == np.float16
+    for b, n in enumerate(lens):
+        r0, nq = (b * S, S) if padded else (bi[b], n)
+        err = np.abs(g[r0:r0 + nq].astype(np.float64) - exp[r0:r0 + nq])
+        assert np.all(err <= 2.0 ** -10 * np.abs(exp[r0:r0 + nq]) + 1e-4), (b, err.max())
+
+
 def test_attention_f32_rows_sum_and_uniform_keys(device):
     """V = const per column: the output is that constant times sum(P) = 1 / (1 + 1e-6 / sum e),
     whatever Q and K are; identical keys give a uniform P."""

@@ -404,6 +404,31 @@ def test_random_whole_encoder_bias_masks_and_operator(device, seed):
         assert mx <= tol[0] and mean <= tol[1], ("th_op", mx, mean)
 
 
+@pytest.mark.parametrize("dtype,head_size,heads", [("fp16", 128, 2), ("fp16", 32, 4),
+                                                   ("fp16", 96, 2), ("fp32", 128, 2),
+                                                   ("fp32", 32, 6), ("fp32", 96, 2)])
+@pytest.mark.parametrize("rm", [True, False])
+def test_head_sizes_other_than_64(device, dtype, head_size, heads, rm):
+    """Head sizes 32, 96 and 128: the QKV projection stays token-major and the generic
+    attention kernel takes over (the reference's unfused path for them)."""
+    _say("head size", dtype, head_size, heads, rm)
+    cfg = workload.EncoderConfig("hs", 4, 70, heads, head_size=head_size, layers=2, dtype=dtype,
+                                 lens=(70, 12, 0, 45), seed=head_size)
+    wl = workload.make_workload(cfg, bias_std=0.05, random_affine=True)
+    layers32 = [{k: np.asarray(v, np.float32) for k, v in w.items()} for w in wl.layers]
+    exp = O.masked_output(O.encoder(wl.x.astype(np.float32), wl.mask.astype(np.float32), layers32,
+                                    heads).numpy(), wl.lens)
+    tol = (2e-4, 2e-5) if dtype == "fp32" else (MAX_ABS, MEAN_ABS)
+    for tag, got in (("c_api", _run_c_api(wl, device, is_remove_padding=rm)),
+                     ("th_op", _run_th_op(wl, device, rm=rm)),
+                     ("whole", _whole_encoder(wl, device, is_remove_padding=rm)(
+                         _dev(wl.x, device), _dev(wl.mask, device)).cpu().numpy())):
+        g = got if rm else O.masked_output(got, wl.lens)
+        mx, mean, pads_zero = O.parity_metrics(g, exp, wl.lens)
+        _say("parity head size %d/%s/%s: max-abs %.3e mean-abs %.3e" % (head_size, dtype, tag, mx, mean))
+        assert mx <= tol[0] and mean <= tol[1] and pads_zero, (tag, mx, mean, pads_zero)
+
+
 @pytest.mark.parametrize("dtype", ["fp16", "fp32"])
 def test_seq_len_one(device, dtype):
     """seq_len 1: batch_idx has one entry more than there are rows (the scratch carve once
