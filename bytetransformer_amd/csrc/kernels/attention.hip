@@ -627,6 +627,8 @@ static int check_att_args(const char *who, const void *qkv, const void *out, con
   BT_REQUIRE(!mask || padded_rows, BT_ERR_INVALID_ARGUMENT,
              "%s: atten_mask is only applied on padded rows (padded_rows != 0)", who);
   BT_REQUIRE(qkv && out && batch_idx, BT_ERR_INVALID_ARGUMENT, "%s: null pointer argument", who);
+  BT_REQUIRE(aligned16({qkv, out, mask}), BT_ERR_INVALID_ARGUMENT,
+             "%s: tensor pointers must be 16-byte aligned", who);
   BT_REQUIRE(B > 0 && S > 0 && heads > 0 && rows_cap > 0, BT_ERR_INVALID_ARGUMENT,
              "%s: batch_size=%d seq_len=%d head_num=%d rows_cap=%d must be positive", who, B, S,
              heads, rows_cap);

@@ -7,6 +7,8 @@
 #include <hip/hip_fp16.h>
 
 #include <cstdarg>
+#include <cstdint>
+#include <initializer_list>
 #include <cstdio>
 
 #include "bt_hip.h"
@@ -75,6 +77,14 @@ int option_attention_xcd_map();     // 1 = XCD-aware workgroup order of the fp16
 int option_prefetch();       // 1 = honour the prefetch hints of the attention entries (default), 0 = ignore
 
 inline hipStream_t as_stream(void *s) { return reinterpret_cast<hipStream_t>(s); }
+
+// Every kernel moves tensors in 16-byte pieces: all tensor pointers of an entry point must
+// be 16-byte aligned (null counts as aligned: nullable arguments are checked elsewhere).
+inline bool aligned16(std::initializer_list<const void *> ptrs) {
+  for (const void *p : ptrs)
+    if (reinterpret_cast<uintptr_t>(p) & 15) return false;
+  return true;
+}
 
 // ---- wave64 reductions ----------------------------------------------------
 __device__ __forceinline__ float wave_sum(float v) {

@@ -493,6 +493,8 @@ int launch_f32_ln(const void *src, const void *residual, const void *bias, const
                   int S, int rows_cap, int H, float eps, hipStream_t s, const char *who) {
   BT_REQUIRE(H > 0 && H % 4 == 0, BT_ERR_UNSUPPORTED, "%s: hidden_dim %d must be a multiple of 4",
              who, H);
+  BT_REQUIRE(aligned16({src, residual, bias, gamma, beta, dst}), BT_ERR_INVALID_ARGUMENT,
+             "%s: tensor pointers must be 16-byte aligned", who);
   const int chunks = H / 4;
   const int nc = (chunks + kWave - 1) / kWave;
   BT_REQUIRE(nc <= 16, BT_ERR_UNSUPPORTED, "%s: hidden_dim %d exceeds 4096", who, H);
@@ -525,6 +527,8 @@ static int launch_generic_attention(const char *who, const void *qkv, void *out,
                                     int size_per_head, float scale, int padded_rows,
                                     hipStream_t s) {
   BT_REQUIRE(qkv && out && batch_idx, BT_ERR_INVALID_ARGUMENT, "%s: null pointer argument", who);
+  BT_REQUIRE(aligned16({qkv, out, atten_mask, attention_bias}), BT_ERR_INVALID_ARGUMENT,
+             "%s: tensor pointers must be 16-byte aligned", who);
   BT_REQUIRE(batch_size > 0 && seq_len > 0 && head_num > 0 && rows_cap >= 0,
              BT_ERR_INVALID_ARGUMENT, "%s: sizes must be positive", who);
   BT_REQUIRE(size_per_head > 0 && size_per_head % 32 == 0 && size_per_head <= 128,
@@ -561,6 +565,8 @@ extern "C" int bt_gemm_f32(const void *a, const int *a_row_index, const void *w,
                            void *c, int gelu, const int *valid_rows, int rows_cap, int rows_hint,
                            int n, int k, void *stream) {
   BT_REQUIRE(a && w && c, BT_ERR_INVALID_ARGUMENT, "bt_gemm_f32: null pointer argument");
+  BT_REQUIRE(aligned16({a, w, c}), BT_ERR_INVALID_ARGUMENT,
+             "bt_gemm_f32: tensor pointers must be 16-byte aligned");
   BT_REQUIRE(rows_cap >= 0 && n > 0 && k > 0, BT_ERR_INVALID_ARGUMENT,
              "bt_gemm_f32: sizes must be positive");
   BT_REQUIRE(n % 4 == 0 && k % 4 == 0, BT_ERR_UNSUPPORTED,

@@ -551,6 +551,8 @@ static int launch_gemm(GemmArgs p, hipStream_t s) {
 static int check_gemm_args(const char *who, const void *a, const void *wt, const void *c,
                            int rows_cap, int n, int k) {
   BT_REQUIRE(a && wt && c, BT_ERR_INVALID_ARGUMENT, "%s: null pointer argument", who);
+  BT_REQUIRE(aligned16({a, wt, c}), BT_ERR_INVALID_ARGUMENT,
+             "%s: tensor pointers must be 16-byte aligned", who);
   BT_REQUIRE(rows_cap >= 0 && n > 0 && k > 0, BT_ERR_INVALID_ARGUMENT,
              "%s: rows_cap=%d n=%d k=%d out of range", who, rows_cap, n, k);
   BT_REQUIRE(k % 64 == 0, BT_ERR_UNSUPPORTED, "%s: k=%d must be a multiple of 64", who, k);

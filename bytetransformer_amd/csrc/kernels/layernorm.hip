@@ -135,6 +135,8 @@ static int launch_ln(const void *src, const void *residual, const void *bias, co
                      hipStream_t s, const char *who) {
   BT_REQUIRE(H > 0 && H % 8 == 0, BT_ERR_UNSUPPORTED, "%s: hidden_dim %d must be a multiple of 8",
              who, H);
+  BT_REQUIRE(aligned16({src, residual, bias, gamma, beta, dst}), BT_ERR_INVALID_ARGUMENT,
+             "%s: tensor pointers must be 16-byte aligned", who);
   const int chunks = H / 8;
   const int nc = (chunks + kWave - 1) / kWave;
   BT_REQUIRE(nc <= 8, BT_ERR_UNSUPPORTED, "%s: hidden_dim %d exceeds 4096", who, H);

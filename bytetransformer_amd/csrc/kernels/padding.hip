@@ -201,6 +201,8 @@ extern "C" int bt_compress(const void *from_tensor, void *to_tensor, const int *
              "bt_compress: sizes must be positive");
   BT_REQUIRE(hidden_dim % 8 == 0, BT_ERR_UNSUPPORTED,
              "bt_compress: hidden_dim %d must be a multiple of 8", hidden_dim);
+  BT_REQUIRE(aligned16({from_tensor, to_tensor}), BT_ERR_INVALID_ARGUMENT,
+             "bt_compress: tensor pointers must be 16-byte aligned");
   const long long rows = (long long)batch_size * seq_len;
   BT_REQUIRE(rows < (1ll << 31), BT_ERR_UNSUPPORTED, "bt_compress: too many rows");
   const int grid = (int)((rows + kRowsPerBlock - 1) / kRowsPerBlock);

@@ -9,6 +9,7 @@
  *     device memory; the caller owns every buffer, scratch included;
  *   - after a non-zero return bt_last_error_string() describes the failure
  *     (thread-local);
+ *   - tensor pointers must be 16-byte aligned (every kernel moves data in 16-byte pieces);
  *   - activations and weights are fp16 (IEEE binary16) unless a dtype argument
  *     says otherwise; "packed" means the M valid token rows of the batch laid
  *     out back to back in (batch, position) order;

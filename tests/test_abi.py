@@ -63,6 +63,10 @@ def test_argument_validation_returns_codes_without_gpu():
     assert lib.bt_add_bias_residual_layernorm_restore(p, p, p, p, p, 0, None, p, 2, 4, 64, 1e-6,
                                                       None) == 1
     assert lib.bt_transpose_weight(None, p, 8, 8, None) == 1
+    odd = ctypes.c_void_p(264)   # 8-byte aligned only
+    assert lib.bt_gemm(odd, p, p, None, 4, 0, 8, 64, None) == 1 and "16-byte aligned" in err()
+    assert lib.bt_add_bias_residual_layernorm(p, odd, None, p, p, p, 0, None, 4, 64, 1e-6, None) == 1
+    assert "16-byte aligned" in err()
     # float entry points
     assert lib.bt_gemm_f32(p, None, p, None, p, 0, None, 4, 0, 6, 8, None) == 2 and "multiples of 4" in err()
     assert lib.bt_gemm_f32(p, None, p, None, p, 1, None, 4, 0, 8, 8, None) == 1 and "gelu needs a bias" in err()
