@@ -34,7 +34,7 @@ void Attention<OpType>::infer(AttentionInferParam infer_param) {
   // reference's non-remove-padding kernels; packed rows use the prefix lengths
   const void *mask = is_remove_padding_ ? nullptr : (const void *)infer_param.atten_mask;
   if (size_per_head_ != 64) {
-    // the fp16 kernels are built for 64-wide heads; other head sizes (32, 96, 128) take the
+    // the fp16 kernels are built for 64-wide heads; other head sizes (multiples of 8 up to 128) take the
     // generic kernel over token-major projections (the reference's unfused path for them)
     check_bt_error(bt_attention_generic_f16(
         infer_param.qkv, infer_param.attention_output, infer_param.et_param.batch_idx,

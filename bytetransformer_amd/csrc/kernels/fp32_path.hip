@@ -213,6 +213,8 @@ struct F32AttArgs {
   float scale;
   int padded_rows;
   int nqb;             // query tiles per sequence
+  int d;               // head size (a multiple of 8, <= the kernel's D = 32 * ND; the
+                       // columns d..D-1 of Q, K and V read as zero)
 };
 
 constexpr int kF32KT = 32;   // keys per tile
@@ -250,10 +252,10 @@ __global__ __launch_bounds__(64 * NW) void f32_attention_kernel(F32AttArgs<T> p)
   if (q0 >= nq || klen <= 0) {
     // padded rows of an empty sequence still get defined output: zeros
     if (q0 < nq) {
-      const int H = p.heads * D;
-      for (int i = threadIdx.x; i < BQ * D; i += THREADS) {
-        const int q = q0 + i / D;
-        if (q < nq) p.out[(size_t)(row_start + q) * H + head * D + i % D] = (T)0.f;
+      const int H = p.heads * p.d;
+      for (int i = threadIdx.x; i < BQ * p.d; i += THREADS) {
+        const int q = q0 + i / p.d;
+        if (q < nq) p.out[(size_t)(row_start + q) * H + head * p.d + i % p.d] = (T)0.f;
       }
     }
     return;
@@ -261,9 +263,10 @@ __global__ __launch_bounds__(64 * NW) void f32_attention_kernel(F32AttArgs<T> p)
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int l32 = lane & 31, half = lane >> 5;
-  const int H = p.heads * D;
+  const int d = p.d;
+  const int H = p.heads * d;
   const size_t ld = (size_t)3 * H;
-  const T *Q = p.qkv + (size_t)row_start * ld + head * D;
+  const T *Q = p.qkv + (size_t)row_start * ld + head * d;
   const T *K = Q + H;
   const T *V = K + H;
 
@@ -275,7 +278,9 @@ __global__ __launch_bounds__(64 * NW) void f32_attention_kernel(F32AttArgs<T> p)
   float qf[D / 2];
 #pragma unroll
   for (int i = 0; i < D / 8; ++i) {
-    const float4_t v = load4(Q + (size_t)qc * ld + half * (D / 2) + 4 * i);
+    const int e = half * (D / 2) + 4 * i;
+    float4_t v = {0.f, 0.f, 0.f, 0.f};
+    if (e < d) v = load4(Q + (size_t)qc * ld + e);
 #pragma unroll
     for (int j = 0; j < 4; ++j) qf[4 * i + j] = v[j];
   }
@@ -289,9 +294,13 @@ __global__ __launch_bounds__(64 * NW) void f32_attention_kernel(F32AttArgs<T> p)
     for (int i = 0; i < NV; ++i) {
       const int idx = tid + THREADS * i;
       const int key = min(k0 + idx / CPR, klen - 1);
-      const size_t off = (size_t)key * ld + 4 * (idx % CPR);
-      rk[i] = load4(K + off);
-      rv[i] = load4(V + off);
+      const int e = 4 * (idx % CPR);
+      const size_t off = (size_t)key * ld + e;
+      rk[i] = rv[i] = float4_t{0.f, 0.f, 0.f, 0.f};
+      if (e < d) {
+        rk[i] = load4(K + off);
+        rv[i] = load4(V + off);
+      }
     }
   };
   auto stash = [&]() {
@@ -412,7 +421,7 @@ __global__ __launch_bounds__(64 * NW) void f32_attention_kernel(F32AttArgs<T> p)
   const float l_all = l_run + __shfl_xor(l_run, 32, 64);
   const float inv = 1.0f / (l_all + 1e-6f);
   // accumulator element i of d-tile dt: d = 32*dt + 8*(i/4) + 4*half + i%4, query = l32
-  T *orow = p.out + (size_t)(row_start + q) * H + head * D;
+  T *orow = p.out + (size_t)(row_start + q) * H + head * d;
 #pragma unroll
   for (int dt = 0; dt < ND; ++dt)
 #pragma unroll
@@ -420,7 +429,7 @@ __global__ __launch_bounds__(64 * NW) void f32_attention_kernel(F32AttArgs<T> p)
       float4_t v;
 #pragma unroll
       for (int r = 0; r < 4; ++r) v[r] = o[dt][4 * g + r] * inv;
-      store4(orow + 32 * dt + 8 * g + 4 * half, v);
+      if (32 * dt + 8 * g + 4 * half < d) store4(orow + 32 * dt + 8 * g + 4 * half, v);
     }
 }
 
@@ -531,9 +540,9 @@ static int launch_generic_attention(const char *who, const void *qkv, void *out,
              "%s: tensor pointers must be 16-byte aligned", who);
   BT_REQUIRE(batch_size > 0 && seq_len > 0 && head_num > 0 && rows_cap >= 0,
              BT_ERR_INVALID_ARGUMENT, "%s: sizes must be positive", who);
-  BT_REQUIRE(size_per_head > 0 && size_per_head % 32 == 0 && size_per_head <= 128,
-             BT_ERR_UNSUPPORTED, "%s: size_per_head %d (supported: 32, 64, 96, 128)", who,
-             size_per_head);
+  BT_REQUIRE(size_per_head > 0 && size_per_head % 8 == 0 && size_per_head <= 128,
+             BT_ERR_UNSUPPORTED, "%s: size_per_head %d (supported: multiples of 8 up to 128)",
+             who, size_per_head);
   BT_REQUIRE(batch_size <= 65535 && head_num <= 65535, BT_ERR_UNSUPPORTED,
              "%s: batch_size / head_num exceed the grid limit", who);
   BT_REQUIRE(!padded_rows || (long long)batch_size * seq_len <= rows_cap, BT_ERR_INVALID_ARGUMENT,
@@ -541,11 +550,12 @@ static int launch_generic_attention(const char *who, const void *qkv, void *out,
   F32AttArgs<T> p{(const T *)qkv, (T *)out, batch_idx, seq_order, (const T *)atten_mask,
                   (const T *)attention_bias, batch_size, seq_len, rows_cap, head_num, scale,
                   padded_rows ? 1 : 0};
+  p.d = size_per_head;
   constexpr int kWaves = 4;    // 128 queries per workgroup (two-wave workgroups measured slower)
   p.nqb = (seq_len + 32 * kWaves - 1) / (32 * kWaves);
   const unsigned grid = ((unsigned)batch_size * head_num + 7) / 8 * 8 * p.nqb;
 #define BT_F32_ATT(ND_) f32_attention_kernel<T, ND_, kWaves><<<grid, 64 * kWaves, 0, s>>>(p)
-  switch (size_per_head / 32) {
+  switch ((size_per_head + 31) / 32) {
     case 1: BT_F32_ATT(1); break;
     case 2: BT_F32_ATT(2); break;
     case 3: BT_F32_ATT(3); break;

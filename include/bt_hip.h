@@ -267,10 +267,10 @@ int bt_gemm_f32(const void *a, const int *a_row_index, const void *w, const void
  * buffer.  atten_mask (nullable, float [B,S,S]) is applied on both row layouts; keys at
  * or past the sequence length are excluded by index on packed rows (they do not exist
  * there) and, without a mask, on padded rows.  seq_order (nullable) as in the fp16
- * entries: issue order only.  size_per_head in {32, 64, 96, 128}.
+ * entries: issue order only.  size_per_head a multiple of 8 up to 128.
  */
 /* The same kernel on fp16 tensors (operands widened to float on chip), for fp16 layers whose
- * head size the fp16 attention entries do not cover: size_per_head in {32, 64, 96, 128}.
+ * head size the fp16 attention entries do not cover: size_per_head a multiple of 8 up to 128.
  * Role of the reference's unfused path for size_per_head != 64 (bert_transformer.h:132-133,
  * attention_nofused.cu:27-114). */
 int bt_attention_generic_f16(const void *qkv, void *attention_output, const int *batch_idx,

@@ -173,6 +173,7 @@ def _naive_attention(qkv, lens, S, heads, d, scale, padded, mask=None, bias=None
 F32_ATT_CASES = [
     ([64, 38], 64, 12, 64), ([154], 256, 12, 64), ([1, 16, 17, 0, 100, 128, 129], 160, 3, 64),
     ([300, 77, 5], 320, 2, 64), ([40, 33], 40, 4, 32), ([70, 9], 72, 2, 128),
+    ([50, 31], 50, 2, 48), ([50, 31], 50, 3, 104),
 ]
 
 
@@ -239,7 +240,9 @@ def test_attention_f32_mask_and_bias(device, padded):
 
 @pytest.mark.parametrize("padded", [False, True])
 @pytest.mark.parametrize("lens,S,heads,d", [([70, 9, 33], 72, 2, 128), ([40, 33], 40, 4, 32),
-                                            ([150, 64, 1], 160, 2, 96), ([64, 38], 64, 3, 64)])
+                                            ([150, 64, 1], 160, 2, 96), ([64, 38], 64, 3, 64),
+                                            ([33, 70], 70, 4, 16), ([100, 5], 100, 2, 80),
+                                            ([64, 64], 64, 3, 8)])
 def test_attention_generic_f16(device, lens, S, heads, d, padded):
     """The same kernel on fp16 tensors (head sizes the fp16 attention kernels do not take):
     inputs rounded to fp16, arithmetic in float, one fp16 rounding of the output."""

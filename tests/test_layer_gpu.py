@@ -406,10 +406,12 @@ def test_random_whole_encoder_bias_masks_and_operator(device, seed):
 
 @pytest.mark.parametrize("dtype,head_size,heads", [("fp16", 128, 2), ("fp16", 32, 4),
                                                    ("fp16", 96, 2), ("fp32", 128, 2),
-                                                   ("fp32", 32, 6), ("fp32", 96, 2)])
+                                                   ("fp32", 32, 6), ("fp32", 96, 2),
+                                                   ("fp16", 16, 4), ("fp16", 80, 4),
+                                                   ("fp32", 48, 4)])
 @pytest.mark.parametrize("rm", [True, False])
 def test_head_sizes_other_than_64(device, dtype, head_size, heads, rm):
-    """Head sizes 32, 96 and 128: the QKV projection stays token-major and the generic
+    """Head sizes other than 64 (multiples of 8 up to 128): the QKV projection stays token-major and the generic
     attention kernel takes over (the reference's unfused path for them)."""
     _say("head size", dtype, head_size, heads, rm)
     cfg = workload.EncoderConfig("hs", 4, 70, heads, head_size=head_size, layers=2, dtype=dtype,
