@@ -71,7 +71,7 @@ def test_argument_validation_returns_codes_without_gpu():
     assert lib.bt_gemm_f32(p, None, p, None, p, 0, None, 4, 0, 6, 8, None) == 2 and "multiples of 4" in err()
     assert lib.bt_gemm_f32(p, None, p, None, p, 1, None, 4, 0, 8, 8, None) == 1 and "gelu needs a bias" in err()
     assert lib.bt_gemm_f32(p, p, p, None, p, 0, None, 4, 0, 8, 8, None) == 1 and "needs valid_rows" in err()
-    assert lib.bt_attention_f32(p, p, p, None, None, None, 1, 16, 16, 12, 48, 0.125, 0, None) == 2
+    assert lib.bt_attention_f32(p, p, p, None, None, None, 1, 16, 16, 12, 44, 0.125, 0, None) == 2
     assert lib.bt_attention_f32(p, p, p, None, None, None, 2, 16, 16, 12, 64, 0.125, 1, None) == 1
     assert lib.bt_add_bias_residual_layernorm_f32(p, p, None, p, p, p, None, 4, 6, 1e-6, None) == 2
     assert lib.bt_add_bias_residual_layernorm_restore_f32(p, p, p, p, p, None, p, 2, 4, 64, 1e-6,
