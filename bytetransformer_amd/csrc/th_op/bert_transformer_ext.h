@@ -8,6 +8,8 @@
 
 #include <hip/hip_runtime_api.h>
 
+#include <memory>
+
 namespace bytetransformer {
 namespace torch_ext {
 using torch::Tensor;
@@ -65,9 +67,9 @@ class BTEncoder : public IBTEncoder {
                bool is_remove_padding = true, bool use_fused_attention = true,
                const ModelType model_type = ModelType::Bert,
                const Tensor attention_bias = Tensor()) override {
-    CHECK_SEQ_LEN(seq_len);
+    check_seq_len(seq_len);
     if (attention_bias.defined()) {
-      CHECK_INPUT(attention_bias, input.scalar_type());
+      check_tensor(attention_bias, "attention_bias", input.scalar_type(), false);
       TORCH_CHECK(attention_bias.dim() == 3 && attention_bias.size(0) == head_num_ &&
                       attention_bias.size(1) == seq_len && attention_bias.size(2) == seq_len,
                   "attention_bias must be [head_num, seq_len, seq_len]");
@@ -170,6 +172,36 @@ class BTEncoder : public IBTEncoder {
   std::vector<Tensor> weights_;
   BertTransformerParam<kOp> param_;
 };
+
+// Names of the twelve per-layer tensors in operator-argument order; gamma / beta
+// (positions 4, 5, 10, 11) may be float next to fp16 weights.
+static const char *const kWeightNames[12] = {
+    "qkv_kernel",     "qkv_bias",    "attr_output_kernel",
+    "attr_output_bias", "attr_output_layernorm_gamma", "attr_output_layernorm_beta",
+    "inter_kernel",   "inter_bias",  "output_kernel",
+    "output_bias",    "output_layernorm_gamma",      "output_layernorm_beta"};
+
+inline bool is_affine_slot(int i) { return i == 4 || i == 5 || i == 10 || i == 11; }
+
+inline void check_weights(const std::vector<Tensor> &w) {
+  TORCH_CHECK(w.size() == 12, "expected 12 weight tensors");
+  const at::ScalarType st = w[0].scalar_type();
+  for (int i = 0; i < 12; ++i) check_tensor(w[i], kWeightNames[i], st, is_affine_slot(i));
+}
+
+// The encoder for the weights' dtype; anything but float / half is refused with the
+// reference's text (ths_op_f.cc:62-64).
+inline std::unique_ptr<IBTEncoder> make_encoder(int64_t head_num, int64_t head_size,
+                                                const std::vector<Tensor> &w) {
+  switch (w[0].scalar_type()) {
+    case at::ScalarType::Float:
+      return std::unique_ptr<IBTEncoder>(new BTEncoder<float>((int)head_num, (int)head_size, w));
+    case at::ScalarType::Half:
+      return std::unique_ptr<IBTEncoder>(new BTEncoder<__half>((int)head_num, (int)head_size, w));
+    default:
+      throw std::runtime_error("Wrong Tensor type.");
+  }
+}
 
 inline void check_layer_shapes(int64_t head_num, int64_t head_size, const std::vector<Tensor> &w) {
   const int64_t H = head_num * head_size;

@@ -26,28 +26,8 @@ class BertTransformer : public torch::jit::CustomClassHolder {
                  attr_output_bias, attr_output_layernorm_gamma, attr_output_layernorm_beta,
                  inter_kernel,   inter_bias,  output_kernel,
                  output_bias,    output_layernorm_gamma,      output_layernorm_beta} {
-    CHECK_INPUT(qkv_kernel, st_);
-    CHECK_INPUT(qkv_bias, st_);
-    CHECK_INPUT(attr_output_kernel, st_);
-    CHECK_INPUT(attr_output_bias, st_);
-    CHECK_INPUT_LOOSE(attr_output_layernorm_gamma);
-    CHECK_INPUT_LOOSE(attr_output_layernorm_beta);
-    CHECK_INPUT(inter_kernel, st_);
-    CHECK_INPUT(inter_bias, st_);
-    CHECK_INPUT(output_kernel, st_);
-    CHECK_INPUT(output_bias, st_);
-    CHECK_INPUT_LOOSE(output_layernorm_gamma);
-    CHECK_INPUT_LOOSE(output_layernorm_beta);
-    switch (st_) {
-      case at::ScalarType::Float:
-        encoder_.reset(new torch_ext::BTEncoder<float>(head_num, head_size, weights_));
-        break;
-      case at::ScalarType::Half:
-        encoder_.reset(new torch_ext::BTEncoder<__half>(head_num, head_size, weights_));
-        break;
-      default:
-        throw std::runtime_error("Wrong Tensor type.");
-    }
+    torch_ext::check_weights(weights_);
+    encoder_ = torch_ext::make_encoder(head_num, head_size, weights_);
     torch_ext::check_layer_shapes(head_num, head_size, weights_);
     head_info_ = torch::empty({2}, torch::dtype(torch::kInt64));
     head_info_[0] = head_num;
@@ -59,8 +39,8 @@ class BertTransformer : public torch::jit::CustomClassHolder {
 
   Tensor forwardv2(Tensor input, Tensor attr_mask, bool is_remove_padding,
                    bool use_fused_attention) {
-    CHECK_INPUT(input, st_);
-    CHECK_INPUT(attr_mask, st_);
+    torch_ext::check_tensor(input, "input", st_, false);
+    torch_ext::check_tensor(attr_mask, "attr_mask", st_, false);
     TORCH_CHECK(input.dim() == 3 && input.size(2) == hidden_,
                 "input must be [batch_size, seq_len, head_num * head_size]");
     const int batch_size = (int)input.size(0), seq_len = (int)input.size(1);
