@@ -96,7 +96,7 @@ def kernel_table(wl, dev, iters):
     wt_1, wt_2 = ops.transpose_weight(w["inter_kernel"]), ops.transpose_weight(w["output_kernel"])
     qkv = ops.gemm_qkv_bias_split(packed, wt_qkv, w["qkv_bias"], heads, valid_rows=vr)
     scale = 1.0 / cfg.head_size ** 0.5
-    att_fn = ops.attention_short if S <= 256 else ops.attention_grouped
+    att_fn = ops.attention_grouped     # the host library's default choice at every length
     att = att_fn(qkv, batch_idx, B, S, scale)
     proj = ops.gemm(att, wt_o, valid_rows=vr)
     inter = ops.gemm_bias_gelu(proj, wt_1, w["inter_bias"], valid_rows=vr)

@@ -31,6 +31,7 @@ static std::atomic<int> g_gemm_tile{-1};
 static std::atomic<int> g_attention_qb{-1};
 static std::atomic<int> g_prefetch{1};
 static std::atomic<int> g_f32_gemm_tile{-1};
+static std::atomic<int> g_attention_short_limit{0};
 static std::atomic<int> g_attention_xcd_map{1};
 int option_attention_xcd_map() { return g_attention_xcd_map.load(std::memory_order_relaxed); }
 int option_f32_gemm_tile() { return g_f32_gemm_tile.load(std::memory_order_relaxed); }
@@ -144,6 +145,10 @@ extern "C" int bt_set_option(const char *name, int value) {
     BT_REQUIRE(value >= -1 && value <= 2, BT_ERR_INVALID_ARGUMENT,
                "bt_set_option: f32_gemm_tile=%d outside [-1, 2]", value);
     g_f32_gemm_tile.store(value);
+  } else if (!strcmp(name, "attention_short_limit")) {
+    BT_REQUIRE(value >= 0 && value <= 512, BT_ERR_INVALID_ARGUMENT,
+               "bt_set_option: attention_short_limit=%d outside [0, 512]", value);
+    g_attention_short_limit.store(value);
   } else if (!strcmp(name, "attention_xcd_map")) {
     BT_REQUIRE(value == 0 || value == 1, BT_ERR_INVALID_ARGUMENT,
                "bt_set_option: attention_xcd_map=%d must be 0 or 1", value);
@@ -154,6 +159,27 @@ extern "C" int bt_set_option(const char *name, int value) {
     g_prefetch.store(value);
   } else {
     set_error("bt_set_option: unknown option '%s'", name);
+    return BT_ERR_INVALID_ARGUMENT;
+  }
+  return BT_OK;
+}
+
+extern "C" int bt_get_option(const char *name, int *value) {
+  BT_REQUIRE(name && value, BT_ERR_INVALID_ARGUMENT, "bt_get_option: null argument");
+  if (!strcmp(name, "gemm_tile")) {
+    *value = g_gemm_tile.load();
+  } else if (!strcmp(name, "attention_qb")) {
+    *value = g_attention_qb.load();
+  } else if (!strcmp(name, "prefetch")) {
+    *value = g_prefetch.load();
+  } else if (!strcmp(name, "f32_gemm_tile")) {
+    *value = g_f32_gemm_tile.load();
+  } else if (!strcmp(name, "attention_short_limit")) {
+    *value = g_attention_short_limit.load();
+  } else if (!strcmp(name, "attention_xcd_map")) {
+    *value = g_attention_xcd_map.load();
+  } else {
+    set_error("bt_get_option: unknown option '%s'", name);
     return BT_ERR_INVALID_ARGUMENT;
   }
   return BT_OK;

@@ -46,6 +46,12 @@ def set_option(name, value):
     _check(kernel_lib().bt_set_option(name.encode(), int(value)))
 
 
+def get_option(name):
+    v = ctypes.c_int(0)
+    _check(kernel_lib().bt_get_option(name.encode(), ctypes.byref(v)))
+    return v.value
+
+
 def build_offsets(mask, want_count=False, out=None, seq_order=None):
     """mask [B,S,S] -> (batch_idx int32[B+1], word_idx int32[B*S], M or None)."""
     B, S = mask.shape[0], mask.shape[1]

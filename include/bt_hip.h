@@ -54,9 +54,15 @@ const char *bt_last_error_string(void);
  *   "prefetch"      1 (default) | 0: honour / ignore the prefetch hint of the attention entries
  *   "f32_gemm_tile" -1 heuristic | 0: 128x128 tile, 8 waves | 1: 128x64, 4 waves | 2: 64x64, 4 waves
  *                   (bt_gemm_f32 only)
+ *   "attention_short_limit"  0 (default) .. 512: the host library sends sequences up to this
+ *                   length to bt_attention_short when use_fused_attention is set; 0 = always
+ *                   the streaming kernel, which measures faster at every length
+ *   "attention_xcd_map"  1 (default) | 0: XCD-aware or plain workgroup order of the fp16
+ *                   attention kernels
  * Process-wide; results do not depend on it beyond fp32 summation order.
  */
 int bt_set_option(const char *name, int value);
+int bt_get_option(const char *name, int *value);
 
 /*
  * Mask prefix sum.  Replaces build_sequence_length_padding_offset_kernelLauncher

@@ -60,10 +60,16 @@ class Attention {
   const ModelType model_type_;
 
  public:
-  // Sequences up to this length take the LDS-resident short kernel when
-  // use_fused_attention is set; longer ones (or use_fused_attention = false)
-  // take the streaming grouped kernel.
-  static constexpr int kShortSeqLimit = 256;
+  // Sequences up to this length take the LDS-resident short kernel (whole K / V in LDS,
+  // exact two-pass softmax) when use_fused_attention is set; longer ones, or
+  // use_fused_attention = false, take the streaming grouped kernel.  The limit is the
+  // process-wide option "attention_short_limit" of the kernel library and defaults to 0:
+  // on MI355X the streaming kernel measures faster at every length and batch size (its
+  // first key tile is in flight while the short kernel still waits for all of K and V).
+  static int short_seq_limit() {
+    int v = 0;
+    return bt_get_option("attention_short_limit", &v) == BT_OK ? v : 0;
+  }
 
   Attention(const int max_batch_size, const int head_num, const int size_per_head,
             const int max_seq_len, const bool use_fused_attention = true,
@@ -82,7 +88,7 @@ class Attention {
   virtual unsigned long long cal_bufsize() const { return 0; }
 
   bool uses_short_kernel(int seq_len) const {
-    return use_fused_attention_ && seq_len <= kShortSeqLimit;
+    return use_fused_attention_ && seq_len <= short_seq_limit();
   }
 
   virtual void infer(AttentionInferParam infer_param);

@@ -51,6 +51,17 @@ def _run_c_api(wl, device, n_layers=None, **kw):
     return out.cpu().numpy()
 
 
+@pytest.fixture(autouse=True)
+def _short_kernel_for_fused_runs():
+    """By default the host sends every length to the streaming attention kernel (the faster
+    one); these tests let use_fused_attention = True select the LDS-resident short kernel up to
+    its capacity again, so that both kernels are covered through the layer."""
+    from bytetransformer_amd import ops
+    ops.set_option("attention_short_limit", 512)
+    yield
+    ops.set_option("attention_short_limit", 0)
+
+
 def _run_th_op(wl, device, n_layers=None, rm=True, fused=True):
     bt.load_th_op()
     layers = wl.layers if n_layers is None else wl.layers[:n_layers]
@@ -442,6 +453,24 @@ def test_seq_len_one(device, dtype):
                                     12).numpy(), wl.lens)
     _check(_run_c_api(wl, device), exp, wl.lens, tag="seq_len 1/" + dtype)
     _check(_run_th_op(wl, device), exp, wl.lens, tag="seq_len 1/th_op/" + dtype)
+
+
+def test_default_dispatch_is_the_streaming_kernel(device):
+    """attention_short_limit defaults to 0: with it the fused flag changes nothing, and the
+    result still matches the oracle."""
+    from bytetransformer_amd import ops
+    ops.set_option("attention_short_limit", 0)
+    assert ops.get_option("attention_short_limit") == 0
+    wl = workload.make_workload(workload.EncoderConfig("dd", 4, 100, 2, layers=1,
+                                                       lens=(100, 30, 64, 7)))
+    a = _run_c_api(wl, device, use_fused_attention=True)
+    b = _run_c_api(wl, device, use_fused_attention=False)
+    assert np.array_equal(a, b)
+    _check(a, _oracle(wl), wl.lens, tag="default dispatch")
+    ops.set_option("attention_short_limit", 512)
+    c = _run_c_api(wl, device, use_fused_attention=True)
+    assert not np.array_equal(a, c)          # another kernel, another rounding
+    _check(c, _oracle(wl), wl.lens, tag="short kernel")
 
 
 def test_th_op_prepack_cache_tracks_weight_updates(device):
