@@ -473,6 +473,52 @@ def test_default_dispatch_is_the_streaming_kernel(device):
     _check(c, _oracle(wl), wl.lens, tag="short kernel")
 
 
+def test_two_threads_two_streams_share_nothing(device):
+    """The operator from two host threads at once, each on its own stream and its own
+    batch: the caches are keyed per stream and every call owns its scratch, so each thread
+    must get exactly what it gets alone."""
+    import threading
+    bt.load_th_op()
+    op = torch.ops.ByteTransformer.BertTransformer
+    jobs = []
+    for seed, (B, S) in enumerate([(4, 96), (6, 130)]):
+        cfg = workload.EncoderConfig("mt%d" % seed, B, S, 2, layers=3, seed=40 + seed)
+        wl = workload.make_workload(cfg, bias_std=0.05, random_affine=True)
+        ws = [[_dev(w[n], device) for n in workload.WEIGHT_NAMES] for w in wl.layers]
+        jobs.append((ws, _dev(wl.x, device), _dev(wl.mask, device)))
+
+    def forward(job):
+        ws, x, m = job
+        h = x
+        for w in ws:
+            h = op(2, 64, *w, h, m, True, True)
+        return h
+
+    alone = [forward(j).clone() for j in jobs]
+    torch.cuda.synchronize()
+    results, errors = [None, None], []
+
+    def worker(i):
+        try:
+            stream = torch.cuda.Stream(device=device)
+            with torch.cuda.stream(stream):
+                for _ in range(30):
+                    out = forward(jobs[i])
+                stream.synchronize()
+            results[i] = out
+        except Exception as exc:   # noqa: BLE001 - reported by the assertion below
+            errors.append(exc)
+
+    threads = [threading.Thread(target=worker, args=(i,)) for i in range(2)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join(timeout=100)
+    assert not errors, errors
+    for i in range(2):
+        assert results[i] is not None and torch.equal(results[i], alone[i])
+
+
 def test_th_op_prepack_cache_tracks_weight_updates(device):
     """The operator caches the k-contiguous weight copies per tensor object; an
     in-place update of a weight (version counter bump) must be picked up, and a
