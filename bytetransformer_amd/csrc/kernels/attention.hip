@@ -16,7 +16,7 @@
 //                             two-pass softmax: P = exp(s-max)/(sum+1e-6) is
 //                             rounded to fp16 before P.V exactly as
 //                             attention_fused.cu:348-381 does.
-//   attention_grouped_kernel  K / V streamed in 64-key tiles through a 3-stage
+//   attention_grouped_kernel  K / V streamed in 64-key tiles through a 2- or 3-stage
 //                             LDS ring with an online softmax; handles any
 //                             length; the [S, S] logits never exist.
 //
@@ -222,14 +222,15 @@ __device__ __forceinline__ float4_t add_terms4(const half_t *mask_row, const hal
 // ---------------------------------------------------------------------------
 constexpr int kKT = 64;                          // keys per streamed tile
 constexpr int kTileHalfs = kKT * kHeadDim;       // one K or V tile
-constexpr int kAttStages = 3;
 
 // QB 16-query blocks per wave; workgroup covers 4*QB*16 queries.  ADD: a mask tensor and / or an
 // attention bias contribute additive terms to the logits.
-template <int QB, bool ADD>
+template <int QB, bool ADD, int STAGES>
 __global__ __launch_bounds__(kAttThreads, 2) void attention_grouped_kernel(AttArgs p) {
   constexpr int BQ = 4 * QB * 16;
-  __shared__ __attribute__((aligned(1024))) half_t ring[kAttStages * 2 * kTileHalfs];
+  constexpr int AHEAD = STAGES - 1;     // tiles in flight beyond the one being consumed
+  static_assert(STAGES == 2 || STAGES == 3, "ring depth");
+  __shared__ __attribute__((aligned(1024))) half_t ring[STAGES * 2 * kTileHalfs];
 
   const AttItem item = att_item(p);
   if (!item.exists) {
@@ -306,7 +307,7 @@ __global__ __launch_bounds__(kAttThreads, 2) void attention_grouped_kernel(AttAr
   const bool wave_live = q0 + wave * QB * 16 < nq;
   const int ntiles = (klen + kKT - 1) / kKT;
   if (ntiles > 0) issue_tile(0, 0);
-  if (ntiles > 1) issue_tile(1, 1);
+  if (AHEAD > 1 && ntiles > 1) issue_tile(1, 1);
 
   const float c = p.scale_log2e;
   // after the mask term is folded in, the logits already are in the exp2 domain
@@ -317,21 +318,21 @@ __global__ __launch_bounds__(kAttThreads, 2) void attention_grouped_kernel(AttAr
   auto process_tile = [&](int t, auto masked_tag) {
     constexpr bool MASKED = decltype(masked_tag)::value;
     // this wave's share of tile t has landed once only tile t+1's four loads are outstanding
-    if (t + 1 < ntiles)
+    if (AHEAD > 1 && t + 1 < ntiles)
       att_wait_vmcnt<4>();
     else
       att_wait_vmcnt<0>();
     asm volatile("" ::: "memory");
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
-    if (t + 2 < ntiles) {
-      int ps = stage + 2;
-      if (ps >= kAttStages) ps -= kAttStages;
-      issue_tile(t + 2, ps);
+    if (t + AHEAD < ntiles) {
+      int ps = stage + AHEAD;
+      if (ps >= STAGES) ps -= STAGES;
+      issue_tile(t + AHEAD, ps);
     }
     // a wave whose queries all lie past the sequence only copies and keeps the barriers
     if (!wave_live) {
-      if (++stage == kAttStages) stage = 0;
+      if (++stage == STAGES) stage = 0;
       return;
     }
     const half_t *sK = ring + stage * 2 * kTileHalfs;
@@ -424,7 +425,7 @@ __global__ __launch_bounds__(kAttThreads, 2) void attention_grouped_kernel(AttAr
       for (int qb = 0; qb < QB; ++qb)
         o[4][qb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ones, pf[kk][qb], o[4][qb], 0, 0, 0);
     }
-    if (++stage == kAttStages) stage = 0;
+    if (++stage == STAGES) stage = 0;
   };
 
   // every tile but the last is full: no masking code on the steady-state path
@@ -702,23 +703,27 @@ extern "C" int bt_attention_grouped(const void *qkv_heads, void *attention_outpu
             nullptr, 0, batch_size, seq_len,
             rows_cap, head_num, scale * kLog2e, padded_rows};
   hipStream_t s = as_stream(stream);
-  // 128-query tiles once there is enough work to fill the chip, else 64
+  // 128-query tiles with a three-deep ring once there is plenty of work (three workgroups
+  // per CU); else 64-query tiles with a two-deep ring: 32 KB of LDS and ~100 registers let
+  // five workgroups share a CU, which hides more of the per-tile dependency chain than the
+  // third stage did (-0.1 to -2.8 % per forward from batch 1 x 256 to batch 16 x 384)
   const long long blocks128 = (long long)((seq_len + 127) / 128) * head_num * batch_size;
   const int qb = option_attention_qb();
-  if (qb == 2 || (qb < 0 && blocks128 >= 512)) {
+  const bool add = a.mask || a.bias;
+  if (qb == 2 || (qb < 0 && blocks128 >= 700)) {
     const unsigned grid = att_grid(a, (seq_len + 127) / 128);
     set_prefetch(a, grid, prefetch, prefetch_bytes);
-    if (a.mask || a.bias)
-      attention_grouped_kernel<2, true><<<grid, kAttThreads, 0, s>>>(a);
+    if (add)
+      attention_grouped_kernel<2, true, 3><<<grid, kAttThreads, 0, s>>>(a);
     else
-      attention_grouped_kernel<2, false><<<grid, kAttThreads, 0, s>>>(a);
+      attention_grouped_kernel<2, false, 3><<<grid, kAttThreads, 0, s>>>(a);
   } else {
     const unsigned grid = att_grid(a, (seq_len + 63) / 64);
     set_prefetch(a, grid, prefetch, prefetch_bytes);
-    if (a.mask || a.bias)
-      attention_grouped_kernel<1, true><<<grid, kAttThreads, 0, s>>>(a);
+    if (add)
+      attention_grouped_kernel<1, true, 2><<<grid, kAttThreads, 0, s>>>(a);
     else
-      attention_grouped_kernel<1, false><<<grid, kAttThreads, 0, s>>>(a);
+      attention_grouped_kernel<1, false, 2><<<grid, kAttThreads, 0, s>>>(a);
   }
   BT_CHECK_LAUNCH("attention_grouped_kernel");
   return BT_OK;
