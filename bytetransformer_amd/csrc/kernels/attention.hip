@@ -54,7 +54,7 @@ struct AttArgs {
   int padded_rows;
   int nqb;             // query tiles per sequence (set by the launcher)
   unsigned nqb_grid;   // host only: workgroups of the launch
-  int xcd_map;         // 1: XCD-aware workgroup order, 0: plain (tile, head, sequence) order
+  int xcd_map;         // 0: plain (tile, head, sequence) order, 1: XCD-aware, 2: XCD-aware and balanced over the CUs
 };
 
 // Which (sequence rank, head, query tile) a workgroup of the 1-D grid works on.  The
@@ -85,6 +85,76 @@ __device__ __forceinline__ AttItem att_item(const AttArgs &p) {
     it.exists = true;
   }
   return it;
+}
+
+// Balanced work list (xcd_map == 2, streaming kernel).  Within an XCD the hardware deals
+// consecutive workgroups to its 32 CUs round-robin (slot s of the XCD lands on CU s % 32),
+// and a launch of up to three workgroups per CU is resident at once, so the static order
+// alone decides what each CU gets.  With a fixed number of query-tile slots per sequence
+// the tile index is s % 4 at 512 tokens: one CU in four received only the last tiles -
+// dead for most sequences - while others held three live ones of the longest sequences.
+// Here the live (pair, query tile) items of the XCD - pairs p = x (mod 8) over the
+// longest-first order as above, the tiles of a pair adjacent - are counted on the device
+// and slot s takes item j = s in even rounds of 32 and the mirrored position in odd
+// rounds, so a CU that drew a long item in one round draws a short one in the next.
+// Every lane of a wave holds one rank: lengths, tile counts and a wave prefix sum invert
+// j -> (rank, head, tile) with the two dependent loads the plain lookup needs as well.
+// Inclusive prefix sum over the 64 lanes with data-parallel-primitive adds only: four
+// shifts inside each row of 16, then lane 15 of rows 0 / 2 into rows 1 / 3 and lane 31
+// into the upper half.
+__device__ __forceinline__ int wave_inclusive_sum(int v) {
+  v += __builtin_amdgcn_update_dpp(0, v, 0x111, 0xf, 0xf, true);   // row_shr:1
+  v += __builtin_amdgcn_update_dpp(0, v, 0x112, 0xf, 0xf, true);   // row_shr:2
+  v += __builtin_amdgcn_update_dpp(0, v, 0x114, 0xf, 0xf, true);   // row_shr:4
+  v += __builtin_amdgcn_update_dpp(0, v, 0x118, 0xf, 0xf, true);   // row_shr:8
+  v += __builtin_amdgcn_update_dpp(0, v, 0x142, 0xa, 0xf, false);  // row_bcast:15 -> rows 1, 3
+  v += __builtin_amdgcn_update_dpp(0, v, 0x143, 0xc, 0xf, false);  // row_bcast:31 -> rows 2, 3
+  return v;
+}
+
+struct AttWork {
+  int b, head, qb, seq_start, len;
+  bool exists;
+};
+template <int BQ>
+__device__ __forceinline__ AttWork att_work_balanced(const AttArgs &p) {
+  AttWork w{0, 0, 0, 0, 0, false};
+  const int lane = threadIdx.x & 63;
+  const int x = blockIdx.x & 7, s = blockIdx.x >> 3;
+  const int round = s >> 5, pos = s & 31;
+  const int j = (round << 5) + ((round & 1) ? 31 - pos : pos);
+  int carry = 0;
+  for (int base = 0; base < p.B; base += 64) {
+    const int r = base + lane;
+    const bool valid = r < p.B;
+    const int seq = valid ? (p.seq_order ? p.seq_order[r] : r) : 0;
+    const int start = p.batch_idx[seq];
+    const int len = valid ? p.batch_idx[seq + 1] - start : 0;
+    const int nq = p.padded_rows ? p.S : len;
+    const int nqb = valid ? min((nq + BQ - 1) / BQ, p.nqb) : 0;
+    const int first = r * p.heads;   // pairs [first, first + heads) belong to rank r
+    const int cnt = ((first + p.heads + 7 - x) >> 3) - ((first + 7 - x) >> 3);
+    const int mine = cnt * nqb;
+    const int incl = wave_inclusive_sum(mine);
+    const int lo = carry + incl - mine;   // first item of this rank
+    const unsigned long long hit = __builtin_amdgcn_ballot_w64(mine > 0 && j >= lo && j < lo + mine);
+    if (hit) {
+      const int src = __builtin_ctzll(hit);
+      const int jj = j - __builtin_amdgcn_readlane(lo, src);
+      const int nqb_s = __builtin_amdgcn_readlane(nqb, src);
+      const int first_s = (base + src) * p.heads;
+      w.b = __builtin_amdgcn_readlane(seq, src);
+      w.seq_start = __builtin_amdgcn_readlane(start, src);
+      w.len = __builtin_amdgcn_readlane(len, src);
+      w.qb = jj % nqb_s;
+      // the (jj / nqb_s)-th head h of the rank with first_s + h = x (mod 8)
+      w.head = ((x - first_s) & 7) + 8 * (jj / nqb_s);
+      w.exists = true;
+      return w;
+    }
+    carry += __builtin_amdgcn_readlane(incl, 63);
+  }
+  return w;
 }
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
@@ -232,18 +302,30 @@ __global__ __launch_bounds__(kAttThreads, 2) void attention_grouped_kernel(AttAr
   static_assert(STAGES == 2 || STAGES == 3, "ring depth");
   __shared__ __attribute__((aligned(1024))) half_t ring[STAGES * 2 * kTileHalfs];
 
-  const AttItem item = att_item(p);
-  if (!item.exists) {
-    prefetch_slice(p);
-    return;
+  int b, head, seq_start, seq_len, qb_index;
+  if (p.xcd_map == 2) {
+    const AttWork w = att_work_balanced<BQ>(p);
+    if (!w.exists) {
+      prefetch_slice(p);
+      return;
+    }
+    b = w.b, head = w.head, seq_start = w.seq_start, seq_len = w.len, qb_index = w.qb;
+  } else {
+    const AttItem item = att_item(p);
+    if (!item.exists) {
+      prefetch_slice(p);
+      return;
+    }
+    b = p.seq_order ? p.seq_order[item.rank] : item.rank, head = item.head;
+    seq_start = p.batch_idx[b];
+    seq_len = p.batch_idx[b + 1] - seq_start;
+    qb_index = item.qb;
   }
-  const int b = p.seq_order ? p.seq_order[item.rank] : item.rank, head = item.head;
-  const int seq_start = p.batch_idx[b];
   // with a mask tensor every one of the S key rows takes part
-  const int klen = ADD && p.mask ? p.S : p.batch_idx[b + 1] - seq_start;
+  const int klen = ADD && p.mask ? p.S : seq_len;
   const int row_start = p.padded_rows ? b * p.S : seq_start;
   const int nq = p.padded_rows ? p.S : klen;
-  const int q0 = item.qb * BQ;
+  const int q0 = qb_index * BQ;
   if (q0 >= nq) {
     prefetch_slice(p);
     return;
@@ -615,10 +697,17 @@ static void set_prefetch(AttArgs &a, unsigned grid, const void *prefetch, unsign
 }
 
 // Size of the 1-D grid for `nqb` query tiles per sequence; fills the mapping fields.
-static unsigned att_grid(AttArgs &a, int nqb) {
+static unsigned att_grid(AttArgs &a, int nqb, bool streaming = false) {
   a.nqb = nqb;
   a.xcd_map = option_attention_xcd_map();
   const unsigned pairs = (unsigned)a.B * a.heads;
+  // The balanced list is the streaming kernel's, and pays from the third round of 32
+  // workgroups per XCD on: up to two rounds its look-up (vector loads and a wave scan
+  // where the plain order needs three scalar loads) cost 0.3-1.5 % per forward.
+  if (a.xcd_map == 2 && (pairs + 7) / 8 * nqb <= 64) a.xcd_map = 1;
+  if (a.xcd_map == 3) a.xcd_map = 2;   // option value 3: the balanced list at any size
+  if (a.xcd_map == 2 && !streaming) a.xcd_map = 1;
+  if (a.xcd_map == 2) return ((pairs + 7) / 8 * nqb + 31) / 32 * 32 * 8;   // whole rounds of 32 per XCD
   return a.xcd_map ? (pairs + 7) / 8 * 8 * nqb : pairs * nqb;
 }
 
@@ -706,19 +795,21 @@ extern "C" int bt_attention_grouped(const void *qkv_heads, void *attention_outpu
   // 128-query tiles with a three-deep ring once there is plenty of work (three workgroups
   // per CU); else 64-query tiles with a two-deep ring: 32 KB of LDS and ~100 registers let
   // five workgroups share a CU, which hides more of the per-tile dependency chain than the
-  // third stage did (-0.1 to -2.8 % per forward from batch 1 x 256 to batch 16 x 384)
+  // third stage did (-0.1 to -2.8 % per forward from batch 1 x 256 to batch 16 x 384; with
+  // the balanced work list also -0.8 to -1.9 % at batch 32 x 256 / 384 and 16 x 768, so the
+  // switch sits at 1300 workgroups of 128 queries; batch 16 x 512 is within 0.3 % either way)
   const long long blocks128 = (long long)((seq_len + 127) / 128) * head_num * batch_size;
   const int qb = option_attention_qb();
   const bool add = a.mask || a.bias;
-  if (qb == 2 || (qb < 0 && blocks128 >= 700)) {
-    const unsigned grid = att_grid(a, (seq_len + 127) / 128);
+  if (qb == 2 || (qb < 0 && blocks128 >= 1300)) {
+    const unsigned grid = att_grid(a, (seq_len + 127) / 128, true);
     set_prefetch(a, grid, prefetch, prefetch_bytes);
     if (add)
       attention_grouped_kernel<2, true, 3><<<grid, kAttThreads, 0, s>>>(a);
     else
       attention_grouped_kernel<2, false, 3><<<grid, kAttThreads, 0, s>>>(a);
   } else {
-    const unsigned grid = att_grid(a, (seq_len + 63) / 64);
+    const unsigned grid = att_grid(a, (seq_len + 63) / 64, true);
     set_prefetch(a, grid, prefetch, prefetch_bytes);
     if (add)
       attention_grouped_kernel<1, true, 2><<<grid, kAttThreads, 0, s>>>(a);

@@ -32,7 +32,7 @@ static std::atomic<int> g_attention_qb{-1};
 static std::atomic<int> g_prefetch{1};
 static std::atomic<int> g_f32_gemm_tile{-1};
 static std::atomic<int> g_attention_short_limit{0};
-static std::atomic<int> g_attention_xcd_map{1};
+static std::atomic<int> g_attention_xcd_map{2};
 int option_attention_xcd_map() { return g_attention_xcd_map.load(std::memory_order_relaxed); }
 int option_f32_gemm_tile() { return g_f32_gemm_tile.load(std::memory_order_relaxed); }
 int option_gemm_tile() { return g_gemm_tile.load(std::memory_order_relaxed); }
@@ -150,8 +150,8 @@ extern "C" int bt_set_option(const char *name, int value) {
                "bt_set_option: attention_short_limit=%d outside [0, 512]", value);
     g_attention_short_limit.store(value);
   } else if (!strcmp(name, "attention_xcd_map")) {
-    BT_REQUIRE(value == 0 || value == 1, BT_ERR_INVALID_ARGUMENT,
-               "bt_set_option: attention_xcd_map=%d must be 0 or 1", value);
+    BT_REQUIRE(value >= 0 && value <= 3, BT_ERR_INVALID_ARGUMENT,
+               "bt_set_option: attention_xcd_map=%d outside [0, 3]", value);
     g_attention_xcd_map.store(value);
   } else if (!strcmp(name, "prefetch")) {
     BT_REQUIRE(value == 0 || value == 1, BT_ERR_INVALID_ARGUMENT,

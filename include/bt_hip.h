@@ -57,8 +57,10 @@ const char *bt_last_error_string(void);
  *   "attention_short_limit"  0 (default) .. 512: the host library sends sequences up to this
  *                   length to bt_attention_short when use_fused_attention is set; 0 = always
  *                   the streaming kernel, which measures faster at every length
- *   "attention_xcd_map"  1 (default) | 0: XCD-aware or plain workgroup order of the fp16
- *                   attention kernels
+ *   "attention_xcd_map"  workgroup order of the fp16 attention kernels: 0 plain | 1 XCD-aware
+ *                   | 2 (default) XCD-aware, and in the streaming kernel the live query
+ *                   tiles are dealt evenly to the CUs once the launch has more than two
+ *                   rounds of workgroups per CU | 3: that balanced order at any size
  * Process-wide; results do not depend on it beyond fp32 summation order.
  */
 int bt_set_option(const char *name, int value);

@@ -397,8 +397,61 @@ def test_attention_packed(device, kind, lens, S, heads, qb):
     assert np.all(g[M:] == 5.0)
 
 
+@pytest.fixture(params=[2, 3], ids=["default-order", "balanced-order"])
+def att_order(request):
+    """Runs a test under the default workgroup order and with the balanced work list
+    forced on (small launches would not use it by themselves)."""
+    ops.set_option("attention_xcd_map", request.param)
+    yield request.param
+    ops.set_option("attention_xcd_map", 2)
+
+
+ORDER_CASES = [
+    ([512, 103, 257, 64, 65, 1, 0, 300], 512, 3),
+    ([33, 2, 47], 47, 5),
+    ([154], 256, 12),
+    (list(np.random.RandomState(7).randint(0, 97, size=70)), 96, 2),    # more sequences than lanes
+    (list(np.random.RandomState(8).randint(1, 193, size=131)), 192, 1),  # three passes of 64 ranks
+]
+
+
+@pytest.mark.parametrize("qb", [1, 2])
+@pytest.mark.parametrize("lens,S,heads", ORDER_CASES)
+def test_attention_workgroup_orders_agree(device, lens, S, heads, qb):
+    """Plain, XCD-aware and balanced workgroup orders (and the identity or longest-first
+    sequence order under each) visit every live query tile exactly once: same bits out,
+    rows past the last token untouched, and the oracle's values."""
+    lens = [int(v) for v in lens]
+    _say("attention orders", len(lens), S, heads, qb)
+    rs = np.random.RandomState(S * 7 + heads)
+    bi, M, qkv = _attention_case(rs, lens, S, heads)
+    scale = 1 / math.sqrt(64)
+    exp = O.attention_packed(qkv[0, :, :M], qkv[1, :, :M], qkv[2, :, :M], bi, scale, 1e-6,
+                             round_p_fp16=True)
+    order = _dev(np.argsort(-np.asarray(lens), kind="stable").astype(np.int32), device)
+    outs = []
+    ops.set_option("attention_qb", qb)
+    try:
+        for mode in (0, 1, 2, 3):
+            ops.set_option("attention_xcd_map", mode)
+            for so in (None, order):
+                out = torch.full((len(lens) * S, heads * 64), 5.0, dtype=torch.float16, device=device)
+                ops.attention_grouped(_dev(qkv, device), _dev(bi, device), len(lens), S, scale, False,
+                                      out=out, seq_order=so)
+                outs.append(out)
+    finally:
+        ops.set_option("attention_qb", -1)
+        ops.set_option("attention_xcd_map", 2)
+    for o in outs[1:]:
+        assert torch.equal(o, outs[0])
+    g = outs[-1].cpu().numpy()
+    err = np.abs(g[:M].astype(np.float64) - exp)
+    assert err.max() <= 4e-3 and err.mean() <= 4e-4, (err.max(), err.mean())
+    assert np.all(g[M:] == 5.0)
+
+
 @pytest.mark.parametrize("kind", ["short", "grouped"])
-def test_attention_padded_rows_mode(device, kind):
+def test_attention_padded_rows_mode(device, kind, att_order):
     """Padded layout: sequence b owns rows [b*S, (b+1)*S); every query row is
     computed against the len_b valid keys."""
     _say("attention padded", kind)
@@ -425,7 +478,7 @@ def test_attention_padded_rows_mode(device, kind):
 
 @pytest.mark.parametrize("kind,S", [("short", 64), ("short", 200), ("grouped", 200),
                                      ("grouped", 70), ("short", 37), ("grouped", 640)])
-def test_attention_arbitrary_mask_on_padded_rows(device, kind, S):
+def test_attention_arbitrary_mask_on_padded_rows(device, kind, S, att_order):
     """With the mask tensor given, every (query, key) pair follows mask[b,q,k]:
     logits are shifted by (mask-1)*10000 as in the reference's non-remove-padding
     kernels - banded, random and fully-masked rows included."""
@@ -458,7 +511,7 @@ def test_attention_arbitrary_mask_on_padded_rows(device, kind, S):
 @pytest.mark.parametrize("kind,S,padded,with_mask", [("short", 64, True, True), ("grouped", 200, True, True),
                                                     ("short", 100, False, False), ("grouped", 300, False, False),
                                                     ("grouped", 130, True, False)])
-def test_attention_bias(device, kind, S, padded, with_mask):
+def test_attention_bias(device, kind, S, padded, with_mask, att_order):
     """attention_bias[h, q, k] is added to the scaled logits (positions relative to
     the sequence start) in the packed and the padded row layout, with and without
     the mask tensor."""
