@@ -794,7 +794,7 @@ extern "C" int bt_attention_grouped(const void *qkv_heads, void *attention_outpu
   hipStream_t s = as_stream(stream);
   // 128-query tiles with a three-deep ring once there is plenty of work (three workgroups
   // per CU); else 64-query tiles with a two-deep ring: 32 KB of LDS and ~100 registers let
-  // five workgroups share a CU, which hides more of the per-tile dependency chain than the
+  // four workgroups share a CU (a build held to 84 registers fits five and measures the same), which hides more of the per-tile dependency chain than the
   // third stage did (-0.1 to -2.8 % per forward from batch 1 x 256 to batch 16 x 384; with
   // the balanced work list also -0.8 to -1.9 % at batch 32 x 256 / 384 and 16 x 768, so the
   // switch sits at 1300 workgroups of 128 queries; batch 16 x 512 is within 0.3 % either way)
