@@ -704,7 +704,9 @@ static unsigned att_grid(AttArgs &a, int nqb, bool streaming = false) {
   // The balanced list is the streaming kernel's, and pays from the third round of 32
   // workgroups per XCD on: up to two rounds its look-up (vector loads and a wave scan
   // where the plain order needs three scalar loads) cost 0.3-1.5 % per forward.
-  if (a.xcd_map == 2 && (pairs + 7) / 8 * nqb <= 64) a.xcd_map = 1;
+  // Its look-up takes one pass (two dependent loads) per 64 sequences: beyond 128 the
+  // plain order stays, and so many sequences even out by themselves.
+  if (a.xcd_map == 2 && ((pairs + 7) / 8 * nqb <= 64 || a.B > 128)) a.xcd_map = 1;
   if (a.xcd_map == 3) a.xcd_map = 2;   // option value 3: the balanced list at any size
   if (a.xcd_map == 2 && !streaming) a.xcd_map = 1;
   if (a.xcd_map == 2) return ((pairs + 7) / 8 * nqb + 31) / 32 * 32 * 8;   // whole rounds of 32 per XCD

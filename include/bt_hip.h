@@ -60,7 +60,8 @@ const char *bt_last_error_string(void);
  *   "attention_xcd_map"  workgroup order of the fp16 attention kernels: 0 plain | 1 XCD-aware
  *                   | 2 (default) XCD-aware, and in the streaming kernel the live query
  *                   tiles are dealt evenly to the CUs once the launch has more than two
- *                   rounds of workgroups per CU | 3: that balanced order at any size
+ *                   rounds of workgroups per CU (batches up to 128 sequences) | 3: that
+ *                   balanced order at any size
  * Process-wide; results do not depend on it beyond fp32 summation order.
  */
 int bt_set_option(const char *name, int value);
