@@ -70,6 +70,14 @@ void BertTransformer<OpType>::bert_infer(BertTransformerInferParam infer_param) 
   const int *valid_rows = nullptr;
   const int *gather = nullptr;
   DataType_ *restore_target = nullptr;
+  // Row capacity of the launches over packed rows that follow the attention.  The
+  // caller's offsets carry the exact live count (the operator's mask plan read it back
+  // once), so these launches are sized for it instead of batch * seq_len: no workgroups
+  // that only find out on the device that their rows do not exist (1.7-2.2 us per layer
+  // at batch 16 x 512), and a short sequence in a long padded row still takes the split-k
+  // FFN2.  The QKV product and the attention keep batch * seq_len: it is the row stride
+  // of the per-head Q/K/V layout and the extent of the gathered input.
+  int packed_cap = rows;
   if (is_remove_padding_) {
     // The packed copy of the input is never materialised: the QKV GEMM and the
     // first LayerNorm read valid token t from the padded input at row word_idx[t]
@@ -78,6 +86,7 @@ void BertTransformer<OpType>::bert_infer(BertTransformerInferParam infer_param) 
     restore_target = transformer_out;
     transformer_out = inner_buf;  // FFN2 output reuses the dead qkv region
     valid_rows = et_param.batch_idx + batch_size;
+    if (rows_hint > 0 && rows_hint < rows) packed_cap = rows_hint;
   }
 
   if constexpr (OpType == OperationType::FP32) {
@@ -154,36 +163,36 @@ void BertTransformer<OpType>::bert_infer(BertTransformerInferParam infer_param) 
   attention_layer_->infer(attention_infer_param);
 
   check_bt_error(
-      bt_gemm(attr_out_buf, wt_proj, attr_matmul_buf, valid_rows, rows, rows_hint, hidden, hidden,
-              stream));
+      bt_gemm(attr_out_buf, wt_proj, attr_matmul_buf, valid_rows, packed_cap, rows_hint, hidden,
+              hidden, stream));
 
   check_bt_error(bt_add_bias_residual_layernorm(
       attr_matmul_buf, from_tensor, gather, param_.attr_output_bias, param_.attr_output_layernorm_gamma,
-      param_.attr_output_layernorm_beta, use_fp32_ ? 1 : 0, valid_rows, rows, hidden,
+      param_.attr_output_layernorm_beta, use_fp32_ ? 1 : 0, valid_rows, packed_cap, hidden,
       layernorm_eps, stream));
 
   check_bt_error(bt_gemm_bias_gelu(attr_matmul_buf, wt_inter, param_.inter_bias, inter_matmul_buf,
-                                   valid_rows, rows, rows_hint, inter, hidden, stream));
+                                   valid_rows, packed_cap, rows_hint, inter, hidden, stream));
 
   // few rows, long k: FFN2 as split-k partial sums that the last LayerNorm folds in
   const long long rows_expected =
       !valid_rows ? rows : (rows_hint > 0 ? rows_hint : (rows * 3LL + 4) / 5);
-  const int splits = splitk_splits(rows, rows_expected, inter);
+  const int splits = splitk_splits(packed_cap, rows_expected, inter);
   if (splits > 1) {
-    check_bt_error(bt_gemm_splitk(inter_matmul_buf, wt_out, splitk_buf, splits, valid_rows, rows,
-                                  hidden, inter, stream));
+    check_bt_error(bt_gemm_splitk(inter_matmul_buf, wt_out, splitk_buf, splits, valid_rows,
+                                  packed_cap, hidden, inter, stream));
     check_bt_error(bt_splitk_layernorm(
         splitk_buf, splits, attr_matmul_buf, nullptr, param_.output_bias,
         param_.output_layernorm_gamma, param_.output_layernorm_beta, use_fp32_ ? 1 : 0,
         is_remove_padding_ ? restore_target : transformer_out,
-        is_remove_padding_ ? et_param.batch_idx : nullptr, nullptr, batch_size, seq_len, rows,
-        hidden, layernorm_eps, stream));
+        is_remove_padding_ ? et_param.batch_idx : nullptr, nullptr, batch_size, seq_len,
+        packed_cap, hidden, layernorm_eps, stream));
     return;
   }
 
   check_bt_error(
-      bt_gemm(inter_matmul_buf, wt_out, transformer_out, valid_rows, rows, rows_hint, hidden, inter,
-              stream));
+      bt_gemm(inter_matmul_buf, wt_out, transformer_out, valid_rows, packed_cap, rows_hint, hidden,
+              inter, stream));
 
   if (is_remove_padding_)
     check_bt_error(bt_add_bias_residual_layernorm_restore(

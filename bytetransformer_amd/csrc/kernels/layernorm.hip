@@ -12,15 +12,15 @@ namespace bt {
 
 constexpr int kLnRowsPerBlock = 4;
 
-// SPLITS > 0: `src` holds SPLITS fp32 partial sums of the row ([SPLITS][rows_cap][H], the
+// SPLITS > 0: `src` holds SPLITS fp32 partial sums of the row ([SPLITS][split_rows][H], the
 // output of a split-k GEMM); their sum, rounded to fp16 once, takes the place of `out`.
 template <int NC, bool RESTORE, bool GB32, int SPLITS>
 __global__ __launch_bounds__(kLnRowsPerBlock *kWave) void layernorm_kernel(
     const half8_t *src, const half8_t *__restrict__ residual,
     const half8_t *__restrict__ bias, const void *__restrict__ gamma,
     const void *__restrict__ beta, half8_t *dst, const int *__restrict__ idx,
-    const int *__restrict__ residual_row_index, int B, int S, int rows_cap, int chunks,
-    float inv_n, float eps) {
+    const int *__restrict__ residual_row_index, int B, int S, int rows_cap, int split_rows,
+    int chunks, float inv_n, float eps) {
   const int r = blockIdx.x * kLnRowsPerBlock + (threadIdx.x >> 6);
   const int lane = threadIdx.x & 63;
   if (r >= rows_cap) return;
@@ -58,8 +58,8 @@ __global__ __launch_bounds__(kLnRowsPerBlock *kWave) void layernorm_kernel(
         float4_t lo = pp[0], hi = pp[1];
 #pragma unroll
         for (int sp = 1; sp < SPLITS; ++sp) {
-          lo += pp[(size_t)sp * rows_cap * chunks * 2];
-          hi += pp[(size_t)sp * rows_cap * chunks * 2 + 1];
+          lo += pp[(size_t)sp * split_rows * chunks * 2];
+          hi += pp[(size_t)sp * split_rows * chunks * 2 + 1];
         }
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
@@ -132,7 +132,7 @@ template <bool RESTORE, int SPLITS = 0>
 static int launch_ln(const void *src, const void *residual, const void *bias, const void *gamma,
                      const void *beta, int gb32, void *dst, const int *idx,
                      const int *residual_row_index, int B, int S, int rows_cap, int H, float eps,
-                     hipStream_t s, const char *who) {
+                     hipStream_t s, const char *who, int split_rows = 0) {
   BT_REQUIRE(H > 0 && H % 8 == 0, BT_ERR_UNSUPPORTED, "%s: hidden_dim %d must be a multiple of 8",
              who, H);
   BT_REQUIRE(aligned16({src, residual, bias, gamma, beta, dst}), BT_ERR_INVALID_ARGUMENT,
@@ -146,7 +146,8 @@ static int launch_ln(const void *src, const void *residual, const void *bias, co
 #define BT_LN_LAUNCH(NC_, GB_)                                                                  \
   layernorm_kernel<NC_, RESTORE, GB_, SPLITS><<<grid, kLnRowsPerBlock * kWave, 0, s>>>(         \
       (const half8_t *)src, (const half8_t *)residual, (const half8_t *)bias, gamma, beta,      \
-      (half8_t *)dst, idx, residual_row_index, B, S, rows_cap, chunks, inv_n, eps)
+      (half8_t *)dst, idx, residual_row_index, B, S, rows_cap, split_rows ? split_rows : rows_cap, \
+      chunks, inv_n, eps)
 #define BT_LN_NC(NC_)              \
   do {                             \
     if (gb32)                      \
@@ -219,18 +220,21 @@ extern "C" int bt_splitk_layernorm(const void *partials, int splits, const void 
   hipStream_t s = as_stream(stream);
   if (batch_idx) {
     // restore mode: dst is the padded [batch_size, seq_len, hidden] output
-    BT_REQUIRE(batch_size > 0 && seq_len > 0 && (long long)batch_size * seq_len == rows_cap,
+    // rows_cap is the row count of one partial-sum slice (what bt_gemm_splitk was given)
+    BT_REQUIRE(batch_size > 0 && seq_len > 0 && (long long)batch_size * seq_len < (1ll << 31) &&
+                   rows_cap > 0 && rows_cap <= batch_size * seq_len,
                BT_ERR_INVALID_ARGUMENT,
-               "bt_splitk_layernorm: restore needs rows_cap == batch_size * seq_len");
+               "bt_splitk_layernorm: restore needs 0 < rows_cap <= batch_size * seq_len");
     BT_REQUIRE(!residual_row_index, BT_ERR_INVALID_ARGUMENT,
                "bt_splitk_layernorm: no residual gather in restore mode");
+    const int padded = batch_size * seq_len;
     return splits == 2
                ? launch_ln<true, 2>(partials, residual, bias, gamma, beta, gamma_beta_fp32, dst,
-                                    batch_idx, nullptr, batch_size, seq_len, rows_cap, hidden_dim,
-                                    eps, s, "bt_splitk_layernorm")
+                                    batch_idx, nullptr, batch_size, seq_len, padded, hidden_dim,
+                                    eps, s, "bt_splitk_layernorm", rows_cap)
                : launch_ln<true, 4>(partials, residual, bias, gamma, beta, gamma_beta_fp32, dst,
-                                    batch_idx, nullptr, batch_size, seq_len, rows_cap, hidden_dim,
-                                    eps, s, "bt_splitk_layernorm");
+                                    batch_idx, nullptr, batch_size, seq_len, padded, hidden_dim,
+                                    eps, s, "bt_splitk_layernorm", rows_cap);
   }
   BT_REQUIRE(!residual_row_index || valid_rows, BT_ERR_INVALID_ARGUMENT,
              "bt_splitk_layernorm: residual_row_index needs valid_rows");

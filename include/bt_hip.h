@@ -236,7 +236,9 @@ int bt_add_bias_residual_layernorm_restore(const void *out, const void *residual
  * partials (summed, rounded to fp16 once) in the place of `out`; splits 2 or 4.
  * batch_idx == NULL: packed rows, dst [rows_cap, hidden] (valid_rows / residual_row_index as
  * in bt_add_bias_residual_layernorm); batch_idx != NULL: dst is the padded
- * [batch_size, seq_len, hidden] output with zero fill, rows_cap == batch_size * seq_len.
+ * [batch_size, seq_len, hidden] output with zero fill, and rows_cap (<= batch_size *
+ * seq_len, >= the live rows) is the row count of one slice of the partials, i.e. the
+ * rows_cap that bt_gemm_splitk was given.
  */
 int bt_gemm_splitk(const void *a, const void *wt, void *partials, int splits,
                    const int *valid_rows, int rows_cap, int n, int k, void *stream);

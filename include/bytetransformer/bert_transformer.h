@@ -63,7 +63,9 @@ struct BertTransformerInferParam {
   // Extension (no counterpart in the reference): offsets already built from this
   // very atten_mask by bt_build_offsets (batch_idx int[batch_size+1], word_idx
   // int[batch_size*seq_len], valid_word_num = their total).  When set, infer()
-  // skips its own mask prefix sum and uses valid_word_num to pick tile shapes.
+  // skips its own mask prefix sum.  valid_word_num must be the exact total (as the
+  // reference's ET_Param carries it) or 0 when the host does not know it: a positive
+  // value sizes the launches over packed rows and picks their tile shapes.
   const ET_Param *offsets = NULL;
   // ... and the matching sequence order (int[batch_size], longest first), or NULL.
   const int *seq_order = NULL;

@@ -54,8 +54,8 @@ typedef struct {
 
 // FFN2 with few rows and a long k runs as a split-k GEMM whose fp32 partial sums the last
 // LayerNorm folds in (bt_gemm_splitk / bt_splitk_layernorm): 4 splits up to 192 expected
-// rows, 2 up to 272, none beyond or when the batch has more than kSplitKMaxRows padded rows
-// (the partials live in a scratch area sized for that).
+// rows, 2 up to 272, none beyond or when the launch is sized for more than kSplitKMaxRows
+// rows (the partials live in a scratch area sized for that many).
 constexpr int kSplitKMaxRows = 512;
 inline int splitk_splits(long long rows_cap, long long rows_expected, int k) {
   static const bool enabled = [] {

@@ -455,6 +455,25 @@ def test_seq_len_one(device, dtype):
     _check(_run_th_op(wl, device), exp, wl.lens, tag="seq_len 1/th_op/" + dtype)
 
 
+@pytest.mark.parametrize("B,S,lens,heads", [
+    # (remove-padding needs a batch of three or more, as in the reference)
+    (3, 1024, (200, 0, 0), 12),         # split-k FFN2 although batch * seq_len is beyond its limit
+    (3, 640, (0, 333, 0), 12),          # the same shape without split-k
+    (4, 256, (256, 1, 100, 17), 4),     # several sequences, one of them full
+    (3, 128, (0, 128, 0), 2),           # empty sequences around a full one
+])
+def test_operator_sizes_packed_launches_for_the_live_rows(device, B, S, lens, heads):
+    """The operator knows the exact number of live rows (its mask plan reads it back) and
+    sizes the launches after the attention for it; the per-layer C entry does not and sizes
+    them for batch * seq_len.  Both must give the oracle's layer, padded rows zero."""
+    ffn = 4 if heads * 64 * 4 >= 2048 else 16    # split-k needs k >= 2048
+    cfg = workload.EncoderConfig("tight", B, S, heads, layers=2, lens=lens, ffn_mult=ffn)
+    wl = workload.make_workload(cfg, bias_std=0.05, random_affine=True)
+    exp = _oracle(wl)
+    _check(_run_th_op(wl, device), exp, wl.lens, tag="live-row capacity/th_op")
+    _check(_run_c_api(wl, device), exp, wl.lens, tag="live-row capacity/c_api")
+
+
 def test_default_dispatch_is_the_streaming_kernel(device):
     """attention_short_limit defaults to 0: with it the fused flag changes nothing, and the
     result still matches the oracle."""
