@@ -103,15 +103,18 @@ void BertTransformer<OpType>::bert_infer(BertTransformerInferParam infer_param) 
     attention_infer_param.seq_order = seq_order;
     attention_layer_->infer(attention_infer_param);
     check_bt_error(bt_gemm_f32(attr_out_buf, nullptr, param_.attr_output_kernel, nullptr,
-                               attr_matmul_buf, 0, valid_rows, rows, rows_hint, hidden, hidden, stream));
+                               attr_matmul_buf, 0, valid_rows, packed_cap, rows_hint, hidden, hidden,
+                               stream));
     check_bt_error(bt_add_bias_residual_layernorm_f32(
         attr_matmul_buf, from_tensor, gather, param_.attr_output_bias,
-        param_.attr_output_layernorm_gamma, param_.attr_output_layernorm_beta, valid_rows, rows,
-        hidden, layernorm_eps, stream));
+        param_.attr_output_layernorm_gamma, param_.attr_output_layernorm_beta, valid_rows,
+        packed_cap, hidden, layernorm_eps, stream));
     check_bt_error(bt_gemm_f32(attr_matmul_buf, nullptr, param_.inter_kernel, param_.inter_bias,
-                               inter_matmul_buf, 1, valid_rows, rows, rows_hint, inter, hidden, stream));
+                               inter_matmul_buf, 1, valid_rows, packed_cap, rows_hint, inter, hidden,
+                               stream));
     check_bt_error(bt_gemm_f32(inter_matmul_buf, nullptr, param_.output_kernel, nullptr,
-                               transformer_out, 0, valid_rows, rows, rows_hint, hidden, inter, stream));
+                               transformer_out, 0, valid_rows, packed_cap, rows_hint, hidden, inter,
+                               stream));
     if (is_remove_padding_)
       check_bt_error(bt_add_bias_residual_layernorm_restore_f32(
           transformer_out, attr_matmul_buf, param_.output_bias, param_.output_layernorm_gamma,
