@@ -355,6 +355,29 @@ def test_random_small_configurations(device, seed):
     assert pads_zero
 
 
+@pytest.mark.parametrize("rm", [True, False])
+def test_balanced_workgroup_order_through_the_layer(device, rm):
+    """The streaming attention kernel with its balanced work list forced on (small launches
+    keep the plain order by themselves): ragged and empty sequences, with and without
+    remove-padding, bit-identical to the default order."""
+    from bytetransformer_amd import ops
+    cfg = workload.EncoderConfig("bal", 7, 200, 3, layers=2, lens=(200, 0, 77, 1, 130, 64, 199))
+    wl = workload.make_workload(cfg, bias_std=0.05, random_affine=True)
+    exp = _oracle(wl)
+    ops.set_option("attention_short_limit", 0)
+    try:
+        ops.set_option("attention_xcd_map", 3)
+        got = _run_c_api(wl, device, is_remove_padding=rm)
+        ops.set_option("attention_xcd_map", 1)
+        ref = _run_c_api(wl, device, is_remove_padding=rm)
+    finally:
+        ops.set_option("attention_xcd_map", 2)
+    assert np.array_equal(got, ref)
+    if not rm:
+        got = O.masked_output(got, wl.lens)
+    _check(got, exp, wl.lens, tag="balanced order rm=%s" % rm)
+
+
 @pytest.mark.parametrize("seed", range(24))
 def test_random_whole_encoder_bias_masks_and_operator(device, seed):
     """Seeded random stacks of 1-3 layers through the whole-encoder entry and the PyTorch
