@@ -206,6 +206,58 @@ def test_gemm_random_shapes_all_tiles_and_auto(device, seed):
         ops.set_option("gemm_tile", -1)
 
 
+@pytest.mark.parametrize("seed", range(6))
+def test_gemm_row_hint_never_changes_the_result(device, seed):
+    """rows_hint only steers the launch (tile shape): with the tile pinned, hints from far
+    too small to too large give the bits of a launch without a hint, for every tile shape
+    and the three epilogues; with the automatic choice the oracle's values."""
+    rs = np.random.RandomState(900 + seed)
+    rows = int(rs.randint(300, 1500))
+    M = int(rs.randint(rows // 2, rows + 1))
+    heads = int(rs.randint(1, 4))
+    H = 64 * heads
+    F = 64 * int(rs.randint(2, 9))
+    _say("gemm hint", seed, rows, M, H, F)
+    a = rs.standard_normal((rows, H)).astype(np.float16)
+    a[M:] = np.float16("nan")
+    w1 = (rs.standard_normal((H, F)) * 0.05).astype(np.float16)
+    wq = (rs.standard_normal((H, 3 * H)) * 0.05).astype(np.float16)
+    b1 = (rs.standard_normal(F) * 0.1).astype(np.float16)
+    bq = (rs.standard_normal(3 * H) * 0.1).astype(np.float16)
+    ad, vr = _dev(a, device), torch.tensor([M], dtype=torch.int32, device=device)
+    wt1, wtq = ops.transpose_weight(_dev(w1, device)), ops.transpose_weight(_dev(wq, device))
+    b1d, bqd = _dev(b1, device), _dev(bq, device)
+    exp = O.gemm(a[:M], w1)
+    tol = _gemm_tol(exp, H, np.abs(a[:M]).max(), np.abs(w1).max())
+
+    def run(hint):
+        o1 = torch.full((rows, F), 3.0, dtype=torch.float16, device=device)
+        o2 = torch.full((rows, F), 3.0, dtype=torch.float16, device=device)
+        o3 = torch.full((3, heads, rows, 64), 3.0, dtype=torch.float16, device=device)
+        ops.gemm(ad, wt1, valid_rows=vr, out=o1, rows_hint=hint)
+        ops.gemm_bias_gelu(ad, wt1, b1d, valid_rows=vr, out=o2, rows_hint=hint)
+        ops.gemm_qkv_bias_split(ad, wtq, bqd, heads, valid_rows=vr, out=o3, rows_hint=hint)
+        return o1, o2, o3
+
+    try:
+        for tile in (0, 1, 2, 3, 4, 5):
+            ops.set_option("gemm_tile", tile)
+            ref = run(0)
+            g = ref[0].cpu().numpy()
+            assert np.all(np.abs(g[:M].astype(np.float64) - exp) <= tol), tile
+            assert np.all(g[M:] == 3.0), tile
+            for hint in (1, 33, M // 3, M - 1, M, rows):
+                for got, want in zip(run(hint), ref):
+                    assert torch.equal(got, want), (tile, hint)
+        ops.set_option("gemm_tile", -1)
+        for hint in (1, M // 3, M, rows):
+            g = run(hint)[0].cpu().numpy()
+            assert np.all(np.abs(g[:M].astype(np.float64) - exp) <= tol), hint
+            assert np.all(g[M:] == 3.0), hint
+    finally:
+        ops.set_option("gemm_tile", -1)
+
+
 @pytest.mark.parametrize("splits,restore,tight", [(2, False, False), (4, False, False),
                                                   (4, True, False), (2, True, False),
                                                   (4, True, True), (2, False, True)])
