@@ -211,13 +211,27 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs &p) {
 
   // ---- computing side -------------------------------------------------------
   const int wm = wave / WN, wn = wave % WN;
+  // The accumulators start from the bias of their column (element 4q + e of block (i, j)
+  // is column n0 + wn*WTN + 32 i + 8 q + 4 (lane >> 5) + e), so the epilogue adds nothing.
+  constexpr bool kHasBias = EPI == kEpiBiasGelu || EPI == kEpiQkvSplit || EPI == kEpiBias;
   float16_t acc[TN][TM];
 #pragma unroll
-  for (int i = 0; i < TN; ++i)
+  for (int i = 0; i < TN; ++i) {
+    float16_t init;
 #pragma unroll
-    for (int j = 0; j < TM; ++j)
+    for (int v = 0; v < 16; ++v) init[v] = 0.f;
+    if (kHasBias) {
 #pragma unroll
-      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+      for (int q = 0; q < 4; ++q) {
+        const int n = min(n0 + wn * WTN + i * 32 + q * 8 + (lane >> 5) * 4, p.N - 4);
+        const half4_t b = *(const half4_t *)(p.bias + n);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) init[4 * q + e] = (float)b[e];
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < TM; ++j) acc[i][j] = init;
+  }
 
   const int fr_row = lane & 31, fr_kc = lane >> 5;
   half8_t fw[2][TN], fa[2][TM];
@@ -303,14 +317,6 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs &p) {
       for (int q = 0; q < 4; ++q) {
         float v0 = acc[i][j][4 * q + 0], v1 = acc[i][j][4 * q + 1];
         float v2 = acc[i][j][4 * q + 2], v3 = acc[i][j][4 * q + 3];
-        if (EPI == kEpiBiasGelu || EPI == kEpiQkvSplit || EPI == kEpiBias) {
-          const int n = min(n0 + wn * WTN + i * 32 + q * 8 + col_in, p.N - 4);
-          const half4_t b = *(const half4_t *)(p.bias + n);
-          v0 += (float)b[0];
-          v1 += (float)b[1];
-          v2 += (float)b[2];
-          v3 += (float)b[3];
-        }
         if (EPI == kEpiBiasGelu) {
           v0 = gelu_tanh_f32(v0);
           v1 = gelu_tanh_f32(v1);
