@@ -32,7 +32,12 @@ void Attention<OpType>::infer(AttentionInferParam infer_param) {
   }
   // on padded rows the mask tensor itself is applied (any 0/1 pattern), as in the
   // reference's non-remove-padding kernels; packed rows use the prefix lengths
-  const void *mask = is_remove_padding_ ? nullptr : (const void *)infer_param.atten_mask;
+  // (unless the caller has checked that it is the plain prefix mask: stopping at the
+  // lengths then gives the same result without reading batch x seq_len^2 mask elements
+  // per head)
+  const void *mask = is_remove_padding_ || infer_param.mask_is_prefix
+                         ? nullptr
+                         : (const void *)infer_param.atten_mask;
   if (size_per_head_ != 64) {
     // the fp16 kernels are built for 64-wide heads; other head sizes (multiples of 8 up to 128) take the
     // generic kernel over token-major projections (the reference's unfused path for them)

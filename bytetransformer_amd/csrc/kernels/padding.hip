@@ -106,6 +106,32 @@ __global__ __launch_bounds__(kOffsetThreads) void build_offsets_kernel(
   }
 }
 
+// ---- is the mask the plain prefix mask of its lengths? ------------------------
+// One wave per mask row (b, i): any element whose on / off state differs from
+// (j < len_b), or an empty sequence, clears the workgroup's slot of `ok`.  Every
+// workgroup writes its own slot each time, so nothing needs clearing beforehand.
+constexpr int kPrefixBlocks = 256;
+constexpr int kPrefixWaves = 4;
+
+template <typename T>
+__global__ __launch_bounds__(kPrefixWaves *kWave) void mask_prefix_kernel(
+    const T *__restrict__ mask, const int *__restrict__ batch_idx, int *__restrict__ ok, int B,
+    int S) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const long long rows = (long long)B * S;
+  int bad = 0;
+  for (long long r = (long long)blockIdx.x * kPrefixWaves + wave; r < rows;
+       r += (long long)gridDim.x * kPrefixWaves) {
+    const int b = (int)(r / S);
+    const int len = batch_idx[b + 1] - batch_idx[b];
+    bad |= len == 0;
+    const T *row = mask + (size_t)r * S;
+    for (int j = lane; j < S; j += kWave) bad |= ((float)row[j] >= 0.5f) != (j < len);
+  }
+  const int any_bad = __syncthreads_or(bad);
+  if (threadIdx.x == 0) ok[blockIdx.x] = !any_bad;
+}
+
 // ---- compress ---------------------------------------------------------------
 // One wave per packed row, 16-byte lanes.  M is read from batch_idx[B]; rows
 // past it retire immediately, so the grid is sized for B*S without a host sync.
@@ -215,6 +241,38 @@ extern "C" int bt_build_offsets(const void *atten_mask, int mask_dtype, int batc
     e = hipStreamSynchronize(s);
     if (e != hipSuccess) return hip_fail(e, "stream synchronize for valid_word_num");
   }
+  return BT_OK;
+}
+
+extern "C" int bt_mask_is_prefix(const void *atten_mask, int mask_dtype, int batch_size,
+                                 int seq_len, const int *batch_idx, int *scratch,
+                                 int *is_prefix_host, void *stream) {
+  BT_REQUIRE(atten_mask && batch_idx && scratch && is_prefix_host, BT_ERR_INVALID_ARGUMENT,
+             "bt_mask_is_prefix: null pointer argument");
+  BT_REQUIRE(batch_size > 0 && seq_len > 0, BT_ERR_INVALID_ARGUMENT,
+             "bt_mask_is_prefix: batch_size=%d seq_len=%d must be positive", batch_size, seq_len);
+  BT_REQUIRE(mask_dtype == BT_F16 || mask_dtype == BT_F32, BT_ERR_INVALID_ARGUMENT,
+             "bt_mask_is_prefix: unknown mask dtype %d", mask_dtype);
+  const long long rows = (long long)batch_size * seq_len;
+  BT_REQUIRE(rows < (1ll << 31), BT_ERR_UNSUPPORTED, "bt_mask_is_prefix: too many rows");
+  hipStream_t s = as_stream(stream);
+  const long long want = (rows + kPrefixWaves - 1) / kPrefixWaves;
+  const int grid = (int)(want < kPrefixBlocks ? want : kPrefixBlocks);
+  if (mask_dtype == BT_F16)
+    mask_prefix_kernel<half_t><<<grid, kPrefixWaves * kWave, 0, s>>>(
+        (const half_t *)atten_mask, batch_idx, scratch, batch_size, seq_len);
+  else
+    mask_prefix_kernel<float><<<grid, kPrefixWaves * kWave, 0, s>>>(
+        (const float *)atten_mask, batch_idx, scratch, batch_size, seq_len);
+  BT_CHECK_LAUNCH("mask_prefix_kernel");
+  int slots[kPrefixBlocks];
+  hipError_t e = hipMemcpyAsync(slots, scratch, grid * sizeof(int), hipMemcpyDeviceToHost, s);
+  if (e != hipSuccess) return hip_fail(e, "copy of the prefix-mask verdict");
+  e = hipStreamSynchronize(s);
+  if (e != hipSuccess) return hip_fail(e, "stream synchronize for the prefix-mask verdict");
+  int all = 1;
+  for (int i = 0; i < grid; ++i) all &= slots[i] != 0;
+  *is_prefix_host = all;
   return BT_OK;
 }
 

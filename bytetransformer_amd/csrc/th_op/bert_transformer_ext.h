@@ -97,12 +97,15 @@ class BTEncoder : public IBTEncoder {
     // captured into a graph, where the host may not wait for the token count)
     MaskPlanCache::Plan plan;
     ET_Param offsets{nullptr, nullptr, 0};
-    if (mask_plan(attr_mask, batch_size, seq_len, stream, &plan)) {
+    // (batches of one and two run on the padded rows whatever the flag says)
+    const bool padded_rows = !is_remove_padding || batch_size <= 2;
+    if (mask_plan(attr_mask, batch_size, seq_len, stream, padded_rows, &plan)) {
       offsets.batch_idx = plan.batch_idx.data_ptr<int>();
       offsets.word_idx = plan.word_idx.data_ptr<int>();
       offsets.valid_word_num = plan.valid_word_num;
       infer_param.offsets = &offsets;
       infer_param.seq_order = plan.seq_order.data_ptr<int>();
+      infer_param.mask_is_prefix = plan.prefix_state == 1;
     }
     encoder.infer(infer_param);
   }
@@ -146,16 +149,32 @@ class BTEncoder : public IBTEncoder {
     return out;
   }
 
+  // want_prefix: the layer will run on the padded rows, where it pays to know whether the
+  // mask is the plain prefix mask of its lengths (one pass over the tensor, once per mask).
   bool mask_plan(const Tensor &mask, int batch_size, int seq_len, hipStream_t stream,
-                 MaskPlanCache::Plan *plan) {
+                 bool want_prefix, MaskPlanCache::Plan *plan) {
     if (!PrepackCache::instance().enabled() || mask.is_inference()) return false;
     hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
     if (hipStreamIsCapturing(stream, &capturing) != hipSuccess ||
         capturing != hipStreamCaptureStatusNone)
       return false;
     auto &cache = MaskPlanCache::instance();
-    if (cache.lookup(mask, stream, plan)) return true;
     auto opts = torch::dtype(torch::kInt32).device(mask.device());
+    auto check_prefix = [&]() {
+      auto scratch = torch::empty({256}, opts);
+      int verdict = 0;
+      check_bt_error(bt_mask_is_prefix(mask.data_ptr(), Traits<kOp>::dtype, batch_size, seq_len,
+                                       plan->batch_idx.data_ptr<int>(), scratch.data_ptr<int>(),
+                                       &verdict, stream));
+      plan->prefix_state = verdict;
+    };
+    if (cache.lookup(mask, stream, plan)) {
+      if (want_prefix && plan->prefix_state < 0) {
+        check_prefix();
+        cache.store(mask, stream, *plan);
+      }
+      return true;
+    }
     plan->batch_idx = torch::empty({(int64_t)batch_size + 1}, opts);
     plan->word_idx = torch::empty({(int64_t)batch_size * seq_len}, opts);
     plan->seq_order = torch::empty({(int64_t)batch_size}, opts);
@@ -163,6 +182,7 @@ class BTEncoder : public IBTEncoder {
                                     plan->batch_idx.data_ptr<int>(), plan->word_idx.data_ptr<int>(),
                                     plan->seq_order.data_ptr<int>(), &plan->valid_word_num,
                                     stream));
+    if (want_prefix) check_prefix();
     cache.store(mask, stream, *plan);
     return true;
   }

@@ -117,6 +117,7 @@ class MaskPlanCache {
   struct Plan {
     torch::Tensor batch_idx, word_idx, seq_order;
     int valid_word_num = 0;
+    int prefix_state = -1;   // is the mask the plain prefix mask of these lengths? -1 = not checked
   };
 
   static MaskPlanCache &instance() {

@@ -67,6 +67,16 @@ def build_offsets(mask, want_count=False, out=None, seq_order=None):
     return batch_idx, word_idx, (cnt.value if want_count else None)
 
 
+def mask_is_prefix(mask, batch_idx):
+    """True when mask [B,S,S] is exactly (j < len_b) in every row and no sequence is empty."""
+    B, S = mask.shape[0], mask.shape[1]
+    scratch = torch.empty(256, dtype=torch.int32, device=mask.device)
+    verdict = ctypes.c_int(-1)
+    _check(kernel_lib().bt_mask_is_prefix(_ptr(mask), _dtype_code(mask), B, S, _ptr(batch_idx),
+                                          _ptr(scratch), ctypes.byref(verdict), _stream()))
+    return bool(verdict.value)
+
+
 def compress(x, batch_idx, word_idx, out=None):
     B, S, H = x.shape
     if out is None:

@@ -85,6 +85,18 @@ int bt_build_offsets(const void *atten_mask, int mask_dtype, int batch_size, int
                      void *stream);
 
 /*
+ * Is atten_mask exactly the prefix mask of the lengths in batch_idx, i.e. for every
+ * batch b and EVERY row i: (mask[b, i, j] >= 0.5) == (j < len_b), with no empty
+ * sequence?  Then the padded-row attention may ignore the tensor and stop at len_b keys,
+ * which gives the same result as applying it (the masked logits' exp is exactly 0).
+ * The reference always applies the tensor on that path (attention_fused.cu:234-237); no
+ * counterpart there.  scratch: device int[256], overwritten.  Waits for the stream and
+ * writes 0 / 1 to *is_prefix_host.
+ */
+int bt_mask_is_prefix(const void *atten_mask, int mask_dtype, int batch_size, int seq_len,
+                      const int *batch_idx, int *scratch, int *is_prefix_host, void *stream);
+
+/*
  * Gather valid rows: to_tensor[t, :] = from_tensor[word_idx[t], :], t < M.
  * Replaces compressBertInput_kernelLauncher (remove_padding.h:104-121).
  * hidden_dim % 8 == 0.  M is read on the device from batch_idx[batch_size].

@@ -43,6 +43,9 @@ struct AttentionInferParam {
   // remaining weights); the attention kernel warms the memory-side cache with it.
   const void *prefetch = nullptr;
   unsigned long long prefetch_bytes = 0;
+  // Extension: atten_mask is known to be the plain prefix mask of et_param's lengths; the
+  // padded rows then need no mask tensor (keys stop at each length: the same result).
+  bool mask_is_prefix = false;
 };
 
 template <OperationType OpType>

@@ -69,6 +69,10 @@ struct BertTransformerInferParam {
   const ET_Param *offsets = NULL;
   // ... and the matching sequence order (int[batch_size], longest first), or NULL.
   const int *seq_order = NULL;
+  // ... and the caller's finding (bt_mask_is_prefix) that atten_mask is exactly the prefix
+  // mask of those offsets: on the padded rows the attention then stops at each length
+  // instead of reading the tensor - the same result, the masked terms being exactly zero.
+  bool mask_is_prefix = false;
 };
 
 template <OperationType OpType>

@@ -401,6 +401,43 @@ def test_gather_fused_into_qkv_gemm_and_layernorm(device):
     assert torch.equal(a, b)
 
 
+@pytest.mark.parametrize("np_dtype", [np.float16, np.float32])
+def test_mask_is_prefix(device, np_dtype):
+    """The verdict is True only for masks that are (j < len_b) in EVERY row, with no empty
+    sequence; one flipped element anywhere - on past the length, off inside it, in a row
+    other than the first - makes it False."""
+    _say("mask_is_prefix", np_dtype.__name__)
+    rs = np.random.RandomState(5)
+    for B, S in ((1, 1), (1, 154), (2, 64), (3, 257), (5, 1024)):
+        lens = rs.randint(1, S + 1, size=B)
+        lens[rs.randint(B)] = S
+        mask = workload.make_mask(lens, S, np_dtype)
+        md = _dev(mask, device)
+        bi, _, _ = ops.build_offsets(md)
+        assert ops.mask_is_prefix(md, bi) is True, (B, S)
+        for trial in range(6):
+            b, i = int(rs.randint(B)), int(rs.randint(1, S)) if S > 1 else 0
+            j = int(rs.randint(S))
+            bad = mask.copy()
+            bad[b, i, j] = 1 - bad[b, i, j]
+            if i == 0:
+                continue        # row 0 defines the lengths: flipping there may give another prefix mask
+            assert ops.mask_is_prefix(_dev(bad, device), bi) is False, (B, S, b, i, j)
+        # values other than 0 / 1 count by the 0.5 threshold, as in the offsets kernel
+        soft = (mask * 0.75 + (1 - mask) * 0.25).astype(np_dtype)
+        assert ops.mask_is_prefix(_dev(soft, device), bi) is True
+    # an empty sequence: the reference's softmax over an all-masked row is not "no keys"
+    lens = np.array([7, 0, 3])
+    md = _dev(workload.make_mask(lens, 9, np_dtype), device)
+    bi, _, _ = ops.build_offsets(md)
+    assert ops.mask_is_prefix(md, bi) is False
+    # a causal mask is not a prefix mask
+    causal = np.tril(np.ones((2, 16, 16), np_dtype))
+    cd = _dev(causal, device)
+    bi, _, _ = ops.build_offsets(cd)
+    assert ops.mask_is_prefix(cd, bi) is False
+
+
 # ---- attention -----------------------------------------------------------------
 def _attention_case(rs, lens, S, heads, scale_q=1.0):
     B = len(lens)

@@ -355,6 +355,22 @@ def test_random_small_configurations(device, seed):
     assert pads_zero
 
 
+@pytest.mark.parametrize("lens", [(90, 17, 64, 1, 33), (90, 0, 64, 1, 33), (40, 90)])
+def test_operator_on_padded_rows_with_a_prefix_mask(device, lens):
+    """On the padded rows the operator checks once per mask whether it is the plain prefix
+    mask; then the attention stops at each length instead of reading the tensor (not with
+    an empty sequence, whose all-masked softmax is not "no keys").  Valid rows match the
+    oracle and the path that always applies the tensor."""
+    cfg = workload.EncoderConfig("pp", len(lens), 90, 3, layers=2, lens=lens)
+    wl = workload.make_workload(cfg, bias_std=0.05, random_affine=True)
+    exp = _oracle(wl)
+    got = O.masked_output(_run_th_op(wl, device, rm=False), wl.lens)
+    _check(got, exp, wl.lens, tag="padded rows/prefix mask/th_op")
+    ref = O.masked_output(_run_c_api(wl, device, is_remove_padding=False), wl.lens)
+    mx, _, _ = O.parity_metrics(got, ref, wl.lens)
+    assert mx <= 8e-3, mx
+
+
 @pytest.mark.parametrize("rm", [True, False])
 def test_balanced_workgroup_order_through_the_layer(device, rm):
     """The streaming attention kernel with its balanced work list forced on (small launches
