@@ -107,8 +107,10 @@ __global__ __launch_bounds__(kOffsetThreads) void build_offsets_kernel(
 }
 
 // ---- is the mask the plain prefix mask of its lengths? ------------------------
-// One wave per mask row (b, i): any element whose on / off state differs from
-// (j < len_b), or an empty sequence, clears the workgroup's slot of `ok`.  Every
+// One wave per mask row (b, i): any element that is not exactly 1 before len_b or not
+// exactly 0 from there on, or an empty sequence, clears the workgroup's slot of `ok`
+// (the padded-row attention shifts a logit by (mask - 1) * 10000: only 1 leaves it alone
+// and only a shift of the full -10000 is certain to vanish in the softmax).  Every
 // workgroup writes its own slot each time, so nothing needs clearing beforehand.
 constexpr int kPrefixBlocks = 256;
 constexpr int kPrefixWaves = 4;
@@ -126,7 +128,7 @@ __global__ __launch_bounds__(kPrefixWaves *kWave) void mask_prefix_kernel(
     const int len = batch_idx[b + 1] - batch_idx[b];
     bad |= len == 0;
     const T *row = mask + (size_t)r * S;
-    for (int j = lane; j < S; j += kWave) bad |= ((float)row[j] >= 0.5f) != (j < len);
+    for (int j = lane; j < S; j += kWave) bad |= (float)row[j] != (j < len ? 1.0f : 0.0f);
   }
   const int any_bad = __syncthreads_or(bad);
   if (threadIdx.x == 0) ok[blockIdx.x] = !any_bad;

@@ -86,9 +86,10 @@ int bt_build_offsets(const void *atten_mask, int mask_dtype, int batch_size, int
 
 /*
  * Is atten_mask exactly the prefix mask of the lengths in batch_idx, i.e. for every
- * batch b and EVERY row i: (mask[b, i, j] >= 0.5) == (j < len_b), with no empty
- * sequence?  Then the padded-row attention may ignore the tensor and stop at len_b keys,
- * which gives the same result as applying it (the masked logits' exp is exactly 0).
+ * batch b and EVERY row i: mask[b, i, j] == 1 for j < len_b and == 0 from there on, with
+ * no empty sequence?  Then the padded-row attention may ignore the tensor and stop at
+ * len_b keys, which gives the same result as applying it (the logits of the ones are not
+ * shifted, the exp of the others is exactly 0).
  * The reference always applies the tensor on that path (attention_fused.cu:234-237); no
  * counterpart there.  scratch: device int[256], overwritten.  Waits for the stream and
  * writes 0 / 1 to *is_prefix_host.

@@ -403,9 +403,9 @@ def test_gather_fused_into_qkv_gemm_and_layernorm(device):
 
 @pytest.mark.parametrize("np_dtype", [np.float16, np.float32])
 def test_mask_is_prefix(device, np_dtype):
-    """The verdict is True only for masks that are (j < len_b) in EVERY row, with no empty
-    sequence; one flipped element anywhere - on past the length, off inside it, in a row
-    other than the first - makes it False."""
+    """The verdict is True only for masks that are exactly 1 for j < len_b and exactly 0
+    beyond in EVERY row, with no empty sequence; one flipped element anywhere - on past
+    the length, off inside it, in a row other than the first - makes it False."""
     _say("mask_is_prefix", np_dtype.__name__)
     rs = np.random.RandomState(5)
     for B, S in ((1, 1), (1, 154), (2, 64), (3, 257), (5, 1024)):
@@ -423,9 +423,14 @@ def test_mask_is_prefix(device, np_dtype):
             if i == 0:
                 continue        # row 0 defines the lengths: flipping there may give another prefix mask
             assert ops.mask_is_prefix(_dev(bad, device), bi) is False, (B, S, b, i, j)
-        # values other than 0 / 1 count by the 0.5 threshold, as in the offsets kernel
+        # only exact ones and zeros qualify: the tensor path shifts a logit by
+        # (mask - 1) * 10000, so 0.75 is not "on" and 0.25 is not certainly "off"
         soft = (mask * 0.75 + (1 - mask) * 0.25).astype(np_dtype)
-        assert ops.mask_is_prefix(_dev(soft, device), bi) is True
+        assert ops.mask_is_prefix(_dev(soft, device), bi) is False
+        if S > 1:
+            almost = mask.copy()
+            almost[0, S - 1, 0] = np_dtype(0.75)
+            assert ops.mask_is_prefix(_dev(almost, device), bi) is False
     # an empty sequence: the reference's softmax over an all-masked row is not "no keys"
     lens = np.array([7, 0, 3])
     md = _dev(workload.make_mask(lens, 9, np_dtype), device)
