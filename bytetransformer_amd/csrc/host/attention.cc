@@ -21,10 +21,12 @@ void Attention<OpType>::infer(AttentionInferParam infer_param) {
   if constexpr (OpType == OperationType::FP32) {
     // float: one streaming kernel over token-major [rows, 3H] projections; the mask tensor
     // is applied on both row layouts, as the reference's float path does
-    // (attention_nofused.cu:85-94)
+    // (attention_nofused.cu:85-94) - unless the caller has found it to be the plain
+    // prefix mask, whose terms are 0 for the keys of the sequence and vanish for the rest
     check_bt_error(bt_attention_f32(infer_param.qkv, infer_param.attention_output,
                                     infer_param.et_param.batch_idx, infer_param.seq_order,
-                                    infer_param.atten_mask, infer_param.attention_bias,
+                                    infer_param.mask_is_prefix ? nullptr : infer_param.atten_mask,
+                                    infer_param.attention_bias,
                                     infer_param.batch_size,
                                     infer_param.seq_len, rows_cap, head_num_, size_per_head_,
                                     scale, padded_rows, infer_param.stream));

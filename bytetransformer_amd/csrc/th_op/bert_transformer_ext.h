@@ -97,9 +97,11 @@ class BTEncoder : public IBTEncoder {
     // captured into a graph, where the host may not wait for the token count)
     MaskPlanCache::Plan plan;
     ET_Param offsets{nullptr, nullptr, 0};
-    // (batches of one and two run on the padded rows whatever the flag says)
-    const bool padded_rows = !is_remove_padding || batch_size <= 2;
-    if (mask_plan(attr_mask, batch_size, seq_len, stream, padded_rows, &plan)) {
+    // (batches of one and two run on the padded rows whatever the flag says; the float
+    // attention applies the mask tensor on both row layouts)
+    const bool mask_tensor_in_use =
+        !is_remove_padding || batch_size <= 2 || kOp == OperationType::FP32;
+    if (mask_plan(attr_mask, batch_size, seq_len, stream, mask_tensor_in_use, &plan)) {
       offsets.batch_idx = plan.batch_idx.data_ptr<int>();
       offsets.word_idx = plan.word_idx.data_ptr<int>();
       offsets.valid_word_num = plan.valid_word_num;
@@ -149,8 +151,8 @@ class BTEncoder : public IBTEncoder {
     return out;
   }
 
-  // want_prefix: the layer will run on the padded rows, where it pays to know whether the
-  // mask is the plain prefix mask of its lengths (one pass over the tensor, once per mask).
+  // want_prefix: the attention of this layer would read the mask tensor, so it pays to know
+  // whether that is the plain prefix mask of its lengths (one pass over it, once per mask).
   bool mask_plan(const Tensor &mask, int batch_size, int seq_len, hipStream_t stream,
                  bool want_prefix, MaskPlanCache::Plan *plan) {
     if (!PrepackCache::instance().enabled() || mask.is_inference()) return false;
