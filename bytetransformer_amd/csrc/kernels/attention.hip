@@ -87,76 +87,6 @@ __device__ __forceinline__ AttItem att_item(const AttArgs &p) {
   return it;
 }
 
-// Balanced work list (xcd_map == 2, streaming kernel).  Within an XCD the hardware deals
-// consecutive workgroups to its 32 CUs round-robin (slot s of the XCD lands on CU s % 32),
-// and a launch of up to three workgroups per CU is resident at once, so the static order
-// alone decides what each CU gets.  With a fixed number of query-tile slots per sequence
-// the tile index is s % 4 at 512 tokens: one CU in four received only the last tiles -
-// dead for most sequences - while others held three live ones of the longest sequences.
-// Here the live (pair, query tile) items of the XCD - pairs p = x (mod 8) over the
-// longest-first order as above, the tiles of a pair adjacent - are counted on the device
-// and slot s takes item j = s in even rounds of 32 and the mirrored position in odd
-// rounds, so a CU that drew a long item in one round draws a short one in the next.
-// Every lane of a wave holds one rank: lengths, tile counts and a wave prefix sum invert
-// j -> (rank, head, tile) with the two dependent loads the plain lookup needs as well.
-// Inclusive prefix sum over the 64 lanes with data-parallel-primitive adds only: four
-// shifts inside each row of 16, then lane 15 of rows 0 / 2 into rows 1 / 3 and lane 31
-// into the upper half.
-__device__ __forceinline__ int wave_inclusive_sum(int v) {
-  v += __builtin_amdgcn_update_dpp(0, v, 0x111, 0xf, 0xf, true);   // row_shr:1
-  v += __builtin_amdgcn_update_dpp(0, v, 0x112, 0xf, 0xf, true);   // row_shr:2
-  v += __builtin_amdgcn_update_dpp(0, v, 0x114, 0xf, 0xf, true);   // row_shr:4
-  v += __builtin_amdgcn_update_dpp(0, v, 0x118, 0xf, 0xf, true);   // row_shr:8
-  v += __builtin_amdgcn_update_dpp(0, v, 0x142, 0xa, 0xf, false);  // row_bcast:15 -> rows 1, 3
-  v += __builtin_amdgcn_update_dpp(0, v, 0x143, 0xc, 0xf, false);  // row_bcast:31 -> rows 2, 3
-  return v;
-}
-
-struct AttWork {
-  int b, head, qb, seq_start, len;
-  bool exists;
-};
-template <int BQ>
-__device__ __forceinline__ AttWork att_work_balanced(const AttArgs &p) {
-  AttWork w{0, 0, 0, 0, 0, false};
-  const int lane = threadIdx.x & 63;
-  const int x = blockIdx.x & 7, s = blockIdx.x >> 3;
-  const int round = s >> 5, pos = s & 31;
-  const int j = (round << 5) + ((round & 1) ? 31 - pos : pos);
-  int carry = 0;
-  for (int base = 0; base < p.B; base += 64) {
-    const int r = base + lane;
-    const bool valid = r < p.B;
-    const int seq = valid ? (p.seq_order ? p.seq_order[r] : r) : 0;
-    const int start = p.batch_idx[seq];
-    const int len = valid ? p.batch_idx[seq + 1] - start : 0;
-    const int nq = p.padded_rows ? p.S : len;
-    const int nqb = valid ? min((nq + BQ - 1) / BQ, p.nqb) : 0;
-    const int first = r * p.heads;   // pairs [first, first + heads) belong to rank r
-    const int cnt = ((first + p.heads + 7 - x) >> 3) - ((first + 7 - x) >> 3);
-    const int mine = cnt * nqb;
-    const int incl = wave_inclusive_sum(mine);
-    const int lo = carry + incl - mine;   // first item of this rank
-    const unsigned long long hit = __builtin_amdgcn_ballot_w64(mine > 0 && j >= lo && j < lo + mine);
-    if (hit) {
-      const int src = __builtin_ctzll(hit);
-      const int jj = j - __builtin_amdgcn_readlane(lo, src);
-      const int nqb_s = __builtin_amdgcn_readlane(nqb, src);
-      const int first_s = (base + src) * p.heads;
-      w.b = __builtin_amdgcn_readlane(seq, src);
-      w.seq_start = __builtin_amdgcn_readlane(start, src);
-      w.len = __builtin_amdgcn_readlane(len, src);
-      w.qb = jj % nqb_s;
-      // the (jj / nqb_s)-th head h of the rank with first_s + h = x (mod 8)
-      w.head = ((x - first_s) & 7) + 8 * (jj / nqb_s);
-      w.exists = true;
-      return w;
-    }
-    carry += __builtin_amdgcn_readlane(incl, 63);
-  }
-  return w;
-}
-
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
 // Reductions over the four 16-lane rows of a wave (lanes l, l^16, l^32, l^48) with the

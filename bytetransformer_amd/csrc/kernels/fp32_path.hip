@@ -213,6 +213,7 @@ struct F32AttArgs {
   float scale;
   int padded_rows;
   int nqb;             // query tiles per sequence
+  int balanced;        // 1: the live query tiles are dealt evenly to the CUs (common.h)
   int d;               // head size (a multiple of 8, <= the kernel's D = 32 * ND; the
                        // columns d..D-1 of Q, K and V read as zero)
 };
@@ -238,17 +239,27 @@ __global__ __launch_bounds__(64 * NW) void f32_attention_kernel(F32AttArgs<T> p)
   // 8 XCDs; XCD x works on the (sequence, head) pairs p = x (mod 8), the query tiles of
   // one pair back to back (its K / V then come from that XCD's L2), so every XCD sees the
   // same mix of sequence lengths however ragged the batch is.
-  const unsigned lin = blockIdx.x, slot = lin >> 3;
-  const unsigned pair = (slot / p.nqb) * 8 + (lin & 7);
-  if (pair >= (unsigned)(p.B * p.heads)) return;
-  const int rank = pair / p.heads, head = pair % p.heads;
-  const int b = p.seq_order ? p.seq_order[rank] : rank;
-  const int seq_start = p.batch_idx[b];
-  const int len = p.batch_idx[b + 1] - seq_start;
+  // Launches of more than two rounds of workgroups per CU take the balanced work list.
+  int b, head, seq_start, len, qb_index;
+  if (p.balanced) {
+    const AttWork w = att_work_balanced<BQ>(p);
+    if (!w.exists) return;
+    b = w.b, head = w.head, seq_start = w.seq_start, len = w.len, qb_index = w.qb;
+  } else {
+    const unsigned lin = blockIdx.x, slot = lin >> 3;
+    const unsigned pair = (slot / p.nqb) * 8 + (lin & 7);
+    if (pair >= (unsigned)(p.B * p.heads)) return;
+    const int rank = pair / p.heads;
+    head = pair % p.heads;
+    b = p.seq_order ? p.seq_order[rank] : rank;
+    seq_start = p.batch_idx[b];
+    len = p.batch_idx[b + 1] - seq_start;
+    qb_index = (int)(slot % p.nqb);
+  }
   const int klen = (p.mask && p.padded_rows) ? p.S : len;
   const int row_start = p.padded_rows ? b * p.S : seq_start;
   const int nq = p.padded_rows ? p.S : len;
-  const int q0 = (int)(slot % p.nqb) * BQ;
+  const int q0 = qb_index * BQ;
   if (q0 >= nq || klen <= 0) {
     // padded rows of an empty sequence still get defined output: zeros
     if (q0 < nq) {
@@ -553,7 +564,12 @@ static int launch_generic_attention(const char *who, const void *qkv, void *out,
   p.d = size_per_head;
   constexpr int kWaves = 4;    // 128 queries per workgroup (two-wave workgroups measured slower)
   p.nqb = (seq_len + 32 * kWaves - 1) / (32 * kWaves);
-  const unsigned grid = ((unsigned)batch_size * head_num + 7) / 8 * 8 * p.nqb;
+  // the conditions of the fp16 streaming kernel: from the third round of 32 workgroups
+  // per XCD on and up to 128 sequences, or always / never by the option
+  const unsigned per_xcd = ((unsigned)batch_size * head_num + 7) / 8 * p.nqb;
+  const int order = option_attention_xcd_map();
+  p.balanced = order == 3 || (order == 2 && per_xcd > 64 && batch_size <= 128);
+  const unsigned grid = p.balanced ? (per_xcd + 31) / 32 * 32 * 8 : per_xcd * 8;
 #define BT_F32_ATT(ND_) f32_attention_kernel<T, ND_, kWaves><<<grid, 64 * kWaves, 0, s>>>(p)
   switch ((size_per_head + 31) / 32) {
     case 1: BT_F32_ATT(1); break;

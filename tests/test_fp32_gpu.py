@@ -32,6 +32,15 @@ def _dev(a, device):
     return torch.from_numpy(np.ascontiguousarray(a)).to(device)
 
 
+@pytest.fixture(params=[2, 3], ids=["default-order", "balanced-order"])
+def att_order(request):
+    """Runs a test under the default workgroup order and with the balanced work list
+    forced on (small launches would not use it by themselves)."""
+    ops.set_option("attention_xcd_map", request.param)
+    yield request.param
+    ops.set_option("attention_xcd_map", 2)
+
+
 # ---- GEMM ------------------------------------------------------------------------
 @pytest.mark.parametrize("rows,M,N,K", [(300, 300, 768, 768), (1000, 777, 2304, 768),
                                         (4920, 4920, 3072, 768), (640, 513, 768, 3072),
@@ -179,7 +188,7 @@ F32_ATT_CASES = [
 
 @pytest.mark.parametrize("padded", [False, True])
 @pytest.mark.parametrize("lens,S,heads,d", F32_ATT_CASES)
-def test_attention_f32(device, lens, S, heads, d, padded):
+def test_attention_f32(device, lens, S, heads, d, padded, att_order):
     _say("attention_f32", lens, S, heads, d, padded)
     rs = np.random.RandomState(S + heads + d)
     B, H = len(lens), heads * d
@@ -212,7 +221,7 @@ def test_attention_f32(device, lens, S, heads, d, padded):
 
 
 @pytest.mark.parametrize("padded", [False, True])
-def test_attention_f32_mask_and_bias(device, padded):
+def test_attention_f32_mask_and_bias(device, padded, att_order):
     """An arbitrary 0/1 mask (every query keeps at least one key) and a bias: the kernel
     must apply both per (query, key), on both row layouts."""
     _say("attention_f32 mask+bias", padded)
@@ -243,7 +252,7 @@ def test_attention_f32_mask_and_bias(device, padded):
                                             ([150, 64, 1], 160, 2, 96), ([64, 38], 64, 3, 64),
                                             ([33, 70], 70, 4, 16), ([100, 5], 100, 2, 80),
                                             ([64, 64], 64, 3, 8)])
-def test_attention_generic_f16(device, lens, S, heads, d, padded):
+def test_attention_generic_f16(device, lens, S, heads, d, padded, att_order):
     """The same kernel on fp16 tensors (head sizes the fp16 attention kernels do not take):
     inputs rounded to fp16, arithmetic in float, one fp16 rounding of the output."""
     _say("attention_generic_f16", lens, S, heads, d, padded)
