@@ -73,7 +73,7 @@ inline int allow_dynamic_lds(Kernel kernel, size_t bytes, std::atomic<bool> (&do
 int option_gemm_tile();      // -1 = heuristic, else index into the tile table
 int option_attention_qb();   // -1 = heuristic, 1 or 2 = query blocks per wave
 int option_f32_gemm_tile();  // -1 = heuristic, else index into the float GEMM's tile table
-int option_attention_xcd_map();     // workgroup order of the fp16 attention: 0 plain, 1 XCD-aware, 2 balanced (default), 3 balanced always
+int option_attention_xcd_map();     // workgroup order of the attention kernels: 0 plain, 1 XCD-aware, 2 balanced (default), 3 balanced always
 int option_prefetch();       // 1 = honour the prefetch hints of the attention entries (default), 0 = ignore
 
 inline hipStream_t as_stream(void *s) { return reinterpret_cast<hipStream_t>(s); }

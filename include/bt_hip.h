@@ -57,8 +57,9 @@ const char *bt_last_error_string(void);
  *   "attention_short_limit"  0 (default) .. 512: the host library sends sequences up to this
  *                   length to bt_attention_short when use_fused_attention is set; 0 = always
  *                   the streaming kernel, which measures faster at every length
- *   "attention_xcd_map"  workgroup order of the fp16 attention kernels: 0 plain | 1 XCD-aware
- *                   | 2 (default) XCD-aware, and in the streaming kernel the live query
+ *   "attention_xcd_map"  workgroup order of the attention kernels: 0 plain (fp16 kernels
+ *                   only) | 1 XCD-aware | 2 (default) XCD-aware, and in the streaming
+ *                   kernels (fp16, float, generic head sizes) the live query
  *                   tiles are dealt evenly to the CUs once the launch has more than two
  *                   rounds of workgroups per CU (batches up to 128 sequences) | 3: that
  *                   balanced order at any size
