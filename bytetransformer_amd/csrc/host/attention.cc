@@ -56,12 +56,24 @@ void Attention<OpType>::infer(AttentionInferParam infer_param) {
                                       infer_param.attention_bias, infer_param.batch_size, infer_param.seq_len, rows_cap, head_num_, size_per_head_,
                                       scale, padded_rows, infer_param.prefetch,
                                       infer_param.prefetch_bytes, infer_param.stream));
-  else
-    check_bt_error(bt_attention_grouped(infer_param.qkv, infer_param.attention_output,
-                                        infer_param.et_param.batch_idx, infer_param.seq_order, mask,
-                                        infer_param.attention_bias, infer_param.batch_size, infer_param.seq_len, rows_cap, head_num_, size_per_head_,
-                                        scale, padded_rows, infer_param.prefetch,
-                                      infer_param.prefetch_bytes, infer_param.stream));
+  else {
+    // A mask tensor in use and no verdict from the caller: one pass over it on the device
+    // (every launch of the layer, a few microseconds) lets the kernel drop it when it is the
+    // plain prefix mask - the usual case, worth 3-15 us of attention per layer.
+    const int *slots = mask ? infer_param.mask_prefix_slots : nullptr;
+    if (mask && !slots && infer_param.buf) {
+      int *verdict = (int *)infer_param.buf;
+      check_bt_error(bt_mask_prefix_slots(mask, Traits_::dtype, infer_param.batch_size,
+                                          infer_param.seq_len, infer_param.et_param.batch_idx,
+                                          verdict, infer_param.stream));
+      slots = verdict;
+    }
+    check_bt_error(bt_attention_grouped(
+        infer_param.qkv, infer_param.attention_output, infer_param.et_param.batch_idx,
+        infer_param.seq_order, mask, infer_param.attention_bias, infer_param.batch_size,
+        infer_param.seq_len, rows_cap, head_num_, size_per_head_, scale, padded_rows,
+        infer_param.prefetch, infer_param.prefetch_bytes, slots, infer_param.stream));
+  }
 }
 
 template class Attention<OperationType::FP32>;

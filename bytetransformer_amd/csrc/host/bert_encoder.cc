@@ -53,7 +53,9 @@ void BertEncoder<OpType>::infer(BertEncoderInferParam<DataType_> ip) {
   et_param.batch_idx = et_param.word_idx + max_rows;
   et_param.valid_word_num = rows;
   int *seq_order = et_param.batch_idx + max_batch_size_ + 1;
-  off += align_up((max_rows * 2 + 2 * (unsigned long long)max_batch_size_ + 2) * sizeof(int), 256);
+  int *mask_slots = seq_order + max_batch_size_;       // int[256], padded path only
+  off += align_up((max_rows * 2 + 2 * (unsigned long long)max_batch_size_ + 2 + 256) * sizeof(int),
+                  256);
   DataType_ *staging = (DataType_ *)(base + off);      // one layer's weights when none were passed
   off += align_up(layer_weight_elems() * sizeof(DataType_), 256);
   float *splitk_buf = (float *)(base + off);
@@ -64,6 +66,13 @@ void BertEncoder<OpType>::infer(BertEncoderInferParam<DataType_> ip) {
   const int *valid_rows = is_remove_padding_ ? et_param.batch_idx + batch_size : nullptr;
   const int rows_hint = ip.valid_rows_hint;
   const int L = (int)layers_.size();
+  // padded rows: the fp16 streaming attention applies the mask tensor unless this one pass
+  // over it (once for all layers) finds the plain prefix mask of the lengths
+  const bool check_mask = !is_remove_padding_ && OpType == OperationType::HALF &&
+                          size_per_head_ == 64;
+  if (check_mask)
+    check_bt_error(bt_mask_prefix_slots(ip.atten_mask, Traits_::dtype, batch_size, seq_len,
+                                        et_param.batch_idx, mask_slots, stream));
 
   for (int l = 0; l < L; ++l) {
     const auto &w = layers_[l];
@@ -134,6 +143,7 @@ void BertEncoder<OpType>::infer(BertEncoderInferParam<DataType_> ip) {
     };
     att.attention_bias = ip.attention_bias;
     att.seq_order = seq_order;
+    if (check_mask) att.mask_prefix_slots = mask_slots;
     // warm the memory-side cache with what follows in memory order: the rest of this
     // layer's weights and, when all layers are pre-packed back to back, the next
     // layer's QKV matrix

@@ -55,6 +55,8 @@ struct AttArgs {
   int nqb;             // query tiles per sequence (set by the launcher)
   unsigned nqb_grid;   // host only: workgroups of the launch
   int xcd_map;         // 0: plain (tile, head, sequence) order, 1: XCD-aware, 2: XCD-aware and balanced over the CUs
+  const int *mask_ok;  // optional int[256] from bt_mask_prefix_slots: all non-zero = the mask
+                       // is the plain prefix mask of the lengths, and is then ignored
 };
 
 // Which (sequence rank, head, query tile) a workgroup of the 1-D grid works on.  The
@@ -251,8 +253,16 @@ __global__ __launch_bounds__(kAttThreads, 2) void attention_grouped_kernel(AttAr
     seq_len = p.batch_idx[b + 1] - seq_start;
     qb_index = item.qb;
   }
+  // A mask tensor that the device-side check found to be the plain prefix mask adds 0 to
+  // the logits of the sequence's keys and removes the others: the lengths say the same.
+  const half_t *mask = ADD ? p.mask : nullptr;
+  if (ADD && mask && p.mask_ok) {
+    const int l = threadIdx.x & 63;
+    const int ok = p.mask_ok[l] & p.mask_ok[l + 64] & p.mask_ok[l + 128] & p.mask_ok[l + 192];
+    if (__builtin_amdgcn_ballot_w64(ok == 0) == 0) mask = nullptr;
+  }
   // with a mask tensor every one of the S key rows takes part
-  const int klen = ADD && p.mask ? p.S : seq_len;
+  const int klen = mask ? p.S : seq_len;
   const int row_start = p.padded_rows ? b * p.S : seq_start;
   const int nq = p.padded_rows ? p.S : klen;
   const int q0 = qb_index * BQ;
@@ -367,7 +377,7 @@ __global__ __launch_bounds__(kAttThreads, 2) void attention_grouped_kernel(AttAr
 #pragma unroll
       for (int qb = 0; qb < QB; ++qb) {
         const int q = min(q0 + (wave * QB + qb) * 16 + lq, p.S - 1);
-        const half_t *mrow = p.mask ? p.mask + ((size_t)b * p.S + q) * p.S : nullptr;
+        const half_t *mrow = mask ? mask + ((size_t)b * p.S + q) * p.S : nullptr;
         const half_t *brow = p.bias ? p.bias + ((size_t)head * p.S + q) * p.S : nullptr;
 #pragma unroll
         for (int kb = 0; kb < 4; ++kb) {
@@ -714,7 +724,7 @@ extern "C" int bt_attention_grouped(const void *qkv_heads, void *attention_outpu
                                     int batch_size, int seq_len, int rows_cap, int head_num,
                                     int size_per_head, float scale, int padded_rows,
                                     const void *prefetch, unsigned long long prefetch_bytes,
-                                    void *stream) {
+                                    const int *mask_prefix_slots, void *stream) {
   int rc = check_att_args("bt_attention_grouped", qkv_heads, attention_output, batch_idx,
                           atten_mask, padded_rows, batch_size, seq_len, rows_cap, head_num,
                           size_per_head);
@@ -723,6 +733,7 @@ extern "C" int bt_attention_grouped(const void *qkv_heads, void *attention_outpu
             (const half_t *)atten_mask, (const half_t *)attention_bias,
             nullptr, 0, batch_size, seq_len,
             rows_cap, head_num, scale * kLog2e, padded_rows};
+  a.mask_ok = a.mask ? mask_prefix_slots : nullptr;
   hipStream_t s = as_stream(stream);
   // 128-query tiles with a three-deep ring once there is plenty of work (three workgroups
   // per CU); else 64-query tiles with a two-deep ring: 32 KB of LDS and ~100 registers let

@@ -246,34 +246,44 @@ extern "C" int bt_build_offsets(const void *atten_mask, int mask_dtype, int batc
   return BT_OK;
 }
 
+extern "C" int bt_mask_prefix_slots(const void *atten_mask, int mask_dtype, int batch_size,
+                                    int seq_len, const int *batch_idx, int *slots, void *stream) {
+  BT_REQUIRE(atten_mask && batch_idx && slots, BT_ERR_INVALID_ARGUMENT,
+             "bt_mask_prefix_slots: null pointer argument");
+  BT_REQUIRE(batch_size > 0 && seq_len > 0, BT_ERR_INVALID_ARGUMENT,
+             "bt_mask_prefix_slots: batch_size=%d seq_len=%d must be positive", batch_size,
+             seq_len);
+  BT_REQUIRE(mask_dtype == BT_F16 || mask_dtype == BT_F32, BT_ERR_INVALID_ARGUMENT,
+             "bt_mask_prefix_slots: unknown mask dtype %d", mask_dtype);
+  BT_REQUIRE((long long)batch_size * seq_len < (1ll << 31), BT_ERR_UNSUPPORTED,
+             "bt_mask_prefix_slots: too many rows");
+  hipStream_t s = as_stream(stream);
+  // always all 256 workgroups: one without rows reports "nothing wrong"
+  if (mask_dtype == BT_F16)
+    mask_prefix_kernel<half_t><<<kPrefixBlocks, kPrefixWaves * kWave, 0, s>>>(
+        (const half_t *)atten_mask, batch_idx, slots, batch_size, seq_len);
+  else
+    mask_prefix_kernel<float><<<kPrefixBlocks, kPrefixWaves * kWave, 0, s>>>(
+        (const float *)atten_mask, batch_idx, slots, batch_size, seq_len);
+  BT_CHECK_LAUNCH("mask_prefix_kernel");
+  return BT_OK;
+}
+
 extern "C" int bt_mask_is_prefix(const void *atten_mask, int mask_dtype, int batch_size,
                                  int seq_len, const int *batch_idx, int *scratch,
                                  int *is_prefix_host, void *stream) {
-  BT_REQUIRE(atten_mask && batch_idx && scratch && is_prefix_host, BT_ERR_INVALID_ARGUMENT,
-             "bt_mask_is_prefix: null pointer argument");
-  BT_REQUIRE(batch_size > 0 && seq_len > 0, BT_ERR_INVALID_ARGUMENT,
-             "bt_mask_is_prefix: batch_size=%d seq_len=%d must be positive", batch_size, seq_len);
-  BT_REQUIRE(mask_dtype == BT_F16 || mask_dtype == BT_F32, BT_ERR_INVALID_ARGUMENT,
-             "bt_mask_is_prefix: unknown mask dtype %d", mask_dtype);
-  const long long rows = (long long)batch_size * seq_len;
-  BT_REQUIRE(rows < (1ll << 31), BT_ERR_UNSUPPORTED, "bt_mask_is_prefix: too many rows");
+  BT_REQUIRE(is_prefix_host, BT_ERR_INVALID_ARGUMENT, "bt_mask_is_prefix: null pointer argument");
+  const int rc = bt_mask_prefix_slots(atten_mask, mask_dtype, batch_size, seq_len, batch_idx,
+                                      scratch, stream);
+  if (rc != BT_OK) return rc;
   hipStream_t s = as_stream(stream);
-  const long long want = (rows + kPrefixWaves - 1) / kPrefixWaves;
-  const int grid = (int)(want < kPrefixBlocks ? want : kPrefixBlocks);
-  if (mask_dtype == BT_F16)
-    mask_prefix_kernel<half_t><<<grid, kPrefixWaves * kWave, 0, s>>>(
-        (const half_t *)atten_mask, batch_idx, scratch, batch_size, seq_len);
-  else
-    mask_prefix_kernel<float><<<grid, kPrefixWaves * kWave, 0, s>>>(
-        (const float *)atten_mask, batch_idx, scratch, batch_size, seq_len);
-  BT_CHECK_LAUNCH("mask_prefix_kernel");
   int slots[kPrefixBlocks];
-  hipError_t e = hipMemcpyAsync(slots, scratch, grid * sizeof(int), hipMemcpyDeviceToHost, s);
+  hipError_t e = hipMemcpyAsync(slots, scratch, sizeof(slots), hipMemcpyDeviceToHost, s);
   if (e != hipSuccess) return hip_fail(e, "copy of the prefix-mask verdict");
   e = hipStreamSynchronize(s);
   if (e != hipSuccess) return hip_fail(e, "stream synchronize for the prefix-mask verdict");
   int all = 1;
-  for (int i = 0; i < grid; ++i) all &= slots[i] != 0;
+  for (int i = 0; i < kPrefixBlocks; ++i) all &= slots[i] != 0;
   *is_prefix_host = all;
   return BT_OK;
 }

@@ -142,7 +142,7 @@ def gemm_qkv_bias_split(a, wt_qkv, bias_qkv, head_num, size_per_head=64, valid_r
 
 
 def _attention(fn, qkv_heads, batch_idx, batch_size, seq_len, scale, padded_rows, out,
-               seq_order=None, mask=None, bias=None, prefetch=None):
+               seq_order=None, mask=None, bias=None, prefetch=None, extra=()):
     _, head_num, rows_cap, d = qkv_heads.shape
     if out is None:
         out = torch.zeros(rows_cap, head_num * d, dtype=qkv_heads.dtype, device=qkv_heads.device)
@@ -151,7 +151,7 @@ def _attention(fn, qkv_heads, batch_idx, batch_size, seq_len, scale, padded_rows
     _check(fn(_ptr(qkv_heads), _ptr(out), _ptr(batch_idx), _ptr(seq_order), _ptr(mask), _ptr(bias),
               batch_size, seq_len, rows_cap, head_num, d, float(scale), int(padded_rows),
               _ptr(prefetch), prefetch.numel() * prefetch.element_size() if prefetch is not None else 0,
-              _stream()))
+              *extra, _stream()))
     return out
 
 
@@ -162,9 +162,22 @@ def attention_short(qkv_heads, batch_idx, batch_size, seq_len, scale, padded_row
 
 
 def attention_grouped(qkv_heads, batch_idx, batch_size, seq_len, scale, padded_rows=False,
-                      out=None, seq_order=None, mask=None, bias=None, prefetch=None):
+                      out=None, seq_order=None, mask=None, bias=None, prefetch=None,
+                      mask_prefix_slots=None):
     return _attention(kernel_lib().bt_attention_grouped, qkv_heads, batch_idx, batch_size,
-                      seq_len, scale, padded_rows, out, seq_order, mask, bias, prefetch)
+                      seq_len, scale, padded_rows, out, seq_order, mask, bias, prefetch,
+                      extra=(_ptr(mask_prefix_slots),))
+
+
+def mask_prefix_slots(mask, batch_idx, out=None):
+    """int32[256] on the device, all ones when mask [B,S,S] is the plain prefix mask of the
+    lengths in batch_idx (asynchronous; attention_grouped takes the array)."""
+    B, S = mask.shape[0], mask.shape[1]
+    if out is None:
+        out = torch.empty(256, dtype=torch.int32, device=mask.device)
+    _check(kernel_lib().bt_mask_prefix_slots(_ptr(mask), _dtype_code(mask), B, S, _ptr(batch_idx),
+                                             _ptr(out), _stream()))
+    return out
 
 
 def add_bias_residual_layernorm(out, residual, bias, gamma, beta, eps=1e-6, valid_rows=None,

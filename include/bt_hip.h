@@ -92,9 +92,16 @@ int bt_build_offsets(const void *atten_mask, int mask_dtype, int batch_size, int
  * len_b keys, which gives the same result as applying it (the logits of the ones are not
  * shifted, the exp of the others is exactly 0).
  * The reference always applies the tensor on that path (attention_fused.cu:234-237); no
- * counterpart there.  scratch: device int[256], overwritten.  Waits for the stream and
- * writes 0 / 1 to *is_prefix_host.
+ * counterpart there.
+ *   bt_mask_prefix_slots  asynchronous: 256 workgroups each write 1 ("nothing wrong in
+ *                         my share of the rows") or 0 to slots[0..255] (device); the
+ *                         mask is the prefix mask when every slot is 1.  The attention
+ *                         entry below takes such an array and decides on the device.
+ *   bt_mask_is_prefix     the same pass into scratch (device int[256]), then waits for
+ *                         the stream and writes the verdict 0 / 1 to *is_prefix_host.
  */
+int bt_mask_prefix_slots(const void *atten_mask, int mask_dtype, int batch_size, int seq_len,
+                         const int *batch_idx, int *slots, void *stream);
 int bt_mask_is_prefix(const void *atten_mask, int mask_dtype, int batch_size, int seq_len,
                       const int *batch_idx, int *scratch, int *is_prefix_host, void *stream);
 
@@ -185,6 +192,11 @@ int bt_gemm_qkv_bias_split(const void *a, const int *a_row_index, const void *wt
  *   seq_order (nullable): a permutation of the sequence indices from
  *                     bt_build_offsets; workgroups are issued in that order so the
  *                     longest sequences start first.  Results do not depend on it.
+ *   mask_prefix_slots (bt_attention_grouped; nullable): the int[256] that
+ *                     bt_mask_prefix_slots filled for this atten_mask earlier on the
+ *                     stream.  When all are 1 the kernel ignores the tensor and stops at
+ *                     the lengths, which gives the same result; decided on the device,
+ *                     so the call stays asynchronous.
  *
  * bt_attention_short keeps the whole logits row of a query tile in registers
  * (exact two-pass softmax, seq_len <= 512).  Replaces wmma_attention[_rm]_kernel
@@ -207,7 +219,8 @@ int bt_attention_grouped(const void *qkv_heads, void *attention_output, const in
                          const int *seq_order, const void *atten_mask, const void *attention_bias,
                          int batch_size, int seq_len, int rows_cap, int head_num,
                          int size_per_head, float scale, int padded_rows, const void *prefetch,
-                         unsigned long long prefetch_bytes, void *stream);
+                         unsigned long long prefetch_bytes, const int *mask_prefix_slots,
+                         void *stream);
 
 /*
  * out = LayerNorm((out + residual) + bias) * gamma + beta, in place on `out`,

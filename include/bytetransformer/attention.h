@@ -46,6 +46,10 @@ struct AttentionInferParam {
   // Extension: atten_mask is known to be the plain prefix mask of et_param's lengths; the
   // padded rows then need no mask tensor (keys stop at each length: the same result).
   bool mask_is_prefix = false;
+  // Extension: or the verdict slots of the device-side check (bt_mask_prefix_slots) of
+  // this mask, already enqueued on the stream; else the layer runs the check itself into
+  // `buf` whenever the mask tensor is in use.
+  const int *mask_prefix_slots = nullptr;
 };
 
 template <OperationType OpType>
@@ -88,7 +92,8 @@ class Attention {
   void initialize(AttentionParam<OpType> param) { param_ = param; }
 
   // Both kernels keep logits and probabilities on chip: no attention scratch.
-  virtual unsigned long long cal_bufsize() const { return 0; }
+  // 256 ints: the verdict slots of the device-side prefix-mask check (padded rows)
+  virtual unsigned long long cal_bufsize() const { return 256 * sizeof(int); }
 
   bool uses_short_kernel(int seq_len) const {
     return use_fused_attention_ && seq_len <= short_seq_limit();

@@ -94,7 +94,8 @@ class BertEncoder {
     const unsigned long long rows = (unsigned long long)max_batch_size_ * max_seq_len_;
     const unsigned long long tensor = rows * head_num_ * size_per_head_;
     unsigned long long n = align_up((6 + intermediate_size_) * tensor * sizeof(DataType_), 256);
-    n += align_up((rows * 2 + 2 * (unsigned long long)max_batch_size_ + 2) * sizeof(int), 256);
+    // (+ 256 ints: the verdict slots of the prefix-mask check of the padded path)
+    n += align_up((rows * 2 + 2 * (unsigned long long)max_batch_size_ + 2 + 256) * sizeof(int), 256);
     n += align_up(layer_weight_elems() * sizeof(DataType_), 256);
     n += align_up(splitk_scratch_bytes(rows, (unsigned long long)head_num_ * size_per_head_), 256);
     return n;

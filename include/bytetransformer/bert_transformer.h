@@ -136,7 +136,7 @@ class BertTransformer {
   // Scratch layout (elements of DataType_, T = max_batch*max_seq*hidden):
   //   [0,3T) qkv heads | [3T,4T) attention out | [4T,5T) projection / LN1 |
   //   [5T,(5+mult)T) FFN1 | word_idx int[B*S] | batch_idx int[B+1] | seq order int[B] |
-  //   pre-packed weights (3+1+2*mult)*H*H | split-k partial sums | attention scratch (none)
+  //   pre-packed weights (3+1+2*mult)*H*H | split-k partial sums | attention scratch (256 ints)
   unsigned long long cal_bufsize() {
     const unsigned long long rows = (unsigned long long)max_batch_size_ * max_seq_len_;
     const unsigned long long hidden = (unsigned long long)head_num_ * size_per_head_;

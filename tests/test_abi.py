@@ -52,8 +52,8 @@ def test_argument_validation_returns_codes_without_gpu():
     assert "needs valid_rows" in err()
     assert lib.bt_attention_short(p, p, p, None, None, None, 1, 1024, 1024, 12, 64, 0.125, 0, None, 0, None) == 2
     assert "exceeds 512" in err()
-    assert lib.bt_attention_grouped(p, p, p, None, None, None, 1, 16, 16, 12, 48, 0.125, 0, None, 0, None) == 2
-    assert lib.bt_attention_grouped(p, p, p, None, p, None, 1, 16, 16, 12, 64, 0.125, 0, None, 0, None) == 1
+    assert lib.bt_attention_grouped(p, p, p, None, None, None, 1, 16, 16, 12, 48, 0.125, 0, None, 0, None, None) == 2
+    assert lib.bt_attention_grouped(p, p, p, None, p, None, 1, 16, 16, 12, 64, 0.125, 0, None, 0, None, None) == 1
     assert "only applied on padded rows" in err()
     assert lib.bt_compress(p, p, p, p, 2, 4, 12, None) == 2 and "multiple of 8" in err()
     assert lib.bt_build_offsets(p, 7, 2, 4, p, p, None, None, None) == 1 and "dtype" in err()

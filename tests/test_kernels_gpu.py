@@ -609,6 +609,47 @@ def test_attention_arbitrary_mask_on_padded_rows(device, kind, S, att_order):
         assert err.max() <= 4e-3, (b, err.max())
 
 
+@pytest.mark.parametrize("qb", [1, 2])
+def test_attention_drops_a_prefix_mask_on_the_device(device, qb, att_order):
+    """The streaming kernel with the verdict slots of the device-side mask check: a plain
+    prefix mask is ignored (keys stop at the lengths: the values of the padded rows'
+    attention over the valid keys, as with the tensor applied); any other mask - one
+    element flipped - is applied exactly as without the slots."""
+    _say("attention mask slots", qb)
+    rs = np.random.RandomState(77 + qb)
+    B, S, heads = 3, 150, 2
+    lens = np.array([150, 40, 97])
+    qkv = rs.standard_normal((3, heads, B * S, 64)).astype(np.float16)
+    mask = workload.make_mask(lens, S, np.float16)
+    qd, md = _dev(qkv, device), _dev(mask, device)
+    bi, _, _ = ops.build_offsets(md)
+    scale = 1 / math.sqrt(64)
+    ops.set_option("attention_qb", qb)
+    try:
+        slots = ops.mask_prefix_slots(md, bi)
+        assert int(slots.min()) == 1
+        with_tensor = ops.attention_grouped(qd, bi, B, S, scale, True, mask=md)
+        dropped = ops.attention_grouped(qd, bi, B, S, scale, True, mask=md, mask_prefix_slots=slots)
+        by_length = ops.attention_grouped(qd, bi, B, S, scale, True)
+        # ignoring the tensor: the mask-free instantiation's values up to the last bits
+        # of the fp32 logits (the additive path folds the scale in another order)
+        d1 = (dropped.float() - by_length.float()).abs().max().item()
+        d2 = (dropped.float() - with_tensor.float()).abs().max().item()
+        assert d1 <= 2e-3 and d2 <= 2e-3, (d1, d2)
+        # a mask that is not a prefix mask: slots say so, and the tensor is applied
+        bad = mask.copy()
+        bad[1, 7, 3] = 0
+        bd = _dev(bad, device)
+        bad_slots = ops.mask_prefix_slots(bd, bi)
+        assert int(bad_slots.min()) == 0
+        a = ops.attention_grouped(qd, bi, B, S, scale, True, mask=bd)
+        b = ops.attention_grouped(qd, bi, B, S, scale, True, mask=bd, mask_prefix_slots=bad_slots)
+        assert torch.equal(a, b)
+        assert not torch.equal(a, with_tensor)
+    finally:
+        ops.set_option("attention_qb", -1)
+
+
 @pytest.mark.parametrize("kind,S,padded,with_mask", [("short", 64, True, True), ("grouped", 200, True, True),
                                                     ("short", 100, False, False), ("grouped", 300, False, False),
                                                     ("grouped", 130, True, False)])
