@@ -25,7 +25,7 @@ void Attention<OpType>::infer(AttentionInferParam infer_param) {
     // prefix mask, whose terms are 0 for the keys of the sequence and vanish for the rest
     check_bt_error(bt_attention_f32(infer_param.qkv, infer_param.attention_output,
                                     infer_param.et_param.batch_idx, infer_param.seq_order,
-                                    infer_param.mask_is_prefix ? nullptr : infer_param.atten_mask,
+                                    infer_param.mask_prefix == 1 ? nullptr : infer_param.atten_mask,
                                     infer_param.attention_bias,
                                     infer_param.batch_size,
                                     infer_param.seq_len, rows_cap, head_num_, size_per_head_,
@@ -37,7 +37,7 @@ void Attention<OpType>::infer(AttentionInferParam infer_param) {
   // (unless the caller has checked that it is the plain prefix mask: stopping at the
   // lengths then gives the same result without reading batch x seq_len^2 mask elements
   // per head)
-  const void *mask = is_remove_padding_ || infer_param.mask_is_prefix
+  const void *mask = is_remove_padding_ || infer_param.mask_prefix == 1
                          ? nullptr
                          : (const void *)infer_param.atten_mask;
   if (size_per_head_ != 64) {
@@ -61,7 +61,7 @@ void Attention<OpType>::infer(AttentionInferParam infer_param) {
     // (every launch of the layer, a few microseconds) lets the kernel drop it when it is the
     // plain prefix mask - the usual case, worth 3-15 us of attention per layer.
     const int *slots = mask ? infer_param.mask_prefix_slots : nullptr;
-    if (mask && !slots && infer_param.buf) {
+    if (mask && !slots && infer_param.mask_prefix < 0 && infer_param.buf) {
       int *verdict = (int *)infer_param.buf;
       check_bt_error(bt_mask_prefix_slots(mask, Traits_::dtype, infer_param.batch_size,
                                           infer_param.seq_len, infer_param.et_param.batch_idx,

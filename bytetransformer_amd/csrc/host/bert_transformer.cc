@@ -101,7 +101,7 @@ void BertTransformer<OpType>::bert_infer(BertTransformerInferParam infer_param) 
     };
     attention_infer_param.attention_bias = infer_param.attention_bias;
     attention_infer_param.seq_order = seq_order;
-    attention_infer_param.mask_is_prefix = infer_param.offsets && infer_param.mask_is_prefix;
+    attention_infer_param.mask_prefix = infer_param.offsets ? infer_param.mask_prefix : -1;
     attention_layer_->infer(attention_infer_param);
     check_bt_error(bt_gemm_f32(attr_out_buf, nullptr, param_.attr_output_kernel, nullptr,
                                attr_matmul_buf, 0, valid_rows, packed_cap, rows_hint, hidden, hidden,
@@ -157,7 +157,7 @@ void BertTransformer<OpType>::bert_infer(BertTransformerInferParam infer_param) 
   };
   attention_infer_param.attention_bias = infer_param.attention_bias;
   attention_infer_param.seq_order = seq_order;
-  attention_infer_param.mask_is_prefix = infer_param.offsets && infer_param.mask_is_prefix;
+  attention_infer_param.mask_prefix = infer_param.offsets ? infer_param.mask_prefix : -1;
   // the three weight matrices the rest of the layer reads, when they lie back to back:
   // the attention kernel pulls them into the memory-side cache while it runs
   if (wt_inter == wt_proj + (size_t)hidden * hidden && wt_out == wt_inter + (size_t)hidden * inter) {

@@ -107,7 +107,7 @@ class BTEncoder : public IBTEncoder {
       offsets.valid_word_num = plan.valid_word_num;
       infer_param.offsets = &offsets;
       infer_param.seq_order = plan.seq_order.data_ptr<int>();
-      infer_param.mask_is_prefix = plan.prefix_state == 1;
+      infer_param.mask_prefix = plan.prefix_state;
     }
     encoder.infer(infer_param);
   }

@@ -43,12 +43,13 @@ struct AttentionInferParam {
   // remaining weights); the attention kernel warms the memory-side cache with it.
   const void *prefetch = nullptr;
   unsigned long long prefetch_bytes = 0;
-  // Extension: atten_mask is known to be the plain prefix mask of et_param's lengths; the
-  // padded rows then need no mask tensor (keys stop at each length: the same result).
-  bool mask_is_prefix = false;
+  // Extension: what the caller knows about atten_mask: 1 = the plain prefix mask of
+  // et_param's lengths (the padded rows then need no mask tensor: keys stop at each length,
+  // the same result), 0 = something else, -1 = not checked.
+  int mask_prefix = -1;
   // Extension: or the verdict slots of the device-side check (bt_mask_prefix_slots) of
-  // this mask, already enqueued on the stream; else the layer runs the check itself into
-  // `buf` whenever the mask tensor is in use.
+  // this mask, already enqueued on the stream; else, with mask_prefix == -1, the layer runs
+  // the check itself into `buf` whenever the mask tensor is in use.
   const int *mask_prefix_slots = nullptr;
 };
 

@@ -69,10 +69,11 @@ struct BertTransformerInferParam {
   const ET_Param *offsets = NULL;
   // ... and the matching sequence order (int[batch_size], longest first), or NULL.
   const int *seq_order = NULL;
-  // ... and the caller's finding (bt_mask_is_prefix) that atten_mask is exactly the prefix
-  // mask of those offsets: on the padded rows the attention then stops at each length
-  // instead of reading the tensor - the same result, the masked terms being exactly zero.
-  bool mask_is_prefix = false;
+  // ... and the caller's finding (bt_mask_is_prefix) about atten_mask: 1 = it is exactly the
+  // prefix mask of those offsets - on the padded rows the attention then stops at each
+  // length instead of reading the tensor, the same result, the masked terms being exactly
+  // zero; 0 = it is not; -1 = not checked (the layer then checks on the device).
+  int mask_prefix = -1;
 };
 
 template <OperationType OpType>
