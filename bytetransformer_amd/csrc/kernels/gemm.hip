@@ -483,8 +483,9 @@ static int launch_gemm(GemmArgs p, hipStream_t s) {
   //   0: 256x256, 2, 2x4, 0   wide outputs: one tile per CU, every wave loads and computes
   //   1: 128x128, 3, 2x2, 4   narrow outputs (projection, FFN2) and small problems
   //   2: 256x128, 3, 4x2, 4   narrow outputs with enough rows to fill the chip
-  //   3: 256x192, 2, 4x2, 0   outputs that split into 192-wide panels but not into a
-  //                           full wave of 256-wide ones (QKV at hidden 768)
+  //   3: 256x192, 2, 4x2, 4   outputs that split into 192-wide panels but not into a
+  //                           full wave of 256-wide ones (QKV at hidden 768); 141 registers
+  //                           leave room for the loader waves (-2 to -4 % against unified)
   //   4:  32x64,  4, 1x2, 2   a few hundred rows or fewer: the k loop of one tile is the
   //                           whole run time, and a small tile has the shortest k-step
   //   5: 128x128, 2, 2x2, 4   tile 1 with a two-deep ring: 64 KB of LDS, so two workgroups
@@ -544,7 +545,7 @@ static int launch_gemm(GemmArgs p, hipStream_t s) {
     case 2:
       return launch_gemm_tile<256, 128, 3, 4, 2, 4, 1, EPI>(p, s);
     case 3:
-      return launch_gemm_tile<256, 192, 2, 4, 2, 0, 1, EPI>(p, s);
+      return launch_gemm_tile<256, 192, 2, 4, 2, 4, 1, EPI>(p, s);
     case 4:
       return launch_gemm_tile<32, 64, 4, 1, 2, 2, 0, EPI>(p, s);
     case 5:

@@ -48,7 +48,7 @@ const char *bt_last_error_string(void);
 /*
  * Tuning knob for experiments and tests; no counterpart in the reference.
  *   "gemm_tile"     -1 heuristic | 0: 256x256 tile, 8 waves | 1: 128x128, 4 computing + 4 loader
- *                   waves | 2: 256x128, 8 + 4 waves | 3: 256x192, 8 waves | 4: 32x64, 2 + 2 waves
+ *                   waves | 2: 256x128, 8 + 4 waves | 3: 256x192, 8 + 4 waves | 4: 32x64, 2 + 2 waves
  *                   | 5: 128x128 with a two-deep ring (two workgroups per CU)
  *   "attention_qb"  -1 heuristic | 1 | 2: 16-query blocks per wave in the grouped kernel
  *   "prefetch"      1 (default) | 0: honour / ignore the prefetch hint of the attention entries
