@@ -91,6 +91,8 @@ HOST_ABI = {
                                          _P, _P, c_int, c_int, _P]),
     "bt_encoder_layer_forward_bias": (c_int, [POINTER(EncoderConfig), POINTER(LayerWeights), _P,
                                               _P, _P, _P, _P, c_int, c_int, _P]),
+    "bt_encoder_layer_forward_static": (c_int, [POINTER(EncoderConfig), POINTER(LayerWeights), _P,
+                                                _P, _P, _P, c_int, c_int, _P]),
     "bt_encoder_forward_bufsize": (c_ulonglong, [POINTER(EncoderConfig)]),
     "bt_encoder_prepack_bytes": (c_ulonglong, [POINTER(EncoderConfig), c_int]),
     "bt_encoder_prepack": (c_int, [POINTER(EncoderConfig), c_int, POINTER(LayerWeights), _P, _P]),

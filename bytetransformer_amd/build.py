@@ -24,6 +24,7 @@ HIPCC = os.path.join(ROCM, "bin", "hipcc")
 
 KERNEL_SOURCES = ["padding.hip", "layernorm.hip", "gemm.hip", "attention.hip", "fp32_path.hip"]
 HOST_SOURCES = ["attention.cc", "bert_transformer.cc", "bert_encoder.cc", "c_api.cc"]
+HOST_DEVICE_SOURCE = "layer_static_scratch.hip"
 TH_OP_SOURCES = ["ths_op_f.cc", "ths_op.cc"]
 
 # Packed-fp32 VALU ops are switched off for every device compile.
@@ -74,8 +75,16 @@ def build_host():
     os.makedirs(LIB, exist_ok=True)
     out = os.path.join(LIB, "libbytetransformer.so")
     srcs = [os.path.join(CSRC, "host", s) for s in HOST_SOURCES]
-    _run(["g++"] + HOST_FLAGS + ["-shared", "-I", INC, "-I", os.path.join(ROCM, "include")] + srcs +
-         ["-L", LIB, "-lbt_hip", "-Wl,-rpath,$ORIGIN", "-o", out])
+    obj_dir = os.path.join(PKG, "_build")
+    os.makedirs(obj_dir, exist_ok=True)
+    # the one file with a device symbol (the static scratch array) goes through hipcc
+    static_obj = os.path.join(obj_dir, "layer_static_scratch.o")
+    _run([HIPCC] + HIP_FLAGS + ["-I", INC, "-I", os.path.join(CSRC, "host"), "-c",
+                                os.path.join(CSRC, "host", HOST_DEVICE_SOURCE), "-o", static_obj])
+    _run(["g++"] + HOST_FLAGS + ["-shared", "-I", INC, "-I", os.path.join(CSRC, "host"),
+                                 "-I", os.path.join(ROCM, "include")] + srcs + [static_obj] +
+         ["-L", LIB, "-lbt_hip", "-L", os.path.join(ROCM, "lib"), "-lamdhip64",
+          "-Wl,-rpath,$ORIGIN", "-o", out])
     return out
 
 

@@ -7,6 +7,7 @@
 
 #include "bytetransformer/bert_encoder.h"
 #include "bytetransformer/bert_transformer.h"
+#include "host_error.h"
 
 namespace {
 thread_local std::string g_error;
@@ -255,5 +256,9 @@ extern "C" int bt_encoder_forward(const bt_encoder_config *cfg, int num_layers,
     return BT_ERR_INVALID_ARGUMENT;
   }
 }
+
+namespace bt_host {
+void set_error(const std::string &message) { g_error = message; }
+}  // namespace bt_host
 
 extern "C" const char *bt_encoder_last_error(void) { return g_error.c_str(); }

@@ -67,6 +67,30 @@ int bt_encoder_layer_forward_bias(const bt_encoder_config *cfg, const bt_layer_w
                                   int batch_size, int seq_len, void *stream);
 
 /*
+ * One encoder layer with NO caller-owned scratch: bt_encoder_layer_forward_bias with
+ * `buf` replaced by a device array that the library itself holds (BT_STATIC_SCRATCH_BYTES
+ * per GPU the library runs on, from the first call on that GPU until the process ends).
+ * No counterpart in the reference; it is for callers that cannot allocate device memory
+ * for the workspace: code under HIP-graph capture, tight serving loops, harnesses that
+ * forbid hipMalloc.  The call allocates nothing (no hipMalloc / hipFree, no allocating
+ * library routine) and never waits for the device.
+ *   - cfg's scratch need (bt_encoder_bufsize) must not exceed BT_STATIC_SCRATCH_BYTES,
+ *     else BT_ERR_UNSUPPORTED with a message stating both sizes (BERT-base fp16 fits up
+ *     to about 1300 padded rows, e.g. batch 1-2 x 512 or batch 4 x 256);
+ *   - every call on one GPU shares that GPU's array: calls that overlap on one GPU (two
+ *     streams, two threads) race; calls on one stream are ordered and safe;
+ *   - the first call on a GPU looks the array's address up (hipGetSymbolAddress): make
+ *     it outside stream capture.
+ * attention_bias is nullable as in bt_encoder_layer_forward_bias; results are identical
+ * to that entry point's.
+ */
+#define BT_STATIC_SCRATCH_BYTES (32ull << 20)
+int bt_encoder_layer_forward_static(const bt_encoder_config *cfg, const bt_layer_weights *weights,
+                                    const void *input, const void *atten_mask,
+                                    const void *attention_bias, void *output, int batch_size,
+                                    int seq_len, void *stream);
+
+/*
  * Whole encoder in one call: num_layers layers (weights[l] = layer l) over one padded
  * batch, hidden state kept on the packed rows between layers.  No counterpart in the
  * reference, whose interface is one layer per call: the mask prefix sum runs once,
