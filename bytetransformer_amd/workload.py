@@ -136,6 +136,36 @@ def make_workload(cfg, layers=None, bias_std=0.0, random_affine=False) -> Worklo
     return Workload(cfg, lens, x, mask, ws)
 
 
+def make_reference_test_workload(batch, seq_len, head_num, head_size=64, avg_seqlen=0, layers=1,
+                                 dtype="fp16", seed=0) -> Workload:
+    """The data of the reference's own test script
+    (unit_test/python_scripts/bert_transformer_test.py:93-114): every one of the 12
+    tensors of a layer and the input drawn from U(-0.4, 0.4) (gamma and beta included),
+    lengths integer-uniform on [2*avg - S, S] when 2*avg > S else on [0, 2*avg]
+    (avg_seqlen 0 = every sequence full)."""
+    np_dtype = np.float16 if dtype == "fp16" else np.float32
+    hidden, ffn = head_num * head_size, 4 * head_num * head_size
+    rs = np.random.RandomState(seed)
+    avg = avg_seqlen if avg_seqlen > 0 else seq_len
+    low, high = (2 * avg - seq_len, seq_len + 1) if 2 * avg > seq_len else (0, 2 * avg + 1)
+    lens = rs.randint(low, high, size=batch).astype(np.int32)
+
+    def uni(*shape):
+        return rs.uniform(-0.4, 0.4, size=shape).astype(np.float32).astype(np_dtype)
+
+    shapes = {"qkv_kernel": (hidden, 3 * hidden), "qkv_bias": (3 * hidden,),
+              "attr_output_kernel": (hidden, hidden), "attr_output_bias": (hidden,),
+              "attr_output_layernorm_gamma": (hidden,), "attr_output_layernorm_beta": (hidden,),
+              "inter_kernel": (hidden, ffn), "inter_bias": (ffn,),
+              "output_kernel": (ffn, hidden), "output_bias": (hidden,),
+              "output_layernorm_gamma": (hidden,), "output_layernorm_beta": (hidden,)}
+    ws = [{n: uni(*shapes[n]) for n in WEIGHT_NAMES} for _ in range(layers)]
+    x = uni(batch, seq_len, hidden)
+    cfg = EncoderConfig("reference-test-data", batch, seq_len, head_num, head_size, layers,
+                        dtype=dtype, lens=tuple(int(v) for v in lens), seed=seed)
+    return Workload(cfg, lens, x, make_mask(lens, seq_len, np_dtype), ws)
+
+
 def layer_flops(cfg: EncoderConfig, lens):
     """Algorithmic flops of one layer: the four dense GEMMs on the M valid
     tokens plus unpadded, non-causal attention (QK^T and PV)."""

@@ -29,12 +29,29 @@ def _dev(a, device):
     return torch.from_numpy(np.ascontiguousarray(a)).to(device)
 
 
+_ORACLE_CACHE = {}
+
+
 def _oracle(wl, n_layers=None, **kw):
+    """The CPU oracle's masked output; memoised on the bytes of every operand, because
+    each test runs once per attention dispatch and the oracle does not depend on it."""
+    import zlib
     layers = wl.layers if n_layers is None else wl.layers[:n_layers]
-    layers32 = [{k: np.asarray(v, np.float32) for k, v in w.items()} for w in layers]
-    out = O.encoder(wl.x.astype(np.float32), wl.mask.astype(np.float32), layers32,
-                    wl.cfg.head_num, **kw)
-    return O.masked_output(out.numpy(), wl.lens)
+    crc = zlib.crc32(np.ascontiguousarray(wl.x).tobytes())
+    crc = zlib.crc32(np.ascontiguousarray(wl.mask).tobytes(), crc)
+    for w in layers:
+        for name in workload.WEIGHT_NAMES:
+            crc = zlib.crc32(np.ascontiguousarray(w[name]).tobytes(), crc)
+    key = (crc, wl.x.shape, wl.cfg.head_num, len(layers), tuple(int(v) for v in wl.lens),
+           repr(sorted(kw.items())))
+    if key not in _ORACLE_CACHE:
+        layers32 = [{k: np.asarray(v, np.float32) for k, v in w.items()} for w in layers]
+        out = O.encoder(wl.x.astype(np.float32), wl.mask.astype(np.float32), layers32,
+                        wl.cfg.head_num, **kw)
+        if len(_ORACLE_CACHE) > 8:
+            _ORACLE_CACHE.clear()
+        _ORACLE_CACHE[key] = O.masked_output(out.numpy(), wl.lens)
+    return _ORACLE_CACHE[key]
 
 
 def _gpu_layers(wl, device, n_layers=None, **kw):
@@ -51,14 +68,16 @@ def _run_c_api(wl, device, n_layers=None, **kw):
     return out.cpu().numpy()
 
 
-@pytest.fixture(autouse=True)
-def _short_kernel_for_fused_runs():
-    """By default the host sends every length to the streaming attention kernel (the faster
-    one); these tests let use_fused_attention = True select the LDS-resident short kernel up to
-    its capacity again, so that both kernels are covered through the layer."""
+@pytest.fixture(autouse=True, params=[0, 512], ids=["default-dispatch", "short-kernel"])
+def attention_short_limit(request):
+    """Every test of this file runs twice.  "default-dispatch": the library as shipped and
+    as the benchmark times it - every length goes to the streaming attention kernel, with
+    its balanced work list and cache warm-up duty on large launches.  "short-kernel":
+    use_fused_attention = True selects the LDS-resident short kernel up to its capacity of
+    512 tokens again, so that both kernels are covered through the layer."""
     from bytetransformer_amd import ops
-    ops.set_option("attention_short_limit", 512)
-    yield
+    ops.set_option("attention_short_limit", request.param)
+    yield request.param
     ops.set_option("attention_short_limit", 0)
 
 
@@ -165,6 +184,14 @@ def test_cfg3_long_sequences_grouped_kernel(device):
     _check(got, exp, wl.lens, tag="cfg3/L2")
 
 
+def test_cfg3_full_depth_twelve_layers(device):
+    """cfg3 at its full depth through the operator (the path the benchmark times)."""
+    _say("cfg3 twelve layers")
+    wl = workload.make_workload("cfg3")
+    assert len(wl.layers) == 12
+    _check(_run_th_op(wl, device), _oracle(wl), wl.lens, tag="cfg3/L12/th_op")
+
+
 def test_cfg4_bert_large_variable_and_fixed(device):
     _say("cfg4")
     wl = workload.make_workload("cfg4", layers=2)
@@ -177,6 +204,40 @@ def test_cfg4_bert_large_variable_and_fixed(device):
     # two roundings of the same math (mask term folded before / after the scale): a few
     # fp16 ulps at |y| in [2, 4) after two layers, far inside the parity budget
     assert np.abs(rm.astype(np.float32) - pad.astype(np.float32)).max() <= 8e-3
+
+
+@pytest.mark.parametrize("name", ["cfg4", "cfg4_fixed"])
+def test_cfg4_full_depth_twenty_four_layers(device, name):
+    """BERT-large at all 24 layers, ragged lengths and the fixed-length twin, through the
+    operator; the fixed-length twin also on the padded rows."""
+    _say(name, "twenty-four layers")
+    wl = workload.make_workload(name)
+    assert len(wl.layers) == 24
+    exp = _oracle(wl)
+    got = _run_th_op(wl, device)
+    _check(got, exp, wl.lens, tag=name + "/L24/th_op")
+    if name == "cfg4_fixed":
+        pad = _run_th_op(wl, device, rm=False)
+        _check(pad, exp, wl.lens, pads_must_be_zero=False, tag=name + "/L24/th_op/padded rows")
+
+
+# ---- the reference's own test distribution -----------------------------------------
+@pytest.mark.parametrize("B,S,heads,avg,layers", [(4, 64, 2, 40, 1), (8, 128, 4, 77, 3),
+                                                  (16, 512, 12, 307, 1), (16, 512, 12, 307, 12)],
+                         ids=["small", "medium-3-layers", "cfg2-shape-1-layer",
+                              "cfg2-shape-12-layers"])
+def test_reference_test_distribution(device, B, S, heads, avg, layers):
+    """The only data the reference's own script ever tests with
+    (unit_test/python_scripts/bert_transformer_test.py:93-114): every weight, bias, gamma,
+    beta and the input drawn from U(-0.4, 0.4), lengths uniform on [2*avg - S, S].
+    Activations there are ~50x larger than with N(0, 0.02) weights (|FFN2 output| ~ 50
+    before the last LayerNorm), so fp16 storage of the intermediates is what is tested."""
+    _say("reference distribution", B, S, heads, avg, layers)
+    wl = workload.make_reference_test_workload(B, S, heads, avg_seqlen=avg, layers=layers, seed=2)
+    exp = _oracle(wl)
+    _check(_run_th_op(wl, device), exp, wl.lens, tag="ref-dist/th_op B%d S%d L%d" % (B, S, layers))
+    if layers == 1:
+        _check(_run_c_api(wl, device), exp, wl.lens, tag="ref-dist/c_api B%d S%d" % (B, S))
 
 
 def test_padded_path_applies_arbitrary_masks(device):
@@ -307,6 +368,22 @@ def test_fp32_gamma_beta_next_to_fp16_weights(device):
             wl.layers[0][n] = wl.layers[0][n].astype(np.float32)
     _check(_run_th_op(wl, device), exp, wl.lens, tag="g32/th_op")
     _check(_run_c_api(wl, device), exp, wl.lens, tag="g32/c_api")
+
+
+@pytest.mark.parametrize("tao", [0.5, 3.0])
+def test_fp16_softmax_temperature(device, tao):
+    """tao != 1 on the fp16 kernels (attention.h:32 of the reference: scale = 1/sqrt(d)/tao),
+    packed rows and padded rows."""
+    _say("fp16 tao", tao)
+    cfg = workload.EncoderConfig("tao", 4, 130, 3, layers=2, lens=(130, 9, 64, 77), seed=17)
+    wl = workload.make_workload(cfg, bias_std=0.05, random_affine=True)
+    for w in wl.layers:     # logits of a few units, so that the temperature matters
+        w["qkv_kernel"] = (w["qkv_kernel"].astype(np.float32) * 6).astype(np.float16)
+    exp = _oracle(wl, tao=tao)
+    assert np.abs(exp - _oracle(wl)).max() > 1e-2        # the temperature is not a no-op
+    _check(_run_c_api(wl, device, tao=tao), exp, wl.lens, tag="tao %.1f/packed" % tao)
+    got = O.masked_output(_run_c_api(wl, device, tao=tao, is_remove_padding=False), wl.lens)
+    _check(got, exp, wl.lens, tag="tao %.1f/padded rows" % tao)
 
 
 def test_ragged_edge_cases(device):
