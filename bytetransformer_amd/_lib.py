@@ -37,6 +37,9 @@ KERNEL_ABI = {
     "bt_build_offsets": (c_int, [_P, c_int, c_int, c_int, _IP, _IP, _IP, POINTER(c_int), _P]),
     "bt_mask_prefix_slots": (c_int, [_P, c_int, c_int, c_int, _IP, _IP, _P]),
     "bt_mask_is_prefix": (c_int, [_P, c_int, c_int, c_int, _IP, _IP, POINTER(c_int), _P]),
+    "bt_layer_prologue": (c_int, [_P, c_int, c_int, c_int, _IP, _IP, _IP, _IP, c_int,
+                                  POINTER(c_void_p), POINTER(c_void_p), POINTER(c_int),
+                                  POINTER(c_int), _P, _P]),
     "bt_compress": (c_int, [_P, _P, _IP, _IP, c_int, c_int, c_int, _P]),
     "bt_transpose_weight": (c_int, [_P, _P, c_int, c_int, _P]),
     "bt_transpose_weights": (c_int, [c_int, POINTER(c_void_p), POINTER(c_void_p), POINTER(c_int),

@@ -60,19 +60,18 @@ void BertEncoder<OpType>::infer(BertEncoderInferParam<DataType_> ip) {
   off += align_up(layer_weight_elems() * sizeof(DataType_), 256);
   float *splitk_buf = (float *)(base + off);
 
-  check_bt_error(bt_build_offsets(ip.atten_mask, Traits_::dtype, batch_size, seq_len,
-                                  et_param.batch_idx, et_param.word_idx, seq_order, nullptr,
-                                  stream));
-  const int *valid_rows = is_remove_padding_ ? et_param.batch_idx + batch_size : nullptr;
-  const int rows_hint = ip.valid_rows_hint;
-  const int L = (int)layers_.size();
-  // padded rows: the fp16 streaming attention applies the mask tensor unless this one pass
+  // padded rows: the fp16 streaming attention applies the mask tensor unless one pass
   // over it (once for all layers) finds the plain prefix mask of the lengths
   const bool check_mask = !is_remove_padding_ && OpType == OperationType::HALF &&
                           size_per_head_ == 64;
-  if (check_mask)
-    check_bt_error(bt_mask_prefix_slots(ip.atten_mask, Traits_::dtype, batch_size, seq_len,
-                                        et_param.batch_idx, mask_slots, stream));
+  // offsets and that verdict in one launch, once per forward
+  check_bt_error(bt_layer_prologue(ip.atten_mask, Traits_::dtype, batch_size, seq_len,
+                                   et_param.batch_idx, et_param.word_idx, seq_order,
+                                   check_mask ? mask_slots : nullptr, 0, nullptr, nullptr, nullptr,
+                                   nullptr, nullptr, stream));
+  const int *valid_rows = is_remove_padding_ ? et_param.batch_idx + batch_size : nullptr;
+  const int rows_hint = ip.valid_rows_hint;
+  const int L = (int)layers_.size();
 
   for (int l = 0; l < L; ++l) {
     const auto &w = layers_[l];

@@ -55,24 +55,54 @@ void BertTransformer<OpType>::bert_infer(BertTransformerInferParam infer_param) 
                   256);
   float *splitk_buf = (float *)(base + off);
 
-  // lengths from the mask (needed on both paths: keys past len_b are excluded),
-  // unless the caller already holds the offsets of this mask
-  int rows_hint = 0;
-  if (infer_param.offsets && infer_param.offsets->batch_idx && infer_param.offsets->word_idx) {
+  // k-contiguous weight copies handed in by the caller (fp16 only), with or without the
+  // fingerprint record that lets the prologue check them against the weights
+  const bool have_prepack = OpType == OperationType::HALF && param_.prepacked_kernels[0] &&
+                            param_.prepacked_kernels[1] && param_.prepacked_kernels[2] &&
+                            param_.prepacked_kernels[3];
+  const bool check_prepack = have_prepack && param_.prepack_state;
+  const void *w_src[4] = {param_.attr_kernel_QKV, param_.attr_output_kernel, param_.inter_kernel,
+                          param_.output_kernel};
+  const int w_k[4] = {hidden, hidden, hidden, inter};
+  const int w_n[4] = {3 * hidden, hidden, inter, hidden};
+
+  // Padded rows, fp16 streaming attention: the mask tensor is applied unless one pass over
+  // it finds the plain prefix mask of its lengths; the prologue leaves that verdict in the
+  // attention's scratch and the kernel decides on the device.
+  int *mask_slots = nullptr;
+  const bool have_offsets =
+      infer_param.offsets && infer_param.offsets->batch_idx && infer_param.offsets->word_idx;
+  if (OpType == OperationType::HALF && !is_remove_padding_ && size_per_head_ == 64 &&
+      !attention_layer_->uses_short_kernel(seq_len) && !(have_offsets && infer_param.mask_prefix >= 0))
+    mask_slots = (int *)(base + inner_buf_size_);
+
+  // One launch ahead of the layer: lengths and offsets from the mask (needed on both
+  // paths: keys past len_b are excluded), the prefix-mask verdict, the check of reused
+  // weight copies.  Rebuilt on every call, as the reference does
+  // (bert_transformer.cu:62-66), unless the caller vouches for offsets of its own.
+  int rows_hint = infer_param.valid_rows_hint > 0 ? infer_param.valid_rows_hint : 0;
+  {
+    void *w_dst[4] = {const_cast<DataType_ *>(param_.prepacked_kernels[0]),
+                      const_cast<DataType_ *>(param_.prepacked_kernels[1]),
+                      const_cast<DataType_ *>(param_.prepacked_kernels[2]),
+                      const_cast<DataType_ *>(param_.prepacked_kernels[3])};
+    if (!have_offsets || mask_slots || check_prepack)
+      check_bt_error(bt_layer_prologue(atten_mask, Traits_::dtype, batch_size, seq_len,
+                                       et_param.batch_idx, et_param.word_idx, seq_order,
+                                       mask_slots, check_prepack ? 4 : 0, w_src, w_dst, w_k, w_n,
+                                       check_prepack ? param_.prepack_state : nullptr, stream));
+  }
+  if (have_offsets) {
     et_param = *infer_param.offsets;
     rows_hint = et_param.valid_word_num;
     seq_order = const_cast<int *>(infer_param.seq_order);
-  } else {
-    check_bt_error(bt_build_offsets(atten_mask, Traits_::dtype, batch_size, seq_len,
-                                    et_param.batch_idx, et_param.word_idx, seq_order, nullptr,
-                                    stream));
   }
   const int *valid_rows = nullptr;
   const int *gather = nullptr;
   DataType_ *restore_target = nullptr;
-  // Row capacity of the launches over packed rows that follow the attention.  The
-  // caller's offsets carry the exact live count (the operator's mask plan read it back
-  // once), so these launches are sized for it instead of batch * seq_len: no workgroups
+  // Row capacity of the launches over packed rows that follow the attention.  A caller
+  // that passes offsets of its own vouches for their exact live count, so these launches
+  // are then sized for it instead of batch * seq_len: no workgroups
   // that only find out on the device that their rows do not exist (1.7-2.2 us per layer
   // at batch 16 x 512), and a short sequence in a long padded row still takes the split-k
   // FFN2.  The QKV product and the attention keep batch * seq_len: it is the row stride
@@ -86,7 +116,7 @@ void BertTransformer<OpType>::bert_infer(BertTransformerInferParam infer_param) 
     restore_target = transformer_out;
     transformer_out = inner_buf;  // FFN2 output reuses the dead qkv region
     valid_rows = et_param.batch_idx + batch_size;
-    if (rows_hint > 0 && rows_hint < rows) packed_cap = rows_hint;
+    if (have_offsets && rows_hint > 0 && rows_hint < rows) packed_cap = rows_hint;
   }
 
   if constexpr (OpType == OperationType::FP32) {
@@ -101,7 +131,7 @@ void BertTransformer<OpType>::bert_infer(BertTransformerInferParam infer_param) 
     };
     attention_infer_param.attention_bias = infer_param.attention_bias;
     attention_infer_param.seq_order = seq_order;
-    attention_infer_param.mask_prefix = infer_param.offsets ? infer_param.mask_prefix : -1;
+    attention_infer_param.mask_prefix = have_offsets ? infer_param.mask_prefix : -1;
     attention_layer_->infer(attention_infer_param);
     check_bt_error(bt_gemm_f32(attr_out_buf, nullptr, param_.attr_output_kernel, nullptr,
                                attr_matmul_buf, 0, valid_rows, packed_cap, rows_hint, hidden, hidden,
@@ -131,20 +161,14 @@ void BertTransformer<OpType>::bert_infer(BertTransformerInferParam infer_param) 
 
   // k-contiguous weight pre-pack: all four matrices in one launch, unless the
   // caller handed in copies it already made
-  const bool have_prepack = param_.prepacked_kernels[0] && param_.prepacked_kernels[1] &&
-                            param_.prepacked_kernels[2] && param_.prepacked_kernels[3];
   if (have_prepack) {
     wt_qkv = const_cast<DataType_ *>(param_.prepacked_kernels[0]);
     wt_proj = const_cast<DataType_ *>(param_.prepacked_kernels[1]);
     wt_inter = const_cast<DataType_ *>(param_.prepacked_kernels[2]);
     wt_out = const_cast<DataType_ *>(param_.prepacked_kernels[3]);
   } else {
-    const void *src[4] = {param_.attr_kernel_QKV, param_.attr_output_kernel, param_.inter_kernel,
-                          param_.output_kernel};
     void *dst[4] = {wt_qkv, wt_proj, wt_inter, wt_out};
-    const int ks[4] = {hidden, hidden, hidden, inter};
-    const int ns[4] = {3 * hidden, hidden, inter, hidden};
-    check_bt_error(bt_transpose_weights(4, src, dst, ks, ns, stream));
+    check_bt_error(bt_transpose_weights(4, w_src, dst, w_k, w_n, stream));
   }
 
   check_bt_error(bt_gemm_qkv_bias_split(from_tensor, gather, wt_qkv,
@@ -157,7 +181,8 @@ void BertTransformer<OpType>::bert_infer(BertTransformerInferParam infer_param) 
   };
   attention_infer_param.attention_bias = infer_param.attention_bias;
   attention_infer_param.seq_order = seq_order;
-  attention_infer_param.mask_prefix = infer_param.offsets ? infer_param.mask_prefix : -1;
+  attention_infer_param.mask_prefix = have_offsets ? infer_param.mask_prefix : -1;
+  attention_infer_param.mask_prefix_slots = mask_slots;
   // the three weight matrices the rest of the layer reads, when they lie back to back:
   // the attention kernel pulls them into the memory-side cache while it runs
   if (wt_inter == wt_proj + (size_t)hidden * hidden && wt_out == wt_inter + (size_t)hidden * inter) {

@@ -110,6 +110,42 @@ __device__ __forceinline__ int wave_inclusive_scan(int v, int lane) {
 }
 
 
+// ---- 64 x 64 tile of the weight pre-pack: wt[n][k] = w[k][n] ---------------------------
+// 256 threads (t = 0..255) move one tile through `tile`; both sides are 16-byte accesses.
+// `live` = false keeps a thread group in step (it meets the barrier) without touching memory.
+constexpr int kTransposePitch = 64 + 2;
+__device__ __forceinline__ void transpose_tile_64(const half_t *__restrict__ w,
+                                                  half_t *__restrict__ wt, int K, int N, int k0,
+                                                  int n0, half_t (*tile)[kTransposePitch], int t,
+                                                  bool live) {
+  // read 64 k-rows x 128 B: thread -> (row = t/8 + 32*i, 16-byte chunk t%8)
+  const int r = t >> 3, c = (t & 7) * 8;
+  if (live) {
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const int k = k0 + r + 32 * i, n = n0 + c;
+      uint4_t v = {0u, 0u, 0u, 0u};
+      if (k < K && n < N) v = *(const uint4_t *)(w + (size_t)k * N + n);
+      const half_t *h = (const half_t *)&v;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) tile[r + 32 * i][c + e] = h[e];
+    }
+  }
+  __syncthreads();
+  if (live) {
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const int n = n0 + r + 32 * i, k = k0 + c;
+      if (n < N && k < K) {
+        half8_t o;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) o[e] = tile[c + e][r + 32 * i];
+        *(half8_t *)(wt + (size_t)n * K + k) = o;
+      }
+    }
+  }
+}
+
 // ---- balanced work list of the streaming attention kernels -------------------------
 // Within an XCD the hardware deals consecutive workgroups to its 32 CUs round-robin
 // (slot s of the XCD lands on CU s % 32), and a launch of a few workgroups per CU is

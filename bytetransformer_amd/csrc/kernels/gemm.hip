@@ -367,36 +367,15 @@ struct TransposeArgs {
 };
 
 __global__ __launch_bounds__(256) void transpose_kernel(TransposeArgs a) {
-  __shared__ half_t tile[64][64 + 2];
+  __shared__ half_t tile[64][kTransposePitch];
   int j = 0;
 #pragma unroll
   for (int i = 1; i < 4; ++i)
     if (i < a.njobs && (int)blockIdx.x >= a.job[i].tile_begin) j = i;
   const TransposeJob jb = a.job[j];
   const int t = blockIdx.x - jb.tile_begin;
-  const int k0 = (t / jb.tiles_n) * 64, n0 = (t % jb.tiles_n) * 64;
-  // read 64 k-rows x 128 B: thread -> (row = tid/8 + 32*i, 16-byte chunk tid%8)
-  const int r = threadIdx.x >> 3, c = (threadIdx.x & 7) * 8;
-#pragma unroll
-  for (int i = 0; i < 2; ++i) {
-    const int k = k0 + r + 32 * i, n = n0 + c;
-    uint4_t v = {0u, 0u, 0u, 0u};
-    if (k < jb.K && n < jb.N) v = *(const uint4_t *)(jb.w + (size_t)k * jb.N + n);
-    const half_t *h = (const half_t *)&v;
-#pragma unroll
-    for (int e = 0; e < 8; ++e) tile[r + 32 * i][c + e] = h[e];
-  }
-  __syncthreads();
-#pragma unroll
-  for (int i = 0; i < 2; ++i) {
-    const int n = n0 + r + 32 * i, k = k0 + c;
-    if (n < jb.N && k < jb.K) {
-      half8_t o;
-#pragma unroll
-      for (int e = 0; e < 8; ++e) o[e] = tile[c + e][r + 32 * i];
-      *(half8_t *)(jb.wt + (size_t)n * jb.K + k) = o;
-    }
-  }
+  transpose_tile_64(jb.w, jb.wt, jb.K, jb.N, (t / jb.tiles_n) * 64, (t % jb.tiles_n) * 64, tile,
+                    threadIdx.x, true);
 }
 
 template <int BM, int BN, int STAGES, int WM, int WN, int NP, int SCHED, int EPI>

@@ -134,6 +134,240 @@ __global__ __launch_bounds__(kPrefixWaves *kWave) void mask_prefix_kernel(
   if (threadIdx.x == 0) ok[blockIdx.x] = !any_bad;
 }
 
+// ---- layer prologue ------------------------------------------------------------
+// Everything a layer has to know before its first product, in ONE launch: the offsets
+// (blocks below `offset_blocks`, the code of build_offsets_kernel), the prefix-mask
+// verdict slots (every block, one wave per mask row; a wave counts the length of its row's
+// sequence itself, so no block waits for another) and the fingerprint of the weight
+// matrices behind a cached pre-pack (every block hashes its share of 16-byte vectors).
+constexpr int kPrologueThreads = 1024;
+constexpr int kPrologueWaves = kPrologueThreads / kWave;
+constexpr int kHealGroups = kPrologueThreads / 256;
+
+// The fingerprint job belongs to a fixed set of blocks (kHashFirst .. kHashFirst +
+// kHashBlocks - 1, whatever the batch size), each owning a fixed range of the 64 x 64 tiles
+// of the weight set: a block hashes its tiles, compares with ITS record and, when they
+// differ, packs ITS tiles again - no block waits for or talks to another.
+constexpr int kHashFirst = 64;     // blocks below build offsets (at most 64 of them)
+constexpr int kHashBlocks = 192;
+constexpr int kHashUnroll = 4;     // tiles in flight per group of 256 lanes (two 16-byte loads per lane each)
+
+struct PrologueWeights {
+  const half_t *w[4];        // [K, N] as the caller stores them
+  half_t *wt[4];             // [N, K] cached copies
+  int K[4], N[4];
+  int tiles_n[4];            // 64 x 64 tiles along n
+  int tile_end[4];           // tiles up to and including matrix i
+  int count;                 // 0 = no weights to check
+  // per hash block b: state[2b] = fingerprint its tiles' copies were made from,
+  // state[2b + 1] = non-zero once that is recorded (zero: this launch records it)
+  unsigned long long *state;
+};
+
+__device__ __forceinline__ unsigned int rotl32(unsigned int v, int s) {
+  return __builtin_amdgcn_alignbit(v, v, 32 - s);
+}
+// 64 bits per 16-byte piece, a function of its four dwords and its position; a fingerprint
+// is the sum of these (commutative: no order between lanes or waves to keep).  With the
+// other three dwords fixed each dword acts on the result through bijections (add, rotate,
+// xor-shift, multiplication by an odd constant), so a change of ONE dword always shows;
+// the two multiplications mix whatever else changes.  About 27 VALU operations per piece:
+// the launch reads a layer's weights at memory speed.
+__device__ __forceinline__ unsigned long long piece_hash(const uint4_t v, unsigned int pos) {
+  unsigned int a = v.x + rotl32(v.z, 15) + pos;
+  unsigned int b = (v.y + rotl32(v.w, 9)) ^ rotl32(pos, 16);
+  a ^= a >> 15;
+  a *= 0x2C1B3C6Du;
+  a ^= a >> 12;
+  b += a;
+  b ^= b >> 16;
+  b *= 0x297A2D39u;
+  b ^= b >> 15;
+  a ^= b;
+  return ((unsigned long long)b << 32) | a;
+}
+__device__ __forceinline__ unsigned long long wave_sum_u64(unsigned long long v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    const unsigned int lo = __shfl_xor((unsigned int)v, o, 64);
+    const unsigned int hi = __shfl_xor((unsigned int)(v >> 32), o, 64);
+    v += ((unsigned long long)hi << 32) | lo;
+  }
+  return v;
+}
+// popcount of row elements >= 0.5 by one wave (the length rule of the offsets)
+template <typename T>
+__device__ __forceinline__ int wave_row_length(const T *__restrict__ row, int S, int lane) {
+  int count = 0;
+  for (int i0 = 0; i0 < S; i0 += kWave) {
+    const int i = i0 + lane;
+    const bool on = (i < S) && ((float)row[i] >= 0.5f);
+    count += __popcll(__ballot(on));
+  }
+  return count;
+}
+
+template <typename T>
+__global__ __launch_bounds__(kPrologueThreads) void layer_prologue_kernel(
+    const T *__restrict__ mask, int *__restrict__ batch_idx, int *__restrict__ word_idx,
+    int *__restrict__ seq_order, int *__restrict__ slots, int B, int S, int offset_blocks,
+    PrologueWeights pw) {
+  extern __shared__ __attribute__((aligned(16))) int smem[];
+  __shared__ unsigned long long s_part[kPrologueWaves];
+  __shared__ int s_heal;
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+
+  // ---- offsets ----
+  if ((int)blockIdx.x < offset_blocks) {
+    int *s_len = smem;          // [B]
+    int *s_off = smem + B;      // [B + 1]
+    for (int b = wave; b < B; b += kPrologueWaves) {
+      const int count = wave_row_length(mask + (size_t)b * S * S, S, lane);
+      if (lane == 0) s_len[b] = count;
+    }
+    __syncthreads();
+    if (wave == 0) {
+      int carry = 0;
+      for (int i0 = 0; i0 < B; i0 += kWave) {
+        const int i = i0 + lane;
+        const int len = i < B ? s_len[i] : 0;
+        const int incl = wave_inclusive_scan(len, lane);
+        if (i < B) s_off[i] = carry + incl - len;
+        carry += __shfl(incl, 63, 64);
+      }
+      if (lane == 0) s_off[B] = carry;
+    }
+    __syncthreads();
+    if (blockIdx.x == 0) {
+      for (int i = tid; i <= B; i += kPrologueThreads) batch_idx[i] = s_off[i];
+      if (seq_order)
+        for (int b = tid; b < B; b += kPrologueThreads) {
+          const int len = s_len[b];
+          int rank = 0;
+          for (int o = 0; o < B; ++o) {
+            const int lo = s_len[o];
+            rank += (lo > len) || (lo == len && o < b);
+          }
+          seq_order[rank] = b;
+        }
+    }
+    for (int b = blockIdx.x; b < B; b += offset_blocks) {
+      const int off = s_off[b], len = s_len[b];
+      for (int i = tid; i < len; i += kPrologueThreads) word_idx[off + i] = b * S + i;
+    }
+  }
+
+  // ---- is the mask the plain prefix mask of its lengths? (mask_prefix_kernel's rule) ----
+  if (slots) {
+    const long long rows = (long long)B * S;
+    constexpr int kVec = 16 / (int)sizeof(T);       // elements per 16-byte load
+    const bool vec = S % kVec == 0 && (reinterpret_cast<uintptr_t>(mask) & 15) == 0;
+    int bad = 0, len_of = -1, len = 0;
+    for (long long r = (long long)blockIdx.x * kPrologueWaves + wave; r < rows;
+         r += (long long)gridDim.x * kPrologueWaves) {
+      const int b = (int)(r / S);
+      if (b != len_of) {
+        len = wave_row_length(mask + (size_t)b * S * S, S, lane);
+        len_of = b;
+      }
+      bad |= len == 0;
+      const T *row = mask + (size_t)r * S;
+      if (vec) {
+        for (int j0 = lane * kVec; j0 < S; j0 += kWave * kVec) {
+          const uint4_t raw = *(const uint4_t *)(row + j0);
+          const T *e = (const T *)&raw;
+#pragma unroll
+          for (int i = 0; i < kVec; ++i) bad |= (float)e[i] != (j0 + i < len ? 1.0f : 0.0f);
+        }
+      } else {
+        for (int j = lane; j < S; j += kWave) bad |= (float)row[j] != (j < len ? 1.0f : 0.0f);
+      }
+    }
+    const int any_bad = __syncthreads_or(bad);
+    if (tid == 0) slots[blockIdx.x] = !any_bad;
+  }
+
+  // ---- do the cached weight copies still belong to these weights? ----
+  if (pw.count > 0 && (int)blockIdx.x >= kHashFirst) {
+    const int hb = blockIdx.x - kHashFirst;
+    const int tiles_all = pw.tile_end[pw.count - 1];
+    const int tile_lo = (int)((long long)tiles_all * hb / kHashBlocks);
+    const int tile_hi = (int)((long long)tiles_all * (hb + 1) / kHashBlocks);
+    // A group of 256 lanes takes one tile at a time: which matrix and where in it is the
+    // same for the whole wave (scalar arithmetic), a lane adds one multiply-add for its
+    // row and two 16-byte loads; kHashUnroll tiles per group are in flight at once.
+    const int group = __builtin_amdgcn_readfirstlane(tid >> 8);
+    const int gt = tid & 255, r0 = gt >> 3, c8 = (gt & 7) * 8;
+    unsigned long long sum = 0;
+#pragma unroll 1
+    for (int tb = tile_lo; tb < tile_hi; tb += kHealGroups * kHashUnroll) {
+      uint4_t v[kHashUnroll][2];
+#pragma unroll
+      for (int i = 0; i < kHashUnroll; ++i) {
+        const int t = tb + i * kHealGroups + group;
+        int j = 0, first = 0;
+#pragma unroll
+        for (int q = 1; q < 4; ++q)
+          if (q < pw.count && t >= pw.tile_end[q - 1]) {
+            j = q;
+            first = pw.tile_end[q - 1];
+          }
+        const int tl = t - first;
+        const int k0 = (tl / pw.tiles_n[j]) * 64, n = (tl % pw.tiles_n[j]) * 64 + c8;
+        const int K = pw.K[j], N = pw.N[j];
+        const half_t *src = pw.w[j];
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+          const int k = k0 + r0 + 32 * h;
+          v[i][h] = uint4_t{0u, 0u, 0u, 0u};
+          if (t < tile_hi && k < K && n < N) v[i][h] = *(const uint4_t *)(src + (size_t)k * N + n);
+        }
+      }
+#pragma unroll
+      for (int i = 0; i < kHashUnroll; ++i) {
+        const int t = tb + i * kHealGroups + group;
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+          if (t < tile_hi)
+            sum += piece_hash(v[i][h], (unsigned int)(((t - tile_lo) << 9) + h * 256 + gt));
+      }
+    }
+    sum = wave_sum_u64(sum);
+    if (lane == 0) s_part[wave] = sum;
+    __syncthreads();
+    if (tid == 0) {
+      unsigned long long now = 0;
+      for (int i = 0; i < kPrologueWaves; ++i) now += s_part[i];
+      s_heal = pw.state[2 * hb + 1] != 0 && now != pw.state[2 * hb];
+      pw.state[2 * hb] = now;
+      pw.state[2 * hb + 1] = 1;
+    }
+    __syncthreads();
+    if (s_heal) {
+      // a write that no host-side bookkeeping saw: this block's tiles are packed again
+      half_t(*tile)[kTransposePitch] =
+          (half_t(*)[kTransposePitch])((half_t *)smem + (size_t)(tid >> 8) * 64 * kTransposePitch);
+#pragma unroll 1
+      for (int t0 = tile_lo; t0 < tile_hi; t0 += kHealGroups) {
+        const int t = t0 + (tid >> 8);
+        int j = 0, first = 0;
+#pragma unroll
+        for (int q = 1; q < 4; ++q)
+          if (q < pw.count && t >= pw.tile_end[q - 1]) {
+            j = q;
+            first = pw.tile_end[q - 1];
+          }
+        const int tl = t - first;
+        transpose_tile_64(pw.w[j], pw.wt[j], pw.K[j], pw.N[j], (tl / pw.tiles_n[j]) * 64,
+                          (tl % pw.tiles_n[j]) * 64, tile, tid & 255, t < tile_hi);
+        __syncthreads();
+      }
+    }
+  }
+}
+
 // ---- compress ---------------------------------------------------------------
 // One wave per packed row, 16-byte lanes.  M is read from batch_idx[B]; rows
 // past it retire immediately, so the grid is sized for B*S without a host sync.
@@ -243,6 +477,76 @@ extern "C" int bt_build_offsets(const void *atten_mask, int mask_dtype, int batc
     e = hipStreamSynchronize(s);
     if (e != hipSuccess) return hip_fail(e, "stream synchronize for valid_word_num");
   }
+  return BT_OK;
+}
+
+extern "C" int bt_layer_prologue(const void *atten_mask, int mask_dtype, int batch_size,
+                                 int seq_len, int *batch_idx, int *word_idx, int *seq_order,
+                                 int *mask_prefix_slots, int weight_count, const void *const *w,
+                                 void *const *wt, const int *k, const int *n,
+                                 unsigned long long *prepack_state, void *stream) {
+  BT_REQUIRE(atten_mask && batch_idx && word_idx, BT_ERR_INVALID_ARGUMENT,
+             "bt_layer_prologue: null pointer argument");
+  BT_REQUIRE(batch_size > 0 && seq_len > 0, BT_ERR_INVALID_ARGUMENT,
+             "bt_layer_prologue: batch_size=%d seq_len=%d must be positive", batch_size, seq_len);
+  BT_REQUIRE(mask_dtype == BT_F16 || mask_dtype == BT_F32, BT_ERR_INVALID_ARGUMENT,
+             "bt_layer_prologue: unknown mask dtype %d", mask_dtype);
+  BT_REQUIRE((long long)batch_size * seq_len < (1ll << 31), BT_ERR_UNSUPPORTED,
+             "bt_layer_prologue: batch_size*seq_len overflows int32");
+  BT_REQUIRE(weight_count >= 0 && weight_count <= 4, BT_ERR_INVALID_ARGUMENT,
+             "bt_layer_prologue: weight_count=%d outside [0, 4]", weight_count);
+  PrologueWeights pw;
+  memset(&pw, 0, sizeof(pw));
+  pw.count = weight_count;
+  if (weight_count > 0) {
+    BT_REQUIRE(w && wt && k && n && prepack_state, BT_ERR_INVALID_ARGUMENT,
+               "bt_layer_prologue: weights to check need w, wt, k, n and prepack_state");
+    BT_REQUIRE((reinterpret_cast<uintptr_t>(prepack_state) & 7) == 0, BT_ERR_INVALID_ARGUMENT,
+               "bt_layer_prologue: prepack_state must be 8-byte aligned");
+    long long tiles = 0;
+    for (int i = 0; i < weight_count; ++i) {
+      BT_REQUIRE(w[i] && wt[i], BT_ERR_INVALID_ARGUMENT,
+                 "bt_layer_prologue: null matrix pointer #%d", i);
+      BT_REQUIRE(aligned16({w[i], wt[i]}), BT_ERR_INVALID_ARGUMENT,
+                 "bt_layer_prologue: matrix pointers must be 16-byte aligned");
+      BT_REQUIRE(k[i] > 0 && n[i] > 0 && k[i] % 8 == 0 && n[i] % 8 == 0, BT_ERR_UNSUPPORTED,
+                 "bt_layer_prologue: k=%d n=%d must be positive multiples of 8", k[i], n[i]);
+      tiles += (long long)((k[i] + 63) / 64) * ((n[i] + 63) / 64);
+      BT_REQUIRE(tiles < (1ll << 21), BT_ERR_UNSUPPORTED,
+                 "bt_layer_prologue: weight matrices beyond 2^21 tiles of 64 x 64");
+      pw.w[i] = (const half_t *)w[i];
+      pw.wt[i] = (half_t *)wt[i];
+      pw.K[i] = k[i];
+      pw.N[i] = n[i];
+      pw.tiles_n[i] = (n[i] + 63) / 64;
+      pw.tile_end[i] = (int)tiles;
+    }
+    for (int i = weight_count; i < 4; ++i) {
+      pw.tiles_n[i] = 1;
+      pw.tile_end[i] = (int)tiles;
+    }
+    pw.state = prepack_state;
+  }
+  size_t smem = (2 * (size_t)batch_size + 1) * sizeof(int);
+  const size_t heal = (size_t)kHealGroups * 64 * kTransposePitch * sizeof(half_t);
+  if (weight_count > 0 && smem < heal) smem = heal;
+  BT_REQUIRE(smem <= 60 * 1024, BT_ERR_UNSUPPORTED,
+             "bt_layer_prologue: batch_size %d too large (limit 7679)", batch_size);
+  hipStream_t s = as_stream(stream);
+  const int offset_blocks = batch_size < 64 ? batch_size : 64;
+  // the verdict slots are an array of kPrefixBlocks entries, one per block; the
+  // fingerprint blocks are the last kHashBlocks of the same grid
+  static_assert(kHashFirst + kHashBlocks == kPrefixBlocks, "one grid for both jobs");
+  const int grid = (mask_prefix_slots || weight_count > 0) ? kPrefixBlocks : offset_blocks;
+  if (mask_dtype == BT_F16)
+    layer_prologue_kernel<half_t><<<grid, kPrologueThreads, smem, s>>>(
+        (const half_t *)atten_mask, batch_idx, word_idx, seq_order, mask_prefix_slots, batch_size,
+        seq_len, offset_blocks, pw);
+  else
+    layer_prologue_kernel<float><<<grid, kPrologueThreads, smem, s>>>(
+        (const float *)atten_mask, batch_idx, word_idx, seq_order, mask_prefix_slots, batch_size,
+        seq_len, offset_blocks, pw);
+  BT_CHECK_LAUNCH("layer_prologue_kernel");
   return BT_OK;
 }
 

@@ -77,10 +77,19 @@ class BTEncoder : public IBTEncoder {
     c10::DeviceGuard device_guard(input.device());
 
     hipStream_t stream = c10::hip::getCurrentHIPStream(input.device().index()).stream();
+    // While the stream is being captured into a graph the caches stay out of it: the graph
+    // would hold pointers into entries that may be dropped before a replay, a copy made
+    // now would only be recorded, not executed, and the host may not wait for a count.
+    // The layer then packs into its own scratch and builds its offsets inside the graph.
+    hipStreamCaptureStatus capture_status = hipStreamCaptureStatusNone;
+    const bool capturing = hipStreamIsCapturing(stream, &capture_status) != hipSuccess ||
+                           capture_status != hipStreamCaptureStatusNone;
     BertTransformerParam<kOp> param = param_;
-    std::vector<Tensor> packed = prepacked_weights(stream);   // keeps the copies alive
-    if (packed.size() == 4)
-      for (int i = 0; i < 4; ++i) param.prepacked_kernels[i] = get_ptr<T>(packed[i]);
+    PrepackCache::Packed packed;   // keeps the copies alive through the call
+    if (!capturing && prepacked_weights(stream, &packed)) {
+      for (int i = 0; i < 4; ++i) param.prepacked_kernels[i] = get_ptr<T>(packed.packed[i]);
+      param.prepack_state = reinterpret_cast<unsigned long long *>(packed.state.data_ptr());
+    }
 
     BertTransformer<kOp> encoder(batch_size, head_num_, head_size_, seq_len, use_fused_attention,
                                  is_remove_padding, use_fp32_, model_type);
@@ -93,100 +102,67 @@ class BTEncoder : public IBTEncoder {
           batch_size, seq_len, nullptr, stream
     };
     infer_param.attention_bias = attention_bias.defined() ? get_ptr<T>(attention_bias) : NULL;
-    // offsets of this mask: cached per mask tensor (never while the stream is being
-    // captured into a graph, where the host may not wait for the token count)
-    MaskPlanCache::Plan plan;
-    ET_Param offsets{nullptr, nullptr, 0};
-    // (batches of one and two run on the padded rows whatever the flag says; the float
-    // attention applies the mask tensor on both row layouts)
-    const bool mask_tensor_in_use =
-        !is_remove_padding || batch_size <= 2 || kOp == OperationType::FP32;
-    if (mask_plan(attr_mask, batch_size, seq_len, stream, mask_tensor_in_use, &plan)) {
-      offsets.batch_idx = plan.batch_idx.data_ptr<int>();
-      offsets.word_idx = plan.word_idx.data_ptr<int>();
-      offsets.valid_word_num = plan.valid_word_num;
-      infer_param.offsets = &offsets;
-      infer_param.seq_order = plan.seq_order.data_ptr<int>();
-      infer_param.mask_prefix = plan.prefix_state;
-    }
+    // The layer rebuilds the offsets from the mask on the device in every call; what the
+    // host keeps per mask tensor is the valid-token count as a hint for tile shapes (the
+    // packed rows only: on the padded rows every row is live).
+    if (!capturing && encoder.is_remove_padding())
+      infer_param.valid_rows_hint = valid_rows_hint(attr_mask, batch_size, seq_len, stream);
     encoder.infer(infer_param);
   }
 
  private:
-  // The four [N, K] weight copies, from the process-wide cache when the same
-  // tensors were seen before, else packed now (one launch) and remembered.
-  // Empty for float, whose kernels read the weights as stored.
-  std::vector<Tensor> prepacked_weights(hipStream_t stream) {
-    std::vector<Tensor> out;
-    if (kOp != OperationType::HALF) return out;
+  // The four [N, K] weight copies and their fingerprint record, from the process-wide
+  // cache when the same tensors were seen before, else packed now (one launch) and
+  // remembered.  False for float, whose kernels read the weights as stored.
+  bool prepacked_weights(hipStream_t stream, PrepackCache::Packed *out) {
+    if (kOp != OperationType::HALF) return false;
     auto &cache = PrepackCache::instance();
-    if (!cache.enabled()) return out;
-    static const int kIdx[4] = {0, 2, 6, 8};
-    for (int i = 0; i < 4; ++i)
-      if (weights_[kIdx[i]].dim() != 2) return out;
-    out.resize(4);
-    bool all_hit = true;
-    for (int i = 0; i < 4; ++i) all_hit = cache.lookup(weights_[kIdx[i]], stream, &out[i]) && all_hit;
-    if (all_hit) return out;
+    if (!cache.enabled()) return false;
+    const Tensor *const w[4] = {&weights_[0], &weights_[2], &weights_[6], &weights_[8]};
+    for (const Tensor *t : w)
+      if (t->dim() != 2) return false;
+    if (cache.lookup(w, stream, out)) return true;
     const void *src[4];
     void *dst[4];
     int ks[4], ns[4];
     // one allocation for the four copies: the layer hands the last three to the
     // attention kernel as one range to warm the cache with
     int64_t total = 0;
-    for (int i = 0; i < 4; ++i) total += weights_[kIdx[i]].numel();
-    Tensor block = torch::empty({total}, weights_[kIdx[0]].options());
+    for (const Tensor *t : w) total += t->numel();
+    out->block = torch::empty({total}, w[0]->options());
     int64_t at = 0;
     for (int i = 0; i < 4; ++i) {
-      const Tensor &w = weights_[kIdx[i]];
-      out[i] = block.narrow(0, at, w.numel()).view({w.size(1), w.size(0)});
-      at += w.numel();
-      src[i] = w.data_ptr();
-      dst[i] = out[i].data_ptr();
-      ks[i] = (int)w.size(0);
-      ns[i] = (int)w.size(1);
+      out->packed[i] = out->block.narrow(0, at, w[i]->numel()).view({w[i]->size(1), w[i]->size(0)});
+      at += w[i]->numel();
+      src[i] = w[i]->data_ptr();
+      dst[i] = out->packed[i].data_ptr();
+      ks[i] = (int)w[i]->size(0);
+      ns[i] = (int)w[i]->size(1);
     }
     check_bt_error(bt_transpose_weights(4, src, dst, ks, ns, stream));
-    for (int i = 0; i < 4; ++i) cache.store(weights_[kIdx[i]], stream, out[i]);
-    return out;
+    // all zero: the prologue of this very call records the fingerprint of what was packed
+    out->state = torch::zeros({BT_PREPACK_STATE_WORDS},
+                              torch::dtype(torch::kInt64).device(w[0]->device()));
+    cache.store(w, stream, *out);
+    return true;
   }
 
-  // want_prefix: the attention of this layer would read the mask tensor, so it pays to know
-  // whether that is the plain prefix mask of its lengths (one pass over it, once per mask).
-  bool mask_plan(const Tensor &mask, int batch_size, int seq_len, hipStream_t stream,
-                 bool want_prefix, MaskPlanCache::Plan *plan) {
-    if (!PrepackCache::instance().enabled() || mask.is_inference()) return false;
-    hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
-    if (hipStreamIsCapturing(stream, &capturing) != hipSuccess ||
-        capturing != hipStreamCaptureStatusNone)
-      return false;
-    auto &cache = MaskPlanCache::instance();
+  // The number of valid tokens of this mask, read back once per mask tensor (the one host
+  // synchronisation; the reference has one in every call, remove_padding.h:99-100).
+  // 0 = unknown.
+  int valid_rows_hint(const Tensor &mask, int batch_size, int seq_len, hipStream_t stream) {
+    if (!PrepackCache::instance().enabled() || mask.is_inference()) return 0;
+    auto &cache = MaskHintCache::instance();
+    int count = 0;
+    if (cache.lookup(mask, stream, &count)) return count;
     auto opts = torch::dtype(torch::kInt32).device(mask.device());
-    auto check_prefix = [&]() {
-      auto scratch = torch::empty({256}, opts);
-      int verdict = 0;
-      check_bt_error(bt_mask_is_prefix(mask.data_ptr(), Traits<kOp>::dtype, batch_size, seq_len,
-                                       plan->batch_idx.data_ptr<int>(), scratch.data_ptr<int>(),
-                                       &verdict, stream));
-      plan->prefix_state = verdict;
-    };
-    if (cache.lookup(mask, stream, plan)) {
-      if (want_prefix && plan->prefix_state < 0) {
-        check_prefix();
-        cache.store(mask, stream, *plan);
-      }
-      return true;
-    }
-    plan->batch_idx = torch::empty({(int64_t)batch_size + 1}, opts);
-    plan->word_idx = torch::empty({(int64_t)batch_size * seq_len}, opts);
-    plan->seq_order = torch::empty({(int64_t)batch_size}, opts);
+    auto batch_idx = torch::empty({(int64_t)batch_size + 1}, opts);
+    auto word_idx = torch::empty({(int64_t)batch_size * seq_len}, opts);
     check_bt_error(bt_build_offsets(mask.data_ptr(), Traits<kOp>::dtype, batch_size, seq_len,
-                                    plan->batch_idx.data_ptr<int>(), plan->word_idx.data_ptr<int>(),
-                                    plan->seq_order.data_ptr<int>(), &plan->valid_word_num,
-                                    stream));
-    if (want_prefix) check_prefix();
-    cache.store(mask, stream, *plan);
-    return true;
+                                    batch_idx.data_ptr<int>(), word_idx.data_ptr<int>(), nullptr,
+                                    &count, stream));
+    cache.store(mask, stream, count);
+    return count;
   }
 
   const int head_num_, head_size_;

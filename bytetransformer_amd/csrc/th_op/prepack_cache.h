@@ -1,19 +1,28 @@
-// Process-wide cache of pre-packed ([N, K], k-contiguous) copies of weight
-// tensors for the PyTorch operator.  The operator is called once per layer with
-// the same weight tensors on every forward, so the transposes are made once and
-// reused for as long as the very same tensor object still holds the very same
-// data: an entry is keyed on the TensorImpl address and is valid only while
-//   - that TensorImpl is still alive (weak reference lock succeeds),
-//   - its version counter is unchanged (any in-place write, also through a
-//     view, bumps it),
-//   - its data pointer, shape and device are unchanged, and
-//   - the calling stream is the one the copy was made on.
-// Anything else re-packs.  Inference tensors carry no version counter and are
-// never cached.  BT_PREPACK_CACHE=0 in the environment disables the cache.
+// Process-wide caches of the PyTorch operator.  The operator is called once per layer
+// with the same weight tensors on every forward and with one mask per forward, so two
+// things are worth keeping between calls - and neither may ever change a result:
+//
+//   PrepackCache   the pre-packed ([N, K], k-contiguous) copies of a layer's four weight
+//                  matrices.  An entry is found through the tensors' identity (TensorImpl
+//                  alive, version counter, data pointer, shape, device, stream unchanged);
+//                  that bookkeeping cannot see a write that goes around the version counter
+//                  (`w.data.copy_()`, DLPack, a raw-pointer kernel), so every reuse is also
+//                  CHECKED ON THE DEVICE: the layer's prologue launch fingerprints the four
+//                  weight tensors and re-packs inside that launch when the fingerprint is
+//                  not the one the copies were made from (bt_layer_prologue).  A hit is
+//                  therefore only ever a saving of time.
+//   MaskHintCache  the number of valid tokens of a mask tensor, read back once per mask
+//                  (one host synchronisation).  It is a HINT: it picks tile shapes, never a
+//                  launch size; the offsets themselves are rebuilt from the mask on the
+//                  device in every call.  A stale count costs time and nothing else.
+//
+// Inference tensors carry no version counter and are never cached.  BT_PREPACK_CACHE=0 in
+// the environment, or set_enabled(false), turns both off; clear() drops every entry.
 #pragma once
 #include <c10/util/intrusive_ptr.h>
 #include <torch/all.h>
 
+#include <atomic>
 #include <cstdlib>
 #include <mutex>
 #include <unordered_map>
@@ -24,48 +33,88 @@
 namespace bytetransformer {
 namespace torch_ext {
 
+// Identity of one tensor as the host can see it.
+struct TensorStamp {
+  c10::weak_intrusive_ptr<c10::TensorImpl> owner{c10::intrusive_ptr<c10::TensorImpl>()};
+  const c10::TensorImpl *impl = nullptr;
+  int64_t version = 0;
+  void *data = nullptr;
+  std::vector<int64_t> sizes;
+  c10::Device device{c10::kCPU};
+
+  static TensorStamp of(const torch::Tensor &t) {
+    TensorStamp s;
+    s.owner = c10::weak_intrusive_ptr<c10::TensorImpl>(t.getIntrusivePtr());
+    s.impl = t.unsafeGetTensorImpl();
+    s.version = t._version();
+    s.data = t.data_ptr();
+    s.sizes = t.sizes().vec();
+    s.device = t.device();
+    return s;
+  }
+  bool expired() const { return owner.expired(); }
+  bool matches(const torch::Tensor &t) const {
+    auto alive = owner.lock();
+    return alive && alive.get() == t.unsafeGetTensorImpl() && version == t._version() &&
+           data == t.data_ptr() && sizes == t.sizes().vec() && device == t.device();
+  }
+};
+
+inline std::atomic<bool> &caches_enabled() {
+  static std::atomic<bool> on{[] {
+    const char *e = std::getenv("BT_PREPACK_CACHE");
+    return !(e && e[0] == '0');
+  }()};
+  return on;
+}
+
 class PrepackCache {
  public:
+  struct Packed {
+    torch::Tensor block;       // the four copies back to back (QKV, projection, FFN1, FFN2)
+    torch::Tensor packed[4];   // views into block, [N, K] each
+    torch::Tensor state;       // int64[BT_PREPACK_STATE_WORDS]: fingerprint record of bt_layer_prologue
+  };
+
   static PrepackCache &instance() {
     static PrepackCache c;
     return c;
   }
 
-  bool enabled() const { return enabled_; }
+  bool enabled() const { return caches_enabled().load(std::memory_order_relaxed); }
 
-  // Returns the [N, K] copy of the 2-D weight `w` ([K, N]); `hit` reports whether
-  // the copy came from the cache.  A miss leaves `packed` undefined.
-  bool lookup(const torch::Tensor &w, void *stream, torch::Tensor *packed) {
-    if (!enabled_ || w.is_inference()) return false;
+  // The copies made from exactly these four tensor objects on this stream, if any.
+  bool lookup(const torch::Tensor *const (&w)[4], void *stream, Packed *out) {
+    if (!enabled()) return false;
+    for (const torch::Tensor *t : w)
+      if (t->is_inference()) return false;
     std::lock_guard<std::mutex> g(mu_);
-    auto it = map_.find(w.unsafeGetTensorImpl());
+    auto it = map_.find(w[0]->unsafeGetTensorImpl());
     if (it == map_.end()) return false;
     Entry &e = it->second;
-    auto alive = e.owner.lock();
-    if (!alive || alive.get() != w.unsafeGetTensorImpl() || e.version != w._version() ||
-        e.data != w.data_ptr() || e.stream != stream || e.k != w.size(0) || e.n != w.size(1) ||
-        e.device != w.device()) {
+    bool ok = e.stream == stream;
+    for (int i = 0; ok && i < 4; ++i) ok = e.stamp[i].matches(*w[i]);
+    if (!ok) {
       map_.erase(it);
+      sweep();
       return false;
     }
-    *packed = e.packed;
+    *out = e.value;
     return true;
   }
 
-  void store(const torch::Tensor &w, void *stream, const torch::Tensor &packed) {
-    if (!enabled_ || w.is_inference()) return;
+  void store(const torch::Tensor *const (&w)[4], void *stream, const Packed &value) {
+    if (!enabled()) return;
+    for (const torch::Tensor *t : w)
+      if (t->is_inference()) return;
     std::lock_guard<std::mutex> g(mu_);
-    if (map_.size() >= kMaxEntries) sweep();
+    sweep();
+    if (map_.size() >= kMaxEntries) map_.clear();
     Entry e;
-    e.owner = c10::weak_intrusive_ptr<c10::TensorImpl>(w.getIntrusivePtr());
-    e.version = w._version();
-    e.data = w.data_ptr();
+    for (int i = 0; i < 4; ++i) e.stamp[i] = TensorStamp::of(*w[i]);
     e.stream = stream;
-    e.k = w.size(0);
-    e.n = w.size(1);
-    e.device = w.device();
-    e.packed = packed;
-    map_[w.unsafeGetTensorImpl()] = std::move(e);
+    e.value = value;
+    map_[w[0]->unsafeGetTensorImpl()] = std::move(e);
   }
 
   void clear() {
@@ -80,94 +129,67 @@ class PrepackCache {
 
  private:
   struct Entry {
-    c10::weak_intrusive_ptr<c10::TensorImpl> owner{c10::intrusive_ptr<c10::TensorImpl>()};
-    int64_t version = 0;
-    void *data = nullptr;
+    TensorStamp stamp[4];
     void *stream = nullptr;
-    int64_t k = 0, n = 0;
-    c10::Device device{c10::kCPU};
-    torch::Tensor packed;
+    Packed value;
   };
   static constexpr size_t kMaxEntries = 1024;
 
-  PrepackCache() {
-    const char *e = std::getenv("BT_PREPACK_CACHE");
-    enabled_ = !(e && e[0] == '0');
-  }
-
-  // drop entries whose weight tensor has died; if everything is alive, start over
+  // Entries whose weights have died hold a layer's worth of device memory each: they go
+  // at every miss and store (a scan of at most kMaxEntries weak pointers).
   void sweep() {
-    for (auto it = map_.begin(); it != map_.end();)
-      it = it->second.owner.expired() ? map_.erase(it) : std::next(it);
-    if (map_.size() >= kMaxEntries) map_.clear();
+    for (auto it = map_.begin(); it != map_.end();) {
+      bool dead = false;
+      for (const TensorStamp &s : it->second.stamp) dead = dead || s.expired();
+      it = dead ? map_.erase(it) : std::next(it);
+    }
   }
 
-  bool enabled_ = true;
   std::mutex mu_;
   std::unordered_map<const c10::TensorImpl *, Entry> map_;
 };
 
-// Offsets of an attention mask (batch_idx, word_idx, valid-token count), cached
-// per mask tensor under the same validity rules as the weight copies.  A model
-// calls the operator once per layer with one mask, so the prefix sum - and the
-// one host synchronisation that fetches the token count used to pick GEMM tile
-// shapes - happens once per mask instead of once per layer.
-class MaskPlanCache {
+class MaskHintCache {
  public:
-  struct Plan {
-    torch::Tensor batch_idx, word_idx, seq_order;
-    int valid_word_num = 0;
-    int prefix_state = -1;   // is the mask the plain prefix mask of these lengths? -1 = not checked
-  };
-
-  static MaskPlanCache &instance() {
-    static MaskPlanCache c;
+  static MaskHintCache &instance() {
+    static MaskHintCache c;
     return c;
   }
 
-  bool lookup(const torch::Tensor &mask, void *stream, Plan *plan) {
+  bool lookup(const torch::Tensor &mask, void *stream, int *valid_word_num) {
     std::lock_guard<std::mutex> g(mu_);
     auto it = map_.find(mask.unsafeGetTensorImpl());
     if (it == map_.end()) return false;
-    Entry &e = it->second;
-    auto alive = e.owner.lock();
-    if (!alive || alive.get() != mask.unsafeGetTensorImpl() || e.version != mask._version() ||
-        e.data != mask.data_ptr() || e.stream != stream || e.sizes != mask.sizes().vec() ||
-        e.device != mask.device()) {
+    if (it->second.stream != stream || !it->second.stamp.matches(mask)) {
       map_.erase(it);
       return false;
     }
-    *plan = e.plan;
+    *valid_word_num = it->second.valid_word_num;
     return true;
   }
 
-  void store(const torch::Tensor &mask, void *stream, const Plan &plan) {
+  void store(const torch::Tensor &mask, void *stream, int valid_word_num) {
     std::lock_guard<std::mutex> g(mu_);
-    if (map_.size() >= kMaxEntries) {
-      for (auto it = map_.begin(); it != map_.end();)
-        it = it->second.owner.expired() ? map_.erase(it) : std::next(it);
-      if (map_.size() >= kMaxEntries) map_.clear();
-    }
+    for (auto it = map_.begin(); it != map_.end();)
+      it = it->second.stamp.expired() ? map_.erase(it) : std::next(it);
+    if (map_.size() >= kMaxEntries) map_.clear();
     Entry e;
-    e.owner = c10::weak_intrusive_ptr<c10::TensorImpl>(mask.getIntrusivePtr());
-    e.version = mask._version();
-    e.data = mask.data_ptr();
+    e.stamp = TensorStamp::of(mask);
     e.stream = stream;
-    e.sizes = mask.sizes().vec();
-    e.device = mask.device();
-    e.plan = plan;
+    e.valid_word_num = valid_word_num;
     map_[mask.unsafeGetTensorImpl()] = std::move(e);
+  }
+
+  void clear() {
+    std::lock_guard<std::mutex> g(mu_);
+    map_.clear();
   }
 
  private:
   struct Entry {
-    c10::weak_intrusive_ptr<c10::TensorImpl> owner{c10::intrusive_ptr<c10::TensorImpl>()};
-    int64_t version = 0;
-    void *data = nullptr;
+    TensorStamp stamp;
     void *stream = nullptr;
-    std::vector<int64_t> sizes;
-    c10::Device device{c10::kCPU};
-    Plan plan;
+    int valid_word_num = 0;
   };
   static constexpr size_t kMaxEntries = 64;
   std::mutex mu_;

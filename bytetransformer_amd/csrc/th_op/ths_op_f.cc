@@ -49,9 +49,23 @@ Tensor bert_transformer_layer(int64_t head_num, int64_t head_size, Tensor qkv_ke
   return output;
 }
 
+// The operator's caches (pre-packed weight copies, valid-token counts of masks): dropped /
+// switched on and off.  They never change a result, so these are for memory and timing.
+void clear_caches() {
+  torch_ext::PrepackCache::instance().clear();
+  torch_ext::MaskHintCache::instance().clear();
+}
+
+void set_caches_enabled(bool enabled) {
+  torch_ext::caches_enabled().store(enabled);
+  if (!enabled) clear_caches();
+}
+
 }  // namespace
 
 TORCH_LIBRARY_FRAGMENT(ByteTransformer, m) {
+  m.def("clear_caches() -> ()", &clear_caches);
+  m.def("set_caches_enabled(bool enabled) -> ()", &set_caches_enabled);
   m.def(
       "BertTransformer(int head_num, int head_size, Tensor qkv_kernel, Tensor qkv_bias, "
       "Tensor attr_output_kernel, Tensor attr_output_bias, Tensor attr_output_layernorm_gamma, "

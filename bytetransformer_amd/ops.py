@@ -9,6 +9,7 @@ import torch
 from ._lib import kernel_lib
 
 BT_F32, BT_F16 = 0, 1
+PREPACK_STATE_WORDS = 384     # BT_PREPACK_STATE_WORDS of include/bt_hip.h
 
 
 class BtError(RuntimeError):
@@ -75,6 +76,36 @@ def mask_is_prefix(mask, batch_idx):
     _check(kernel_lib().bt_mask_is_prefix(_ptr(mask), _dtype_code(mask), B, S, _ptr(batch_idx),
                                           _ptr(scratch), ctypes.byref(verdict), _stream()))
     return bool(verdict.value)
+
+
+def layer_prologue(mask, want_slots=False, weights=None, packed=None, state=None, out=None):
+    """bt_layer_prologue: offsets of `mask`, optionally the prefix-mask verdict slots and the
+    check of pre-packed copies `packed` against `weights` (fingerprint record `state`,
+    int64[PREPACK_STATE_WORDS], zero when the copies were made).  Returns (batch_idx, word_idx, seq_order, slots or None); `out` = such a
+    tuple to write into."""
+    B, S = mask.shape[0], mask.shape[1]
+    dev = mask.device
+    if out is not None:
+        batch_idx, word_idx, seq_order, slots = out
+    else:
+        batch_idx = torch.empty(B + 1, dtype=torch.int32, device=dev)
+        word_idx = torch.empty(B * S, dtype=torch.int32, device=dev)
+        seq_order = torch.empty(B, dtype=torch.int32, device=dev)
+        slots = torch.full((256,), -1, dtype=torch.int32, device=dev) if want_slots else None
+    n = len(weights) if weights else 0
+    if n:
+        src = (ctypes.c_void_p * n)(*[_ptr(w).value for w in weights])
+        dst = (ctypes.c_void_p * n)(*[_ptr(w).value for w in packed])
+        ks = (ctypes.c_int * n)(*[w.shape[0] for w in weights])
+        ns = (ctypes.c_int * n)(*[w.shape[1] for w in weights])
+        if state.dtype != torch.int64 or state.numel() != PREPACK_STATE_WORDS:
+            raise BtError("state must be an int64[%d] tensor" % PREPACK_STATE_WORDS)
+    else:
+        src = dst = ks = ns = None
+    _check(kernel_lib().bt_layer_prologue(
+        _ptr(mask), _dtype_code(mask), B, S, _ptr(batch_idx), _ptr(word_idx), _ptr(seq_order),
+        _ptr(slots), n, src, dst, ks, ns, _ptr(state) if n else None, _stream()))
+    return batch_idx, word_idx, seq_order, slots
 
 
 def compress(x, batch_idx, word_idx, out=None):

@@ -106,6 +106,30 @@ int bt_mask_is_prefix(const void *atten_mask, int mask_dtype, int batch_size, in
                       const int *batch_idx, int *scratch, int *is_prefix_host, void *stream);
 
 /*
+ * Layer prologue: what one layer has to know before its first product, in ONE launch.
+ * No counterpart in the reference, which rebuilds the offsets on every call
+ * (bert_transformer.cu:62-66) and reads the weights as stored.
+ *   - the offsets of bt_build_offsets (batch_idx, word_idx, seq_order; same rules);
+ *   - mask_prefix_slots (nullable): the int[256] verdict of bt_mask_prefix_slots for the
+ *     lengths of this very mask;
+ *   - weight_count in [0, 4] matrices w[i] ([k[i], n[i]] as the caller stores them) whose
+ *     pre-packed copies wt[i] ([n[i], k[i]], bt_transpose_weights) are being reused from an
+ *     earlier call: 192 workgroups each fingerprint their fixed share of the w[i] (64 bits
+ *     over every dword and its position) and compare with their record in prepack_state;
+ *     a workgroup whose fingerprint moved - the weights were overwritten in a way the owner
+ *     of the copies did not see - packs its share again inside this launch, so later
+ *     launches of the stream never read copies of other weights.  prepack_state: device
+ *     unsigned long long[BT_PREPACK_STATE_WORDS], all zero when the copies are made (the
+ *     first prologue then records the fingerprints), owned by whoever owns the copies and
+ *     used by one stream at a time.
+ */
+#define BT_PREPACK_STATE_WORDS 384
+int bt_layer_prologue(const void *atten_mask, int mask_dtype, int batch_size, int seq_len,
+                      int *batch_idx, int *word_idx, int *seq_order, int *mask_prefix_slots,
+                      int weight_count, const void *const *w, void *const *wt, const int *k,
+                      const int *n, unsigned long long *prepack_state, void *stream);
+
+/*
  * Gather valid rows: to_tensor[t, :] = from_tensor[word_idx[t], :], t < M.
  * Replaces compressBertInput_kernelLauncher (remove_padding.h:104-121).
  * hidden_dim % 8 == 0.  M is read on the device from batch_idx[batch_size].

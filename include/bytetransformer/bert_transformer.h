@@ -45,6 +45,12 @@ class BertTransformerParam {
   // infer() uses them and skips its own pre-pack launch; the caller vouches that
   // they match the *_kernel tensors above.
   const DataType_ *prepacked_kernels[4] = {nullptr, nullptr, nullptr, nullptr};
+  // ... and, optionally, the fingerprint record of those copies (device unsigned long
+  // long[BT_PREPACK_STATE_WORDS], all zero when the copies were made; see bt_layer_prologue).  When set, every
+  // infer() checks on the device that the *_kernel tensors still hold what the copies were
+  // made from and makes the copies again if not, so a caller that reuses copies across calls
+  // need not vouch for anything.  One stream at a time.
+  unsigned long long *prepack_state = nullptr;
 };
 
 template <typename T>
@@ -74,6 +80,10 @@ struct BertTransformerInferParam {
   // length instead of reading the tensor, the same result, the masked terms being exactly
   // zero; 0 = it is not; -1 = not checked (the layer then checks on the device).
   int mask_prefix = -1;
+  // Extension: the number of valid tokens the caller expects (0 = unknown) when it passes
+  // no offsets.  A hint: it picks tile shapes and the split-k FFN2, never a launch size, so
+  // a wrong value costs time and nothing else.
+  int valid_rows_hint = 0;
 };
 
 template <OperationType OpType>

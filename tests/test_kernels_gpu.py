@@ -46,6 +46,95 @@ def test_build_offsets_bit_exact(device, B, S, dtype):
     assert np.array_equal(g_wi.cpu().numpy()[:M], wi)
 
 
+@pytest.mark.parametrize("B,S,dtype", [(1, 256, np.float16), (16, 512, np.float16),
+                                       (3, 7, np.float32), (70, 33, np.float16),
+                                       (130, 100, np.float16), (2, 1024, np.float16)])
+@pytest.mark.parametrize("kind", ["prefix", "ragged-rows", "empty-sequence"])
+def test_layer_prologue_offsets_and_prefix_verdict(device, B, S, dtype, kind):
+    """bt_layer_prologue = bt_build_offsets + bt_mask_prefix_slots in one launch: offsets
+    bit-exact with the oracle, the verdict equal to the stand-alone check's."""
+    _say("prologue", B, S, dtype, kind)
+    rs = np.random.RandomState(B * 1000 + S)
+    lens = rs.randint(1, S + 1, size=B)
+    lens[0] = S
+    if kind == "empty-sequence" and B > 1:
+        lens[B - 1] = 0
+    mask = workload.make_mask(lens, S, dtype).copy()
+    if kind == "ragged-rows" and S > 1:
+        mask[B // 2, S - 1, 0] = 1 - mask[B // 2, S - 1, 0]      # one element off in the last row
+    bi, wi, M = O.build_offsets(mask)
+    m = _dev(mask, device)
+    g_bi, g_wi, order, slots = ops.layer_prologue(m, want_slots=True)
+    assert np.array_equal(g_bi.cpu().numpy(), bi)
+    assert np.array_equal(g_wi.cpu().numpy()[:M], wi)
+    assert order.cpu().numpy().tolist() == np.argsort(-lens.astype(np.int64), kind="stable").tolist()
+    sl = slots.cpu().numpy()
+    assert set(np.unique(sl).tolist()) <= {0, 1}              # every slot was written
+    expect = kind == "prefix" or (kind == "empty-sequence" and B == 1) or \
+        (kind == "ragged-rows" and S == 1)
+    assert bool(sl.all()) == expect
+    assert ops.mask_is_prefix(m, g_bi) == expect
+    # without the slots (packed rows): the small grid, same offsets
+    g_bi2, g_wi2, order2, none = ops.layer_prologue(m)
+    assert none is None and torch.equal(g_bi2, g_bi) and torch.equal(order2, order)
+    assert torch.equal(g_wi2[:M], g_wi[:M])
+
+
+def test_layer_prologue_repacks_weights_that_changed_behind_the_copies(device):
+    """The fingerprint check of reused weight copies: the first prologue records, an
+    unchanged weight set leaves the copies alone, ANY change of the weights - a whole
+    matrix or one element - is seen on the device and the copies are made again."""
+    _say("prologue fingerprint")
+    rs = np.random.RandomState(5)
+    shapes = [(128, 384), (128, 128), (128, 512), (512, 128)]
+    ws = [_dev(rs.standard_normal(s).astype(np.float16), device) for s in shapes]
+    packed = ops.transpose_weights(ws)
+    state = torch.zeros(ops.PREPACK_STATE_WORDS, dtype=torch.int64, device=device)
+    mask = _dev(workload.make_mask([5, 9, 3], 9, np.float16), device)
+
+    def run():
+        ops.layer_prologue(mask, weights=ws, packed=packed, state=state)
+        torch.cuda.synchronize()
+        st = state.cpu().numpy().reshape(-1, 2)
+        assert (st[:, 1] == 1).all()                  # every share has a record
+        return st[:, 0].copy()
+
+    def copies_match():
+        return all(torch.equal(p, w.t().contiguous()) for p, w in zip(packed, ws))
+
+    fp0 = run()
+    assert (fp0 != 0).sum() >= 40                     # 48 tiles over 192 shares: most hold one
+    # poison one copy: unchanged fingerprints must NOT trigger a re-pack
+    keep = packed[1].clone()
+    packed[1].fill_(7)
+    assert np.array_equal(run(), fp0) and torch.equal(packed[1], torch.full_like(keep, 7))
+    packed[1].copy_(keep)
+    # a whole matrix rewritten without any host-side bookkeeping
+    ws[2].data.copy_(_dev(rs.standard_normal(shapes[2]).astype(np.float16), device))
+    assert not copies_match()
+    fp1 = run()
+    assert (fp1 != fp0).sum() >= 8 and copies_match()  # FFN1's 16 tiles moved, nothing else
+    # one element of the last matrix: exactly one share notices
+    ws[3].data[511, 127] += 1
+    fp2 = run()
+    assert (fp2 != fp1).sum() == 1 and copies_match()
+    # two elements of one tile swapped (the position is part of the fingerprint)
+    a, b = ws[0].data[0, 0].clone(), ws[0].data[5, 7].clone()
+    ws[0].data[0, 0], ws[0].data[5, 7] = b, a
+    fp3 = run()
+    assert ((fp3 != fp2).sum() == 1) == bool(a != b) and copies_match()
+    # shapes that do not fill their last tiles
+    odd = [_dev(rs.standard_normal(sh).astype(np.float16), device) for sh in [(72, 200), (200, 72)]]
+    odd_packed = ops.transpose_weights(odd)
+    odd_state = torch.zeros(ops.PREPACK_STATE_WORDS, dtype=torch.int64, device=device)
+    ops.layer_prologue(mask, weights=odd, packed=odd_packed, state=odd_state)
+    odd[0].data[71, 199] += 1
+    odd[1].data.mul_(-1)
+    ops.layer_prologue(mask, weights=odd, packed=odd_packed, state=odd_state)
+    torch.cuda.synchronize()
+    assert all(torch.equal(p, w.t().contiguous()) for p, w in zip(odd_packed, odd))
+
+
 def test_build_offsets_threshold(device):
     S = 70
     mask = np.zeros((2, S, S), np.float16)

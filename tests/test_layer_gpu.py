@@ -694,6 +694,100 @@ def test_th_op_prepack_cache_tracks_weight_updates(device):
         _check(d.cpu().numpy(), _oracle(wl2), wl2.lens, tag="cache/new-tensors")
 
 
+def test_th_op_caches_cannot_change_results(device):
+    """Writes that go around the version counter (`t.data.copy_()`, the way DLPack consumers
+    and raw-pointer kernels write too) between two operator calls: weights, the mask on the
+    packed rows and the mask on the padded rows.  The second result must be what the operator
+    gives with its caches switched off."""
+    _say("caches vs raw writes")
+    bt.load_th_op()
+    op = torch.ops.ByteTransformer.BertTransformer
+    for B, S, lens, lens2 in [(4, 64, (64, 20, 33, 50), (30, 64, 64, 50)),
+                              (2, 72, (72, 31), (40, 72))]:
+        cfg = workload.EncoderConfig("raw", B, S, 2, layers=1, lens=lens, seed=3)
+        wl = workload.make_workload(cfg, bias_std=0.05, random_affine=True)
+        w = [_dev(wl.layers[0][n], device) for n in workload.WEIGHT_NAMES]
+        x, m = _dev(wl.x, device), _dev(wl.mask, device)
+        first = op(2, 64, *w, x, m, True, True)
+        versions = [t._version for t in w] + [m._version]
+        # every matrix and the mask rewritten behind the operator's back
+        other = workload.make_workload(workload.EncoderConfig("raw2", B, S, 2, layers=1, lens=lens2,
+                                                              seed=4),
+                                       bias_std=0.05, random_affine=True)
+        for i in (0, 2, 6, 8):
+            w[i].data.copy_(_dev(other.layers[0][workload.WEIGHT_NAMES[i]], device))
+        m.data.copy_(_dev(other.mask, device))
+        assert [t._version for t in w] + [m._version] == versions       # nothing the host can see
+        second = op(2, 64, *w, x, m, True, True)
+        torch.ops.ByteTransformer.set_caches_enabled(False)
+        try:
+            plain = op(2, 64, *w, x, m, True, True)
+        finally:
+            torch.ops.ByteTransformer.set_caches_enabled(True)
+        assert not torch.equal(first, second)
+        assert torch.equal(second, plain)
+        mixed = {n: (other.layers[0][n] if i in (0, 2, 6, 8) else wl.layers[0][n])
+                 for i, n in enumerate(workload.WEIGHT_NAMES)}
+        wl2 = workload.Workload(cfg, np.array(lens2), wl.x, other.mask, [mixed])
+        got = second.cpu().numpy()
+        _check(got if B > 2 else O.masked_output(got, wl2.lens), _oracle(wl2), wl2.lens,
+               tag="raw writes B=%d" % B)
+        # one element of one weight
+        w[8].data[5, 7] += 0.5
+        third = op(2, 64, *w, x, m, True, True)
+        torch.ops.ByteTransformer.set_caches_enabled(False)
+        try:
+            plain = op(2, 64, *w, x, m, True, True)
+        finally:
+            torch.ops.ByteTransformer.set_caches_enabled(True)
+        assert torch.equal(third, plain) and not torch.equal(third, second)
+    torch.ops.ByteTransformer.clear_caches()
+
+
+def test_th_op_under_graph_capture(device):
+    """Two operator layers captured with torch.cuda.graph (the caches stay out of a
+    capture: the layer packs its weights and builds its offsets inside the graph), replayed
+    with other lengths and inputs written into the same buffers, eager work in between."""
+    _say("operator under capture")
+    bt.load_th_op()
+    op = torch.ops.ByteTransformer.BertTransformer
+    cfg = workload.EncoderConfig("cap", 5, 80, 2, layers=2, lens=(80, 20, 33, 50, 7), seed=6)
+    wl = workload.make_workload(cfg, bias_std=0.05, random_affine=True)
+    ws = [[_dev(w[n], device) for n in workload.WEIGHT_NAMES] for w in wl.layers]
+    x, m = _dev(wl.x, device), _dev(wl.mask, device)
+
+    def forward():
+        h = x
+        for w in ws:
+            h = op(2, 64, *w, h, m, True, True)
+        return h
+
+    side = torch.cuda.Stream(device=device)
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):          # warm-up on the capture stream, as torch asks for
+        forward()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        out = forward()
+    rs = np.random.RandomState(1)
+    for it in range(3):
+        lens = np.array(cfg.lens) if it == 0 else rs.randint(1, cfg.seq_len + 1, cfg.batch)
+        xn = (wl.x if it == 0 else rs.standard_normal(wl.x.shape)).astype(np.float16)
+        mask = workload.make_mask(lens, cfg.seq_len, np.float16)
+        x.copy_(_dev(xn, device))
+        m.copy_(_dev(mask, device))
+        graph.replay()
+        torch.cuda.synchronize()
+        got = out.cpu().numpy()
+        eager = forward()                   # eager work (cached copies) between the replays
+        torch.cuda.synchronize()
+        cur = workload.Workload(cfg, lens, xn, mask, wl.layers)
+        _check(got, _oracle(cur), lens, tag="captured operator, replay %d" % it)
+        assert np.array_equal(got, eager.cpu().numpy())
+
+
 def test_torchscript_class_forward_and_pickle(device):
     """torch.classes.ByteTransformer.BertTransformer: forward == functional
     operator, forwardv2 flags, TorchScript save/load round trip (pickle state =
