@@ -12,8 +12,11 @@ Prints ONE JSON line.  A "step" is one full L-layer forward over the synthetic
 batch; inputs and weights are resident in HBM before the timed region; the
 timed region is bracketed by torch.cuda.synchronize().  The same line carries
 the roofline of the dominant kernel (live HIP-event timing of that kernel at
-the workload's shape) and the CPU baseline (the oracle's PyTorch fp32 encoder on
-the host cores, bounded sample).
+the workload's shape), the CPU baseline (the oracle's PyTorch fp32 encoder on
+the host cores, bounded sample), the parity of the last timed forward against one
+complete forward of that oracle (the run fails outside max-abs 2e-2 / mean-abs 2e-3),
+the vendor GEMM library on the same shapes and the torch-free per-layer time of the
+C++ API (the stand-alone driver as a child process).
 """
 import argparse
 import json
@@ -160,6 +163,19 @@ def kernel_table(wl, dev, iters):
     rows.append(("copy_calibration_64MiB",
                  lambda: ops.compress(calib_src, c_bi, c_wi, out=calib_dst), "hbm",
                  2 * calib_src.numel() * 2))
+    # A plain copy moving as many bytes as each memory-bound kernel of the layer moves: what
+    # a launch of that size can reach at all (the row gather over an identity index).
+    def same_size_copy(name, total_bytes):
+        r = max(1, int(total_bytes) // (2 * H * 2))          # rows: read + write of r*H halfs
+        src = torch.empty(1, r, H, dtype=torch.float16, device=dev).normal_()
+        dst = torch.empty(r, H, dtype=torch.float16, device=dev)
+        bi = torch.tensor([0, r], dtype=torch.int32, device=dev)
+        wi = torch.arange(r, dtype=torch.int32, device=dev)
+        rows.append((name, lambda: ops.compress(src, bi, wi, out=dst), "hbm", 2 * r * H * 2))
+
+    same_size_copy("copy_same_bytes_as_layernorm", 3 * M * H * 2)
+    same_size_copy("copy_same_bytes_as_layernorm_restore", 2 * M * H * 2 + T * H * 2)
+    same_size_copy("copy_same_bytes_as_compress", 2 * M * H * 2)
     # The memory-bound kernels at a size where the launch cost (a few us, the same for
     # a plain copy) no longer dominates: 16x the rows of the workload.
     big = 16 * T
@@ -176,7 +192,82 @@ def kernel_table(wl, dev, iters):
             ach, peak, unit = work / (ms * 1e-3) / 1e9, HBM_PEAK_GBS, "GB/s"
         table[name] = {"us": round(ms * 1e3, 2), "bound": bound, "achieved": round(ach, 2),
                        "peak": peak, "unit": unit, "frac": round(ach / peak, 4)}
+    # each memory-bound kernel against the plain copy of the same byte count
+    for kern, ref in (("layernorm", "copy_same_bytes_as_layernorm"),
+                      ("layernorm_restore", "copy_same_bytes_as_layernorm_restore"),
+                      ("compress", "copy_same_bytes_as_compress")):
+        table[kern]["vs_same_size_copy"] = round(table[kern]["achieved"] / table[ref]["achieved"], 3)
     return table
+
+
+def hipblaslt_calibration(wl, dev, iters):
+    """torch.matmul (hipBLASLt / rocBLAS behind PyTorch-ROCm) on the layer's four GEMM
+    shapes at the workload's row count and on 8192^3: what the vendor library reaches on
+    this box next to the in-tree kernels.  fp16 in and out, no epilogue."""
+    import torch
+    cfg = wl.cfg
+    H, F, M = cfg.hidden, cfg.ffn_mult * cfg.hidden, wl.valid_tokens
+    out = {}
+    for name, (m, n, k) in (("qkv", (M, 3 * H, H)), ("proj", (M, H, H)), ("ffn1", (M, F, H)),
+                            ("ffn2", (M, H, F)), ("square_8192", (8192, 8192, 8192))):
+        a = torch.empty(m, k, dtype=torch.float16, device=dev).normal_()
+        b = torch.empty(k, n, dtype=torch.float16, device=dev).normal_(std=0.02)
+        c = torch.empty(m, n, dtype=torch.float16, device=dev)
+        ms = time_kernel(lambda: torch.matmul(a, b, out=c), max(5, iters // 5 if m >= 8192 else iters))
+        tf = 2.0 * m * n * k / (ms * 1e-3) / 1e12
+        out[name] = {"m": m, "n": n, "k": k, "us": round(ms * 1e3, 2), "tflops": round(tf, 1),
+                     "frac": round(tf / MFMA_F16_PEAK_TFLOPS, 4)}
+    return out
+
+
+def cpp_api_layer_ms(wl, iters=50):
+    """Per-layer time of the C++ BertTransformer::infer loop without torch or Python: the
+    stand-alone driver on synthetic tensors of the workload's shape and lengths (the
+    reference's own timing loop, unit_test/bert_transformer_test.cc:190-202).  Runs as a
+    child process; None when the driver is not built."""
+    import re
+    import subprocess
+    import bytetransformer_amd as bt
+    exe = os.path.join(bt.lib_dir(), "bert_transformer_test")
+    if not os.path.exists(exe):
+        return None
+    cfg = wl.cfg
+    cmd = [exe, str(cfg.batch), str(cfg.seq_len), str(cfg.head_num), str(cfg.head_size),
+           "--synthetic", "--lens", ",".join(str(int(v)) for v in wl.lens), "--iters", str(iters)]
+    try:
+        res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True,
+                             timeout=120)
+    except (OSError, subprocess.TimeoutExpired) as exc:
+        print("bench: C++ driver failed (%s)" % exc, file=sys.stderr)
+        return None
+    m = re.search(r"layer time costs ([0-9.]+) ms", res.stdout)
+    if res.returncode != 0 or not m:
+        print("bench: C++ driver failed:\n%s" % res.stdout[-500:], file=sys.stderr)
+        return None
+    return float(m.group(1))
+
+
+def oracle_forward(wl):
+    """One complete forward of the CPU oracle (fp32 PyTorch restatement of the reference's
+    encoder script) on the workload; returns (masked output, seconds per layer list)."""
+    import numpy as np
+    import torch
+    from oracle import bert_oracle as O
+    cores = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "0")) or 10 ** 6)
+    torch.set_num_threads(cores)
+    x = torch.from_numpy(wl.x.astype(np.float32))
+    mask = torch.from_numpy(wl.mask.astype(np.float32))
+    layers32 = [{k: torch.from_numpy(np.asarray(v, np.float32)) for k, v in w.items()}
+                for w in wl.layers]
+    times = []
+    with torch.no_grad():
+        O.encoder_layer(x, mask, layers32[0], wl.cfg.head_num)       # warm-up
+        h = x
+        for w in layers32:
+            t0 = time.perf_counter()
+            h = O.encoder_layer(h, mask, w, wl.cfg.head_num)
+            times.append(time.perf_counter() - t0)
+    return O.masked_output(h.numpy(), wl.lens), times, cores
 
 
 def measured_traffic(workload_name, kernel):
@@ -191,32 +282,32 @@ def measured_traffic(workload_name, kernel):
         return None
 
 
-def cpu_baseline(wl, budget_s=25.0, target_s=10.0):
-    """The oracle's PyTorch fp32 encoder on the padded batch, all host cores: whole
-    forwards repeated until about target_s of CPU work is done, cut off inside a
-    forward at budget_s (at least one layer is timed)."""
+def cpu_baseline(wl, first_pass_times, cores, target_s=10.0, budget_s=25.0):
+    """The oracle's PyTorch fp32 encoder on the padded batch, all host cores.  The first
+    complete forward (whose output the parity check uses) is already timed layer by layer;
+    further whole layers are run until about target_s of CPU work is done (cut off at
+    budget_s)."""
     import numpy as np
     import torch
     from oracle import bert_oracle as O
-    cores = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "0")) or 10 ** 6)
     torch.set_num_threads(cores)
     x = torch.from_numpy(wl.x.astype(np.float32))
     mask = torch.from_numpy(wl.mask.astype(np.float32))
     layers32 = [{k: torch.from_numpy(np.asarray(v, np.float32)) for k, v in w.items()}
                 for w in wl.layers]
+    done, el = len(first_pass_times), float(sum(first_pass_times))
     with torch.no_grad():
-        O.encoder_layer(x, mask, layers32[0], wl.cfg.head_num)       # warm-up
-        done, t0 = 0, time.perf_counter()
-        while True:
+        while el < target_s:
             h = x
             for w in layers32:
+                t0 = time.perf_counter()
                 h = O.encoder_layer(h, mask, w, wl.cfg.head_num)
+                el += time.perf_counter() - t0
                 done += 1
-                if time.perf_counter() - t0 > budget_s:
+                if el > budget_s:
                     break
-            if time.perf_counter() - t0 > target_s:
+            if el > budget_s:
                 break
-        el = time.perf_counter() - t0
     ms_full = el / done * len(layers32) * 1e3
     return {"value": round(ms_full, 1), "unit": "ms", "cores": cores, "kind": "port",
             "sample": "%d layer passes (%.1f forwards of %d layers) of the same padded batch timed "
@@ -235,12 +326,15 @@ def main():
     import torch
     import bytetransformer_amd as bt
     from bytetransformer_amd import workload
+    from oracle import bert_oracle as O
 
+    wl = workload.make_workload(args.workload)
+    cfg = wl.cfg
+    # the torch-free C++ loop runs as a child process, before this process touches the GPU
+    cpp_layer_ms = cpp_api_layer_ms(wl)
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     dev = torch.device("cuda:0")
     bt.load_th_op()
-    wl = workload.make_workload(args.workload)
-    cfg = wl.cfg
     t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dev)
     layers = [[t(w[n]) for n in workload.WEIGHT_NAMES] for w in wl.layers]
     x, mask = t(wl.x), t(wl.mask)
@@ -257,9 +351,21 @@ def main():
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for _ in range(args.steps):
-        forward()
+        last = forward()
     torch.cuda.synchronize()
     ms = (time.perf_counter() - t0) * 1e3 / args.steps
+
+    # parity of what was just timed: the last timed forward's output against one complete
+    # forward of the CPU oracle on the same inputs (budget of the fp16 configurations)
+    expect, oracle_times, cores = oracle_forward(wl)
+    got = last.cpu().numpy()
+    if cfg.batch <= 2:                      # padded rows: rows past the lengths are not zeroed
+        got = O.masked_output(got, wl.lens)
+    mx, mean, pads_zero = O.parity_metrics(got, expect, wl.lens)
+    parity = {"max_abs": float("%.4g" % mx), "mean_abs": float("%.4g" % mean),
+              "pads_zero": bool(pads_zero), "tolerance": {"max_abs": 2e-2, "mean_abs": 2e-3},
+              "against": "CPU oracle, one complete %d-layer forward on the same inputs" % cfg.layers}
+    parity["ok"] = bool(mx <= 2e-2 and mean <= 2e-3 and pads_zero)
 
     def timed(fn):
         for _ in range(args.warmup):
@@ -312,7 +418,10 @@ def main():
     d = kernels[dominant]
     roofline = {"kernel": dominant, "bound": d["bound"], "achieved": d["achieved"],
                 "peak": d["peak"], "unit": d["unit"], "frac": d["frac"],
-                "traffic": measured_traffic(args.workload, dominant), "launch_us": d["us"]}
+                "traffic": measured_traffic(args.workload, dominant),
+                "traffic_source": "profiles/traffic.json (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE "
+                                  "runs of this command, not measured in this run)",
+                "launch_us": d["us"]}
     pub = PUBLISHED_A100_MS.get(args.workload)
     line = {
         "metric": "ms per %d-layer BERT fwd, bs%d, avg len 0.6*max (valid-token throughput alongside)"
@@ -330,12 +439,17 @@ def main():
         "tokens_per_s": round(wl.valid_tokens / (ms * 1e-3), 1),
         "model_tflops": round(cfg.layers * (gemm_f + attn_f) / (ms * 1e-3) / 1e12, 2),
         "roofline": roofline,
+        "parity": parity,
         "other_entry_points": other,
+        "cpp_api_layer_ms": cpp_layer_ms,
+        "hipblaslt_calibration": hipblaslt_calibration(wl, dev, args.kernel_iters),
         "kernels": kernels,
     }
     if not args.no_cpu_baseline:
-        line["cpu_baseline"] = cpu_baseline(wl)
+        line["cpu_baseline"] = cpu_baseline(wl, oracle_times, cores)
     print(json.dumps(line))
+    if not parity["ok"]:
+        sys.exit("bench.py: the timed operator's output is outside the parity budget: %s" % parity)
 
 
 if __name__ == "__main__":

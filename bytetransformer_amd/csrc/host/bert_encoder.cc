@@ -37,6 +37,9 @@ void BertEncoder<OpType>::infer(BertEncoderInferParam<DataType_> ip) {
 
   const int hidden = head_num_ * size_per_head_, inter = hidden * intermediate_size_;
   const int rows = batch_size * seq_len;
+  if (OpType == OperationType::HALF && hidden % 64 != 0)
+    throw std::runtime_error("[BT][ERROR] BertEncoder: fp16 layers need head_num * size_per_head "
+                             "to be a multiple of 64, got " + std::to_string(hidden));
   const size_t tensor = (size_t)rows * hidden;
   const unsigned long long max_rows = (unsigned long long)max_batch_size_ * max_seq_len_;
   const unsigned long long max_tensor = max_rows * hidden;

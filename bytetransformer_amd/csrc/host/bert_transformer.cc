@@ -27,6 +27,11 @@ void BertTransformer<OpType>::bert_infer(BertTransformerInferParam infer_param) 
   const int hidden = head_num_ * size_per_head_;
   const int inter = hidden * param_.intermediate_size;
   const int rows = batch_size * seq_len;
+  // the fp16 products step through k in tiles of 64 (the float layer has no such rule)
+  if (OpType == OperationType::HALF && hidden % 64 != 0)
+    throw std::runtime_error("[BT][ERROR] BertTransformer: fp16 layers need head_num * "
+                             "size_per_head to be a multiple of 64, got " +
+                             std::to_string(hidden));
   const size_t tensor = (size_t)rows * hidden;
 
   // carve the scratch with the maxima, exactly as cal_bufsize() laid it out

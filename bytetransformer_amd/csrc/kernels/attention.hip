@@ -136,7 +136,9 @@ __device__ __forceinline__ void prefetch_slice(const AttArgs &p) {
   if (blockIdx.x < z0) return;
   const unsigned long long duty = gridDim.x - z0;
   const unsigned long long me = blockIdx.x - z0;
-  const unsigned long long lines = (p.prefetch_bytes + 127) / 128;
+  // one dword at the start of each 128-byte line; a last line of fewer than four bytes is
+  // left alone, so no byte outside the range is read
+  const unsigned long long lines = (p.prefetch_bytes + 124) / 128;
   const unsigned long long per = (lines + duty - 1) / duty;
   const unsigned long long first = me * per;
   const unsigned long long last = first + per < lines ? first + per : lines;
@@ -630,7 +632,7 @@ static void set_prefetch(AttArgs &a, unsigned grid, const void *prefetch, unsign
   a.prefetch_bytes = 0;
   if (!prefetch || !bytes || !option_prefetch()) return;
   const unsigned long long duty = grid - (unsigned long long)grid * 3 / 4;
-  if (grid < 512) return;
+  if (grid < (unsigned)option_prefetch_min_grid()) return;
   const unsigned long long cap = duty * 4 * kAttThreads * 128;
   a.prefetch = (const char *)prefetch;
   a.prefetch_bytes = bytes < cap ? bytes : cap;

@@ -75,6 +75,7 @@ int option_attention_qb();   // -1 = heuristic, 1 or 2 = query blocks per wave
 int option_f32_gemm_tile();  // -1 = heuristic, else index into the float GEMM's tile table
 int option_attention_xcd_map();     // workgroup order of the attention kernels: 0 plain, 1 XCD-aware, 2 balanced (default), 3 balanced always
 int option_prefetch();       // 1 = honour the prefetch hints of the attention entries (default), 0 = ignore
+int option_prefetch_min_grid();   // attention launches of fewer workgroups skip the cache warm-up (default 512)
 
 inline hipStream_t as_stream(void *s) { return reinterpret_cast<hipStream_t>(s); }
 

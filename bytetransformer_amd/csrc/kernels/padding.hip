@@ -30,6 +30,7 @@ int hip_fail(hipError_t e, const char *what) {
 static std::atomic<int> g_gemm_tile{-1};
 static std::atomic<int> g_attention_qb{-1};
 static std::atomic<int> g_prefetch{1};
+static std::atomic<int> g_prefetch_min_grid{512};
 static std::atomic<int> g_f32_gemm_tile{-1};
 static std::atomic<int> g_attention_short_limit{0};
 static std::atomic<int> g_attention_xcd_map{2};
@@ -38,6 +39,7 @@ int option_f32_gemm_tile() { return g_f32_gemm_tile.load(std::memory_order_relax
 int option_gemm_tile() { return g_gemm_tile.load(std::memory_order_relaxed); }
 int option_attention_qb() { return g_attention_qb.load(std::memory_order_relaxed); }
 int option_prefetch() { return g_prefetch.load(std::memory_order_relaxed); }
+int option_prefetch_min_grid() { return g_prefetch_min_grid.load(std::memory_order_relaxed); }
 
 // ---- offsets ----------------------------------------------------------------
 constexpr int kOffsetThreads = 1024;
@@ -419,6 +421,10 @@ extern "C" int bt_set_option(const char *name, int value) {
     BT_REQUIRE(value == 0 || value == 1, BT_ERR_INVALID_ARGUMENT,
                "bt_set_option: prefetch=%d must be 0 or 1", value);
     g_prefetch.store(value);
+  } else if (!strcmp(name, "prefetch_min_grid")) {
+    BT_REQUIRE(value >= 1 && value <= (1 << 20), BT_ERR_INVALID_ARGUMENT,
+               "bt_set_option: prefetch_min_grid=%d outside [1, 2^20]", value);
+    g_prefetch_min_grid.store(value);
   } else {
     set_error("bt_set_option: unknown option '%s'", name);
     return BT_ERR_INVALID_ARGUMENT;
@@ -434,6 +440,8 @@ extern "C" int bt_get_option(const char *name, int *value) {
     *value = g_attention_qb.load();
   } else if (!strcmp(name, "prefetch")) {
     *value = g_prefetch.load();
+  } else if (!strcmp(name, "prefetch_min_grid")) {
+    *value = g_prefetch_min_grid.load();
   } else if (!strcmp(name, "f32_gemm_tile")) {
     *value = g_f32_gemm_tile.load();
   } else if (!strcmp(name, "attention_short_limit")) {

@@ -204,6 +204,9 @@ inline std::unique_ptr<IBTEncoder> make_encoder(int64_t head_num, int64_t head_s
 inline void check_layer_shapes(int64_t head_num, int64_t head_size, const std::vector<Tensor> &w) {
   const int64_t H = head_num * head_size;
   TORCH_CHECK(head_num > 0 && head_size > 0, "head_num and head_size must be positive");
+  TORCH_CHECK(w[0].scalar_type() != at::ScalarType::Half || H % 64 == 0,
+              "fp16 layers need head_num * head_size to be a multiple of 64, got ", H,
+              " (float tensors have no such rule)");
   TORCH_CHECK(w[0].dim() == 2 && w[0].size(0) == H && w[0].size(1) == 3 * H,
               "qkv_kernel must be [hidden_dim, 3 * hidden_dim]");
   TORCH_CHECK(w[1].numel() == 3 * H, "qkv_bias must have 3 * hidden_dim elements");

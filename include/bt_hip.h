@@ -52,6 +52,8 @@ const char *bt_last_error_string(void);
  *                   | 5: 128x128 with a two-deep ring (two workgroups per CU)
  *   "attention_qb"  -1 heuristic | 1 | 2: 16-query blocks per wave in the grouped kernel
  *   "prefetch"      1 (default) | 0: honour / ignore the prefetch hint of the attention entries
+ *   "prefetch_min_grid"  512 (default): attention launches of fewer workgroups ignore the hint
+ *                   (there the warm-up costs more than it returns); 1 = every launch honours it
  *   "f32_gemm_tile" -1 heuristic | 0: 128x128 tile, 8 waves | 1: 128x64, 4 waves | 2: 64x64, 4 waves
  *                   (bt_gemm_f32 only)
  *   "attention_short_limit"  0 (default) .. 512: the host library sends sequences up to this

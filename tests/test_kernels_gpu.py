@@ -809,6 +809,27 @@ def test_attention_prefetch_hint_changes_nothing(device, kind, lens, S):
         assert torch.equal(got[:M], base[:M])
     finally:
         ops.set_option("prefetch", 1)
+    # Small launches skip the warm-up by themselves; force it on so that the duty
+    # workgroups really run here.  The range sits inside a larger allocation (guard bytes on
+    # both sides, so a stray line would still land in owned memory), starts on a line
+    # boundary or 16 bytes into one, and ends 0-5 bytes into a line: the last touched dword
+    # must lie inside the range.
+    assert ops.get_option("prefetch_min_grid") == 512
+    ops.set_option("prefetch_min_grid", 1)
+    try:
+        guard = 4096
+        for nbytes in (1, 2, 3, 4, 5, 127, 128, 129, 130, 131, 132, 4099, 1000003, (8 << 20) + 2):
+            for lead in (0, 16):
+                whole = torch.full((guard + lead + nbytes + guard,), 7, dtype=torch.uint8,
+                                   device=device)
+                warm = whole[guard + lead:guard + lead + nbytes]
+                got = fn(_dev(qkv, device), _dev(bi, device), len(lens), S, 0.125, False,
+                         prefetch=warm)
+                torch.cuda.synchronize()
+                assert torch.equal(got[:M], base[:M]), (nbytes, lead)
+                assert bool((whole == 7).all())
+    finally:
+        ops.set_option("prefetch_min_grid", 512)
 
 
 def test_attention_large_logits_do_not_overflow(device):

@@ -558,6 +558,26 @@ def test_head_sizes_other_than_64(device, dtype, head_size, heads, rm):
         assert mx <= tol[0] and mean <= tol[1] and pads_zero, (tag, mx, mean, pads_zero)
 
 
+def test_hidden_size_rule_of_the_fp16_layer(device):
+    """head_num * head_size must be a multiple of 64 on fp16 (the MFMA products step
+    through k in tiles of 64); the float layer takes 12 x 40 = 480."""
+    bt.load_th_op()
+    cfg = workload.EncoderConfig("h480", 3, 33, 12, head_size=40, layers=1, lens=(33, 7, 20))
+    wl = workload.make_workload(cfg, bias_std=0.05, random_affine=True)
+    with pytest.raises(RuntimeError, match="multiple of 64"):
+        _run_th_op(wl, device)
+    with pytest.raises(RuntimeError, match="multiple of 64"):
+        _run_c_api(wl, device)
+    with pytest.raises(RuntimeError, match="multiple of 64"):
+        _whole_encoder(wl, device)(_dev(wl.x, device), _dev(wl.mask, device))
+    cfg32 = workload.EncoderConfig("h480f", 3, 33, 12, head_size=40, layers=1, dtype="fp32",
+                                   lens=(33, 7, 20))
+    wl32 = workload.make_workload(cfg32, bias_std=0.05, random_affine=True)
+    exp = O.masked_output(O.encoder(wl32.x, wl32.mask, wl32.layers, 12).numpy(), wl32.lens)
+    mx, mean, pads_zero = O.parity_metrics(_run_th_op(wl32, device), exp, wl32.lens)
+    assert mx <= 2e-4 and mean <= 2e-5 and pads_zero, (mx, mean)
+
+
 @pytest.mark.parametrize("dtype", ["fp16", "fp32"])
 def test_seq_len_one(device, dtype):
     """seq_len 1: batch_idx has one entry more than there are rows (the scratch carve once
