@@ -37,8 +37,8 @@ KERNEL_ABI = {
     "bt_build_offsets": (c_int, [_P, c_int, c_int, c_int, _IP, _IP, _IP, POINTER(c_int), _P]),
     "bt_mask_prefix_slots": (c_int, [_P, c_int, c_int, c_int, _IP, _IP, _P]),
     "bt_mask_is_prefix": (c_int, [_P, c_int, c_int, c_int, _IP, _IP, POINTER(c_int), _P]),
-    "bt_layer_prologue": (c_int, [_P, c_int, c_int, c_int, _IP, _IP, _IP, _IP, c_int,
-                                  POINTER(c_void_p), POINTER(c_void_p), POINTER(c_int),
+    "bt_layer_prologue": (c_int, [_P, c_int, c_int, c_int, _IP, _IP, _IP, _IP, _P, c_int, c_int,
+                                  c_int, POINTER(c_void_p), POINTER(c_void_p), POINTER(c_int),
                                   POINTER(c_int), _P, _P]),
     "bt_compress": (c_int, [_P, _P, _IP, _IP, c_int, c_int, c_int, _P]),
     "bt_transpose_weight": (c_int, [_P, _P, c_int, c_int, _P]),
@@ -51,7 +51,9 @@ KERNEL_ABI = {
     "bt_attention_short": (c_int, [_P, _P, _IP, _IP, _P, _P, c_int, c_int, c_int, c_int, c_int,
                                    c_float, c_int, _P, c_ulonglong, _P]),
     "bt_attention_grouped": (c_int, [_P, _P, _IP, _IP, _P, _P, c_int, c_int, c_int, c_int, c_int,
-                                     c_float, c_int, _P, c_ulonglong, _IP, _P]),
+                                     c_float, c_int, _P, c_ulonglong, _IP, _P, _P]),
+    "bt_attention_worklist_bytes": (c_ulonglong, [c_int, c_int, c_int]),
+    "bt_attention_worklist": (c_int, [_IP, _IP, c_int, c_int, c_int, c_int, _P, _P]),
     "bt_add_bias_residual_layernorm": (c_int, [_P, _P, _IP, _P, _P, _P, c_int, _IP, c_int, c_int,
                                                c_float, _P]),
     "bt_add_bias_residual_layernorm_restore": (c_int, [_P, _P, _P, _P, _P, c_int, _P, _IP, c_int,

@@ -72,7 +72,8 @@ void Attention<OpType>::infer(AttentionInferParam infer_param) {
         infer_param.qkv, infer_param.attention_output, infer_param.et_param.batch_idx,
         infer_param.seq_order, mask, infer_param.attention_bias, infer_param.batch_size,
         infer_param.seq_len, rows_cap, head_num_, size_per_head_, scale, padded_rows,
-        infer_param.prefetch, infer_param.prefetch_bytes, slots, infer_param.stream));
+        infer_param.prefetch, infer_param.prefetch_bytes, slots, infer_param.work_list,
+        infer_param.stream));
   }
 }
 

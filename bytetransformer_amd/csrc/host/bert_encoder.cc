@@ -62,6 +62,13 @@ void BertEncoder<OpType>::infer(BertEncoderInferParam<DataType_> ip) {
   DataType_ *staging = (DataType_ *)(base + off);      // one layer's weights when none were passed
   off += align_up(layer_weight_elems() * sizeof(DataType_), 256);
   float *splitk_buf = (float *)(base + off);
+  off += align_up(splitk_scratch_bytes(max_rows, (unsigned long long)hidden), 256);
+  // the streaming attention's balanced work list: built once per forward beside the offsets
+  void *work_list = nullptr;
+  if (OpType == OperationType::HALF && size_per_head_ == 64 &&
+      !attention_layer_->uses_short_kernel(seq_len) &&
+      bt_attention_worklist_bytes(batch_size, seq_len, head_num_) > 0)
+    work_list = base + off;
 
   // padded rows: the fp16 streaming attention applies the mask tensor unless one pass
   // over it (once for all layers) finds the plain prefix mask of the lengths
@@ -70,7 +77,8 @@ void BertEncoder<OpType>::infer(BertEncoderInferParam<DataType_> ip) {
   // offsets and that verdict in one launch, once per forward
   check_bt_error(bt_layer_prologue(ip.atten_mask, Traits_::dtype, batch_size, seq_len,
                                    et_param.batch_idx, et_param.word_idx, seq_order,
-                                   check_mask ? mask_slots : nullptr, 0, nullptr, nullptr, nullptr,
+                                   check_mask ? mask_slots : nullptr, work_list, head_num_,
+                                   is_remove_padding_ ? 0 : 1, 0, nullptr, nullptr, nullptr,
                                    nullptr, nullptr, stream));
   const int *valid_rows = is_remove_padding_ ? et_param.batch_idx + batch_size : nullptr;
   const int rows_hint = ip.valid_rows_hint;
@@ -146,6 +154,7 @@ void BertEncoder<OpType>::infer(BertEncoderInferParam<DataType_> ip) {
     att.attention_bias = ip.attention_bias;
     att.seq_order = seq_order;
     if (check_mask) att.mask_prefix_slots = mask_slots;
+    att.work_list = work_list;
     // warm the memory-side cache with what follows in memory order: the rest of this
     // layer's weights and, when all layers are pre-packed back to back, the next
     // layer's QKV matrix

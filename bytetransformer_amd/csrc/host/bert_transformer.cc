@@ -81,6 +81,14 @@ void BertTransformer<OpType>::bert_infer(BertTransformerInferParam infer_param) 
       !attention_layer_->uses_short_kernel(seq_len) && !(have_offsets && infer_param.mask_prefix >= 0))
     mask_slots = (int *)(base + inner_buf_size_);
 
+  // The streaming attention's balanced work list, when a launch of this shape uses one: the
+  // prologue builds it beside the offsets, the kernel then finds its work with one load.
+  void *work_list = nullptr;
+  if (OpType == OperationType::HALF && size_per_head_ == 64 && !have_offsets &&
+      !attention_layer_->uses_short_kernel(seq_len) &&
+      bt_attention_worklist_bytes(batch_size, seq_len, head_num_) > 0)
+    work_list = base + inner_buf_size_ + Attention<OpType>::work_list_offset();
+
   // One launch ahead of the layer: lengths and offsets from the mask (needed on both
   // paths: keys past len_b are excluded), the prefix-mask verdict, the check of reused
   // weight copies.  Rebuilt on every call, as the reference does
@@ -94,7 +102,8 @@ void BertTransformer<OpType>::bert_infer(BertTransformerInferParam infer_param) 
     if (!have_offsets || mask_slots || check_prepack)
       check_bt_error(bt_layer_prologue(atten_mask, Traits_::dtype, batch_size, seq_len,
                                        et_param.batch_idx, et_param.word_idx, seq_order,
-                                       mask_slots, check_prepack ? 4 : 0, w_src, w_dst, w_k, w_n,
+                                       mask_slots, work_list, head_num_, is_remove_padding_ ? 0 : 1,
+                                       check_prepack ? 4 : 0, w_src, w_dst, w_k, w_n,
                                        check_prepack ? param_.prepack_state : nullptr, stream));
   }
   if (have_offsets) {
@@ -188,6 +197,7 @@ void BertTransformer<OpType>::bert_infer(BertTransformerInferParam infer_param) 
   attention_infer_param.seq_order = seq_order;
   attention_infer_param.mask_prefix = have_offsets ? infer_param.mask_prefix : -1;
   attention_infer_param.mask_prefix_slots = mask_slots;
+  attention_infer_param.work_list = work_list;
   // the three weight matrices the rest of the layer reads, when they lie back to back:
   // the attention kernel pulls them into the memory-side cache while it runs
   if (wt_inter == wt_proj + (size_t)hidden * hidden && wt_out == wt_inter + (size_t)hidden * inter) {

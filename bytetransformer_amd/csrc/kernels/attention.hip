@@ -57,6 +57,8 @@ struct AttArgs {
   int xcd_map;         // 0: plain (tile, head, sequence) order, 1: XCD-aware, 2: XCD-aware and balanced over the CUs
   const int *mask_ok;  // optional int[256] from bt_mask_prefix_slots: all non-zero = the mask
                        // is the plain prefix mask of the lengths, and is then ignored
+  const int4 *work_list;   // optional: entry w of bt_attention_worklist = what workgroup w of the
+                           // balanced order works on {sequence or -1, head | tile << 16, first row, length}
 };
 
 // Which (sequence rank, head, query tile) a workgroup of the 1-D grid works on.  The
@@ -229,16 +231,32 @@ constexpr int kTileHalfs = kKT * kHeadDim;       // one K or V tile
 
 // QB 16-query blocks per wave; workgroup covers 4*QB*16 queries.  ADD: a mask tensor and / or an
 // attention bias contribute additive terms to the logits.
-template <int QB, bool ADD, int STAGES>
-__global__ __launch_bounds__(kAttThreads, 2) void attention_grouped_kernel(AttArgs p) {
+// KS = 2 (key split): eight waves; waves 4-7 work on the same queries as waves 0-3 but on
+// the other 64-key half of every 128-key ring slot, with their own running maximum, sum
+// and output, and the two halves are merged through LDS at the end.  The dependency chain
+// of a query tile - what bounds a launch of a few workgroups per CU, where the longest
+// sequence's workgroups finish last - is half as long, and twice the waves hide it.
+template <int QB, bool ADD, int STAGES, int KS = 1>
+__global__ __launch_bounds__(kAttThreads * KS, KS == 1 ? 2 : 4) void attention_grouped_kernel(AttArgs p) {
   constexpr int BQ = 4 * QB * 16;
   constexpr int AHEAD = STAGES - 1;     // tiles in flight beyond the one being consumed
+  constexpr int kSlotKeys = kKT * KS;   // keys per ring slot
+  constexpr int kSlotHalfs = KS * 2 * kTileHalfs;
   static_assert(STAGES == 2 || STAGES == 3, "ring depth");
-  __shared__ __attribute__((aligned(1024))) half_t ring[STAGES * 2 * kTileHalfs];
+  static_assert(KS == 1 || KS == 2, "key split");
+  __shared__ __attribute__((aligned(1024))) half_t ring[STAGES * kSlotHalfs];
 
   int b, head, seq_start, seq_len, qb_index;
-  if (p.xcd_map == 2) {
-    const AttWork w = att_work_balanced<BQ>(p);
+  if (p.xcd_map == 2 && p.work_list) {
+    // the balanced order, looked up by an earlier launch: one scalar load
+    const int4 w = p.work_list[blockIdx.x];
+    if (w.x < 0) {
+      prefetch_slice(p);
+      return;
+    }
+    b = w.x, head = w.y & 0xffff, qb_index = w.y >> 16, seq_start = w.z, seq_len = w.w;
+  } else if (p.xcd_map == 2) {
+    const AttWork w = att_work_balanced<BQ>(p, blockIdx.x);
     if (!w.exists) {
       prefetch_slice(p);
       return;
@@ -273,7 +291,10 @@ __global__ __launch_bounds__(kAttThreads, 2) void attention_grouped_kernel(AttAr
     return;
   }
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave_all = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wave = wave_all & 3;        // which 16-query blocks
+  const int grp = wave_all >> 2;        // which 64-key half of a ring slot (KS = 2)
   const int lq = lane & 15, lg = lane >> 4;
 
   const size_t head_stride = (size_t)p.rows_cap * kHeadDim;
@@ -294,24 +315,25 @@ __global__ __launch_bounds__(kAttThreads, 2) void attention_grouped_kernel(AttAr
     }
   }
 
-  // Tile copy: 16 load instructions per tile (8 rows each; 0-7 = K, 8-15 = V),
+  // Slot copy: 16 load instructions per 64-key tile (8 rows each; 0-7 = K, 8-15 = V),
   // four per wave.  Lane -> (row, slot) and fetches the chunk the swizzle puts
   // in that slot.
   const int ld_row = lane >> 3, ld_slot = lane & 7;
   auto issue_tile = [&](int t, int stage) {
-    half_t *sbase = ring + stage * 2 * kTileHalfs;
-    const int k0 = t * kKT;
+    half_t *sbase = ring + stage * kSlotHalfs;
+    const int k0 = t * kSlotKeys;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      const int id = i * 4 + wave;          // 0..15
+      const int id_all = i * 4 * KS + wave_all;   // 0 .. 16 KS - 1
+      const int sub = id_all >> 4, id = id_all & 15;
       const int row = (id & 7) * 8 + ld_row;
-      const int key = min(k0 + row, klen - 1);
+      const int key = min(k0 + sub * kKT + row, klen - 1);
       if (id < 8)
         lds_dma16(K + (size_t)key * kHeadDim + ((ld_slot ^ swz_k(row)) << 3),
-                  sbase + (id & 7) * 8 * kHeadDim);
+                  sbase + sub * 2 * kTileHalfs + (id & 7) * 8 * kHeadDim);
       else
         lds_dma16(V + (size_t)key * kHeadDim + ((ld_slot ^ swz_v(row)) << 3),
-                  sbase + kTileHalfs + (id & 7) * 8 * kHeadDim);
+                  sbase + sub * 2 * kTileHalfs + kTileHalfs + (id & 7) * 8 * kHeadDim);
     }
   };
 
@@ -329,7 +351,7 @@ __global__ __launch_bounds__(kAttThreads, 2) void attention_grouped_kernel(AttAr
   const half8_t ones = {1, 1, 1, 1, 1, 1, 1, 1};
 
   const bool wave_live = q0 + wave * QB * 16 < nq;
-  const int ntiles = (klen + kKT - 1) / kKT;
+  const int ntiles = (klen + kSlotKeys - 1) / kSlotKeys;
   if (ntiles > 0) issue_tile(0, 0);
   if (AHEAD > 1 && ntiles > 1) issue_tile(1, 1);
 
@@ -354,12 +376,14 @@ __global__ __launch_bounds__(kAttThreads, 2) void attention_grouped_kernel(AttAr
       if (ps >= STAGES) ps -= STAGES;
       issue_tile(t + AHEAD, ps);
     }
-    // a wave whose queries all lie past the sequence only copies and keeps the barriers
-    if (!wave_live) {
+    // a wave whose queries all lie past the sequence, or whose half of the slot lies past
+    // the last key, only copies and keeps the barriers
+    const int k0 = t * kSlotKeys + grp * kKT;
+    if (!wave_live || (KS > 1 && k0 >= klen)) {
       if (++stage == STAGES) stage = 0;
       return;
     }
-    const half_t *sK = ring + stage * 2 * kTileHalfs;
+    const half_t *sK = ring + stage * kSlotHalfs + grp * 2 * kTileHalfs;
     const half_t *sV = sK + kTileHalfs;
 
     // S^T = K . Q^T for this tile: 4 key blocks x QB query blocks
@@ -375,7 +399,6 @@ __global__ __launch_bounds__(kAttThreads, 2) void attention_grouped_kernel(AttAr
       }
     }
     if (ADD) {
-      const int k0 = t * kKT;
 #pragma unroll
       for (int qb = 0; qb < QB; ++qb) {
         const int q = min(q0 + (wave * QB + qb) * 16 + lq, p.S - 1);
@@ -390,7 +413,6 @@ __global__ __launch_bounds__(kAttThreads, 2) void attention_grouped_kernel(AttAr
       }
     }
     if (MASKED) {
-      const int k0 = t * kKT;
 #pragma unroll
       for (int kb = 0; kb < 4; ++kb)
 #pragma unroll
@@ -455,10 +477,44 @@ __global__ __launch_bounds__(kAttThreads, 2) void attention_grouped_kernel(AttAr
   // every tile but the last is full: no masking code on the steady-state path
   for (int t = 0; t + 1 < ntiles; ++t) process_tile(t, std::false_type{});
   if (ntiles > 0) {
-    if (klen % kKT == 0)
+    if (klen % kSlotKeys == 0)
       process_tile(ntiles - 1, std::false_type{});
     else
       process_tile(ntiles - 1, std::true_type{});
+  }
+
+  if (KS > 1) {
+    // fold the second key half into the first: waves 4-7 hand over maximum, sum and output
+    // through the ring (lane-major, one word per lane and item: no bank conflicts)
+    float *xch = (float *)ring + (size_t)wave * (21 * QB) * 64 + lane;
+    __syncthreads();           // every wave is done reading the ring
+    if (grp == 1) {
+#pragma unroll
+      for (int qb = 0; qb < QB; ++qb) {
+        xch[(qb * 21 + 20) * 64] = m_run[qb];
+#pragma unroll
+        for (int db = 0; db < 5; ++db)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) xch[(qb * 21 + db * 4 + r) * 64] = o[db][qb][r];
+      }
+    }
+    __syncthreads();
+    if (grp == 1) {
+      prefetch_slice(p);
+      return;
+    }
+#pragma unroll
+    for (int qb = 0; qb < QB; ++qb) {
+      const float m_other = xch[(qb * 21 + 20) * 64];
+      const float m_new = fmaxf(m_run[qb], m_other);
+      const float a_mine = fast_exp2((m_run[qb] - m_new) * cs);
+      const float a_other = fast_exp2((m_other - m_new) * cs);
+#pragma unroll
+      for (int db = 0; db < 5; ++db)
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+          o[db][qb][r] = o[db][qb][r] * a_mine + xch[(qb * 21 + db * 4 + r) * 64] * a_other;
+    }
   }
 
   // O / (l + 1e-6) -> fp16, token-major [row][head*64 + d]
@@ -476,6 +532,17 @@ __global__ __launch_bounds__(kAttThreads, 2) void attention_grouped_kernel(AttAr
     }
   }
   prefetch_slice(p);
+}
+
+// The balanced order of a launch of `entries` workgroups as a list: one wave per entry.
+template <int BQ>
+__global__ __launch_bounds__(kAttThreads) void attention_worklist_kernel(AttArgs p, int4 *list,
+                                                                        unsigned entries) {
+  const unsigned e = blockIdx.x * (kAttThreads / 64) + (threadIdx.x >> 6);
+  if (e >= entries) return;
+  const AttWork w = att_work_balanced<BQ>(p, e);
+  if ((threadIdx.x & 63) == 0)
+    list[e] = w.exists ? int4{w.b, w.head | (w.qb << 16), w.seq_start, w.len} : int4{-1, 0, 0, 0};
 }
 
 // ---------------------------------------------------------------------------
@@ -720,46 +787,117 @@ extern "C" int bt_attention_short(const void *qkv_heads, void *attention_output,
   return launch_short<32>(a, s);
 }
 
+namespace bt {
+// Shape of a streaming-attention launch: 128-query tiles with a three-deep ring once there
+// is plenty of work (three workgroups per CU); else 64-query tiles with a two-deep ring: 32 KB
+// of LDS and ~100 registers let four workgroups share a CU (a build held to 84 registers fits
+// five and measures the same), which hides more of the per-tile dependency chain than the
+// third stage did (-0.1 to -2.8 % per forward from batch 1 x 256 to batch 16 x 384; with the
+// balanced work list also -0.8 to -1.9 % at batch 32 x 256 / 384 and 16 x 768, so the switch
+// sits at 1300 workgroups of 128 queries; batch 16 x 512 is within 0.3 % either way).
+struct GroupedPlan {
+  bool wide;        // 128-query tiles
+  unsigned grid;
+};
+static GroupedPlan plan_grouped(AttArgs &a, int batch_size, int seq_len, int head_num) {
+  const long long blocks128 = (long long)((seq_len + 127) / 128) * head_num * batch_size;
+  const int qb = option_attention_qb();
+  GroupedPlan plan;
+  plan.wide = qb == 2 || (qb < 0 && blocks128 >= 1300);
+  plan.grid = att_grid(a, plan.wide ? (seq_len + 127) / 128 : (seq_len + 63) / 64, true);
+  return plan;
+}
+AttListPlan att_worklist_plan(int B, int S, int heads) {
+  AttListPlan out{0, 64, 0};
+  if (B <= 0 || S <= 0 || heads <= 0) return out;
+  AttArgs a{};
+  a.B = B, a.S = S, a.heads = heads;
+  const GroupedPlan plan = plan_grouped(a, B, S, heads);
+  out.bq = plan.wide ? 128 : 64;
+  out.nqb = a.nqb;
+  out.entries = a.xcd_map == 2 ? plan.grid : 0;
+  return out;
+}
+}  // namespace bt
+
+extern "C" unsigned long long bt_attention_worklist_bytes(int batch_size, int seq_len,
+                                                          int head_num) {
+  return (unsigned long long)att_worklist_plan(batch_size, seq_len, head_num).entries *
+         sizeof(int4);
+}
+
+extern "C" int bt_attention_worklist(const int *batch_idx, const int *seq_order, int batch_size,
+                                     int seq_len, int head_num, int padded_rows, void *work_list,
+                                     void *stream) {
+  BT_REQUIRE(batch_idx && work_list, BT_ERR_INVALID_ARGUMENT,
+             "bt_attention_worklist: null pointer argument");
+  BT_REQUIRE(batch_size > 0 && seq_len > 0 && head_num > 0, BT_ERR_INVALID_ARGUMENT,
+             "bt_attention_worklist: sizes must be positive");
+  BT_REQUIRE(aligned16({work_list}), BT_ERR_INVALID_ARGUMENT,
+             "bt_attention_worklist: work_list must be 16-byte aligned");
+  AttArgs a{};
+  a.batch_idx = batch_idx, a.seq_order = seq_order;
+  a.B = batch_size, a.S = seq_len, a.heads = head_num, a.padded_rows = padded_rows;
+  const GroupedPlan plan = plan_grouped(a, batch_size, seq_len, head_num);
+  BT_REQUIRE(a.xcd_map == 2, BT_ERR_INVALID_ARGUMENT,
+             "bt_attention_worklist: launches of this shape take no work list "
+             "(bt_attention_worklist_bytes is 0)");
+  const unsigned blocks = (plan.grid + kAttThreads / 64 - 1) / (kAttThreads / 64);
+  if (plan.wide)
+    attention_worklist_kernel<128><<<blocks, kAttThreads, 0, as_stream(stream)>>>(
+        a, (int4 *)work_list, plan.grid);
+  else
+    attention_worklist_kernel<64><<<blocks, kAttThreads, 0, as_stream(stream)>>>(
+        a, (int4 *)work_list, plan.grid);
+  BT_CHECK_LAUNCH("attention_worklist_kernel");
+  return BT_OK;
+}
+
 extern "C" int bt_attention_grouped(const void *qkv_heads, void *attention_output,
                                     const int *batch_idx, const int *seq_order,
                                     const void *atten_mask, const void *attention_bias,
                                     int batch_size, int seq_len, int rows_cap, int head_num,
                                     int size_per_head, float scale, int padded_rows,
                                     const void *prefetch, unsigned long long prefetch_bytes,
-                                    const int *mask_prefix_slots, void *stream) {
+                                    const int *mask_prefix_slots, const void *work_list,
+                                    void *stream) {
   int rc = check_att_args("bt_attention_grouped", qkv_heads, attention_output, batch_idx,
                           atten_mask, padded_rows, batch_size, seq_len, rows_cap, head_num,
                           size_per_head);
   if (rc) return rc;
+  BT_REQUIRE(aligned16({work_list}), BT_ERR_INVALID_ARGUMENT,
+             "bt_attention_grouped: work_list must be 16-byte aligned");
   AttArgs a{(const half_t *)qkv_heads, (half_t *)attention_output, batch_idx, seq_order,
             (const half_t *)atten_mask, (const half_t *)attention_bias,
             nullptr, 0, batch_size, seq_len,
             rows_cap, head_num, scale * kLog2e, padded_rows};
   a.mask_ok = a.mask ? mask_prefix_slots : nullptr;
+  a.work_list = (const int4 *)work_list;   // read only when the launch uses the balanced order
   hipStream_t s = as_stream(stream);
-  // 128-query tiles with a three-deep ring once there is plenty of work (three workgroups
-  // per CU); else 64-query tiles with a two-deep ring: 32 KB of LDS and ~100 registers let
-  // four workgroups share a CU (a build held to 84 registers fits five and measures the same), which hides more of the per-tile dependency chain than the
-  // third stage did (-0.1 to -2.8 % per forward from batch 1 x 256 to batch 16 x 384; with
-  // the balanced work list also -0.8 to -1.9 % at batch 32 x 256 / 384 and 16 x 768, so the
-  // switch sits at 1300 workgroups of 128 queries; batch 16 x 512 is within 0.3 % either way)
-  const long long blocks128 = (long long)((seq_len + 127) / 128) * head_num * batch_size;
-  const int qb = option_attention_qb();
   const bool add = a.mask || a.bias;
-  if (qb == 2 || (qb < 0 && blocks128 >= 1300)) {
-    const unsigned grid = att_grid(a, (seq_len + 127) / 128, true);
-    set_prefetch(a, grid, prefetch, prefetch_bytes);
+  const GroupedPlan plan = plan_grouped(a, batch_size, seq_len, head_num);
+  const unsigned grid = plan.grid;
+  set_prefetch(a, grid, prefetch, prefetch_bytes);
+  if (plan.wide) {
     if (add)
       attention_grouped_kernel<2, true, 3><<<grid, kAttThreads, 0, s>>>(a);
     else
       attention_grouped_kernel<2, false, 3><<<grid, kAttThreads, 0, s>>>(a);
   } else {
-    const unsigned grid = att_grid(a, (seq_len + 63) / 64, true);
-    set_prefetch(a, grid, prefetch, prefetch_bytes);
-    if (add)
+    // eight waves over two key halves: pays for a few long sequences that leave most CUs
+    // with one workgroup or none (batch 1 x 1024: 9.9 -> 8.7 us); with several workgroups
+    // per CU the four-wave form is faster (batch 16 x 512: 16.3 against 19.6 us)
+    const int ks = option_attention_key_split();
+    if (ks == 1 || (ks < 0 && seq_len >= 512 && grid <= 256)) {
+      if (add)
+        attention_grouped_kernel<1, true, 2, 2><<<grid, 2 * kAttThreads, 0, s>>>(a);
+      else
+        attention_grouped_kernel<1, false, 2, 2><<<grid, 2 * kAttThreads, 0, s>>>(a);
+    } else if (add) {
       attention_grouped_kernel<1, true, 2><<<grid, kAttThreads, 0, s>>>(a);
-    else
+    } else {
       attention_grouped_kernel<1, false, 2><<<grid, kAttThreads, 0, s>>>(a);
+    }
   }
   BT_CHECK_LAUNCH("attention_grouped_kernel");
   return BT_OK;

@@ -75,6 +75,7 @@ int option_attention_qb();   // -1 = heuristic, 1 or 2 = query blocks per wave
 int option_f32_gemm_tile();  // -1 = heuristic, else index into the float GEMM's tile table
 int option_attention_xcd_map();     // workgroup order of the attention kernels: 0 plain, 1 XCD-aware, 2 balanced (default), 3 balanced always
 int option_prefetch();       // 1 = honour the prefetch hints of the attention entries (default), 0 = ignore
+int option_attention_key_split();  // streaming attention, 64-query tiles: -1 heuristic, 0 four waves, 1 eight waves over two key halves
 int option_prefetch_min_grid();   // attention launches of fewer workgroups skip the cache warm-up (default 512)
 
 inline hipStream_t as_stream(void *s) { return reinterpret_cast<hipStream_t>(s); }
@@ -180,11 +181,26 @@ struct AttWork {
   int b, head, qb, seq_start, len;
   bool exists;
 };
+// Shape of the balanced order of a streaming-attention launch over (B, S, heads): entries =
+// workgroups of the launch (0: such a launch does not use the balanced order), bq = queries
+// per tile (64 or 128), nqb = tile slots per sequence.  One function decides for the
+// attention launcher and for whoever builds the list ahead of it.
+struct AttListPlan {
+  unsigned entries;
+  int bq, nqb;
+};
+AttListPlan att_worklist_plan(int B, int S, int heads);
+// Arguments of att_work_balanced when the offsets come from somewhere else than a kernel's
+// own argument struct (the layer prologue builds the list from lengths it holds in LDS).
+struct AttListArgs {
+  int B, S, heads, nqb, padded_rows;
+  const int *batch_idx, *seq_order;
+};
 template <int BQ, typename Args>
-__device__ __forceinline__ AttWork att_work_balanced(const Args &p) {
+__device__ __forceinline__ AttWork att_work_balanced(const Args &p, unsigned int workgroup) {
   AttWork w{0, 0, 0, 0, 0, false};
   const int lane = threadIdx.x & 63;
-  const int x = blockIdx.x & 7, s = blockIdx.x >> 3;
+  const int x = workgroup & 7, s = workgroup >> 3;
   const int round = s >> 5, pos = s & 31;
   const int j = (round << 5) + ((round & 1) ? 31 - pos : pos);
   int carry = 0;

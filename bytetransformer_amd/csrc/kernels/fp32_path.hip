@@ -242,7 +242,7 @@ __global__ __launch_bounds__(64 * NW) void f32_attention_kernel(F32AttArgs<T> p)
   // Launches of more than two rounds of workgroups per CU take the balanced work list.
   int b, head, seq_start, len, qb_index;
   if (p.balanced) {
-    const AttWork w = att_work_balanced<BQ>(p);
+    const AttWork w = att_work_balanced<BQ>(p, blockIdx.x);
     if (!w.exists) return;
     b = w.b, head = w.head, seq_start = w.seq_start, len = w.len, qb_index = w.qb;
   } else {

@@ -31,6 +31,8 @@ static std::atomic<int> g_gemm_tile{-1};
 static std::atomic<int> g_attention_qb{-1};
 static std::atomic<int> g_prefetch{1};
 static std::atomic<int> g_prefetch_min_grid{512};
+static std::atomic<int> g_attention_key_split{-1};
+static std::atomic<int> g_prepack_check{2};
 static std::atomic<int> g_f32_gemm_tile{-1};
 static std::atomic<int> g_attention_short_limit{0};
 static std::atomic<int> g_attention_xcd_map{2};
@@ -40,6 +42,7 @@ int option_gemm_tile() { return g_gemm_tile.load(std::memory_order_relaxed); }
 int option_attention_qb() { return g_attention_qb.load(std::memory_order_relaxed); }
 int option_prefetch() { return g_prefetch.load(std::memory_order_relaxed); }
 int option_prefetch_min_grid() { return g_prefetch_min_grid.load(std::memory_order_relaxed); }
+int option_attention_key_split() { return g_attention_key_split.load(std::memory_order_relaxed); }
 
 // ---- offsets ----------------------------------------------------------------
 constexpr int kOffsetThreads = 1024;
@@ -161,9 +164,19 @@ struct PrologueWeights {
   int tiles_n[4];            // 64 x 64 tiles along n
   int tile_end[4];           // tiles up to and including matrix i
   int count;                 // 0 = no weights to check
+  int sample_mask;           // 0: every row of every tile is fingerprinted; else 4 rows of its 64
   // per hash block b: state[2b] = fingerprint its tiles' copies were made from,
   // state[2b + 1] = non-zero once that is recorded (zero: this launch records it)
   unsigned long long *state;
+};
+
+// The attention's balanced work list, built by blocks of their own beyond the others
+// (kListBlocks of them, each with its own copy of the lengths in LDS): one wave per entry.
+constexpr int kListBlocks = 48;
+struct PrologueList {
+  int4 *list;           // null: none
+  unsigned entries;
+  int bq, nqb, heads, padded_rows;
 };
 
 __device__ __forceinline__ unsigned int rotl32(unsigned int v, int s) {
@@ -213,7 +226,7 @@ template <typename T>
 __global__ __launch_bounds__(kPrologueThreads) void layer_prologue_kernel(
     const T *__restrict__ mask, int *__restrict__ batch_idx, int *__restrict__ word_idx,
     int *__restrict__ seq_order, int *__restrict__ slots, int B, int S, int offset_blocks,
-    PrologueWeights pw) {
+    PrologueWeights pw, PrologueList pl) {
   extern __shared__ __attribute__((aligned(16))) int smem[];
   __shared__ unsigned long long s_part[kPrologueWaves];
   __shared__ int s_heal;
@@ -221,10 +234,12 @@ __global__ __launch_bounds__(kPrologueThreads) void layer_prologue_kernel(
   const int lane = tid & 63;
   const int wave = tid >> 6;
 
-  // ---- offsets ----
-  if ((int)blockIdx.x < offset_blocks) {
+  // ---- offsets (and, in the list blocks, the attention's work list) ----
+  const bool list_block = pl.list && blockIdx.x >= gridDim.x - kListBlocks;
+  if ((int)blockIdx.x < offset_blocks || list_block) {
     int *s_len = smem;          // [B]
     int *s_off = smem + B;      // [B + 1]
+    int *s_order = smem + 2 * B + 1;   // [B] rank -> sequence, longest first
     for (int b = wave; b < B; b += kPrologueWaves) {
       const int count = wave_row_length(mask + (size_t)b * S * S, S, lane);
       if (lane == 0) s_len[b] = count;
@@ -241,19 +256,33 @@ __global__ __launch_bounds__(kPrologueThreads) void layer_prologue_kernel(
       }
       if (lane == 0) s_off[B] = carry;
     }
+    // sequences by descending length (ties by index): rank by counting
+    if (blockIdx.x == 0 || list_block)
+      for (int b = tid; b < B; b += kPrologueThreads) {
+        const int len = s_len[b];
+        int rank = 0;
+        for (int o = 0; o < B; ++o) {
+          const int lo = s_len[o];
+          rank += (lo > len) || (lo == len && o < b);
+        }
+        s_order[rank] = b;
+      }
     __syncthreads();
+    if (list_block) {
+      AttListArgs la{B, S, pl.heads, pl.nqb, pl.padded_rows, s_off, s_order};
+      const unsigned first = (blockIdx.x - (gridDim.x - kListBlocks)) * kPrologueWaves + wave;
+      for (unsigned e = first; e < pl.entries; e += kListBlocks * kPrologueWaves) {
+        const AttWork w = pl.bq == 128 ? att_work_balanced<128>(la, e) : att_work_balanced<64>(la, e);
+        if (lane == 0)
+          pl.list[e] = w.exists ? int4{w.b, w.head | (w.qb << 16), w.seq_start, w.len}
+                                : int4{-1, 0, 0, 0};
+      }
+      return;     // a list block has no other job
+    }
     if (blockIdx.x == 0) {
       for (int i = tid; i <= B; i += kPrologueThreads) batch_idx[i] = s_off[i];
       if (seq_order)
-        for (int b = tid; b < B; b += kPrologueThreads) {
-          const int len = s_len[b];
-          int rank = 0;
-          for (int o = 0; o < B; ++o) {
-            const int lo = s_len[o];
-            rank += (lo > len) || (lo == len && o < b);
-          }
-          seq_order[rank] = b;
-        }
+        for (int b = tid; b < B; b += kPrologueThreads) seq_order[b] = s_order[b];
     }
     for (int b = blockIdx.x; b < B; b += offset_blocks) {
       const int off = s_off[b], len = s_len[b];
@@ -268,7 +297,7 @@ __global__ __launch_bounds__(kPrologueThreads) void layer_prologue_kernel(
     const bool vec = S % kVec == 0 && (reinterpret_cast<uintptr_t>(mask) & 15) == 0;
     int bad = 0, len_of = -1, len = 0;
     for (long long r = (long long)blockIdx.x * kPrologueWaves + wave; r < rows;
-         r += (long long)gridDim.x * kPrologueWaves) {
+         r += (long long)kPrefixBlocks * kPrologueWaves) {
       const int b = (int)(r / S);
       if (b != len_of) {
         len = wave_row_length(mask + (size_t)b * S * S, S, lane);
@@ -324,7 +353,8 @@ __global__ __launch_bounds__(kPrologueThreads) void layer_prologue_kernel(
         for (int h = 0; h < 2; ++h) {
           const int k = k0 + r0 + 32 * h;
           v[i][h] = uint4_t{0u, 0u, 0u, 0u};
-          if (t < tile_hi && k < K && n < N) v[i][h] = *(const uint4_t *)(src + (size_t)k * N + n);
+          if (t < tile_hi && (!pw.sample_mask || (h == 0 && (r0 & 7) == 0)) && k < K && n < N)
+            v[i][h] = *(const uint4_t *)(src + (size_t)k * N + n);
         }
       }
 #pragma unroll
@@ -332,7 +362,7 @@ __global__ __launch_bounds__(kPrologueThreads) void layer_prologue_kernel(
         const int t = tb + i * kHealGroups + group;
 #pragma unroll
         for (int h = 0; h < 2; ++h)
-          if (t < tile_hi)
+          if (t < tile_hi && (!pw.sample_mask || (h == 0 && (r0 & 7) == 0)))
             sum += piece_hash(v[i][h], (unsigned int)(((t - tile_lo) << 9) + h * 256 + gt));
       }
     }
@@ -421,6 +451,14 @@ extern "C" int bt_set_option(const char *name, int value) {
     BT_REQUIRE(value == 0 || value == 1, BT_ERR_INVALID_ARGUMENT,
                "bt_set_option: prefetch=%d must be 0 or 1", value);
     g_prefetch.store(value);
+  } else if (!strcmp(name, "attention_key_split")) {
+    BT_REQUIRE(value >= -1 && value <= 1, BT_ERR_INVALID_ARGUMENT,
+               "bt_set_option: attention_key_split=%d must be -1, 0 or 1", value);
+    g_attention_key_split.store(value);
+  } else if (!strcmp(name, "prepack_check")) {
+    BT_REQUIRE(value >= 0 && value <= 2, BT_ERR_INVALID_ARGUMENT,
+               "bt_set_option: prepack_check=%d must be 0, 1 or 2", value);
+    g_prepack_check.store(value);
   } else if (!strcmp(name, "prefetch_min_grid")) {
     BT_REQUIRE(value >= 1 && value <= (1 << 20), BT_ERR_INVALID_ARGUMENT,
                "bt_set_option: prefetch_min_grid=%d outside [1, 2^20]", value);
@@ -442,6 +480,10 @@ extern "C" int bt_get_option(const char *name, int *value) {
     *value = g_prefetch.load();
   } else if (!strcmp(name, "prefetch_min_grid")) {
     *value = g_prefetch_min_grid.load();
+  } else if (!strcmp(name, "attention_key_split")) {
+    *value = g_attention_key_split.load();
+  } else if (!strcmp(name, "prepack_check")) {
+    *value = g_prepack_check.load();
   } else if (!strcmp(name, "f32_gemm_tile")) {
     *value = g_f32_gemm_tile.load();
   } else if (!strcmp(name, "attention_short_limit")) {
@@ -490,7 +532,8 @@ extern "C" int bt_build_offsets(const void *atten_mask, int mask_dtype, int batc
 
 extern "C" int bt_layer_prologue(const void *atten_mask, int mask_dtype, int batch_size,
                                  int seq_len, int *batch_idx, int *word_idx, int *seq_order,
-                                 int *mask_prefix_slots, int weight_count, const void *const *w,
+                                 int *mask_prefix_slots, void *attention_work_list, int head_num,
+                                 int padded_rows, int weight_count, const void *const *w,
                                  void *const *wt, const int *k, const int *n,
                                  unsigned long long *prepack_state, void *stream) {
   BT_REQUIRE(atten_mask && batch_idx && word_idx, BT_ERR_INVALID_ARGUMENT,
@@ -505,7 +548,12 @@ extern "C" int bt_layer_prologue(const void *atten_mask, int mask_dtype, int bat
              "bt_layer_prologue: weight_count=%d outside [0, 4]", weight_count);
   PrologueWeights pw;
   memset(&pw, 0, sizeof(pw));
+  // option "prepack_check": 2 = the weights are fingerprinted whole, 1 = four rows of every
+  // 64 x 64 tile, 0 = the copies are taken on trust (the caller's bookkeeping decides alone)
+  const int check = g_prepack_check.load(std::memory_order_relaxed);
+  if (check == 0) weight_count = 0;
   pw.count = weight_count;
+  pw.sample_mask = check == 1 ? 15 : 0;
   if (weight_count > 0) {
     BT_REQUIRE(w && wt && k && n && prepack_state, BT_ERR_INVALID_ARGUMENT,
                "bt_layer_prologue: weights to check need w, wt, k, n and prepack_state");
@@ -535,25 +583,44 @@ extern "C" int bt_layer_prologue(const void *atten_mask, int mask_dtype, int bat
     }
     pw.state = prepack_state;
   }
-  size_t smem = (2 * (size_t)batch_size + 1) * sizeof(int);
+  // the attention's balanced work list, when a launch of this shape uses one
+  PrologueList pl;
+  memset(&pl, 0, sizeof(pl));
+  if (attention_work_list) {
+    BT_REQUIRE(head_num > 0, BT_ERR_INVALID_ARGUMENT,
+               "bt_layer_prologue: attention_work_list needs head_num");
+    BT_REQUIRE(aligned16({attention_work_list}), BT_ERR_INVALID_ARGUMENT,
+               "bt_layer_prologue: attention_work_list must be 16-byte aligned");
+    const AttListPlan plan = att_worklist_plan(batch_size, seq_len, head_num);
+    if (plan.entries > 0) {
+      pl.list = (int4 *)attention_work_list;
+      pl.entries = plan.entries;
+      pl.bq = plan.bq;
+      pl.nqb = plan.nqb;
+      pl.heads = head_num;
+      pl.padded_rows = padded_rows;
+    }
+  }
+  size_t smem = (3 * (size_t)batch_size + 1) * sizeof(int);
   const size_t heal = (size_t)kHealGroups * 64 * kTransposePitch * sizeof(half_t);
   if (weight_count > 0 && smem < heal) smem = heal;
   BT_REQUIRE(smem <= 60 * 1024, BT_ERR_UNSUPPORTED,
-             "bt_layer_prologue: batch_size %d too large (limit 7679)", batch_size);
+             "bt_layer_prologue: batch_size %d too large (limit 5119)", batch_size);
   hipStream_t s = as_stream(stream);
   const int offset_blocks = batch_size < 64 ? batch_size : 64;
   // the verdict slots are an array of kPrefixBlocks entries, one per block; the
   // fingerprint blocks are the last kHashBlocks of the same grid
   static_assert(kHashFirst + kHashBlocks == kPrefixBlocks, "one grid for both jobs");
-  const int grid = (mask_prefix_slots || weight_count > 0) ? kPrefixBlocks : offset_blocks;
+  const int grid = ((mask_prefix_slots || weight_count > 0) ? kPrefixBlocks : offset_blocks) +
+                   (pl.list ? kListBlocks : 0);
   if (mask_dtype == BT_F16)
     layer_prologue_kernel<half_t><<<grid, kPrologueThreads, smem, s>>>(
         (const half_t *)atten_mask, batch_idx, word_idx, seq_order, mask_prefix_slots, batch_size,
-        seq_len, offset_blocks, pw);
+        seq_len, offset_blocks, pw, pl);
   else
     layer_prologue_kernel<float><<<grid, kPrologueThreads, smem, s>>>(
         (const float *)atten_mask, batch_idx, word_idx, seq_order, mask_prefix_slots, batch_size,
-        seq_len, offset_blocks, pw);
+        seq_len, offset_blocks, pw, pl);
   BT_CHECK_LAUNCH("layer_prologue_kernel");
   return BT_OK;
 }

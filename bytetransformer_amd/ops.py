@@ -78,11 +78,13 @@ def mask_is_prefix(mask, batch_idx):
     return bool(verdict.value)
 
 
-def layer_prologue(mask, want_slots=False, weights=None, packed=None, state=None, out=None):
+def layer_prologue(mask, want_slots=False, weights=None, packed=None, state=None, out=None,
+                   work_list=None, head_num=0, padded_rows=False):
     """bt_layer_prologue: offsets of `mask`, optionally the prefix-mask verdict slots and the
     check of pre-packed copies `packed` against `weights` (fingerprint record `state`,
     int64[PREPACK_STATE_WORDS], zero when the copies were made).  Returns (batch_idx, word_idx, seq_order, slots or None); `out` = such a
-    tuple to write into."""
+    tuple to write into.  work_list (int32[entries, 4], with head_num and padded_rows): also
+    filled with the attention's balanced order, as attention_worklist would."""
     B, S = mask.shape[0], mask.shape[1]
     dev = mask.device
     if out is not None:
@@ -104,7 +106,8 @@ def layer_prologue(mask, want_slots=False, weights=None, packed=None, state=None
         src = dst = ks = ns = None
     _check(kernel_lib().bt_layer_prologue(
         _ptr(mask), _dtype_code(mask), B, S, _ptr(batch_idx), _ptr(word_idx), _ptr(seq_order),
-        _ptr(slots), n, src, dst, ks, ns, _ptr(state) if n else None, _stream()))
+        _ptr(slots), _ptr(work_list), int(head_num), int(padded_rows), n, src, dst, ks, ns,
+        _ptr(state) if n else None, _stream()))
     return batch_idx, word_idx, seq_order, slots
 
 
@@ -194,10 +197,24 @@ def attention_short(qkv_heads, batch_idx, batch_size, seq_len, scale, padded_row
 
 def attention_grouped(qkv_heads, batch_idx, batch_size, seq_len, scale, padded_rows=False,
                       out=None, seq_order=None, mask=None, bias=None, prefetch=None,
-                      mask_prefix_slots=None):
+                      mask_prefix_slots=None, work_list=None):
     return _attention(kernel_lib().bt_attention_grouped, qkv_heads, batch_idx, batch_size,
                       seq_len, scale, padded_rows, out, seq_order, mask, bias, prefetch,
-                      extra=(_ptr(mask_prefix_slots),))
+                      extra=(_ptr(mask_prefix_slots), _ptr(work_list)))
+
+
+def attention_worklist(batch_idx, batch_size, seq_len, head_num, padded_rows=False, seq_order=None):
+    """The balanced workgroup order of attention_grouped for this shape and these offsets as
+    a list (int32[entries, 4]) to pass as work_list, or None when launches of this shape do
+    not use that order."""
+    lib = kernel_lib()
+    nbytes = lib.bt_attention_worklist_bytes(batch_size, seq_len, head_num)
+    if nbytes == 0:
+        return None
+    wl = torch.empty(nbytes // 16, 4, dtype=torch.int32, device=batch_idx.device)
+    _check(lib.bt_attention_worklist(_ptr(batch_idx), _ptr(seq_order), batch_size, seq_len,
+                                     head_num, int(padded_rows), _ptr(wl), _stream()))
+    return wl
 
 
 def mask_prefix_slots(mask, batch_idx, out=None):

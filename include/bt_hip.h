@@ -51,6 +51,15 @@ const char *bt_last_error_string(void);
  *                   waves | 2: 256x128, 8 + 4 waves | 3: 256x192, 8 + 4 waves | 4: 32x64, 2 + 2 waves
  *                   | 5: 128x128 with a two-deep ring (two workgroups per CU)
  *   "attention_qb"  -1 heuristic | 1 | 2: 16-query blocks per wave in the grouped kernel
+ *   "attention_key_split"  -1 heuristic | 0 | 1: the 64-query streaming attention with four waves,
+ *                   or with eight: two groups of four take alternate 64-key halves of every ring
+ *                   slot and are merged at the end
+ *   "prepack_check" 2 (default) | 1 | 0: how bt_layer_prologue checks reused weight copies:
+ *                   the weights are fingerprinted whole | four rows of every 64 x 64 tile
+ *                   (a write that touches every row is still seen, at a sixteenth of the
+ *                   reads) | not at all (the caller's bookkeeping is trusted).  The one option
+ *                   that can change results: below 2, a write to the weights that the caller's
+ *                   bookkeeping misses can leave stale copies in use
  *   "prefetch"      1 (default) | 0: honour / ignore the prefetch hint of the attention entries
  *   "prefetch_min_grid"  512 (default): attention launches of fewer workgroups ignore the hint
  *                   (there the warm-up costs more than it returns); 1 = every launch honours it
@@ -114,6 +123,9 @@ int bt_mask_is_prefix(const void *atten_mask, int mask_dtype, int batch_size, in
  *   - the offsets of bt_build_offsets (batch_idx, word_idx, seq_order; same rules);
  *   - mask_prefix_slots (nullable): the int[256] verdict of bt_mask_prefix_slots for the
  *     lengths of this very mask;
+ *   - attention_work_list (nullable; needs head_num and padded_rows): the list of
+ *     bt_attention_worklist for these offsets, when launches of this shape use one
+ *     (bt_attention_worklist_bytes > 0; else nothing is written);
  *   - weight_count in [0, 4] matrices w[i] ([k[i], n[i]] as the caller stores them) whose
  *     pre-packed copies wt[i] ([n[i], k[i]], bt_transpose_weights) are being reused from an
  *     earlier call: 192 workgroups each fingerprint their fixed share of the w[i] (64 bits
@@ -128,8 +140,9 @@ int bt_mask_is_prefix(const void *atten_mask, int mask_dtype, int batch_size, in
 #define BT_PREPACK_STATE_WORDS 384
 int bt_layer_prologue(const void *atten_mask, int mask_dtype, int batch_size, int seq_len,
                       int *batch_idx, int *word_idx, int *seq_order, int *mask_prefix_slots,
-                      int weight_count, const void *const *w, void *const *wt, const int *k,
-                      const int *n, unsigned long long *prepack_state, void *stream);
+                      void *attention_work_list, int head_num, int padded_rows, int weight_count,
+                      const void *const *w, void *const *wt, const int *k, const int *n,
+                      unsigned long long *prepack_state, void *stream);
 
 /*
  * Gather valid rows: to_tensor[t, :] = from_tensor[word_idx[t], :], t < M.
@@ -218,6 +231,7 @@ int bt_gemm_qkv_bias_split(const void *a, const int *a_row_index, const void *wt
  *   seq_order (nullable): a permutation of the sequence indices from
  *                     bt_build_offsets; workgroups are issued in that order so the
  *                     longest sequences start first.  Results do not depend on it.
+ *   work_list (bt_attention_grouped; nullable): see bt_attention_worklist below.
  *   mask_prefix_slots (bt_attention_grouped; nullable): the int[256] that
  *                     bt_mask_prefix_slots filled for this atten_mask earlier on the
  *                     stream.  When all are 1 the kernel ignores the tensor and stops at
@@ -246,7 +260,23 @@ int bt_attention_grouped(const void *qkv_heads, void *attention_output, const in
                          int batch_size, int seq_len, int rows_cap, int head_num,
                          int size_per_head, float scale, int padded_rows, const void *prefetch,
                          unsigned long long prefetch_bytes, const int *mask_prefix_slots,
-                         void *stream);
+                         const void *work_list, void *stream);
+
+/*
+ * The balanced workgroup order of bt_attention_grouped (option "attention_xcd_map" 2) as a
+ * list, so that a forward of many layers looks it up once instead of in every workgroup of
+ * every layer: entry w = what workgroup w works on.  No counterpart in the reference.
+ *   bt_attention_worklist_bytes  bytes of the list for a launch of this shape, 0 when such a
+ *                                launch does not use the balanced order (few workgroups, more
+ *                                than 128 sequences, another option value)
+ *   bt_attention_worklist        fills it from batch_idx / seq_order (asynchronous); pass the
+ *                                same shape, padded_rows and offsets to bt_attention_grouped
+ *                                with the list (work_list there is nullable and only a time
+ *                                saver: results do not depend on it)
+ */
+unsigned long long bt_attention_worklist_bytes(int batch_size, int seq_len, int head_num);
+int bt_attention_worklist(const int *batch_idx, const int *seq_order, int batch_size, int seq_len,
+                          int head_num, int padded_rows, void *work_list, void *stream);
 
 /*
  * out = LayerNorm((out + residual) + bias) * gamma + beta, in place on `out`,

@@ -51,6 +51,10 @@ struct AttentionInferParam {
   // this mask, already enqueued on the stream; else, with mask_prefix == -1, the layer runs
   // the check itself into `buf` whenever the mask tensor is in use.
   const int *mask_prefix_slots = nullptr;
+  // Extension: the balanced workgroup order of the streaming kernel as a list
+  // (bt_attention_worklist for this shape and these offsets), or null: the kernel then
+  // looks its work up itself.
+  const void *work_list = nullptr;
 };
 
 template <OperationType OpType>
@@ -92,9 +96,18 @@ class Attention {
 
   void initialize(AttentionParam<OpType> param) { param_ = param; }
 
-  // Both kernels keep logits and probabilities on chip: no attention scratch.
-  // 256 ints: the verdict slots of the device-side prefix-mask check (padded rows)
-  virtual unsigned long long cal_bufsize() const { return 256 * sizeof(int); }
+  // Both kernels keep logits and probabilities on chip.  Scratch: 256 ints, the verdict slots
+  // of the device-side prefix-mask check (padded rows), then the streaming kernel's work
+  // list (16 bytes per workgroup of its largest launch).
+  static unsigned long long work_list_offset() { return 256 * sizeof(int); }
+  unsigned long long work_list_capacity() const {
+    const unsigned long long pairs8 = ((unsigned long long)max_batch_size_ * head_num_ + 7) / 8;
+    const unsigned long long slots = (pairs8 * ((max_seq_len_ + 63) / 64) + 31) / 32 * 32 * 8;
+    return slots * 16;
+  }
+  virtual unsigned long long cal_bufsize() const {
+    return work_list_offset() + work_list_capacity();
+  }
 
   bool uses_short_kernel(int seq_len) const {
     return use_fused_attention_ && seq_len <= short_seq_limit();

@@ -89,7 +89,8 @@ class BertEncoder {
   // Scratch (elements of DataType_, T = max_batch*max_seq*hidden): [0,3T) qkv heads |
   // [3T,4T) attention out | [4T,5T) projection / LN1 | [5T,6T) packed hidden state |
   // [6T,(6+mult)T) FFN1 | word_idx int[B*S] | batch_idx int[B+1] | seq order int[B] |
-  // one layer's pre-packed weights (used only when the caller passes none) | split-k partial sums
+  // one layer's pre-packed weights (used only when the caller passes none) | split-k partial
+  // sums | the streaming attention's work list
   unsigned long long cal_bufsize() const {
     const unsigned long long rows = (unsigned long long)max_batch_size_ * max_seq_len_;
     const unsigned long long tensor = rows * head_num_ * size_per_head_;
@@ -98,6 +99,7 @@ class BertEncoder {
     n += align_up((rows * 2 + 2 * (unsigned long long)max_batch_size_ + 2 + 256) * sizeof(int), 256);
     n += align_up(layer_weight_elems() * sizeof(DataType_), 256);
     n += align_up(splitk_scratch_bytes(rows, (unsigned long long)head_num_ * size_per_head_), 256);
+    n += align_up(attention_layer_->work_list_capacity(), 256);   // the attention's work list
     return n;
   }
 

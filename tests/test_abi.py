@@ -52,8 +52,8 @@ def test_argument_validation_returns_codes_without_gpu():
     assert "needs valid_rows" in err()
     assert lib.bt_attention_short(p, p, p, None, None, None, 1, 1024, 1024, 12, 64, 0.125, 0, None, 0, None) == 2
     assert "exceeds 512" in err()
-    assert lib.bt_attention_grouped(p, p, p, None, None, None, 1, 16, 16, 12, 48, 0.125, 0, None, 0, None, None) == 2
-    assert lib.bt_attention_grouped(p, p, p, None, p, None, 1, 16, 16, 12, 64, 0.125, 0, None, 0, None, None) == 1
+    assert lib.bt_attention_grouped(p, p, p, None, None, None, 1, 16, 16, 12, 48, 0.125, 0, None, 0, None, None, None) == 2
+    assert lib.bt_attention_grouped(p, p, p, None, p, None, 1, 16, 16, 12, 64, 0.125, 0, None, 0, None, None, None) == 1
     assert "only applied on padded rows" in err()
     assert lib.bt_compress(p, p, p, p, 2, 4, 12, None) == 2 and "multiple of 8" in err()
     assert lib.bt_build_offsets(p, 7, 2, 4, p, p, None, None, None) == 1 and "dtype" in err()
@@ -84,9 +84,11 @@ def test_encoder_c_api_validation_and_bufsize():
     need = lib.bt_encoder_bufsize(ctypes.byref(cfg))
     T = 16 * 512 * 768
     # nine activation tensors + two index arrays + the pre-packed weights + the split-k area
+    # + the attention's work list (16 bytes per workgroup of its largest launch)
     splitk = 4 * 512 * 768 * 4
-    assert need >= 9 * T * 2 + 2 * 16 * 512 * 4 + 12 * 768 * 768 * 2 + splitk
-    assert need < 9 * T * 2 + 2 * 16 * 512 * 4 + 12 * 768 * 768 * 2 + splitk + 8192
+    work_list = (16 * 12 // 8) * (512 // 64) * 8 * 16
+    assert need >= 9 * T * 2 + 2 * 16 * 512 * 4 + 12 * 768 * 768 * 2 + splitk + work_list
+    assert need < 9 * T * 2 + 2 * 16 * 512 * 4 + 12 * 768 * 768 * 2 + splitk + work_list + 8192
     f32 = _lib.EncoderConfig(0, 16, 512, 12, 64, 4, 1, 1, 0, 1.0, 1e-6)   # float: twice the bytes
     need32 = lib.bt_encoder_bufsize(ctypes.byref(f32))
     assert 2 * need - 4 * 16 * 512 * 4 - splitk - 8192 < need32 < 2 * need

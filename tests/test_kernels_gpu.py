@@ -123,6 +123,26 @@ def test_layer_prologue_repacks_weights_that_changed_behind_the_copies(device):
     ws[0].data[0, 0], ws[0].data[5, 7] = b, a
     fp3 = run()
     assert ((fp3 != fp2).sum() == 1) == bool(a != b) and copies_match()
+    # option prepack_check: 1 = four rows of every tile are fingerprinted (a rewrite of a whole
+    # matrix is still seen), 0 = the copies are taken on trust (nothing is read or repaired)
+    ops.set_option("prepack_check", 1)
+    try:
+        sampled = torch.zeros(ops.PREPACK_STATE_WORDS, dtype=torch.int64, device=device)
+        ops.layer_prologue(mask, weights=ws, packed=packed, state=sampled)
+        ws[1].data.copy_(_dev(rs.standard_normal(shapes[1]).astype(np.float16), device))
+        ops.layer_prologue(mask, weights=ws, packed=packed, state=sampled)
+        torch.cuda.synchronize()
+        assert copies_match()
+        ops.set_option("prepack_check", 0)
+        before = [p.clone() for p in packed]
+        ws[1].data.copy_(_dev(rs.standard_normal(shapes[1]).astype(np.float16), device))
+        untouched = sampled.clone()
+        ops.layer_prologue(mask, weights=ws, packed=packed, state=sampled)
+        torch.cuda.synchronize()
+        assert torch.equal(sampled, untouched) and all(torch.equal(a, b) for a, b in zip(packed, before))
+    finally:
+        ops.set_option("prepack_check", 2)
+    assert ops.get_option("prepack_check") == 2
     # shapes that do not fill their last tiles
     odd = [_dev(rs.standard_normal(sh).astype(np.float16), device) for sh in [(72, 200), (200, 72)]]
     odd_packed = ops.transpose_weights(odd)
@@ -533,6 +553,16 @@ def test_mask_is_prefix(device, np_dtype):
 
 
 # ---- attention -----------------------------------------------------------------
+@pytest.fixture(autouse=True, params=[0, 1], ids=["four-waves", "key-split"])
+def attention_key_split(request):
+    """The streaming attention kernel's 64-query variant exists with four waves and with
+    eight (two key halves merged at the end); every test of this file runs under both
+    (the option does not touch the other kernels)."""
+    ops.set_option("attention_key_split", request.param)
+    yield request.param
+    ops.set_option("attention_key_split", -1)
+
+
 def _attention_case(rs, lens, S, heads, scale_q=1.0):
     B = len(lens)
     bi = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
@@ -696,6 +726,56 @@ def test_attention_arbitrary_mask_on_padded_rows(device, kind, S, att_order):
         exp = np.einsum("hqk,hkd->qhd", p, v).reshape(S, heads * 64)
         err = np.abs(g[b * S:(b + 1) * S] - exp)
         assert err.max() <= 4e-3, (b, err.max())
+
+
+@pytest.mark.parametrize("qb", [1, 2])
+@pytest.mark.parametrize("lens,S,heads,padded", [
+    ([512, 103, 257, 64, 65, 1, 0, 300], 512, 3, False),
+    (list(np.random.RandomState(7).randint(0, 97, size=70)), 96, 2, False),
+    ([200, 77, 130, 5], 200, 12, True),
+])
+def test_attention_work_list(device, lens, S, heads, padded, qb):
+    """The balanced order as a list: the stand-alone builder and the layer prologue write
+    the same entries, every live query tile appears exactly once, and the kernel gives the
+    same bits with the list as with its own look-up."""
+    lens = [int(v) for v in lens]
+    _say("attention work list", len(lens), S, heads, padded, qb)
+    rs = np.random.RandomState(S + heads)
+    B = len(lens)
+    mask = _dev(workload.make_mask(lens, S, np.float16), device)
+    ops.set_option("attention_qb", qb)
+    ops.set_option("attention_xcd_map", 3)          # the balanced order at any size
+    try:
+        order = torch.empty(B, dtype=torch.int32, device=device)
+        bi, wi, _ = ops.build_offsets(mask, seq_order=order)
+        wl = ops.attention_worklist(bi, B, S, heads, padded, seq_order=order)
+        assert wl is not None
+        wl2 = torch.full_like(wl, -7)
+        ops.layer_prologue(mask, work_list=wl2, head_num=heads, padded_rows=padded)
+        assert torch.equal(wl, wl2)
+        e = wl.cpu().numpy()
+        live = e[e[:, 0] >= 0]
+        bq = 64 * qb
+        want = set()
+        for b, n in enumerate(lens):
+            nq = S if padded else n
+            for h in range(heads):
+                for t in range((nq + bq - 1) // bq):
+                    want.add((b, h, t))
+        got = [(int(r[0]), int(r[1]) & 0xffff, int(r[1]) >> 16) for r in live]
+        assert len(got) == len(set(got)) and set(got) == want
+        starts = np.concatenate([[0], np.cumsum(lens)])
+        assert all(int(r[2]) == starts[int(r[0])] and int(r[3]) == lens[int(r[0])] for r in live)
+        qkv = _dev(rs.standard_normal((3, heads, B * S, 64)).astype(np.float16), device)
+        a = ops.attention_grouped(qkv, bi, B, S, 0.125, padded, seq_order=order)
+        b_ = ops.attention_grouped(qkv, bi, B, S, 0.125, padded, seq_order=order, work_list=wl)
+        rows = B * S if padded else int(starts[-1])
+        assert torch.equal(a[:rows], b_[:rows])
+    finally:
+        ops.set_option("attention_qb", -1)
+        ops.set_option("attention_xcd_map", 2)
+    # a shape whose launches keep the plain order takes no list
+    assert ops.attention_worklist(bi, 1, 64, 2, False) is None
 
 
 @pytest.mark.parametrize("qb", [1, 2])
