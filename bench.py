@@ -41,6 +41,9 @@ def parse():
     ap.add_argument("--workload", default="cfg2",
                     choices=["cfg1", "cfg2", "cfg3", "cfg4", "cfg4_fixed"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-cpp-driver", action="store_true",
+                    help="skip the child process that times the C++ API (profilers that "
+                         "initialise the GPU before this program starts forbid spawning it)")
     ap.add_argument("--kernel-iters", type=int, default=50)
     return ap.parse_args()
 
@@ -331,7 +334,7 @@ def main():
     wl = workload.make_workload(args.workload)
     cfg = wl.cfg
     # the torch-free C++ loop runs as a child process, before this process touches the GPU
-    cpp_layer_ms = cpp_api_layer_ms(wl)
+    cpp_layer_ms = None if args.no_cpp_driver else cpp_api_layer_ms(wl)
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     dev = torch.device("cuda:0")
     bt.load_th_op()

@@ -345,7 +345,280 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs &p) {
   }
 }
 
+// ---- persistent form ---------------------------------------------------------------
+// The launch has about one workgroup per CU and every workgroup takes SEVERAL tiles of its
+// XCD's range, running ONE software pipeline over all their k-steps: the loads of the next
+// tile's first stages are in flight while the current tile's accumulators are stored, and
+// a tile's stores drain to memory under the next tile's products instead of in one burst of
+// the whole launch at its end.  (One tile per workgroup leaves the matrix pipe idle from
+// the first store instruction on: with 228 tiles on 256 CUs the last 7 us of the 31 us of
+// the FFN1 product at batch 16 x 512 are 29.5 MB of stores.)  The grid no longer depends
+// on the row count: a workgroup counts its tiles from the device-side row count.
+template <int BM, int BN, int STAGES, int WM, int WN, int NP, int SCHED, int EPI>
+__device__ __forceinline__ void gemm_tiles_flat(const GemmArgs &p) {
+  constexpr int BK = kBK;
+  constexpr int NW = WM * WN;
+  constexpr int NL = NP > 0 ? NP : NW;
+  constexpr int WTM = BM / WM, WTN = BN / WN;
+  constexpr int TM = WTM / 32, TN = WTN / 32;
+  constexpr int ROWS = BM + BN;
+  constexpr int NI = ROWS / 8 / NL;
+  constexpr int NIA = BM / 8 / NL;
+  constexpr int STAGE_HALFS = ROWS * BK;
+  static_assert(BM % (8 * NL) == 0 && BN % (8 * NL) == 0, "tile rows must split evenly over the loading waves");
+  static_assert(STAGES >= 2 && STAGES <= 5 && (STAGES - 2) * NI < 64, "pipeline depth");
+  static_assert(EPI != kEpiPartial, "split-k launches keep one tile per workgroup");
+  constexpr int YOUNG = STAGES - 2;
+  constexpr int EP = WTN + 8;   // pitch (halfs) of the wave-private staging tile
+  static_assert((size_t)NW * 32 * EP <= (size_t)STAGE_HALFS, "staging fits one stage of the ring");
+
+  extern __shared__ __attribute__((aligned(1024))) half_t gemm_smem[];
+  half_t *smem = gemm_smem;
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int M = p.valid_rows ? min(*p.valid_rows, p.rows_cap) : p.rows_cap;
+
+  // XCD x owns the contiguous range [x * per, (x + 1) * per) of the live tiles; its
+  // workgroups take them round-robin
+  const int live = ((M + BM - 1) / BM) * p.tiles_n;
+  const int per = (live + 7) >> 3;
+  const int wgx = (int)(gridDim.x >> 3);                 // workgroups per XCD
+  const int lo = (int)(blockIdx.x & 7) * per;
+  const int hi = min(lo + per, live);
+  const int L0 = lo + (int)(blockIdx.x >> 3);
+  if (L0 >= hi) return;
+  const int n_my = (hi - L0 + wgx - 1) / wgx;
+  const int nk = p.K / BK;
+  const int total = n_my * nk;                           // k-steps of this workgroup
+
+  // ---- loading side: a cursor (tile, k-step) STAGES - 1 steps ahead of the products ----
+  const bool loader = NP == 0 || wave >= NW;
+  const int lw = NP == 0 ? wave : wave - NW;
+  const bool gather = p.a_row_index != nullptr;
+  rsrc_t rs_a = make_rsrc(p.a, 0), rs_w = make_rsrc(p.wt, 0);
+  constexpr bool kHasBias = EPI == kEpiBiasGelu || EPI == kEpiQkvSplit || EPI == kEpiBias;
+  // The bias of a tile's columns reaches the computing waves through LDS, fetched by the
+  // first loading wave together with the tile's first k-step: a global load in a computing
+  // wave after its stores would wait for every one of them to complete - the very wait this
+  // form of the kernel exists to avoid.  (Only the first tile's bias is loaded directly.)
+  half_t *s_bias = smem + STAGES * STAGE_HALFS;          // [BN]
+  const rsrc_t rs_bias = make_rsrc(kHasBias ? p.bias : p.wt, kHasBias ? (size_t)p.N * sizeof(half_t) : 0);
+  int voff[NI];
+  int idx_next[NIA];   // gathered A rows of the tile after the one being loaded
+  int ld_L = L0, ld_kt = 0, ld_left = loader ? total : 0;
+  auto fetch_indices = [&](int Lt) {
+    const int m0 = (Lt / p.tiles_n) * BM;
+#pragma unroll
+    for (int i = 0; i < NIA; ++i) {
+      const int r = (i * NL + lw) * 8 + (lane >> 3);
+      idx_next[i] = p.a_row_index[min(m0 + r, M - 1)];   // live rows only hold valid indices
+    }
+  };
+  auto load_setup = [&](int Lt, bool more, bool bias_to_lds) {
+    const int tm = Lt / p.tiles_n, tn = Lt - tm * p.tiles_n;
+    const int m0 = tm * BM, n0 = tn * BN;
+    if (kHasBias && bias_to_lds && lw == 0) {
+      // 4 bytes per lane and instruction: 128 columns each
+#pragma unroll
+      for (int i = 0; i < BN / 128; ++i)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(
+            rs_bias, (__attribute__((address_space(3))) void *)(s_bias + i * 128), 4,
+            (lane + i * 64) * 4, n0 * (int)sizeof(half_t), 0, 0);
+    }
+    rs_a = gather ? make_rsrc(p.a, (size_t)p.rows_cap * p.K * sizeof(half_t))
+                  : make_rsrc(p.a + (size_t)m0 * p.K, (size_t)(p.rows_cap - m0) * p.K * sizeof(half_t));
+    rs_w = make_rsrc(p.wt + (size_t)n0 * p.K, (size_t)(p.N - n0) * p.K * sizeof(half_t));
+    if (gather) {
+#pragma unroll
+      for (int i = 0; i < NIA; ++i) {
+        const int r = (i * NL + lw) * 8 + (lane >> 3);
+        const int kc = (lane & 7) ^ swz(r);
+        voff[i] = (idx_next[i] * p.K + kc * 8) * (int)sizeof(half_t);
+      }
+      if (more) fetch_indices(Lt + wgx);
+    }
+  };
+  if (loader) {
+#pragma unroll
+    for (int i = 0; i < NI; ++i) {
+      const int r = (i * NL + lw) * 8 + (lane >> 3);
+      const int kc = (lane & 7) ^ swz(r);
+      const int row = i < NIA ? r : r - BM;
+      voff[i] = (row * p.K + kc * 8) * (int)sizeof(half_t);
+    }
+    if (gather) fetch_indices(L0);
+    load_setup(L0, n_my > 1, false);
+  }
+  // issues the loads of the cursor's k-step into `stage` and moves the cursor on
+  auto issue_next = [&](int stage) {
+    if (ld_left == 0) return;
+    issue_stage_loads<NI, NIA>(rs_a, rs_w, voff, smem + stage * STAGE_HALFS + lw * 8 * BK,
+                               NL * 8 * BK, ld_kt * BK * (int)sizeof(half_t));
+    --ld_left;
+    if (++ld_kt == nk) {
+      ld_kt = 0;
+      ld_L += wgx;
+      if (ld_left) load_setup(ld_L, ld_left > nk, true);
+    }
+  };
+  if (loader) {
+#pragma unroll
+    for (int s = 0; s < STAGES - 1; ++s) issue_next(s);
+  }
+
+  if (NP > 0 && wave >= NW) {
+    // pure loader: one barrier per k-step in step with the computing waves, one more at
+    // the end of every tile (the computing waves then overlay the consumed stage)
+    int stage = 0, kt = 0;
+    for (int g = 0; g < total; ++g) {
+      wait_stages<NI, YOUNG>(total - 1 - g);
+      asm volatile("" ::: "memory");
+      __builtin_amdgcn_s_barrier();
+      asm volatile("" ::: "memory");
+      int ps = stage + STAGES - 1;
+      if (ps >= STAGES) ps -= STAGES;
+      issue_next(ps);
+      if (++kt == nk) {
+        kt = 0;
+        __builtin_amdgcn_s_barrier();
+      }
+      if (++stage == STAGES) stage = 0;
+    }
+    return;
+  }
+
+  // ---- computing side ---------------------------------------------------------------
+  const int wm = wave / WN, wn = wave % WN;
+  // The accumulators of a tile start from the bias of their columns (element 4q + e of
+  // block (i, j) is column n0 + wn*WTN + 32 i + 8 q + 4 (lane >> 5) + e).
+  float16_t acc[TN][TM];
+  auto init_acc = [&](const half_t *bias_of_tile, int n_limit) {
+#pragma unroll
+    for (int i = 0; i < TN; ++i) {
+      float16_t init;
+#pragma unroll
+      for (int v = 0; v < 16; ++v) init[v] = 0.f;
+      if (kHasBias) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const int n = min(wn * WTN + i * 32 + q * 8 + (lane >> 5) * 4, n_limit);
+          const half4_t b = *(const half4_t *)(bias_of_tile + n);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) init[4 * q + e] = (float)b[e];
+        }
+      }
+#pragma unroll
+      for (int j = 0; j < TM; ++j) acc[i][j] = init;
+    }
+  };
+  int cL = L0;
+  {
+    const int n0 = (cL % p.tiles_n) * BN;
+    init_acc(kHasBias ? p.bias + n0 : nullptr, p.N - 4 - n0);   // the first tile: straight from memory
+  }
+
+  const int fr_row = lane & 31, fr_kc = lane >> 5;
+  half8_t fw[2][TN], fa[2][TM];
+  auto load_frags = [&](int st, int ks, int b) {
+    const half_t *sA = smem + st * STAGE_HALFS;
+    const half_t *sB = sA + BM * BK;
+#pragma unroll
+    for (int i = 0; i < TN; ++i) {
+      const int r = wn * WTN + i * 32 + fr_row;
+      fw[b][i] = *(const half8_t *)(sB + r * BK + (((2 * ks + fr_kc) ^ swz(r + BM)) * 8));
+    }
+#pragma unroll
+    for (int j = 0; j < TM; ++j) {
+      const int r = wm * WTM + j * 32 + fr_row;
+      fa[b][j] = *(const half8_t *)(sA + r * BK + (((2 * ks + fr_kc) ^ swz(r)) * 8));
+    }
+  };
+  const int row_in = lane & 31, col_in = (lane >> 5) * 4;
+  constexpr int CPRW = WTN / 8;   // 16-byte chunks per staged row
+  constexpr int RPS = 64 / CPRW;  // rows per store instruction
+  const int sr = lane / CPRW, sc = (lane % CPRW) * 8;
+
+  int stage = 0, kt = 0;
+  for (int g = 0; g < total; ++g) {
+    if (NP == 0) wait_stages<NI, YOUNG>(total - 1 - g);
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_barrier();   // everyone's k-step g is in LDS; the stage of step g-1 is free again
+    asm volatile("" ::: "memory");
+    if (NP == 0) {
+      int ps = stage + STAGES - 1;
+      if (ps >= STAGES) ps -= STAGES;
+      issue_next(ps);
+    }
+    load_frags(stage, 0, 0);
+    if (SCHED == 0) __builtin_amdgcn_iglp_opt(0);
+    if (SCHED == 1) __builtin_amdgcn_iglp_opt(1);
+#pragma unroll
+    for (int ks = 0; ks < BK / 16; ++ks) {
+      if (ks + 1 < BK / 16) load_frags(stage, ks + 1, (ks + 1) & 1);
+#pragma unroll
+      for (int i = 0; i < TN; ++i)
+#pragma unroll
+        for (int j = 0; j < TM; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fw[ks & 1][i], fa[ks & 1][j],
+                                                            acc[i][j], 0, 0, 0);
+    }
+    if (++kt == nk) {
+      // ---- this tile is complete: store it, start the next from its bias ----
+      kt = 0;
+      const int tm = cL / p.tiles_n, tn = cL - tm * p.tiles_n;
+      const int m0 = tm * BM, n0 = tn * BN;
+      __builtin_amdgcn_s_barrier();   // all waves are done reading this stage: it becomes the staging area
+      half_t *st = smem + stage * STAGE_HALFS + wave * 32 * EP;
+#pragma unroll
+      for (int j = 0; j < TM; ++j) {
+#pragma unroll
+        for (int i = 0; i < TN; ++i) {
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            float v0 = acc[i][j][4 * q + 0], v1 = acc[i][j][4 * q + 1];
+            float v2 = acc[i][j][4 * q + 2], v3 = acc[i][j][4 * q + 3];
+            if (EPI == kEpiBiasGelu) {
+              v0 = gelu_tanh_f32(v0);
+              v1 = gelu_tanh_f32(v1);
+              v2 = gelu_tanh_f32(v2);
+              v3 = gelu_tanh_f32(v3);
+            }
+            *(half4_t *)(st + row_in * EP + i * 32 + q * 8 + col_in) =
+                half4_t{(half_t)v0, (half_t)v1, (half_t)v2, (half_t)v3};
+          }
+        }
+#pragma unroll
+        for (int r0 = 0; r0 < 32; r0 += RPS) {
+          const int r = r0 + sr;
+          if (sr >= RPS || r >= 32) continue;   // lanes left over when 64 % CPRW != 0
+          const int m = m0 + wm * WTM + j * 32 + r, n = n0 + wn * WTN + sc;
+          const uint4_t v = *(const uint4_t *)(st + r * EP + sc);
+          if (m < M && n < p.N) {
+            if (EPI == kEpiQkvSplit) {
+              // column n = which*H + g*64 + dd  ->  [which*heads + g][m][dd]
+              *(uint4_t *)(p.c + ((size_t)(n >> 6) * p.rows_cap + m) * 64 + (n & 63)) = v;
+            } else {
+              *(uint4_t *)(p.c + (size_t)m * p.N + n) = v;
+            }
+          }
+        }
+      }
+      cL += wgx;
+      if (g + 1 < total) init_acc(s_bias, BN - 4);   // from LDS, where the loading side has put it
+    }
+    if (++stage == STAGES) stage = 0;
+  }
+}
+
 #endif  // __HIP_DEVICE_COMPILE__
+
+template <int BM, int BN, int STAGES, int WM, int WN, int NP, int SCHED, int EPI>
+__global__ __launch_bounds__((WM * WN + NP) * 64) void gemm_flat_kernel(GemmArgs p) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  gemm_tiles_flat<BM, BN, STAGES, WM, WN, NP, SCHED, EPI>(p);
+#endif
+}
 
 template <int BM, int BN, int STAGES, int WM, int WN, int NP, int SCHED, int EPI>
 __global__ __launch_bounds__((WM * WN + NP) * 64) void gemm_kernel(GemmArgs p) {
@@ -394,6 +667,30 @@ static int launch_gemm_tile(GemmArgs p, hipStream_t s, int splits = 1) {
   return BT_OK;
 }
 
+static int cu_count();
+
+// Persistent launch: about one workgroup per CU (a multiple of 8, one share per XCD), each
+// looping over its tiles on the device.
+template <int BM, int BN, int STAGES, int WM, int WN, int NP, int SCHED, int EPI>
+static int launch_gemm_flat(GemmArgs p, hipStream_t s) {
+  constexpr size_t smem = (size_t)STAGES * (BM + BN) * kBK * sizeof(half_t) + BN * sizeof(half_t);
+  static_assert(smem <= 160 * 1024, "LDS budget");
+  static std::atomic<bool> configured[kMaxDevices];
+  const int rc = allow_dynamic_lds(gemm_flat_kernel<BM, BN, STAGES, WM, WN, NP, SCHED, EPI>, smem,
+                                   configured, "hipFuncSetAttribute(gemm_flat_kernel)");
+  if (rc != BT_OK) return rc;
+  const int tiles_m = (p.rows_cap + BM - 1) / BM;
+  p.tiles_n = (p.N + BN - 1) / BN;
+  const long long tiles = (long long)tiles_m * p.tiles_n;
+  const int per_cu = smem <= 80 * 1024 ? 2 : 1;          // workgroups that fit one CU's LDS
+  long long wgs = (long long)cu_count() * per_cu;
+  if (wgs > tiles) wgs = tiles;
+  const dim3 grid((unsigned)((wgs + 7) / 8 * 8));
+  gemm_flat_kernel<BM, BN, STAGES, WM, WN, NP, SCHED, EPI><<<grid, (WM * WN + NP) * 64, smem, s>>>(p);
+  BT_CHECK_LAUNCH("gemm_flat_kernel");
+  return BT_OK;
+}
+
 static int cu_count() {
   static const int cus = [] {
     int dev = 0, n = 0;
@@ -417,43 +714,24 @@ static long long estimated_rows(const GemmArgs &p) {
 
 #include "gemm_tuned.inc"
 
-// Measured time of tile t between two table rows (0 = not measured at one of them).
-static float tuned_time(const float *lo, const float *hi, float w, int t) {
-  if (t < 0 || t >= kTunedTiles || lo[t] <= 0.f || hi[t] <= 0.f) return 0.f;
-  return lo[t] + (hi[t] - lo[t]) * w;
-}
-
-// Tile with the smallest measured time for this weight shape at m rows, times
-// interpolated linearly between the measured row counts; -1 when the shape is not in
-// the table or m lies beyond it (the analytic model then decides).
-static int tuned_choice(long long m, int n, int k, int epi, const float **row_lo,
-                        const float **row_hi, float *weight) {
-  if (cu_count() != 256) return -1;     // the table was measured on a 256-CU part
+// Measured times of every tile for this weight shape at the first table row of at least m
+// rows, or nullptr when the shape is not in the table or m lies outside it (the analytic
+// model then decides alone).  The rows are kTunedStep apart, the height of the tallest
+// tile, so the row used has the same number of row tiles as m or one more: run time moves
+// in steps with the number of rounds of workgroups, and interpolating between two row
+// counts on either side of such a step would describe neither.
+static const float *tuned_times(long long m, int n, int k, int epi) {
+  if (cu_count() != 256) return nullptr;     // the table was measured on a 256-CU part
+  // below about a thousand rows a launch is latency bound and a loop of identical
+  // launches says little about the layer sequence
+  if (m < 1024 || m > kTunedRows[kTunedPoints - 1]) return nullptr;
   for (const TunedShape &ts : kTunedShapes) {
     if (ts.n != n || ts.k != k || ts.epi != epi) continue;
-    // below about a thousand rows a launch is latency bound and a loop of identical
-    // launches says little about the layer sequence: the model decides there
-    if (m > kTunedRows[kTunedPoints - 1] || m < 1024) return -1;
-    int hi = 0;
-    while (hi < kTunedPoints - 1 && kTunedRows[hi] < m) ++hi;
-    const int lo = hi > 0 && kTunedRows[hi] > m ? hi - 1 : hi;
-    const float w = hi == lo ? 0.f
-                             : (float)(m - kTunedRows[lo]) / (float)(kTunedRows[hi] - kTunedRows[lo]);
-    *row_lo = ts.us[lo];
-    *row_hi = ts.us[hi];
-    *weight = w;
-    int best = -1;
-    float best_us = 0.f;
-    for (int t = 0; t < kTunedTiles; ++t) {
-      const float us = tuned_time(ts.us[lo], ts.us[hi], w, t);
-      if (us > 0.f && (best < 0 || us < best_us)) {
-        best = t;
-        best_us = us;
-      }
-    }
-    return best;
+    int at = 0;
+    while (at < kTunedPoints - 1 && kTunedRows[at] < m) ++at;
+    return ts.us[at];
   }
-  return -1;
+  return nullptr;
 }
 
 template <int EPI>
@@ -470,6 +748,9 @@ static int launch_gemm(GemmArgs p, hipStream_t s) {
   //   5: 128x128, 2, 2x2, 4   tile 1 with a two-deep ring: 64 KB of LDS, so two workgroups
   //                           share a CU and one's fill and epilogue hide under the other's
   //                           k loop; pays when tile 1 would need several rounds
+  //   6, 7, 8                 tiles 2, 1 and 0 in the persistent form (gemm_tiles_flat); never
+  //                           the model's choice, only the measured table's, and there
+  //                           within a few per cent of the one-tile-per-workgroup form
   // The choice minimises rounds x (k-steps x time of one k-step + fill and epilogue) with
   // the per-tile constants below, for the estimated live rows; for the weight shapes of
   // BERT-base and BERT-large a table of measured times (gemm_tuned.inc) then overrides it
@@ -510,12 +791,13 @@ static int launch_gemm(GemmArgs p, hipStream_t s) {
     // the table overrides the model only for a clear win: the timings come from a loop
     // of identical launches, and differences of a few per cent do not carry over to the
     // layer sequence
-    const float *lo = nullptr, *hi = nullptr;
-    float w = 0.f;
-    const int tuned = tuned_choice(estimated_rows(p), p.N, p.K, EPI, &lo, &hi, &w);
-    if (tuned >= 0 && tuned != choice) {
-      const float t_model = tuned_time(lo, hi, w, choice), t_tuned = tuned_time(lo, hi, w, tuned);
-      if (t_model <= 0.f || t_tuned < 0.96f * t_model) choice = tuned;
+    if (const float *us = tuned_times(estimated_rows(p), p.N, p.K, EPI)) {
+      int tuned = -1;
+      for (int t = 0; t < kTunedTiles; ++t)
+        if (us[t] > 0.f && (tuned < 0 || us[t] < us[tuned])) tuned = t;
+      const float t_model = choice < kTunedTiles ? us[choice] : 0.f;
+      if (tuned >= 0 && tuned != choice && (t_model <= 0.f || us[tuned] < 0.96f * t_model))
+        choice = tuned;
     }
   }
   switch (choice) {
@@ -529,6 +811,12 @@ static int launch_gemm(GemmArgs p, hipStream_t s) {
       return launch_gemm_tile<32, 64, 4, 1, 2, 2, 0, EPI>(p, s);
     case 5:
       return launch_gemm_tile<128, 128, 2, 2, 2, 4, 0, EPI>(p, s);
+    case 6:
+      return launch_gemm_flat<256, 128, 3, 4, 2, 4, 1, EPI>(p, s);
+    case 7:
+      return launch_gemm_flat<128, 128, 3, 2, 2, 4, 0, EPI>(p, s);
+    case 8:
+      return launch_gemm_flat<256, 256, 2, 2, 4, 0, 1, EPI>(p, s);
     default:
       return launch_gemm_tile<128, 128, 3, 2, 2, 4, 0, EPI>(p, s);
   }

@@ -428,8 +428,8 @@ extern "C" const char *bt_last_error_string(void) { return g_last_error.c_str();
 extern "C" int bt_set_option(const char *name, int value) {
   BT_REQUIRE(name, BT_ERR_INVALID_ARGUMENT, "bt_set_option: null name");
   if (!strcmp(name, "gemm_tile")) {
-    BT_REQUIRE(value >= -1 && value <= 5, BT_ERR_INVALID_ARGUMENT,
-               "bt_set_option: gemm_tile=%d outside [-1, 5]", value);
+    BT_REQUIRE(value >= -1 && value <= 8, BT_ERR_INVALID_ARGUMENT,
+               "bt_set_option: gemm_tile=%d outside [-1, 8]", value);
     g_gemm_tile.store(value);
   } else if (!strcmp(name, "attention_qb")) {
     BT_REQUIRE(value == -1 || value == 1 || value == 2, BT_ERR_INVALID_ARGUMENT,

@@ -11,10 +11,10 @@ import json
 import os
 import sys
 
-M_GRID = (154, 300, 600, 900, 1200, 1500, 1800, 2400, 3000, 3600, 4809, 6000, 7400, 9830, 12288,
-          16384)
+M_STEP = 256                     # the tallest tile: run time steps with the count of row tiles
+M_GRID = tuple(range(M_STEP, 16384 + 1, M_STEP))
 HIDDEN = (768, 1024)
-TILES = (0, 1, 2, 3, 4, 5)
+TILES = (0, 1, 2, 3, 4, 5, 6, 7, 8)
 EPI_CODE = {"plain": 0, "gelu": 1, "qkv": 2}     # enum Epilogue of gemm.hip
 SMALL_TILE_MAX_ROWS = 3000      # the 32x64 tile is not worth timing beyond this
 INC = os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc", "kernels", "gemm_tuned.inc")
@@ -42,14 +42,17 @@ def _time_kernel(fn, iters):
 
 
 def measure(iters=32):
-    """Each weight shape with the epilogue the layer uses it with (QKV: bias + head split,
-    FFN1: bias + GELU, the two others plain), and with the weights cold: the launches of one
-    timing loop walk through enough copies of the weight matrix to exceed the memory-side
-    cache, as the layers of a model do."""
+    """Each weight shape as the layer launches it: with its epilogue (QKV: bias + head
+    split, FFN1: bias + GELU, the two others plain), with a row capacity of m / 0.6 (the
+    padded batch: launches are sized for batch x seq_len rows, of which m are live), the
+    QKV product gathering its rows from the padded input through a word_idx of 16 runs, and
+    with the weights cold: the launches of one timing loop walk through enough copies of
+    the weight matrix to exceed the memory-side cache, as the layers of a model do."""
     import torch
     from . import ops
     dev = torch.device("cuda:0")
-    rows_cap = max(M_GRID)
+    cap_of = lambda m: (int(m / 0.6) + 255) // 256 * 256
+    rows_cap = cap_of(max(M_GRID))
     out = []
     try:
         for h in HIDDEN:
@@ -65,18 +68,25 @@ def measure(iters=32):
                 for m in M_GRID:
                     vr = torch.tensor([m], dtype=torch.int32, device=dev)
                     turn = [0]
+                    cap = cap_of(m)
+                    # 16 sequences of cap / 16 padded rows each, m / 16 of them valid
+                    runs = [torch.arange(b * (cap // 16), b * (cap // 16) + (m * (b + 1)) // 16
+                                         - (m * b) // 16, dtype=torch.int32) for b in range(16)]
+                    word_idx = torch.cat(runs + [torch.zeros(cap - m, dtype=torch.int32)]).to(dev)
 
                     def call():
                         wt = wts[turn[0] % copies]
                         turn[0] += 1
                         if epi == "qkv":
-                            ops.gemm_qkv_bias_split(a, wt, bias, heads, valid_rows=vr, rows_hint=m,
-                                                    out=c.view(3, heads, rows_cap, 64))
+                            ops.gemm_qkv_bias_split(a[:cap], wt, bias, heads, valid_rows=vr,
+                                                    rows_hint=m, a_row_index=word_idx,
+                                                    out=c[:3 * cap * k].view(3, heads, cap, 64))
                         elif epi == "gelu":
-                            ops.gemm_bias_gelu(a, wt, bias, valid_rows=vr, rows_hint=m,
-                                               out=c.view(rows_cap, n))
+                            ops.gemm_bias_gelu(a[:cap], wt, bias, valid_rows=vr, rows_hint=m,
+                                               out=c[:cap * n].view(cap, n))
                         else:
-                            ops.gemm(a, wt, valid_rows=vr, rows_hint=m, out=c.view(rows_cap, n))
+                            ops.gemm(a[:cap], wt, valid_rows=vr, rows_hint=m,
+                                     out=c[:cap * n].view(cap, n))
 
                     ops.set_option("gemm_tile", 1)
                     _time_kernel(call, 8)      # warm the clocks for this shape
@@ -103,6 +113,7 @@ def write_inc(rows, path=INC):
              "// at kTunedRows live rows, per weight shape.  Do not edit by hand.",
              "constexpr int kTunedPoints = %d;" % len(M_GRID),
              "constexpr int kTunedTiles = %d;" % len(TILES),
+             "constexpr int kTunedStep = %d;" % M_STEP,
              "static const int kTunedRows[kTunedPoints] = {%s};" % ", ".join(map(str, M_GRID)),
              "struct TunedShape {", "  int n, k, epi;   // epi: the Epilogue the shape was timed with", "  float us[kTunedPoints][kTunedTiles];", "};",
              "static const TunedShape kTunedShapes[] = {"]

@@ -50,6 +50,8 @@ const char *bt_last_error_string(void);
  *   "gemm_tile"     -1 heuristic | 0: 256x256 tile, 8 waves | 1: 128x128, 4 computing + 4 loader
  *                   waves | 2: 256x128, 8 + 4 waves | 3: 256x192, 8 + 4 waves | 4: 32x64, 2 + 2 waves
  *                   | 5: 128x128 with a two-deep ring (two workgroups per CU)
+ *                   | 6, 7, 8: tiles 2, 1, 0 as persistent workgroups (about one per CU, each
+ *                   running one load pipeline over several tiles of its XCD's range)
  *   "attention_qb"  -1 heuristic | 1 | 2: 16-query blocks per wave in the grouped kernel
  *   "attention_key_split"  -1 heuristic | 0 | 1: the 64-query streaming attention with four waves,
  *                   or with eight: two groups of four take alternate 64-key halves of every ring

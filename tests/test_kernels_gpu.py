@@ -262,7 +262,7 @@ def _gemm_tol(exp, K, amax, wmax):
     return 2.0 ** -10 * np.abs(exp) + 4 * K * 2.0 ** -24 * amax * wmax + 1e-6
 
 
-@pytest.mark.parametrize("tile", [0, 1, 2, 3, 4, 5])
+@pytest.mark.parametrize("tile", [0, 1, 2, 3, 4, 5, 6, 7, 8])
 @pytest.mark.parametrize("rows,M,N,K", [(300, 300, 768, 768), (1000, 777, 2304, 768),
                                         (520, 513, 768, 3072), (64, 1, 136, 64),
                                         (257, 257, 3072, 768)])
@@ -304,7 +304,7 @@ def test_gemm_random_shapes_all_tiles_and_auto(device, seed):
     wt = ops.transpose_weight(_dev(w, device))
     vr = torch.tensor([M], dtype=torch.int32, device=device)
     try:
-        for tile in (-1, 0, 1, 2, 3, 4, 5):
+        for tile in (-1, 0, 1, 2, 3, 4, 5, 6, 7, 8):
             ops.set_option("gemm_tile", tile)
             out = torch.full((rows, N), 3.0, dtype=torch.float16, device=device)
             g = ops.gemm(_dev(a, device), wt, valid_rows=vr, out=out, rows_hint=M).cpu().numpy()
@@ -428,7 +428,7 @@ def test_splitk_gemm_and_layernorm(device, splits, restore, tight):
         assert np.abs(ref[:M].astype(np.float32) - g[:M].astype(np.float32)).max() <= 2e-2
 
 
-@pytest.mark.parametrize("tile", [0, 1, 2, 3, 4, 5])
+@pytest.mark.parametrize("tile", [0, 1, 2, 3, 4, 5, 6, 7, 8])
 def test_gemm_bias_gelu(device, tile):
     _say("gemm_bias_gelu", tile)
     rs = np.random.RandomState(tile)
@@ -450,7 +450,7 @@ def test_gemm_bias_gelu(device, tile):
     assert np.all(g[M:] == 0)
 
 
-@pytest.mark.parametrize("tile", [0, 1, 2, 3, 4, 5])
+@pytest.mark.parametrize("tile", [0, 1, 2, 3, 4, 5, 6, 7, 8])
 @pytest.mark.parametrize("heads", [12, 16])
 def test_gemm_qkv_bias_split(device, tile, heads):
     _say("gemm_qkv", tile, heads)
