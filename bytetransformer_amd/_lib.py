@@ -3,7 +3,7 @@ PyTorch operator library.  Nothing is built here: run
 `python -m bytetransformer_amd.build` first."""
 import ctypes
 import os
-from ctypes import POINTER, c_char_p, c_float, c_int, c_ulonglong, c_void_p
+from ctypes import POINTER, c_char_p, c_float, c_int, c_longlong, c_ulonglong, c_void_p
 
 _DIR = os.path.join(os.path.dirname(os.path.abspath(__file__)), "lib")
 
@@ -39,26 +39,29 @@ KERNEL_ABI = {
     "bt_mask_is_prefix": (c_int, [_P, c_int, c_int, c_int, _IP, _IP, POINTER(c_int), _P]),
     "bt_layer_prologue": (c_int, [_P, c_int, c_int, c_int, _IP, _IP, _IP, _IP, _P, c_int, c_int,
                                   c_int, POINTER(c_void_p), POINTER(c_void_p), POINTER(c_int),
-                                  POINTER(c_int), _P, _P]),
+                                  POINTER(c_int), _P]),
+    "bt_gemm_prepack_pays": (c_int, [c_longlong, c_int, c_int, c_int]),
     "bt_compress": (c_int, [_P, _P, _IP, _IP, c_int, c_int, c_int, _P]),
     "bt_transpose_weight": (c_int, [_P, _P, c_int, c_int, _P]),
     "bt_transpose_weights": (c_int, [c_int, POINTER(c_void_p), POINTER(c_void_p), POINTER(c_int),
                                      POINTER(c_int), _P]),
-    "bt_gemm": (c_int, [_P, _P, _P, _IP, c_int, c_int, c_int, c_int, _P]),
-    "bt_gemm_bias_gelu": (c_int, [_P, _P, _P, _P, _IP, c_int, c_int, c_int, c_int, _P]),
+    "bt_gemm": (c_int, [_P, _P, _P, _IP, c_int, c_int, c_int, c_int, c_int, _P]),
+    "bt_gemm_bias_gelu": (c_int, [_P, _P, _P, _P, _IP, c_int, c_int, c_int, c_int, c_int, _P]),
     "bt_gemm_qkv_bias_split": (c_int, [_P, _IP, _P, _P, _P, _IP, c_int, c_int, c_int, c_int,
-                                       _P]),
+                                       c_int, _P]),
     "bt_attention_short": (c_int, [_P, _P, _IP, _IP, _P, _P, c_int, c_int, c_int, c_int, c_int,
-                                   c_float, c_int, _P, c_ulonglong, _P]),
+                                   c_float, c_int, POINTER(c_void_p), POINTER(c_ulonglong), c_int,
+                                   _P]),
     "bt_attention_grouped": (c_int, [_P, _P, _IP, _IP, _P, _P, c_int, c_int, c_int, c_int, c_int,
-                                     c_float, c_int, _P, c_ulonglong, _IP, _P, _P]),
+                                     c_float, c_int, POINTER(c_void_p), POINTER(c_ulonglong),
+                                     c_int, _IP, _P, _P]),
     "bt_attention_worklist_bytes": (c_ulonglong, [c_int, c_int, c_int]),
     "bt_attention_worklist": (c_int, [_IP, _IP, c_int, c_int, c_int, c_int, _P, _P]),
     "bt_add_bias_residual_layernorm": (c_int, [_P, _P, _IP, _P, _P, _P, c_int, _IP, c_int, c_int,
                                                c_float, _P]),
     "bt_add_bias_residual_layernorm_restore": (c_int, [_P, _P, _P, _P, _P, c_int, _P, _IP, c_int,
                                                        c_int, c_int, c_float, _P]),
-    "bt_gemm_splitk": (c_int, [_P, _P, _P, c_int, _IP, c_int, c_int, c_int, _P]),
+    "bt_gemm_splitk": (c_int, [_P, _P, _P, c_int, _IP, c_int, c_int, c_int, c_int, _P]),
     "bt_splitk_layernorm": (c_int, [_P, c_int, _P, _IP, _P, _P, _P, c_int, _P, _IP, _IP, c_int,
                                     c_int, c_int, c_int, c_float, _P]),
     "bt_gemm_f32": (c_int, [_P, _IP, _P, _P, _P, c_int, _IP, c_int, c_int, c_int, c_int, _P]),

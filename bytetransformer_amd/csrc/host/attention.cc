@@ -55,7 +55,8 @@ void Attention<OpType>::infer(AttentionInferParam infer_param) {
                                       infer_param.et_param.batch_idx, infer_param.seq_order, mask,
                                       infer_param.attention_bias, infer_param.batch_size, infer_param.seq_len, rows_cap, head_num_, size_per_head_,
                                       scale, padded_rows, infer_param.prefetch,
-                                      infer_param.prefetch_bytes, infer_param.stream));
+                                      infer_param.prefetch_bytes, infer_param.prefetch_count,
+                                      infer_param.stream));
   else {
     // A mask tensor in use and no verdict from the caller: one pass over it on the device
     // (every launch of the layer, a few microseconds) lets the kernel drop it when it is the
@@ -72,7 +73,8 @@ void Attention<OpType>::infer(AttentionInferParam infer_param) {
         infer_param.qkv, infer_param.attention_output, infer_param.et_param.batch_idx,
         infer_param.seq_order, mask, infer_param.attention_bias, infer_param.batch_size,
         infer_param.seq_len, rows_cap, head_num_, size_per_head_, scale, padded_rows,
-        infer_param.prefetch, infer_param.prefetch_bytes, slots, infer_param.work_list,
+        infer_param.prefetch, infer_param.prefetch_bytes, infer_param.prefetch_count, slots,
+        infer_param.work_list,
         infer_param.stream));
   }
 }

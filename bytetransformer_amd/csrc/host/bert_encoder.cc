@@ -59,7 +59,6 @@ void BertEncoder<OpType>::infer(BertEncoderInferParam<DataType_> ip) {
   int *mask_slots = seq_order + max_batch_size_;       // int[256], padded path only
   off += align_up((max_rows * 2 + 2 * (unsigned long long)max_batch_size_ + 2 + 256) * sizeof(int),
                   256);
-  DataType_ *staging = (DataType_ *)(base + off);      // one layer's weights when none were passed
   off += align_up(layer_weight_elems() * sizeof(DataType_), 256);
   float *splitk_buf = (float *)(base + off);
   off += align_up(splitk_scratch_bytes(max_rows, (unsigned long long)hidden), 256);
@@ -79,7 +78,7 @@ void BertEncoder<OpType>::infer(BertEncoderInferParam<DataType_> ip) {
                                    et_param.batch_idx, et_param.word_idx, seq_order,
                                    check_mask ? mask_slots : nullptr, work_list, head_num_,
                                    is_remove_padding_ ? 0 : 1, 0, nullptr, nullptr, nullptr,
-                                   nullptr, nullptr, stream));
+                                   nullptr, stream));
   const int *valid_rows = is_remove_padding_ ? et_param.batch_idx + batch_size : nullptr;
   const int rows_hint = ip.valid_rows_hint;
   const int L = (int)layers_.size();
@@ -127,26 +126,21 @@ void BertEncoder<OpType>::infer(BertEncoderInferParam<DataType_> ip) {
       continue;
     }
 
-    const DataType_ *wt_qkv;
+    // pre-packed copies made when the encoder was created (its weights are private and
+    // immutable), else the [k, n] weights as they are stored
+    const int weight_kn = ip.prepacked ? 0 : 1;
+    const DataType_ *wt_qkv = w.attr_kernel_QKV, *wt_proj = w.attr_output_kernel,
+                    *wt_inter = w.inter_kernel, *wt_out = w.output_kernel;
     if (ip.prepacked) {
       wt_qkv = (const DataType_ *)ip.prepacked + (size_t)l * layer_weight_elems();
-    } else {
-      DataType_ *d = staging;
-      const void *src[4] = {w.attr_kernel_QKV, w.attr_output_kernel, w.inter_kernel, w.output_kernel};
-      void *dst[4] = {d, d + (size_t)3 * hidden * hidden, d + (size_t)4 * hidden * hidden,
-                      d + (size_t)4 * hidden * hidden + (size_t)hidden * inter};
-      const int ks[4] = {hidden, hidden, hidden, inter};
-      const int ns[4] = {3 * hidden, hidden, inter, hidden};
-      check_bt_error(bt_transpose_weights(4, src, dst, ks, ns, stream));
-      wt_qkv = staging;
+      wt_proj = wt_qkv + (size_t)3 * hidden * hidden;
+      wt_inter = wt_proj + (size_t)hidden * hidden;
+      wt_out = wt_inter + (size_t)hidden * inter;
     }
-    const DataType_ *wt_proj = wt_qkv + (size_t)3 * hidden * hidden;
-    const DataType_ *wt_inter = wt_proj + (size_t)hidden * hidden;
-    const DataType_ *wt_out = wt_inter + (size_t)hidden * inter;
 
     check_bt_error(bt_gemm_qkv_bias_split(x, gather, wt_qkv, w.attention_param.attr_bias_QKV,
                                           qkv_buf, valid_rows, rows, rows_hint, head_num_,
-                                          size_per_head_, stream));
+                                          size_per_head_, weight_kn, stream));
 
     struct AttentionInferParam<DataType_> att {
       qkv_buf, ip.atten_mask, attr_out_buf, nullptr, batch_size, seq_len, nullptr, stream, et_param
@@ -158,19 +152,36 @@ void BertEncoder<OpType>::infer(BertEncoderInferParam<DataType_> ip) {
     // warm the memory-side cache with what follows in memory order: the rest of this
     // layer's weights and, when all layers are pre-packed back to back, the next
     // layer's QKV matrix
-    att.prefetch = wt_proj;
-    att.prefetch_bytes = ((size_t)hidden * hidden + 2 * (size_t)hidden * inter) * sizeof(DataType_);
-    if (ip.prepacked && l + 1 < L) att.prefetch_bytes += (size_t)3 * hidden * hidden * sizeof(DataType_);
+    if (ip.prepacked) {
+      att.prefetch[0] = wt_proj;
+      att.prefetch_bytes[0] = ((size_t)hidden * hidden + 2 * (size_t)hidden * inter) * sizeof(DataType_);
+      if (l + 1 < L) att.prefetch_bytes[0] += (size_t)3 * hidden * hidden * sizeof(DataType_);
+      att.prefetch_count = 1;
+    } else {
+      const void *next[3] = {wt_proj, wt_inter, wt_out};
+      const size_t elems[3] = {(size_t)hidden * hidden, (size_t)hidden * inter, (size_t)hidden * inter};
+      for (int i = 0; i < 3; ++i) {
+        att.prefetch[i] = next[i];
+        att.prefetch_bytes[i] = elems[i] * sizeof(DataType_);
+      }
+      att.prefetch_count = 3;
+      if (l + 1 < L) {
+        att.prefetch[3] = layers_[l + 1].attr_kernel_QKV;
+        att.prefetch_bytes[3] = (size_t)3 * hidden * hidden * sizeof(DataType_);
+        att.prefetch_count = 4;
+      }
+    }
     attention_layer_->infer(att);
 
     check_bt_error(bt_gemm(attr_out_buf, wt_proj, attr_matmul_buf, valid_rows, rows, rows_hint,
-                           hidden, hidden, stream));
+                           hidden, hidden, weight_kn, stream));
     check_bt_error(bt_add_bias_residual_layernorm(
         attr_matmul_buf, x, gather, w.attr_output_bias, w.attr_output_layernorm_gamma,
         w.attr_output_layernorm_beta, use_fp32_ ? 1 : 0, valid_rows, rows, hidden, layernorm_eps,
         stream));
     check_bt_error(bt_gemm_bias_gelu(attr_matmul_buf, wt_inter, w.inter_bias, inter_matmul_buf,
-                                     valid_rows, rows, rows_hint, inter, hidden, stream));
+                                     valid_rows, rows, rows_hint, inter, hidden, weight_kn,
+                                     stream));
 
     // few rows, long k: FFN2 as split-k partial sums that the last LayerNorm folds in
     const long long rows_expected =
@@ -179,7 +190,7 @@ void BertEncoder<OpType>::infer(BertEncoderInferParam<DataType_> ip) {
     if (splits > 1) {
       const bool restore = last && is_remove_padding_;
       check_bt_error(bt_gemm_splitk(inter_matmul_buf, wt_out, splitk_buf, splits, valid_rows, rows,
-                                    hidden, inter, stream));
+                                    hidden, inter, weight_kn, stream));
       check_bt_error(bt_splitk_layernorm(
           splitk_buf, splits, attr_matmul_buf, nullptr, w.output_bias, w.output_layernorm_gamma,
           w.output_layernorm_beta, use_fp32_ ? 1 : 0,
@@ -189,7 +200,7 @@ void BertEncoder<OpType>::infer(BertEncoderInferParam<DataType_> ip) {
       continue;
     }
     check_bt_error(bt_gemm(inter_matmul_buf, wt_out, ffn2_out, valid_rows, rows, rows_hint, hidden,
-                           inter, stream));
+                           inter, weight_kn, stream));
     if (last && is_remove_padding_)
       check_bt_error(bt_add_bias_residual_layernorm_restore(
           ffn2_out, attr_matmul_buf, w.output_bias, w.output_layernorm_gamma,

@@ -51,25 +51,52 @@ void BertTransformer<OpType>::bert_infer(BertTransformerInferParam infer_param) 
   et_param.valid_word_num = rows;
   int *seq_order = et_param.batch_idx + max_batch_size_ + 1;   // int[max_batch_size]
   off += align_up((max_rows * 2 + 2 * (unsigned long long)max_batch_size_ + 2) * sizeof(int), 256);
-  DataType_ *wt_qkv = (DataType_ *)(base + off);
-  DataType_ *wt_proj = wt_qkv + (size_t)3 * hidden * hidden;
-  DataType_ *wt_inter = wt_proj + (size_t)hidden * hidden;
-  DataType_ *wt_out = wt_inter + (size_t)hidden * inter;
+  // The four products read the [k, n] weights as the caller stores them, exactly as the
+  // reference hands them to cuBLAS (gemm.cu:27-39): nothing is kept between calls and
+  // nothing can go stale.  Where the measured tile table says that a product of this size
+  // runs faster on a k-contiguous copy even after paying for the copy, the prologue launch
+  // makes that copy in the scratch, afresh in every call.  A caller that owns
+  // k-contiguous copies of immutable weights (prepacked_kernels) passes those instead.
+  const bool have_prepack = OpType == OperationType::HALF && param_.prepacked_kernels[0] &&
+                            param_.prepacked_kernels[1] && param_.prepacked_kernels[2] &&
+                            param_.prepacked_kernels[3];
+  const DataType_ *w_use[4] = {param_.attr_kernel_QKV, param_.attr_output_kernel,
+                               param_.inter_kernel, param_.output_kernel};
+  int w_kn[4] = {1, 1, 1, 1};
+  const int w_k[4] = {hidden, hidden, hidden, inter};
+  const int w_n[4] = {3 * hidden, hidden, inter, hidden};
+  const void *pack_src[4];
+  void *pack_dst[4];
+  int pack_k[4], pack_n[4], pack_count = 0;
+  if (have_prepack) {
+    for (int i = 0; i < 4; ++i) {
+      w_use[i] = param_.prepacked_kernels[i];
+      w_kn[i] = 0;
+    }
+  } else if (OpType == OperationType::HALF) {
+    const long long live = infer_param.valid_rows_hint > 0 ? infer_param.valid_rows_hint
+                           : is_remove_padding_            ? (rows * 3LL + 4) / 5
+                                                           : rows;
+    const int epilogue[4] = {size_per_head_ == 64 ? BT_EPILOGUE_QKV_SPLIT : -1,
+                             BT_EPILOGUE_PLAIN, BT_EPILOGUE_BIAS_GELU, BT_EPILOGUE_PLAIN};
+    DataType_ *slot = (DataType_ *)(base + off);
+    for (int i = 0; i < 4; ++i) {
+      if (epilogue[i] >= 0 && bt_gemm_prepack_pays(live, w_n[i], w_k[i], epilogue[i])) {
+        pack_src[pack_count] = w_use[i];
+        pack_dst[pack_count] = slot;
+        pack_k[pack_count] = w_k[i];
+        pack_n[pack_count] = w_n[i];
+        ++pack_count;
+        w_use[i] = slot;
+        w_kn[i] = 0;
+      }
+      slot += (size_t)w_k[i] * w_n[i];
+    }
+  }
   off += align_up((4 + 2 * (unsigned long long)param_.intermediate_size) * hidden * hidden *
                       sizeof(DataType_),
                   256);
   float *splitk_buf = (float *)(base + off);
-
-  // k-contiguous weight copies handed in by the caller (fp16 only), with or without the
-  // fingerprint record that lets the prologue check them against the weights
-  const bool have_prepack = OpType == OperationType::HALF && param_.prepacked_kernels[0] &&
-                            param_.prepacked_kernels[1] && param_.prepacked_kernels[2] &&
-                            param_.prepacked_kernels[3];
-  const bool check_prepack = have_prepack && param_.prepack_state;
-  const void *w_src[4] = {param_.attr_kernel_QKV, param_.attr_output_kernel, param_.inter_kernel,
-                          param_.output_kernel};
-  const int w_k[4] = {hidden, hidden, hidden, inter};
-  const int w_n[4] = {3 * hidden, hidden, inter, hidden};
 
   // Padded rows, fp16 streaming attention: the mask tensor is applied unless one pass over
   // it finds the plain prefix mask of its lengths; the prologue leaves that verdict in the
@@ -90,22 +117,15 @@ void BertTransformer<OpType>::bert_infer(BertTransformerInferParam infer_param) 
     work_list = base + inner_buf_size_ + Attention<OpType>::work_list_offset();
 
   // One launch ahead of the layer: lengths and offsets from the mask (needed on both
-  // paths: keys past len_b are excluded), the prefix-mask verdict, the check of reused
-  // weight copies.  Rebuilt on every call, as the reference does
-  // (bert_transformer.cu:62-66), unless the caller vouches for offsets of its own.
+  // paths: keys past len_b are excluded), the prefix-mask verdict, the weight copies.
+  // Rebuilt on every call, as the reference does (bert_transformer.cu:62-66), unless the
+  // caller vouches for offsets of its own.
   int rows_hint = infer_param.valid_rows_hint > 0 ? infer_param.valid_rows_hint : 0;
-  {
-    void *w_dst[4] = {const_cast<DataType_ *>(param_.prepacked_kernels[0]),
-                      const_cast<DataType_ *>(param_.prepacked_kernels[1]),
-                      const_cast<DataType_ *>(param_.prepacked_kernels[2]),
-                      const_cast<DataType_ *>(param_.prepacked_kernels[3])};
-    if (!have_offsets || mask_slots || check_prepack)
-      check_bt_error(bt_layer_prologue(atten_mask, Traits_::dtype, batch_size, seq_len,
-                                       et_param.batch_idx, et_param.word_idx, seq_order,
-                                       mask_slots, work_list, head_num_, is_remove_padding_ ? 0 : 1,
-                                       check_prepack ? 4 : 0, w_src, w_dst, w_k, w_n,
-                                       check_prepack ? param_.prepack_state : nullptr, stream));
-  }
+  if (!have_offsets || mask_slots || pack_count > 0)
+    check_bt_error(bt_layer_prologue(atten_mask, Traits_::dtype, batch_size, seq_len,
+                                     et_param.batch_idx, et_param.word_idx, seq_order,
+                                     mask_slots, work_list, head_num_, is_remove_padding_ ? 0 : 1,
+                                     pack_count, pack_src, pack_dst, pack_k, pack_n, stream));
   if (have_offsets) {
     et_param = *infer_param.offsets;
     rows_hint = et_param.valid_word_num;
@@ -173,21 +193,12 @@ void BertTransformer<OpType>::bert_infer(BertTransformerInferParam infer_param) 
     return;
   }
 
-  // k-contiguous weight pre-pack: all four matrices in one launch, unless the
-  // caller handed in copies it already made
-  if (have_prepack) {
-    wt_qkv = const_cast<DataType_ *>(param_.prepacked_kernels[0]);
-    wt_proj = const_cast<DataType_ *>(param_.prepacked_kernels[1]);
-    wt_inter = const_cast<DataType_ *>(param_.prepacked_kernels[2]);
-    wt_out = const_cast<DataType_ *>(param_.prepacked_kernels[3]);
-  } else {
-    void *dst[4] = {wt_qkv, wt_proj, wt_inter, wt_out};
-    check_bt_error(bt_transpose_weights(4, w_src, dst, w_k, w_n, stream));
-  }
+  const DataType_ *wt_qkv = w_use[0], *wt_proj = w_use[1], *wt_inter = w_use[2], *wt_out = w_use[3];
 
   check_bt_error(bt_gemm_qkv_bias_split(from_tensor, gather, wt_qkv,
                                         param_.attention_param.attr_bias_QKV, qkv_buf, valid_rows,
-                                        rows, rows_hint, head_num_, size_per_head_, stream));
+                                        rows, rows_hint, head_num_, size_per_head_, w_kn[0],
+                                        stream));
 
   struct AttentionInferParam<DataType_> attention_infer_param {
     qkv_buf, atten_mask, attr_out_buf, base + inner_buf_size_, batch_size, seq_len,
@@ -198,18 +209,21 @@ void BertTransformer<OpType>::bert_infer(BertTransformerInferParam infer_param) 
   attention_infer_param.mask_prefix = have_offsets ? infer_param.mask_prefix : -1;
   attention_infer_param.mask_prefix_slots = mask_slots;
   attention_infer_param.work_list = work_list;
-  // the three weight matrices the rest of the layer reads, when they lie back to back:
-  // the attention kernel pulls them into the memory-side cache while it runs
-  if (wt_inter == wt_proj + (size_t)hidden * hidden && wt_out == wt_inter + (size_t)hidden * inter) {
-    attention_infer_param.prefetch = wt_proj;
-    attention_infer_param.prefetch_bytes =
-        ((size_t)hidden * hidden + 2 * (size_t)hidden * inter) * sizeof(DataType_);
+  // the three weight matrices the rest of the layer reads (as stored, or the copies of
+  // this call): the attention kernel pulls them into the memory-side cache while it runs
+  {
+    const size_t elems[3] = {(size_t)hidden * hidden, (size_t)hidden * inter, (size_t)hidden * inter};
+    for (int i = 0; i < 3; ++i) {
+      attention_infer_param.prefetch[i] = w_use[i + 1];
+      attention_infer_param.prefetch_bytes[i] = elems[i] * sizeof(DataType_);
+    }
+    attention_infer_param.prefetch_count = 3;
   }
   attention_layer_->infer(attention_infer_param);
 
   check_bt_error(
       bt_gemm(attr_out_buf, wt_proj, attr_matmul_buf, valid_rows, packed_cap, rows_hint, hidden,
-              hidden, stream));
+              hidden, w_kn[1], stream));
 
   check_bt_error(bt_add_bias_residual_layernorm(
       attr_matmul_buf, from_tensor, gather, param_.attr_output_bias, param_.attr_output_layernorm_gamma,
@@ -217,7 +231,8 @@ void BertTransformer<OpType>::bert_infer(BertTransformerInferParam infer_param) 
       layernorm_eps, stream));
 
   check_bt_error(bt_gemm_bias_gelu(attr_matmul_buf, wt_inter, param_.inter_bias, inter_matmul_buf,
-                                   valid_rows, packed_cap, rows_hint, inter, hidden, stream));
+                                   valid_rows, packed_cap, rows_hint, inter, hidden, w_kn[2],
+                                   stream));
 
   // few rows, long k: FFN2 as split-k partial sums that the last LayerNorm folds in
   const long long rows_expected =
@@ -225,7 +240,7 @@ void BertTransformer<OpType>::bert_infer(BertTransformerInferParam infer_param) 
   const int splits = splitk_splits(packed_cap, rows_expected, inter);
   if (splits > 1) {
     check_bt_error(bt_gemm_splitk(inter_matmul_buf, wt_out, splitk_buf, splits, valid_rows,
-                                  packed_cap, hidden, inter, stream));
+                                  packed_cap, hidden, inter, w_kn[3], stream));
     check_bt_error(bt_splitk_layernorm(
         splitk_buf, splits, attr_matmul_buf, nullptr, param_.output_bias,
         param_.output_layernorm_gamma, param_.output_layernorm_beta, use_fp32_ ? 1 : 0,
@@ -237,7 +252,7 @@ void BertTransformer<OpType>::bert_infer(BertTransformerInferParam infer_param) 
 
   check_bt_error(
       bt_gemm(inter_matmul_buf, wt_out, transformer_out, valid_rows, packed_cap, rows_hint, hidden,
-              inter, stream));
+              inter, w_kn[3], stream));
 
   if (is_remove_padding_)
     check_bt_error(bt_add_bias_residual_layernorm_restore(

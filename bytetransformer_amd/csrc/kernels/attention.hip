@@ -36,8 +36,9 @@ constexpr int kHeadDim = 64;
 constexpr float kNegBig = -1.0e30f;
 constexpr float kLog2e = 1.4426950408889634f;
 
-typedef __fp16 fp16x4_t __attribute__((ext_vector_type(4)));
 typedef float float2_t __attribute__((ext_vector_type(2)));
+
+constexpr int kPrefetchRanges = 4;
 
 struct AttArgs {
   const half_t *qkv;   // [3][heads][rows_cap][64]
@@ -47,8 +48,11 @@ struct AttArgs {
   const half_t *mask;     // optional [B,S,S] 0/1 mask, padded rows only: every key of the
                           // sequence's S rows takes part, shifted by (mask-1)*10000
   const half_t *bias;     // optional [heads,S,S] term added to the scaled logits
-  const char *prefetch;   // optional: memory the NEXT kernels will read (weights); touched
-  unsigned long long prefetch_bytes;   // line by line so it sits in the memory-side cache
+  // optional: up to kPrefetchRanges ranges that the NEXT kernels will read (weights),
+  // touched line by line so they sit in the memory-side cache: range r holds the 128-byte
+  // lines [pf_end[r - 1], pf_end[r]) of their concatenation (pf_end[last] = 0: none)
+  const char *pf_base[kPrefetchRanges];
+  unsigned pf_end[kPrefetchRanges];
   int B, S, rows_cap, heads;
   float scale_log2e;   // scale * log2(e)
   int padded_rows;
@@ -130,23 +134,29 @@ __device__ __forceinline__ float rows_sum(float x) {
 
 // Cache warm-up on behalf of later kernels: the workgroups of the last quarter of the
 // issue order (short sequences and dead tiles, which retire early) each touch one
-// dword per 128-byte line of their slice of [prefetch, prefetch + bytes).  The loads
-// are the wave's last instructions; nothing reads their results.
+// dword per 128-byte line of their slice of the ranges.  The loads are the wave's last
+// instructions; nothing reads their results.
 __device__ __forceinline__ void prefetch_slice(const AttArgs &p) {
-  if (!p.prefetch) return;
+  const unsigned lines = p.pf_end[kPrefetchRanges - 1];
+  if (!lines) return;
   const unsigned z0 = (unsigned)((unsigned long long)gridDim.x * 3 / 4);
   if (blockIdx.x < z0) return;
-  const unsigned long long duty = gridDim.x - z0;
-  const unsigned long long me = blockIdx.x - z0;
-  // one dword at the start of each 128-byte line; a last line of fewer than four bytes is
-  // left alone, so no byte outside the range is read
-  const unsigned long long lines = (p.prefetch_bytes + 124) / 128;
-  const unsigned long long per = (lines + duty - 1) / duty;
-  const unsigned long long first = me * per;
-  const unsigned long long last = first + per < lines ? first + per : lines;
-  for (unsigned long long l = first + threadIdx.x; l < last; l += blockDim.x) {
+  const unsigned duty = gridDim.x - z0;
+  const unsigned me = blockIdx.x - z0;
+  const unsigned per = (lines + duty - 1) / duty;
+  const unsigned first = me * per;
+  const unsigned last = first + per < lines ? first + per : lines;
+  for (unsigned l = first + threadIdx.x; l < last; l += blockDim.x) {
+    const char *base = p.pf_base[0];
+    unsigned begin = 0;
+#pragma unroll
+    for (int r = 1; r < kPrefetchRanges; ++r)
+      if (l >= p.pf_end[r - 1]) {
+        base = p.pf_base[r];
+        begin = p.pf_end[r - 1];
+      }
     unsigned sink;
-    const char *addr = p.prefetch + l * 128;
+    const char *addr = base + (unsigned long long)(l - begin) * 128;
     asm volatile("global_load_dword %0, %1, off" : "=v"(sink) : "v"(addr) : "memory");
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -694,15 +704,34 @@ __global__ __launch_bounds__(kAttThreads) void attention_short_kernel(AttArgs p)
 // and up) and a loss of 2-3 % with smaller grids, which therefore skip it.  Each
 // duty workgroup (last quarter of the issue order; a half measured 0.7 % slower) touches at most four
 // lines per thread; the range is cut to that.
-static void set_prefetch(AttArgs &a, unsigned grid, const void *prefetch, unsigned long long bytes) {
-  a.prefetch = nullptr;
-  a.prefetch_bytes = 0;
-  if (!prefetch || !bytes || !option_prefetch()) return;
+static int set_prefetch(AttArgs &a, unsigned grid, const void *const *prefetch,
+                        const unsigned long long *bytes, int count) {
+  for (int r = 0; r < kPrefetchRanges; ++r) {
+    a.pf_base[r] = nullptr;
+    a.pf_end[r] = 0;
+  }
+  BT_REQUIRE(count >= 0 && count <= kPrefetchRanges, BT_ERR_INVALID_ARGUMENT,
+             "attention: prefetch_count=%d outside [0, %d]", count, kPrefetchRanges);
+  BT_REQUIRE(count == 0 || (prefetch && bytes), BT_ERR_INVALID_ARGUMENT,
+             "attention: prefetch ranges need their pointers and sizes");
+  if (!count || !option_prefetch()) return BT_OK;
+  if (grid < (unsigned)option_prefetch_min_grid()) return BT_OK;
   const unsigned long long duty = grid - (unsigned long long)grid * 3 / 4;
-  if (grid < (unsigned)option_prefetch_min_grid()) return;
-  const unsigned long long cap = duty * 4 * kAttThreads * 128;
-  a.prefetch = (const char *)prefetch;
-  a.prefetch_bytes = bytes < cap ? bytes : cap;
+  unsigned long long left = duty * 4 * kAttThreads;   // lines the duty workgroups take on
+  unsigned end = 0;
+  for (int r = 0; r < kPrefetchRanges; ++r) {
+    if (r < count && prefetch[r] && left) {
+      // one dword at the start of each 128-byte line; a last line of fewer than four bytes
+      // is left alone, so no byte outside the range is read
+      unsigned long long lines = (bytes[r] + 124) / 128;
+      if (lines > left) lines = left;
+      left -= lines;
+      a.pf_base[r] = (const char *)prefetch[r];
+      end += (unsigned)lines;
+    }
+    a.pf_end[r] = end;
+  }
+  return BT_OK;
 }
 
 // Size of the 1-D grid for `nqb` query tiles per sequence; fills the mapping fields.
@@ -766,7 +795,8 @@ extern "C" int bt_attention_short(const void *qkv_heads, void *attention_output,
                                   const void *atten_mask, const void *attention_bias,
                                   int batch_size, int seq_len, int rows_cap, int head_num,
                                   int size_per_head, float scale, int padded_rows,
-                                  const void *prefetch, unsigned long long prefetch_bytes,
+                                  const void *const *prefetch,
+                                  const unsigned long long *prefetch_bytes, int prefetch_count,
                                   void *stream) {
   int rc = check_att_args("bt_attention_short", qkv_heads, attention_output, batch_idx, atten_mask,
                           padded_rows, batch_size, seq_len, rows_cap, head_num, size_per_head);
@@ -775,11 +805,12 @@ extern "C" int bt_attention_short(const void *qkv_heads, void *attention_output,
              "bt_attention_short: seq_len=%d exceeds 512, use bt_attention_grouped", seq_len);
   AttArgs a{(const half_t *)qkv_heads, (half_t *)attention_output, batch_idx, seq_order,
             (const half_t *)atten_mask, (const half_t *)attention_bias,
-            nullptr, 0, batch_size, seq_len,
+            {}, {}, batch_size, seq_len,
             rows_cap, head_num, scale * kLog2e, padded_rows};
   hipStream_t s = as_stream(stream);
   a.nqb_grid = att_grid(a, (seq_len + 63) / 64);
-  set_prefetch(a, a.nqb_grid, prefetch, prefetch_bytes);
+  rc = set_prefetch(a, a.nqb_grid, prefetch, prefetch_bytes, prefetch_count);
+  if (rc) return rc;
   if (seq_len <= 64) return launch_short<4>(a, s);
   if (seq_len <= 128) return launch_short<8>(a, s);
   if (seq_len <= 256) return launch_short<16>(a, s);
@@ -858,7 +889,8 @@ extern "C" int bt_attention_grouped(const void *qkv_heads, void *attention_outpu
                                     const void *atten_mask, const void *attention_bias,
                                     int batch_size, int seq_len, int rows_cap, int head_num,
                                     int size_per_head, float scale, int padded_rows,
-                                    const void *prefetch, unsigned long long prefetch_bytes,
+                                    const void *const *prefetch,
+                                    const unsigned long long *prefetch_bytes, int prefetch_count,
                                     const int *mask_prefix_slots, const void *work_list,
                                     void *stream) {
   int rc = check_att_args("bt_attention_grouped", qkv_heads, attention_output, batch_idx,
@@ -869,7 +901,7 @@ extern "C" int bt_attention_grouped(const void *qkv_heads, void *attention_outpu
              "bt_attention_grouped: work_list must be 16-byte aligned");
   AttArgs a{(const half_t *)qkv_heads, (half_t *)attention_output, batch_idx, seq_order,
             (const half_t *)atten_mask, (const half_t *)attention_bias,
-            nullptr, 0, batch_size, seq_len,
+            {}, {}, batch_size, seq_len,
             rows_cap, head_num, scale * kLog2e, padded_rows};
   a.mask_ok = a.mask ? mask_prefix_slots : nullptr;
   a.work_list = (const int4 *)work_list;   // read only when the launch uses the balanced order
@@ -877,7 +909,8 @@ extern "C" int bt_attention_grouped(const void *qkv_heads, void *attention_outpu
   const bool add = a.mask || a.bias;
   const GroupedPlan plan = plan_grouped(a, batch_size, seq_len, head_num);
   const unsigned grid = plan.grid;
-  set_prefetch(a, grid, prefetch, prefetch_bytes);
+  rc = set_prefetch(a, grid, prefetch, prefetch_bytes, prefetch_count);
+  if (rc) return rc;
   if (plan.wide) {
     if (add)
       attention_grouped_kernel<2, true, 3><<<grid, kAttThreads, 0, s>>>(a);

@@ -21,6 +21,7 @@ typedef _Float16 half_t;
 typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
 typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
 typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+typedef __fp16 fp16x4_t __attribute__((ext_vector_type(4)));   // element type of the LDS transpose-read builtin
 typedef float float4_t __attribute__((ext_vector_type(4)));
 typedef float float16_t __attribute__((ext_vector_type(16)));
 typedef unsigned int uint4_t __attribute__((ext_vector_type(4)));
@@ -71,6 +72,7 @@ inline int allow_dynamic_lds(Kernel kernel, size_t bytes, std::atomic<bool> (&do
 }
 
 int option_gemm_tile();      // -1 = heuristic, else index into the tile table
+int option_layer_prepack();  // -1 = by the measured table, 0 = never, 1 = always
 int option_attention_qb();   // -1 = heuristic, 1 or 2 = query blocks per wave
 int option_f32_gemm_tile();  // -1 = heuristic, else index into the float GEMM's tile table
 int option_attention_xcd_map();     // workgroup order of the attention kernels: 0 plain, 1 XCD-aware, 2 balanced (default), 3 balanced always

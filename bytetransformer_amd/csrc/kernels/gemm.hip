@@ -1,7 +1,8 @@
 // fp16 MFMA GEMM family for gfx950: C[rows, N] = A[rows, K] . W[K, N] with
 // fp32 accumulation and three fused epilogues (plain store, +bias+tanh-GELU,
-// +bias with the Q/K/V head split).  Both operands are consumed k-contiguous:
-// A as stored, W through the [N, K] pre-pack made by bt_transpose_weights.
+// +bias with the Q/K/V head split).  A is consumed k-contiguous as stored; W either
+// as the row-major [K, N] matrix itself (its LDS tile is read with the LDS transpose
+// read) or through the k-contiguous [N, K] pre-pack made by bt_transpose_weights.
 //
 // Structure of one workgroup (tile BM x BN, BK = 64):
 //   * global -> LDS copies are 16-byte buffer loads with an LDS destination: no
@@ -39,7 +40,7 @@ enum Epilogue { kEpiPlain = 0, kEpiBiasGelu = 1, kEpiQkvSplit = 2, kEpiPartial =
 
 struct GemmArgs {
   const half_t *a;      // [rows_cap, K]
-  const half_t *wt;     // [N, K]
+  const half_t *wt;     // [N, K] (pre-packed), or [K, N] as the layer's weights are stored (w_kn)
   const half_t *bias;   // [N] or null
   half_t *c;            // [rows_cap, N]  (or [3][heads][rows_cap][64] for the QKV split)
   const int *valid_rows;
@@ -48,6 +49,7 @@ struct GemmArgs {
   int tiles_n;
   int rows_hint;        // host-side estimate of the live rows (0 = unknown); tile choice only
   float *c32;           // kEpiPartial only: [splits][rows_cap][N]
+  int w_kn;             // 1: wt is the row-major [K, N] matrix itself
 };
 
 __device__ __forceinline__ float gelu_tanh_f32(float x) {
@@ -65,6 +67,18 @@ __device__ __forceinline__ float gelu_tanh_f32(float x) {
 __device__ __forceinline__ int swz(int row) { return (row >> 1) & 7; }
 
 constexpr int kBK = 64;   // k extent of one LDS tile (halfs) = 8 chunks of 16 bytes
+
+// A [K, N] weight tile sits in LDS as 64 k-rows of BN halfs and is read with the LDS
+// transpose read: the 32 lanes of one pass fetch 4 consecutive k-rows x 64 bytes.  Rows are
+// BN / 32 segments of 64 bytes long; with a multiple of four segments per row the four rows
+// start on the same bank and the segment is XORed with row & 3, with an odd multiple of
+// two (BN = 64, 192) rows r and r + 2 do and bit 0 of the segment is XORed with bit 1 of the
+// row.  Returned in 16-byte chunks (the unit a loading lane moves).
+template <int BN>
+__device__ __forceinline__ int swz_kn(int k_row) {
+  static_assert(BN % 64 == 0, "whole 64-byte segment pairs");
+  return (BN / 32) % 4 == 0 ? (k_row & 3) << 2 : ((k_row >> 1) & 1) << 2;
+}
 
 template <int N>
 __device__ __forceinline__ void wait_vmcnt() {
@@ -101,15 +115,46 @@ __device__ __forceinline__ rsrc_t make_rsrc(const void *base, size_t bytes) {
 // lds + i * lds_step; the first NIA instructions read A, the rest W.
 template <int NI, int NIA>
 __device__ __forceinline__ void issue_stage_loads(rsrc_t rs_a, rsrc_t rs_w, const int (&voff)[NI],
-                                                  half_t *lds, int lds_step, int k_bytes) {
+                                                  half_t *lds, int lds_step, int k_bytes,
+                                                  int k_bytes_w) {
 #pragma unroll
   for (int i = 0; i < NI; ++i)
     __builtin_amdgcn_raw_ptr_buffer_load_lds(i < NIA ? rs_a : rs_w,
                                              (__attribute__((address_space(3))) void *)(lds + i * lds_step),
-                                             16, voff[i], k_bytes, 0, 0);
+                                             16, voff[i], i < NIA ? k_bytes : k_bytes_w, 0, 0);
 }
 
-template <int BM, int BN, int STAGES, int WM, int WN, int NP, int SCHED, int EPI>
+// Byte offset, from the first element of a [K, N] weight tile (k-step 0, first column of
+// the tile), of the 16 bytes that a loading lane moves with the load that fills bytes
+// [1024 g, 1024 g + 1024) of the tile's LDS image; the tile has `cols` columns inside the
+// matrix, and chunks past them get an offset outside every descriptor (they read as zero).
+template <int BN>
+__device__ __forceinline__ int kn_load_offset(int g, int lane, int N, int cols) {
+  constexpr int CPR = BN / 8;                       // 16-byte chunks per k-row
+  const int slot = g * 64 + lane;
+  const int k_row = slot / CPR, c = (slot % CPR) ^ swz_kn<BN>(k_row);
+  return c * 8 < cols ? (k_row * N + c * 8) * (int)sizeof(half_t) : 0x7ffffff0;
+}
+
+// Weight operand of one 32x32x16 MFMA (32 columns from n_base, 16 k-rows from k_base) out
+// of the LDS image of a [K, N] tile: lane l holds column n_base + (l & 31) at k-rows
+// k_base + 8 (l >> 5) .. + 7, gathered by two transpose reads of 4 k-rows x 16 columns per
+// 16 lanes.  `lane_part` = kn_frag_lane_part(lane).
+template <int BN>
+__device__ __forceinline__ half8_t load_kn_frag(const half_t *sW, int n_base, int k_base, int lane) {
+  const int lq = lane & 15, g2 = lane >> 4;
+  const int k_row = k_base + 8 * (g2 >> 1) + (lq >> 2);
+  const int col = n_base + 16 * (g2 & 1) + 4 * (lq & 3);
+  const half_t *p0 = sW + k_row * BN + (((col >> 3) ^ swz_kn<BN>(k_row)) << 3) + (col & 7);
+  const fp16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4f16(
+      (__attribute__((address_space(3))) fp16x4_t *)p0);
+  const fp16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4f16(
+      (__attribute__((address_space(3))) fp16x4_t *)(p0 + 4 * BN));   // rows + 4: same swizzle term
+  const half4_t l4 = __builtin_bit_cast(half4_t, lo), h4 = __builtin_bit_cast(half4_t, hi);
+  return half8_t{l4[0], l4[1], l4[2], l4[3], h4[0], h4[1], h4[2], h4[3]};
+}
+
+template <int BM, int BN, int STAGES, int WM, int WN, int NP, int SCHED, int EPI, bool WKN>
 __device__ __forceinline__ void gemm_tile(const GemmArgs &p) {
   constexpr int BK = kBK;
   constexpr int NW = WM * WN;                   // waves that run the MFMAs
@@ -167,8 +212,13 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs &p) {
       gather ? make_rsrc(p.a + k_first, ((size_t)p.rows_cap * p.K - k_first) * sizeof(half_t))
              : make_rsrc(p.a + (size_t)m0 * p.K + k_first,
                          ((size_t)(p.rows_cap - m0) * p.K - k_first) * sizeof(half_t));
-  const rsrc_t rs_w = make_rsrc(p.wt + (size_t)n0 * p.K + k_first,
-                                ((size_t)(p.N - n0) * p.K - k_first) * sizeof(half_t));
+  // the weight tile: BN rows of 64 k ([N, K] pre-pack), or 64 k-rows of BN columns ([K, N]);
+  // 1 KB per load instruction either way
+  const rsrc_t rs_w =
+      WKN ? make_rsrc(p.wt + (size_t)k_first * p.N + n0,
+                      ((size_t)(p.K - k_first) * p.N - n0) * sizeof(half_t))
+          : make_rsrc(p.wt + (size_t)n0 * p.K + k_first,
+                      ((size_t)(p.N - n0) * p.K - k_first) * sizeof(half_t));
   int voff[NI];
   if (loader) {
 #pragma unroll
@@ -178,11 +228,13 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs &p) {
       int row = i < NIA ? r : r - BM;
       if (i < NIA && gather) row = p.a_row_index[min(m0 + r, M - 1)];   // live rows only hold valid indices
       voff[i] = (row * p.K + kc * 8) * (int)sizeof(half_t);
+      if (WKN && i >= NIA) voff[i] = kn_load_offset<BN>((i - NIA) * NL + lw, lane, p.N, p.N - n0);
     }
   }
+  const int w_step_bytes = (WKN ? BK * p.N : BK) * (int)sizeof(half_t);   // one k-step further
 #define BT_ISSUE_LOADS(kt, stage)                                                        \
   issue_stage_loads<NI, NIA>(rs_a, rs_w, voff, smem + (stage)*STAGE_HALFS + lw * 8 * BK, \
-                             NL * 8 * BK, (kt)*BK * (int)sizeof(half_t))
+                             NL * 8 * BK, (kt)*BK * (int)sizeof(half_t), (kt)*w_step_bytes)
 
   if (loader) {
 #pragma unroll
@@ -241,7 +293,10 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs &p) {
 #pragma unroll
     for (int i = 0; i < TN; ++i) {
       const int r = wn * WTN + i * 32 + fr_row;
-      fw[b][i] = *(const half8_t *)(sB + r * BK + (((2 * ks + fr_kc) ^ swz(r + BM)) * 8));
+      if (WKN)
+        fw[b][i] = load_kn_frag<BN>(sB, wn * WTN + i * 32, 16 * ks, lane);
+      else
+        fw[b][i] = *(const half8_t *)(sB + r * BK + (((2 * ks + fr_kc) ^ swz(r + BM)) * 8));
     }
 #pragma unroll
     for (int j = 0; j < TM; ++j) {
@@ -354,7 +409,7 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs &p) {
 // the first store instruction on: with 228 tiles on 256 CUs the last 7 us of the 31 us of
 // the FFN1 product at batch 16 x 512 are 29.5 MB of stores.)  The grid no longer depends
 // on the row count: a workgroup counts its tiles from the device-side row count.
-template <int BM, int BN, int STAGES, int WM, int WN, int NP, int SCHED, int EPI>
+template <int BM, int BN, int STAGES, int WM, int WN, int NP, int SCHED, int EPI, bool WKN>
 __device__ __forceinline__ void gemm_tiles_flat(const GemmArgs &p) {
   constexpr int BK = kBK;
   constexpr int NW = WM * WN;
@@ -428,7 +483,14 @@ __device__ __forceinline__ void gemm_tiles_flat(const GemmArgs &p) {
     }
     rs_a = gather ? make_rsrc(p.a, (size_t)p.rows_cap * p.K * sizeof(half_t))
                   : make_rsrc(p.a + (size_t)m0 * p.K, (size_t)(p.rows_cap - m0) * p.K * sizeof(half_t));
-    rs_w = make_rsrc(p.wt + (size_t)n0 * p.K, (size_t)(p.N - n0) * p.K * sizeof(half_t));
+    rs_w = WKN ? make_rsrc(p.wt + n0, ((size_t)p.K * p.N - n0) * sizeof(half_t))
+               : make_rsrc(p.wt + (size_t)n0 * p.K, (size_t)(p.N - n0) * p.K * sizeof(half_t));
+    if (WKN && (p.N % BN) != 0) {
+      // the column mask of the weight loads depends on the tile's first column
+#pragma unroll
+      for (int i = NIA; i < NI; ++i)
+        voff[i] = kn_load_offset<BN>((i - NIA) * NL + lw, lane, p.N, p.N - n0);
+    }
     if (gather) {
 #pragma unroll
       for (int i = 0; i < NIA; ++i) {
@@ -446,6 +508,7 @@ __device__ __forceinline__ void gemm_tiles_flat(const GemmArgs &p) {
       const int kc = (lane & 7) ^ swz(r);
       const int row = i < NIA ? r : r - BM;
       voff[i] = (row * p.K + kc * 8) * (int)sizeof(half_t);
+      if (WKN && i >= NIA) voff[i] = kn_load_offset<BN>((i - NIA) * NL + lw, lane, p.N, BN);
     }
     if (gather) fetch_indices(L0);
     load_setup(L0, n_my > 1, false);
@@ -454,7 +517,8 @@ __device__ __forceinline__ void gemm_tiles_flat(const GemmArgs &p) {
   auto issue_next = [&](int stage) {
     if (ld_left == 0) return;
     issue_stage_loads<NI, NIA>(rs_a, rs_w, voff, smem + stage * STAGE_HALFS + lw * 8 * BK,
-                               NL * 8 * BK, ld_kt * BK * (int)sizeof(half_t));
+                               NL * 8 * BK, ld_kt * BK * (int)sizeof(half_t),
+                               ld_kt * (WKN ? BK * p.N : BK) * (int)sizeof(half_t));
     --ld_left;
     if (++ld_kt == nk) {
       ld_kt = 0;
@@ -526,7 +590,10 @@ __device__ __forceinline__ void gemm_tiles_flat(const GemmArgs &p) {
 #pragma unroll
     for (int i = 0; i < TN; ++i) {
       const int r = wn * WTN + i * 32 + fr_row;
-      fw[b][i] = *(const half8_t *)(sB + r * BK + (((2 * ks + fr_kc) ^ swz(r + BM)) * 8));
+      if (WKN)
+        fw[b][i] = load_kn_frag<BN>(sB, wn * WTN + i * 32, 16 * ks, lane);
+      else
+        fw[b][i] = *(const half8_t *)(sB + r * BK + (((2 * ks + fr_kc) ^ swz(r + BM)) * 8));
     }
 #pragma unroll
     for (int j = 0; j < TM; ++j) {
@@ -613,17 +680,17 @@ __device__ __forceinline__ void gemm_tiles_flat(const GemmArgs &p) {
 
 #endif  // __HIP_DEVICE_COMPILE__
 
-template <int BM, int BN, int STAGES, int WM, int WN, int NP, int SCHED, int EPI>
+template <int BM, int BN, int STAGES, int WM, int WN, int NP, int SCHED, int EPI, bool WKN>
 __global__ __launch_bounds__((WM * WN + NP) * 64) void gemm_flat_kernel(GemmArgs p) {
 #if defined(__HIP_DEVICE_COMPILE__)
-  gemm_tiles_flat<BM, BN, STAGES, WM, WN, NP, SCHED, EPI>(p);
+  gemm_tiles_flat<BM, BN, STAGES, WM, WN, NP, SCHED, EPI, WKN>(p);
 #endif
 }
 
-template <int BM, int BN, int STAGES, int WM, int WN, int NP, int SCHED, int EPI>
+template <int BM, int BN, int STAGES, int WM, int WN, int NP, int SCHED, int EPI, bool WKN>
 __global__ __launch_bounds__((WM * WN + NP) * 64) void gemm_kernel(GemmArgs p) {
 #if defined(__HIP_DEVICE_COMPILE__)
-  gemm_tile<BM, BN, STAGES, WM, WN, NP, SCHED, EPI>(p);
+  gemm_tile<BM, BN, STAGES, WM, WN, NP, SCHED, EPI, WKN>(p);
 #endif
 }
 
@@ -651,33 +718,40 @@ __global__ __launch_bounds__(256) void transpose_kernel(TransposeArgs a) {
                     threadIdx.x, true);
 }
 
-template <int BM, int BN, int STAGES, int WM, int WN, int NP, int SCHED, int EPI>
-static int launch_gemm_tile(GemmArgs p, hipStream_t s, int splits = 1) {
+template <int BM, int BN, int STAGES, int WM, int WN, int NP, int SCHED, int EPI, bool WKN>
+static int launch_gemm_tile_as(GemmArgs p, hipStream_t s, int splits) {
   constexpr size_t smem = (size_t)STAGES * (BM + BN) * kBK * sizeof(half_t);
   static_assert(smem <= 160 * 1024, "LDS budget");
   static std::atomic<bool> configured[kMaxDevices];
-  const int rc = allow_dynamic_lds(gemm_kernel<BM, BN, STAGES, WM, WN, NP, SCHED, EPI>, smem,
+  const int rc = allow_dynamic_lds(gemm_kernel<BM, BN, STAGES, WM, WN, NP, SCHED, EPI, WKN>, smem,
                                    configured, "hipFuncSetAttribute(gemm_kernel)");
   if (rc != BT_OK) return rc;
   const int tiles_m = (p.rows_cap + BM - 1) / BM;
   p.tiles_n = (p.N + BN - 1) / BN;
   const dim3 grid((tiles_m * p.tiles_n + 7) / 8 * 8, splits);
-  gemm_kernel<BM, BN, STAGES, WM, WN, NP, SCHED, EPI><<<grid, (WM * WN + NP) * 64, smem, s>>>(p);
+  gemm_kernel<BM, BN, STAGES, WM, WN, NP, SCHED, EPI, WKN>
+      <<<grid, (WM * WN + NP) * 64, smem, s>>>(p);
   BT_CHECK_LAUNCH("gemm_kernel");
   return BT_OK;
+}
+
+template <int BM, int BN, int STAGES, int WM, int WN, int NP, int SCHED, int EPI>
+static int launch_gemm_tile(GemmArgs p, hipStream_t s, int splits = 1) {
+  return p.w_kn ? launch_gemm_tile_as<BM, BN, STAGES, WM, WN, NP, SCHED, EPI, true>(p, s, splits)
+                : launch_gemm_tile_as<BM, BN, STAGES, WM, WN, NP, SCHED, EPI, false>(p, s, splits);
 }
 
 static int cu_count();
 
 // Persistent launch: about one workgroup per CU (a multiple of 8, one share per XCD), each
 // looping over its tiles on the device.
-template <int BM, int BN, int STAGES, int WM, int WN, int NP, int SCHED, int EPI>
-static int launch_gemm_flat(GemmArgs p, hipStream_t s) {
+template <int BM, int BN, int STAGES, int WM, int WN, int NP, int SCHED, int EPI, bool WKN>
+static int launch_gemm_flat_as(GemmArgs p, hipStream_t s) {
   constexpr size_t smem = (size_t)STAGES * (BM + BN) * kBK * sizeof(half_t) + BN * sizeof(half_t);
   static_assert(smem <= 160 * 1024, "LDS budget");
   static std::atomic<bool> configured[kMaxDevices];
-  const int rc = allow_dynamic_lds(gemm_flat_kernel<BM, BN, STAGES, WM, WN, NP, SCHED, EPI>, smem,
-                                   configured, "hipFuncSetAttribute(gemm_flat_kernel)");
+  const int rc = allow_dynamic_lds(gemm_flat_kernel<BM, BN, STAGES, WM, WN, NP, SCHED, EPI, WKN>,
+                                   smem, configured, "hipFuncSetAttribute(gemm_flat_kernel)");
   if (rc != BT_OK) return rc;
   const int tiles_m = (p.rows_cap + BM - 1) / BM;
   p.tiles_n = (p.N + BN - 1) / BN;
@@ -686,9 +760,16 @@ static int launch_gemm_flat(GemmArgs p, hipStream_t s) {
   long long wgs = (long long)cu_count() * per_cu;
   if (wgs > tiles) wgs = tiles;
   const dim3 grid((unsigned)((wgs + 7) / 8 * 8));
-  gemm_flat_kernel<BM, BN, STAGES, WM, WN, NP, SCHED, EPI><<<grid, (WM * WN + NP) * 64, smem, s>>>(p);
+  gemm_flat_kernel<BM, BN, STAGES, WM, WN, NP, SCHED, EPI, WKN>
+      <<<grid, (WM * WN + NP) * 64, smem, s>>>(p);
   BT_CHECK_LAUNCH("gemm_flat_kernel");
   return BT_OK;
+}
+
+template <int BM, int BN, int STAGES, int WM, int WN, int NP, int SCHED, int EPI>
+static int launch_gemm_flat(GemmArgs p, hipStream_t s) {
+  return p.w_kn ? launch_gemm_flat_as<BM, BN, STAGES, WM, WN, NP, SCHED, EPI, true>(p, s)
+                : launch_gemm_flat_as<BM, BN, STAGES, WM, WN, NP, SCHED, EPI, false>(p, s);
 }
 
 static int cu_count() {
@@ -720,13 +801,13 @@ static long long estimated_rows(const GemmArgs &p) {
 // tile, so the row used has the same number of row tiles as m or one more: run time moves
 // in steps with the number of rounds of workgroups, and interpolating between two row
 // counts on either side of such a step would describe neither.
-static const float *tuned_times(long long m, int n, int k, int epi) {
+static const float *tuned_times(long long m, int n, int k, int epi, int kn) {
   if (cu_count() != 256) return nullptr;     // the table was measured on a 256-CU part
   // below about a thousand rows a launch is latency bound and a loop of identical
   // launches says little about the layer sequence
   if (m < 1024 || m > kTunedRows[kTunedPoints - 1]) return nullptr;
   for (const TunedShape &ts : kTunedShapes) {
-    if (ts.n != n || ts.k != k || ts.epi != epi) continue;
+    if (ts.n != n || ts.k != k || ts.epi != epi || ts.kn != kn) continue;
     int at = 0;
     while (at < kTunedPoints - 1 && kTunedRows[at] < m) ++at;
     return ts.us[at];
@@ -791,7 +872,7 @@ static int launch_gemm(GemmArgs p, hipStream_t s) {
     // the table overrides the model only for a clear win: the timings come from a loop
     // of identical launches, and differences of a few per cent do not carry over to the
     // layer sequence
-    if (const float *us = tuned_times(estimated_rows(p), p.N, p.K, EPI)) {
+    if (const float *us = tuned_times(estimated_rows(p), p.N, p.K, EPI, p.w_kn)) {
       int tuned = -1;
       for (int t = 0; t < kTunedTiles; ++t)
         if (us[t] > 0.f && (tuned < 0 || us[t] < us[tuned])) tuned = t;
@@ -823,7 +904,7 @@ static int launch_gemm(GemmArgs p, hipStream_t s) {
 }
 
 static int check_gemm_args(const char *who, const void *a, const void *wt, const void *c,
-                           int rows_cap, int n, int k) {
+                           int rows_cap, int n, int k, int weight_kn) {
   BT_REQUIRE(a && wt && c, BT_ERR_INVALID_ARGUMENT, "%s: null pointer argument", who);
   BT_REQUIRE(aligned16({a, wt, c}), BT_ERR_INVALID_ARGUMENT,
              "%s: tensor pointers must be 16-byte aligned", who);
@@ -833,6 +914,11 @@ static int check_gemm_args(const char *who, const void *a, const void *wt, const
   BT_REQUIRE(n % 8 == 0, BT_ERR_UNSUPPORTED, "%s: n=%d must be a multiple of 8", who, n);
   // a 256-row tile is addressed with 32-bit byte offsets from its first row
   BT_REQUIRE(k <= (1 << 21), BT_ERR_UNSUPPORTED, "%s: k=%d is beyond 2^21", who, k);
+  BT_REQUIRE(weight_kn == 0 || weight_kn == 1, BT_ERR_INVALID_ARGUMENT,
+             "%s: weight_kn=%d must be 0 ([n, k] pre-pack) or 1 ([k, n] as stored)", who, weight_kn);
+  // a [k, n] weight is addressed with 32-bit byte offsets from its first row
+  BT_REQUIRE(!weight_kn || (long long)n * k * 2 <= 0x7fffffffLL, BT_ERR_UNSUPPORTED,
+             "%s: a [k, n] weight of %d x %d halfs is beyond 2 GiB", who, k, n);
   return BT_OK;
 }
 
@@ -870,53 +956,76 @@ extern "C" int bt_transpose_weight(const void *w, void *wt, int k, int n, void *
   return bt_transpose_weights(1, ws, wts, &k, &n, stream);
 }
 
+extern "C" int bt_gemm_prepack_pays(long long rows, int n, int k, int epilogue) {
+  const int forced = option_layer_prepack();
+  if (forced >= 0) return forced;
+  const float *nk = tuned_times(rows, n, k, epilogue, 0), *kn = tuned_times(rows, n, k, epilogue, 1);
+  if (!nk || !kn) return 0;
+  float best_nk = 0.f, best_kn = 0.f;
+  for (int t = 0; t < kTunedTiles; ++t) {
+    if (nk[t] > 0.f && (best_nk == 0.f || nk[t] < best_nk)) best_nk = nk[t];
+    if (kn[t] > 0.f && (best_kn == 0.f || kn[t] < best_kn)) best_kn = kn[t];
+  }
+  if (best_nk == 0.f || best_kn == 0.f) return 0;
+  // the copy is made inside the layer's prologue launch, beside the offsets: measured in
+  // the layer sequence it adds about 0.5 us per megabyte of weight to that launch (2.4 us
+  // for FFN1 of BERT-base, 7.4 us for all four matrices); asked to return a microsecond more
+  const float pack_us = 0.5e-6f * (float)n * (float)k * sizeof(half_t);
+  return best_nk + pack_us + 1.0f < best_kn ? 1 : 0;
+}
+
 extern "C" int bt_gemm(const void *a, const void *wt, void *c, const int *valid_rows,
-                       int rows_cap, int rows_hint, int n, int k, void *stream) {
-  int rc = check_gemm_args("bt_gemm", a, wt, c, rows_cap, n, k);
+                       int rows_cap, int rows_hint, int n, int k, int weight_kn, void *stream) {
+  int rc = check_gemm_args("bt_gemm", a, wt, c, rows_cap, n, k, weight_kn);
   if (rc) return rc;
   if (rows_cap == 0) return BT_OK;
   GemmArgs p{(const half_t *)a, (const half_t *)wt, nullptr, (half_t *)c, valid_rows, nullptr,
-             rows_cap,          n,                  k,       0,           rows_hint};
+             rows_cap,          n,                  k,       0,           rows_hint,
+             nullptr,           weight_kn};
   return launch_gemm<kEpiPlain>(p, as_stream(stream));
 }
 
 extern "C" int bt_gemm_splitk(const void *a, const void *wt, void *partials, int splits,
-                              const int *valid_rows, int rows_cap, int n, int k, void *stream) {
-  int rc = check_gemm_args("bt_gemm_splitk", a, wt, partials, rows_cap, n, k);
+                              const int *valid_rows, int rows_cap, int n, int k, int weight_kn,
+                              void *stream) {
+  int rc = check_gemm_args("bt_gemm_splitk", a, wt, partials, rows_cap, n, k, weight_kn);
   if (rc) return rc;
   BT_REQUIRE(splits >= 1 && splits <= 16 && k % (splits * kBK) == 0, BT_ERR_INVALID_ARGUMENT,
              "bt_gemm_splitk: splits=%d must lie in [1, 16] and divide k / 64 = %d", splits,
              k / kBK);
   if (rows_cap == 0) return BT_OK;
   GemmArgs p{(const half_t *)a, (const half_t *)wt, nullptr, nullptr, valid_rows, nullptr,
-             rows_cap,          n,                  k,       0,       0,          (float *)partials};
+             rows_cap,          n,                  k,       0,       0,          (float *)partials,
+             weight_kn};
   // the small tile only: splitting k is for launches whose k loop is the whole run time
   return launch_gemm_tile<32, 64, 4, 1, 2, 2, 0, kEpiPartial>(p, as_stream(stream), splits);
 }
 
 extern "C" int bt_gemm_bias_gelu(const void *a, const void *wt, const void *bias, void *c,
                                  const int *valid_rows, int rows_cap, int rows_hint, int n, int k,
-                                 void *stream) {
-  int rc = check_gemm_args("bt_gemm_bias_gelu", a, wt, c, rows_cap, n, k);
+                                 int weight_kn, void *stream) {
+  int rc = check_gemm_args("bt_gemm_bias_gelu", a, wt, c, rows_cap, n, k, weight_kn);
   if (rc) return rc;
   BT_REQUIRE(bias, BT_ERR_INVALID_ARGUMENT, "bt_gemm_bias_gelu: null bias");
   if (rows_cap == 0) return BT_OK;
   GemmArgs p{(const half_t *)a, (const half_t *)wt, (const half_t *)bias, (half_t *)c, valid_rows,
              nullptr,           rows_cap,           n,                    k,           0,
-             rows_hint};
+             rows_hint,         nullptr,            weight_kn};
   return launch_gemm<kEpiBiasGelu>(p, as_stream(stream));
 }
 
 extern "C" int bt_gemm_qkv_bias_split(const void *a, const int *a_row_index, const void *wt_qkv,
                                       const void *bias_qkv, void *qkv_heads,
                                       const int *valid_rows, int rows_cap, int rows_hint,
-                                      int head_num, int size_per_head, void *stream) {
+                                      int head_num, int size_per_head, int weight_kn,
+                                      void *stream) {
   BT_REQUIRE(head_num > 0, BT_ERR_INVALID_ARGUMENT, "bt_gemm_qkv_bias_split: head_num=%d",
              head_num);
   BT_REQUIRE(size_per_head > 0, BT_ERR_INVALID_ARGUMENT,
              "bt_gemm_qkv_bias_split: size_per_head=%d", size_per_head);
   const int H = head_num * size_per_head;
-  int rc = check_gemm_args("bt_gemm_qkv_bias_split", a, wt_qkv, qkv_heads, rows_cap, 3 * H, H);
+  int rc = check_gemm_args("bt_gemm_qkv_bias_split", a, wt_qkv, qkv_heads, rows_cap, 3 * H, H,
+                           weight_kn);
   if (rc) return rc;
   BT_REQUIRE(bias_qkv, BT_ERR_INVALID_ARGUMENT, "bt_gemm_qkv_bias_split: null bias");
   if (rows_cap == 0) return BT_OK;
@@ -926,7 +1035,8 @@ extern "C" int bt_gemm_qkv_bias_split(const void *a, const int *a_row_index, con
   BT_REQUIRE(!a_row_index || (long long)rows_cap * H * 2 <= 0x7fffffffLL, BT_ERR_UNSUPPORTED,
              "bt_gemm_qkv_bias_split: a gathered input of %d x %d halfs is beyond 2 GiB", rows_cap, H);
   GemmArgs p{(const half_t *)a, (const half_t *)wt_qkv, (const half_t *)bias_qkv,
-             (half_t *)qkv_heads, valid_rows, a_row_index, rows_cap, 3 * H, H, 0, rows_hint};
+             (half_t *)qkv_heads, valid_rows, a_row_index, rows_cap, 3 * H, H, 0, rows_hint,
+             nullptr, weight_kn};
   // the head-major split is the layout of the fp16 attention kernels, which are built for
   // 64-wide heads; any other head size keeps the projections token-major [rows_cap, 3H]
   // for bt_attention_generic_f16

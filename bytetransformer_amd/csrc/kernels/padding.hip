@@ -32,7 +32,7 @@ static std::atomic<int> g_attention_qb{-1};
 static std::atomic<int> g_prefetch{1};
 static std::atomic<int> g_prefetch_min_grid{512};
 static std::atomic<int> g_attention_key_split{-1};
-static std::atomic<int> g_prepack_check{2};
+static std::atomic<int> g_layer_prepack{-1};
 static std::atomic<int> g_f32_gemm_tile{-1};
 static std::atomic<int> g_attention_short_limit{0};
 static std::atomic<int> g_attention_xcd_map{2};
@@ -43,10 +43,48 @@ int option_attention_qb() { return g_attention_qb.load(std::memory_order_relaxed
 int option_prefetch() { return g_prefetch.load(std::memory_order_relaxed); }
 int option_prefetch_min_grid() { return g_prefetch_min_grid.load(std::memory_order_relaxed); }
 int option_attention_key_split() { return g_attention_key_split.load(std::memory_order_relaxed); }
+int option_layer_prepack() { return g_layer_prepack.load(std::memory_order_relaxed); }
 
 // ---- offsets ----------------------------------------------------------------
 constexpr int kOffsetThreads = 1024;
 constexpr int kOffsetWaves = kOffsetThreads / kWave;
+
+// Number of row elements >= 0.5 (the length rule of the offsets), counted by one wave.
+// A mask row that has not been touched since the last layer comes from HBM: the wave
+// fetches it with 16-byte loads, four per lane in flight (a row of up to 2048 halfs is one
+// round trip; element by element a 512-token row was eight dependent ones).
+template <typename T>
+__device__ __forceinline__ int wave_row_length(const T *__restrict__ row, int S, int lane) {
+  constexpr int kVec = 16 / (int)sizeof(T);
+  int count = 0;
+  if (S % kVec == 0 && (reinterpret_cast<uintptr_t>(row) & 15) == 0) {
+    constexpr int kUnroll = 4;
+    for (int j0 = 0; j0 < S; j0 += kWave * kVec * kUnroll) {
+      uint4_t raw[kUnroll];
+#pragma unroll
+      for (int u = 0; u < kUnroll; ++u) {
+        const int j = j0 + (u * kWave + lane) * kVec;
+        raw[u] = uint4_t{0u, 0u, 0u, 0u};
+        if (j < S) raw[u] = *(const uint4_t *)(row + j);
+      }
+#pragma unroll
+      for (int u = 0; u < kUnroll; ++u) {
+        const T *e = (const T *)&raw[u];
+#pragma unroll
+        for (int i = 0; i < kVec; ++i) count += (float)e[i] >= 0.5f;
+      }
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) count += __shfl_xor(count, o, 64);
+    return count;
+  }
+  for (int i0 = 0; i0 < S; i0 += kWave) {
+    const int i = i0 + lane;
+    const bool on = (i < S) && ((float)row[i] >= 0.5f);
+    count += __popcll(__ballot(on));
+  }
+  return count;
+}
 
 // Every block recomputes all B lengths (B*S mask elements, a few KB) and the
 // exclusive scan, then writes word_idx for the sequences it owns; block 0 also
@@ -65,13 +103,7 @@ __global__ __launch_bounds__(kOffsetThreads) void build_offsets_kernel(
 
   // one wave per sequence: count row-0 mask elements >= 0.5 with a 64-wide ballot
   for (int b = wave; b < B; b += kOffsetWaves) {
-    const T *row = mask + (size_t)b * S * S;
-    int count = 0;
-    for (int i0 = 0; i0 < S; i0 += kWave) {
-      int i = i0 + lane;
-      bool on = (i < S) && ((float)row[i] >= 0.5f);
-      count += __popcll(__ballot(on));
-    }
+    const int count = wave_row_length(mask + (size_t)b * S * S, S, lane);
     if (lane == 0) s_len[b] = count;
   }
   __syncthreads();
@@ -140,34 +172,28 @@ __global__ __launch_bounds__(kPrefixWaves *kWave) void mask_prefix_kernel(
 }
 
 // ---- layer prologue ------------------------------------------------------------
-// Everything a layer has to know before its first product, in ONE launch: the offsets
+// Everything a layer needs before its first product, in ONE launch: the offsets
 // (blocks below `offset_blocks`, the code of build_offsets_kernel), the prefix-mask
 // verdict slots (every block, one wave per mask row; a wave counts the length of its row's
-// sequence itself, so no block waits for another) and the fingerprint of the weight
-// matrices behind a cached pre-pack (every block hashes its share of 16-byte vectors).
+// sequence itself, so no block waits for another) and the k-contiguous copies of those
+// weight matrices whose product runs faster on one (made afresh in every call, from the
+// weights as they are at that moment: nothing is kept between calls).
 constexpr int kPrologueThreads = 1024;
 constexpr int kPrologueWaves = kPrologueThreads / kWave;
-constexpr int kHealGroups = kPrologueThreads / 256;
+constexpr int kPackGroups = kPrologueThreads / 256;   // 64 x 64 tiles one block transposes at a time
 
-// The fingerprint job belongs to a fixed set of blocks (kHashFirst .. kHashFirst +
-// kHashBlocks - 1, whatever the batch size), each owning a fixed range of the 64 x 64 tiles
-// of the weight set: a block hashes its tiles, compares with ITS record and, when they
-// differ, packs ITS tiles again - no block waits for or talks to another.
-constexpr int kHashFirst = 64;     // blocks below build offsets (at most 64 of them)
-constexpr int kHashBlocks = 192;
-constexpr int kHashUnroll = 4;     // tiles in flight per group of 256 lanes (two 16-byte loads per lane each)
+// The pre-pack job belongs to a fixed set of blocks (kPackFirst .. kPackFirst + kPackBlocks
+// - 1, whatever the batch size), each with an equal share of the 64 x 64 tiles.
+constexpr int kPackFirst = 64;     // blocks below build offsets (at most 64 of them)
+constexpr int kPackBlocks = 192;
 
 struct PrologueWeights {
   const half_t *w[4];        // [K, N] as the caller stores them
-  half_t *wt[4];             // [N, K] cached copies
+  half_t *wt[4];             // [N, K] copies to make
   int K[4], N[4];
   int tiles_n[4];            // 64 x 64 tiles along n
   int tile_end[4];           // tiles up to and including matrix i
-  int count;                 // 0 = no weights to check
-  int sample_mask;           // 0: every row of every tile is fingerprinted; else 4 rows of its 64
-  // per hash block b: state[2b] = fingerprint its tiles' copies were made from,
-  // state[2b + 1] = non-zero once that is recorded (zero: this launch records it)
-  unsigned long long *state;
+  int count;                 // 0 = none
 };
 
 // The attention's balanced work list, built by blocks of their own beyond the others
@@ -179,57 +205,12 @@ struct PrologueList {
   int bq, nqb, heads, padded_rows;
 };
 
-__device__ __forceinline__ unsigned int rotl32(unsigned int v, int s) {
-  return __builtin_amdgcn_alignbit(v, v, 32 - s);
-}
-// 64 bits per 16-byte piece, a function of its four dwords and its position; a fingerprint
-// is the sum of these (commutative: no order between lanes or waves to keep).  With the
-// other three dwords fixed each dword acts on the result through bijections (add, rotate,
-// xor-shift, multiplication by an odd constant), so a change of ONE dword always shows;
-// the two multiplications mix whatever else changes.  About 27 VALU operations per piece:
-// the launch reads a layer's weights at memory speed.
-__device__ __forceinline__ unsigned long long piece_hash(const uint4_t v, unsigned int pos) {
-  unsigned int a = v.x + rotl32(v.z, 15) + pos;
-  unsigned int b = (v.y + rotl32(v.w, 9)) ^ rotl32(pos, 16);
-  a ^= a >> 15;
-  a *= 0x2C1B3C6Du;
-  a ^= a >> 12;
-  b += a;
-  b ^= b >> 16;
-  b *= 0x297A2D39u;
-  b ^= b >> 15;
-  a ^= b;
-  return ((unsigned long long)b << 32) | a;
-}
-__device__ __forceinline__ unsigned long long wave_sum_u64(unsigned long long v) {
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) {
-    const unsigned int lo = __shfl_xor((unsigned int)v, o, 64);
-    const unsigned int hi = __shfl_xor((unsigned int)(v >> 32), o, 64);
-    v += ((unsigned long long)hi << 32) | lo;
-  }
-  return v;
-}
-// popcount of row elements >= 0.5 by one wave (the length rule of the offsets)
-template <typename T>
-__device__ __forceinline__ int wave_row_length(const T *__restrict__ row, int S, int lane) {
-  int count = 0;
-  for (int i0 = 0; i0 < S; i0 += kWave) {
-    const int i = i0 + lane;
-    const bool on = (i < S) && ((float)row[i] >= 0.5f);
-    count += __popcll(__ballot(on));
-  }
-  return count;
-}
-
 template <typename T>
 __global__ __launch_bounds__(kPrologueThreads) void layer_prologue_kernel(
     const T *__restrict__ mask, int *__restrict__ batch_idx, int *__restrict__ word_idx,
     int *__restrict__ seq_order, int *__restrict__ slots, int B, int S, int offset_blocks,
     PrologueWeights pw, PrologueList pl) {
   extern __shared__ __attribute__((aligned(16))) int smem[];
-  __shared__ unsigned long long s_part[kPrologueWaves];
-  __shared__ int s_heal;
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
@@ -320,82 +301,30 @@ __global__ __launch_bounds__(kPrologueThreads) void layer_prologue_kernel(
     if (tid == 0) slots[blockIdx.x] = !any_bad;
   }
 
-  // ---- do the cached weight copies still belong to these weights? ----
-  if (pw.count > 0 && (int)blockIdx.x >= kHashFirst) {
-    const int hb = blockIdx.x - kHashFirst;
+  // ---- k-contiguous copies of the weights that were asked for ----
+  if (pw.count > 0 && (int)blockIdx.x >= kPackFirst) {
+    const int pb = blockIdx.x - kPackFirst;
     const int tiles_all = pw.tile_end[pw.count - 1];
-    const int tile_lo = (int)((long long)tiles_all * hb / kHashBlocks);
-    const int tile_hi = (int)((long long)tiles_all * (hb + 1) / kHashBlocks);
-    // A group of 256 lanes takes one tile at a time: which matrix and where in it is the
-    // same for the whole wave (scalar arithmetic), a lane adds one multiply-add for its
-    // row and two 16-byte loads; kHashUnroll tiles per group are in flight at once.
-    const int group = __builtin_amdgcn_readfirstlane(tid >> 8);
-    const int gt = tid & 255, r0 = gt >> 3, c8 = (gt & 7) * 8;
-    unsigned long long sum = 0;
+    const int tile_lo = (int)((long long)tiles_all * pb / kPackBlocks);
+    const int tile_hi = (int)((long long)tiles_all * (pb + 1) / kPackBlocks);
+    // a group of 256 lanes takes one tile at a time; which matrix and where in it is the
+    // same for the whole group (scalar arithmetic)
+    half_t(*tile)[kTransposePitch] =
+        (half_t(*)[kTransposePitch])((half_t *)smem + (size_t)(tid >> 8) * 64 * kTransposePitch);
 #pragma unroll 1
-    for (int tb = tile_lo; tb < tile_hi; tb += kHealGroups * kHashUnroll) {
-      uint4_t v[kHashUnroll][2];
+    for (int t0 = tile_lo; t0 < tile_hi; t0 += kPackGroups) {
+      const int t = t0 + (tid >> 8);
+      int j = 0, first = 0;
 #pragma unroll
-      for (int i = 0; i < kHashUnroll; ++i) {
-        const int t = tb + i * kHealGroups + group;
-        int j = 0, first = 0;
-#pragma unroll
-        for (int q = 1; q < 4; ++q)
-          if (q < pw.count && t >= pw.tile_end[q - 1]) {
-            j = q;
-            first = pw.tile_end[q - 1];
-          }
-        const int tl = t - first;
-        const int k0 = (tl / pw.tiles_n[j]) * 64, n = (tl % pw.tiles_n[j]) * 64 + c8;
-        const int K = pw.K[j], N = pw.N[j];
-        const half_t *src = pw.w[j];
-#pragma unroll
-        for (int h = 0; h < 2; ++h) {
-          const int k = k0 + r0 + 32 * h;
-          v[i][h] = uint4_t{0u, 0u, 0u, 0u};
-          if (t < tile_hi && (!pw.sample_mask || (h == 0 && (r0 & 7) == 0)) && k < K && n < N)
-            v[i][h] = *(const uint4_t *)(src + (size_t)k * N + n);
+      for (int q = 1; q < 4; ++q)
+        if (q < pw.count && t >= pw.tile_end[q - 1]) {
+          j = q;
+          first = pw.tile_end[q - 1];
         }
-      }
-#pragma unroll
-      for (int i = 0; i < kHashUnroll; ++i) {
-        const int t = tb + i * kHealGroups + group;
-#pragma unroll
-        for (int h = 0; h < 2; ++h)
-          if (t < tile_hi && (!pw.sample_mask || (h == 0 && (r0 & 7) == 0)))
-            sum += piece_hash(v[i][h], (unsigned int)(((t - tile_lo) << 9) + h * 256 + gt));
-      }
-    }
-    sum = wave_sum_u64(sum);
-    if (lane == 0) s_part[wave] = sum;
-    __syncthreads();
-    if (tid == 0) {
-      unsigned long long now = 0;
-      for (int i = 0; i < kPrologueWaves; ++i) now += s_part[i];
-      s_heal = pw.state[2 * hb + 1] != 0 && now != pw.state[2 * hb];
-      pw.state[2 * hb] = now;
-      pw.state[2 * hb + 1] = 1;
-    }
-    __syncthreads();
-    if (s_heal) {
-      // a write that no host-side bookkeeping saw: this block's tiles are packed again
-      half_t(*tile)[kTransposePitch] =
-          (half_t(*)[kTransposePitch])((half_t *)smem + (size_t)(tid >> 8) * 64 * kTransposePitch);
-#pragma unroll 1
-      for (int t0 = tile_lo; t0 < tile_hi; t0 += kHealGroups) {
-        const int t = t0 + (tid >> 8);
-        int j = 0, first = 0;
-#pragma unroll
-        for (int q = 1; q < 4; ++q)
-          if (q < pw.count && t >= pw.tile_end[q - 1]) {
-            j = q;
-            first = pw.tile_end[q - 1];
-          }
-        const int tl = t - first;
-        transpose_tile_64(pw.w[j], pw.wt[j], pw.K[j], pw.N[j], (tl / pw.tiles_n[j]) * 64,
-                          (tl % pw.tiles_n[j]) * 64, tile, tid & 255, t < tile_hi);
-        __syncthreads();
-      }
+      const int tl = t - first;
+      transpose_tile_64(pw.w[j], pw.wt[j], pw.K[j], pw.N[j], (tl / pw.tiles_n[j]) * 64,
+                        (tl % pw.tiles_n[j]) * 64, tile, tid & 255, t < tile_hi);
+      __syncthreads();
     }
   }
 }
@@ -455,10 +384,10 @@ extern "C" int bt_set_option(const char *name, int value) {
     BT_REQUIRE(value >= -1 && value <= 1, BT_ERR_INVALID_ARGUMENT,
                "bt_set_option: attention_key_split=%d must be -1, 0 or 1", value);
     g_attention_key_split.store(value);
-  } else if (!strcmp(name, "prepack_check")) {
-    BT_REQUIRE(value >= 0 && value <= 2, BT_ERR_INVALID_ARGUMENT,
-               "bt_set_option: prepack_check=%d must be 0, 1 or 2", value);
-    g_prepack_check.store(value);
+  } else if (!strcmp(name, "layer_prepack")) {
+    BT_REQUIRE(value >= -1 && value <= 1, BT_ERR_INVALID_ARGUMENT,
+               "bt_set_option: layer_prepack=%d must be -1, 0 or 1", value);
+    g_layer_prepack.store(value);
   } else if (!strcmp(name, "prefetch_min_grid")) {
     BT_REQUIRE(value >= 1 && value <= (1 << 20), BT_ERR_INVALID_ARGUMENT,
                "bt_set_option: prefetch_min_grid=%d outside [1, 2^20]", value);
@@ -482,8 +411,8 @@ extern "C" int bt_get_option(const char *name, int *value) {
     *value = g_prefetch_min_grid.load();
   } else if (!strcmp(name, "attention_key_split")) {
     *value = g_attention_key_split.load();
-  } else if (!strcmp(name, "prepack_check")) {
-    *value = g_prepack_check.load();
+  } else if (!strcmp(name, "layer_prepack")) {
+    *value = g_layer_prepack.load();
   } else if (!strcmp(name, "f32_gemm_tile")) {
     *value = g_f32_gemm_tile.load();
   } else if (!strcmp(name, "attention_short_limit")) {
@@ -534,8 +463,7 @@ extern "C" int bt_layer_prologue(const void *atten_mask, int mask_dtype, int bat
                                  int seq_len, int *batch_idx, int *word_idx, int *seq_order,
                                  int *mask_prefix_slots, void *attention_work_list, int head_num,
                                  int padded_rows, int weight_count, const void *const *w,
-                                 void *const *wt, const int *k, const int *n,
-                                 unsigned long long *prepack_state, void *stream) {
+                                 void *const *wt, const int *k, const int *n, void *stream) {
   BT_REQUIRE(atten_mask && batch_idx && word_idx, BT_ERR_INVALID_ARGUMENT,
              "bt_layer_prologue: null pointer argument");
   BT_REQUIRE(batch_size > 0 && seq_len > 0, BT_ERR_INVALID_ARGUMENT,
@@ -548,17 +476,10 @@ extern "C" int bt_layer_prologue(const void *atten_mask, int mask_dtype, int bat
              "bt_layer_prologue: weight_count=%d outside [0, 4]", weight_count);
   PrologueWeights pw;
   memset(&pw, 0, sizeof(pw));
-  // option "prepack_check": 2 = the weights are fingerprinted whole, 1 = four rows of every
-  // 64 x 64 tile, 0 = the copies are taken on trust (the caller's bookkeeping decides alone)
-  const int check = g_prepack_check.load(std::memory_order_relaxed);
-  if (check == 0) weight_count = 0;
   pw.count = weight_count;
-  pw.sample_mask = check == 1 ? 15 : 0;
   if (weight_count > 0) {
-    BT_REQUIRE(w && wt && k && n && prepack_state, BT_ERR_INVALID_ARGUMENT,
-               "bt_layer_prologue: weights to check need w, wt, k, n and prepack_state");
-    BT_REQUIRE((reinterpret_cast<uintptr_t>(prepack_state) & 7) == 0, BT_ERR_INVALID_ARGUMENT,
-               "bt_layer_prologue: prepack_state must be 8-byte aligned");
+    BT_REQUIRE(w && wt && k && n, BT_ERR_INVALID_ARGUMENT,
+               "bt_layer_prologue: weights to pre-pack need w, wt, k and n");
     long long tiles = 0;
     for (int i = 0; i < weight_count; ++i) {
       BT_REQUIRE(w[i] && wt[i], BT_ERR_INVALID_ARGUMENT,
@@ -581,7 +502,6 @@ extern "C" int bt_layer_prologue(const void *atten_mask, int mask_dtype, int bat
       pw.tiles_n[i] = 1;
       pw.tile_end[i] = (int)tiles;
     }
-    pw.state = prepack_state;
   }
   // the attention's balanced work list, when a launch of this shape uses one
   PrologueList pl;
@@ -602,15 +522,15 @@ extern "C" int bt_layer_prologue(const void *atten_mask, int mask_dtype, int bat
     }
   }
   size_t smem = (3 * (size_t)batch_size + 1) * sizeof(int);
-  const size_t heal = (size_t)kHealGroups * 64 * kTransposePitch * sizeof(half_t);
-  if (weight_count > 0 && smem < heal) smem = heal;
+  const size_t pack = (size_t)kPackGroups * 64 * kTransposePitch * sizeof(half_t);
+  if (weight_count > 0 && smem < pack) smem = pack;
   BT_REQUIRE(smem <= 60 * 1024, BT_ERR_UNSUPPORTED,
              "bt_layer_prologue: batch_size %d too large (limit 5119)", batch_size);
   hipStream_t s = as_stream(stream);
   const int offset_blocks = batch_size < 64 ? batch_size : 64;
   // the verdict slots are an array of kPrefixBlocks entries, one per block; the
-  // fingerprint blocks are the last kHashBlocks of the same grid
-  static_assert(kHashFirst + kHashBlocks == kPrefixBlocks, "one grid for both jobs");
+  // pre-pack blocks are the last kPackBlocks of the same grid
+  static_assert(kPackFirst + kPackBlocks == kPrefixBlocks, "one grid for both jobs");
   const int grid = ((mask_prefix_slots || weight_count > 0) ? kPrefixBlocks : offset_blocks) +
                    (pl.list ? kListBlocks : 0);
   if (mask_dtype == BT_F16)

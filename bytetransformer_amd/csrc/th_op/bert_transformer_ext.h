@@ -3,7 +3,7 @@
 // bytetransformer/th_op/bert_transformer_ext.h:30-117.
 #pragma once
 #include "bytetransformer/bert_transformer.h"
-#include "prepack_cache.h"
+#include "mask_hint_cache.h"
 #include "util.h"
 
 #include <hip/hip_runtime_api.h>
@@ -77,19 +77,12 @@ class BTEncoder : public IBTEncoder {
     c10::DeviceGuard device_guard(input.device());
 
     hipStream_t stream = c10::hip::getCurrentHIPStream(input.device().index()).stream();
-    // While the stream is being captured into a graph the caches stay out of it: the graph
-    // would hold pointers into entries that may be dropped before a replay, a copy made
-    // now would only be recorded, not executed, and the host may not wait for a count.
-    // The layer then packs into its own scratch and builds its offsets inside the graph.
+    // While the stream is being captured into a graph the host may not wait for a count:
+    // the layer then goes without the row-count hint.
     hipStreamCaptureStatus capture_status = hipStreamCaptureStatusNone;
     const bool capturing = hipStreamIsCapturing(stream, &capture_status) != hipSuccess ||
                            capture_status != hipStreamCaptureStatusNone;
-    BertTransformerParam<kOp> param = param_;
-    PrepackCache::Packed packed;   // keeps the copies alive through the call
-    if (!capturing && prepacked_weights(stream, &packed)) {
-      for (int i = 0; i < 4; ++i) param.prepacked_kernels[i] = get_ptr<T>(packed.packed[i]);
-      param.prepack_state = reinterpret_cast<unsigned long long *>(packed.state.data_ptr());
-    }
+    const BertTransformerParam<kOp> &param = param_;
 
     BertTransformer<kOp> encoder(batch_size, head_num_, head_size_, seq_len, use_fused_attention,
                                  is_remove_padding, use_fp32_, model_type);
@@ -102,56 +95,21 @@ class BTEncoder : public IBTEncoder {
           batch_size, seq_len, nullptr, stream
     };
     infer_param.attention_bias = attention_bias.defined() ? get_ptr<T>(attention_bias) : NULL;
-    // The layer rebuilds the offsets from the mask on the device in every call; what the
-    // host keeps per mask tensor is the valid-token count as a hint for tile shapes (the
-    // packed rows only: on the padded rows every row is live).
+    // The layer reads the weights as they are and rebuilds the offsets from the mask on the
+    // device, in every call; all the host keeps between calls is the valid-token count per
+    // mask tensor, as a hint for tile shapes (the packed rows only: on the padded rows
+    // every row is live).
     if (!capturing && encoder.is_remove_padding())
       infer_param.valid_rows_hint = valid_rows_hint(attr_mask, batch_size, seq_len, stream);
     encoder.infer(infer_param);
   }
 
  private:
-  // The four [N, K] weight copies and their fingerprint record, from the process-wide
-  // cache when the same tensors were seen before, else packed now (one launch) and
-  // remembered.  False for float, whose kernels read the weights as stored.
-  bool prepacked_weights(hipStream_t stream, PrepackCache::Packed *out) {
-    if (kOp != OperationType::HALF) return false;
-    auto &cache = PrepackCache::instance();
-    if (!cache.enabled()) return false;
-    const Tensor *const w[4] = {&weights_[0], &weights_[2], &weights_[6], &weights_[8]};
-    for (const Tensor *t : w)
-      if (t->dim() != 2) return false;
-    if (cache.lookup(w, stream, out)) return true;
-    const void *src[4];
-    void *dst[4];
-    int ks[4], ns[4];
-    // one allocation for the four copies: the layer hands the last three to the
-    // attention kernel as one range to warm the cache with
-    int64_t total = 0;
-    for (const Tensor *t : w) total += t->numel();
-    out->block = torch::empty({total}, w[0]->options());
-    int64_t at = 0;
-    for (int i = 0; i < 4; ++i) {
-      out->packed[i] = out->block.narrow(0, at, w[i]->numel()).view({w[i]->size(1), w[i]->size(0)});
-      at += w[i]->numel();
-      src[i] = w[i]->data_ptr();
-      dst[i] = out->packed[i].data_ptr();
-      ks[i] = (int)w[i]->size(0);
-      ns[i] = (int)w[i]->size(1);
-    }
-    check_bt_error(bt_transpose_weights(4, src, dst, ks, ns, stream));
-    // all zero: the prologue of this very call records the fingerprint of what was packed
-    out->state = torch::zeros({BT_PREPACK_STATE_WORDS},
-                              torch::dtype(torch::kInt64).device(w[0]->device()));
-    cache.store(w, stream, *out);
-    return true;
-  }
-
   // The number of valid tokens of this mask, read back once per mask tensor (the one host
   // synchronisation; the reference has one in every call, remove_padding.h:99-100).
   // 0 = unknown.
   int valid_rows_hint(const Tensor &mask, int batch_size, int seq_len, hipStream_t stream) {
-    if (!PrepackCache::instance().enabled() || mask.is_inference()) return 0;
+    if (!caches_enabled().load(std::memory_order_relaxed) || mask.is_inference()) return 0;
     auto &cache = MaskHintCache::instance();
     int count = 0;
     if (cache.lookup(mask, stream, &count)) return count;

@@ -49,12 +49,9 @@ Tensor bert_transformer_layer(int64_t head_num, int64_t head_size, Tensor qkv_ke
   return output;
 }
 
-// The operator's caches (pre-packed weight copies, valid-token counts of masks): dropped /
-// switched on and off.  They never change a result, so these are for memory and timing.
-void clear_caches() {
-  torch_ext::PrepackCache::instance().clear();
-  torch_ext::MaskHintCache::instance().clear();
-}
+// The operator's cache (valid-token counts of mask tensors, a hint for tile shapes): dropped /
+// switched on and off.  It never changes a result, so these are for timing experiments.
+void clear_caches() { torch_ext::MaskHintCache::instance().clear(); }
 
 void set_caches_enabled(bool enabled) {
   torch_ext::caches_enabled().store(enabled);

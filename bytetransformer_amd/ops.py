@@ -9,7 +9,6 @@ import torch
 from ._lib import kernel_lib
 
 BT_F32, BT_F16 = 0, 1
-PREPACK_STATE_WORDS = 384     # BT_PREPACK_STATE_WORDS of include/bt_hip.h
 
 
 class BtError(RuntimeError):
@@ -78,13 +77,13 @@ def mask_is_prefix(mask, batch_idx):
     return bool(verdict.value)
 
 
-def layer_prologue(mask, want_slots=False, weights=None, packed=None, state=None, out=None,
+def layer_prologue(mask, want_slots=False, weights=None, packed=None, out=None,
                    work_list=None, head_num=0, padded_rows=False):
     """bt_layer_prologue: offsets of `mask`, optionally the prefix-mask verdict slots and the
-    check of pre-packed copies `packed` against `weights` (fingerprint record `state`,
-    int64[PREPACK_STATE_WORDS], zero when the copies were made).  Returns (batch_idx, word_idx, seq_order, slots or None); `out` = such a
-    tuple to write into.  work_list (int32[entries, 4], with head_num and padded_rows): also
-    filled with the attention's balanced order, as attention_worklist would."""
+    [n, k] copies `packed` of the [k, n] `weights` (up to four).  Returns (batch_idx,
+    word_idx, seq_order, slots or None); `out` = such a tuple to write into.  work_list
+    (int32[entries, 4], with head_num and padded_rows): also filled with the attention's
+    balanced order, as attention_worklist would."""
     B, S = mask.shape[0], mask.shape[1]
     dev = mask.device
     if out is not None:
@@ -96,19 +95,25 @@ def layer_prologue(mask, want_slots=False, weights=None, packed=None, state=None
         slots = torch.full((256,), -1, dtype=torch.int32, device=dev) if want_slots else None
     n = len(weights) if weights else 0
     if n:
+        for w, t in zip(weights, packed):
+            if tuple(t.shape) != tuple(w.shape[::-1]) or t.dtype != w.dtype:
+                raise ValueError("packed copies must be the [n, k] counterparts of the weights")
         src = (ctypes.c_void_p * n)(*[_ptr(w).value for w in weights])
         dst = (ctypes.c_void_p * n)(*[_ptr(w).value for w in packed])
         ks = (ctypes.c_int * n)(*[w.shape[0] for w in weights])
         ns = (ctypes.c_int * n)(*[w.shape[1] for w in weights])
-        if state.dtype != torch.int64 or state.numel() != PREPACK_STATE_WORDS:
-            raise BtError("state must be an int64[%d] tensor" % PREPACK_STATE_WORDS)
     else:
         src = dst = ks = ns = None
     _check(kernel_lib().bt_layer_prologue(
         _ptr(mask), _dtype_code(mask), B, S, _ptr(batch_idx), _ptr(word_idx), _ptr(seq_order),
         _ptr(slots), _ptr(work_list), int(head_num), int(padded_rows), n, src, dst, ks, ns,
-        _ptr(state) if n else None, _stream()))
+        _stream()))
     return batch_idx, word_idx, seq_order, slots
+
+
+def gemm_prepack_pays(rows, n, k, epilogue):
+    """bt_gemm_prepack_pays; epilogue: 0 plain, 1 bias + GELU, 2 QKV split."""
+    return bool(kernel_lib().bt_gemm_prepack_pays(int(rows), int(n), int(k), int(epilogue)))
 
 
 def compress(x, batch_idx, word_idx, out=None):
@@ -142,36 +147,61 @@ def transpose_weights(ws, out=None):
     return wts
 
 
-def gemm(a, wt, valid_rows=None, out=None, rows_hint=0):
+def _gemm_shapes(who, a, w, w_kn, out, out_elems_per_row=None):
+    """Shapes the launch is derived from must agree before anything is launched: a weight
+    passed in the wrong layout would otherwise make the kernel write past `out`."""
     rows, K = a.shape
-    N = wt.shape[0]
+    wk, N = w.shape if w_kn else w.shape[::-1]
+    if wk != K:
+        raise ValueError("%s: the weight must be %s with k = %d, got %s"
+                         % (who, "[k, n]" if w_kn else "the [n, k] pre-pack", K, tuple(w.shape)))
+    if out is not None and out.numel() < rows * (out_elems_per_row or N):
+        raise ValueError("%s: out holds %d elements, the launch writes up to %d"
+                         % (who, out.numel(), rows * (out_elems_per_row or N)))
+    return rows, N, K
+
+
+def gemm(a, wt, valid_rows=None, out=None, rows_hint=0, w_kn=False):
+    """a . w; `wt` is the [n, k] pre-pack, or with w_kn the [k, n] weight itself."""
+    rows, N, K = _gemm_shapes("gemm", a, wt, w_kn, out)
     if out is None:
         out = torch.zeros(rows, N, dtype=a.dtype, device=a.device)
     _check(kernel_lib().bt_gemm(_ptr(a), _ptr(wt), _ptr(out), _ptr(valid_rows), rows,
-                                int(rows_hint), N, K, _stream()))
+                                int(rows_hint), N, K, int(w_kn), _stream()))
     return out
 
 
-def gemm_bias_gelu(a, wt, bias, valid_rows=None, out=None, rows_hint=0):
-    rows, K = a.shape
-    N = wt.shape[0]
+def gemm_bias_gelu(a, wt, bias, valid_rows=None, out=None, rows_hint=0, w_kn=False):
+    rows, N, K = _gemm_shapes("gemm_bias_gelu", a, wt, w_kn, out)
+    if bias.numel() != N:
+        raise ValueError("gemm_bias_gelu: bias must have %d elements" % N)
     if out is None:
         out = torch.zeros(rows, N, dtype=a.dtype, device=a.device)
     _check(kernel_lib().bt_gemm_bias_gelu(_ptr(a), _ptr(wt), _ptr(bias), _ptr(out),
                                           _ptr(valid_rows), rows, int(rows_hint), N, K,
-                                          _stream()))
+                                          int(w_kn), _stream()))
     return out
 
 
 def gemm_qkv_bias_split(a, wt_qkv, bias_qkv, head_num, size_per_head=64, valid_rows=None,
-                        out=None, a_row_index=None, rows_cap=None, rows_hint=0):
+                        out=None, a_row_index=None, rows_cap=None, rows_hint=0, w_kn=False):
     rows = a.shape[0] if rows_cap is None else rows_cap
+    H = head_num * size_per_head
+    want = (H, 3 * H) if w_kn else (3 * H, H)
+    if tuple(wt_qkv.shape) != want or a.shape[1] != H or bias_qkv.numel() != 3 * H:
+        raise ValueError("gemm_qkv_bias_split: a [*, %d], weight %s and bias [%d] expected"
+                         % (H, list(want), 3 * H))
+    if a_row_index is None and a.shape[0] < rows:
+        raise ValueError("gemm_qkv_bias_split: a has fewer rows than rows_cap")
+    if out is not None and out.numel() < rows * 3 * H:
+        raise ValueError("gemm_qkv_bias_split: out holds %d elements, the launch writes up to %d"
+                         % (out.numel(), rows * 3 * H))
     if out is None:
         out = torch.zeros(3, head_num, rows, size_per_head, dtype=a.dtype, device=a.device)
     _check(kernel_lib().bt_gemm_qkv_bias_split(_ptr(a), _ptr(a_row_index), _ptr(wt_qkv),
                                                _ptr(bias_qkv), _ptr(out),
                                                _ptr(valid_rows), rows, int(rows_hint), head_num,
-                                               size_per_head, _stream()))
+                                               size_per_head, int(w_kn), _stream()))
     return out
 
 
@@ -182,10 +212,16 @@ def _attention(fn, qkv_heads, batch_idx, batch_size, seq_len, scale, padded_rows
         out = torch.zeros(rows_cap, head_num * d, dtype=qkv_heads.dtype, device=qkv_heads.device)
     if bias is not None and tuple(bias.shape) != (head_num, seq_len, seq_len):
         raise ValueError("attention bias must be [head_num, seq_len, seq_len]")
+    # prefetch: one tensor or up to four, the ranges later kernels will read
+    ranges = [] if prefetch is None else ([prefetch] if torch.is_tensor(prefetch) else list(prefetch))
+    n = len(ranges)
+    ptrs = (ctypes.c_void_p * max(n, 1))(*[t.data_ptr() for t in ranges])
+    sizes = (ctypes.c_ulonglong * max(n, 1))(*[t.numel() * t.element_size() for t in ranges])
+    for t in ranges:
+        _ptr(t)
     _check(fn(_ptr(qkv_heads), _ptr(out), _ptr(batch_idx), _ptr(seq_order), _ptr(mask), _ptr(bias),
               batch_size, seq_len, rows_cap, head_num, d, float(scale), int(padded_rows),
-              _ptr(prefetch), prefetch.numel() * prefetch.element_size() if prefetch is not None else 0,
-              *extra, _stream()))
+              ptrs, sizes, n, *extra, _stream()))
     return out
 
 
@@ -249,14 +285,16 @@ def add_bias_residual_layernorm_restore(out, residual, bias, gamma, beta, batch_
     return out_padded
 
 
-def gemm_splitk(a, wt, splits, valid_rows=None, out=None):
-    """fp32 partial sums [splits, rows, N] of a . wt^T over `splits` k ranges."""
-    rows, K = a.shape
-    N = wt.shape[0]
+def gemm_splitk(a, wt, splits, valid_rows=None, out=None, w_kn=False):
+    """fp32 partial sums [splits, rows, N] of a . w over `splits` k ranges."""
+    rows, N, K = _gemm_shapes("gemm_splitk", a, wt, w_kn, None)
+    if out is not None and out.numel() < splits * rows * N:
+        raise ValueError("gemm_splitk: out holds %d elements, the launch writes up to %d"
+                         % (out.numel(), splits * rows * N))
     if out is None:
         out = torch.zeros(splits, rows, N, dtype=torch.float32, device=a.device)
     _check(kernel_lib().bt_gemm_splitk(_ptr(a), _ptr(wt), _ptr(out), int(splits), _ptr(valid_rows),
-                                       rows, N, K, _stream()))
+                                       rows, N, K, int(w_kn), _stream()))
     return out
 
 

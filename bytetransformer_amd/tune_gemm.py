@@ -1,10 +1,11 @@
 """Measures every fp16 GEMM tile shape of libbt_hip.so over a grid of row counts for
-the four weight shapes of BERT-base and BERT-large, and writes the table the launcher
-consults (csrc/kernels/gemm_tuned.inc; rebuild the kernels afterwards).
+the four weight shapes of BERT-base and BERT-large, in both weight layouts ([k, n] as
+stored and the [n, k] pre-pack), and writes the table the launcher consults (csrc/kernels/gemm_tuned.inc; rebuild the kernels afterwards).
 
-    python -m bytetransformer_amd.tune_gemm [--json timings.json] [--from-json timings.json]
+    python -m bytetransformer_amd.tune_gemm [--json timings.json] [--from-json run1.json run2.json ...]
 
-Needs a GPU unless --from-json replays earlier measurements.  Shapes outside the table
+Needs a GPU unless --from-json replays earlier measurements; several runs (ideally from
+several machines) are merged by the median of each entry.  Shapes outside the table
 keep using the launcher's analytic cost model."""
 import argparse
 import json
@@ -47,7 +48,8 @@ def measure(iters=32):
     padded batch: launches are sized for batch x seq_len rows, of which m are live), the
     QKV product gathering its rows from the padded input through a word_idx of 16 runs, and
     with the weights cold: the launches of one timing loop walk through enough copies of
-    the weight matrix to exceed the memory-side cache, as the layers of a model do."""
+    the weight matrix to exceed the memory-side cache, as the layers of a model do.  Every
+    shape is timed with the weight in both layouts."""
     import torch
     from . import ops
     dev = torch.device("cuda:0")
@@ -61,8 +63,8 @@ def measure(iters=32):
                               ("plain", h, 4 * h)):
                 a = torch.randn(rows_cap, k, device=dev).half()
                 copies = min(iters, max(2, -(-300 * 2 ** 20 // (n * k * 2))))
-                wts = [ops.transpose_weight((torch.randn(k, n, device=dev) * 0.02).half())
-                       for _ in range(copies)]
+                ws = [(torch.randn(k, n, device=dev) * 0.02).half() for _ in range(copies)]
+                wts = [ops.transpose_weight(w) for w in ws]
                 bias = torch.zeros(n, device=dev, dtype=torch.float16)
                 c = torch.empty(rows_cap * n, device=dev, dtype=torch.float16)
                 for m in M_GRID:
@@ -74,51 +76,73 @@ def measure(iters=32):
                                          - (m * b) // 16, dtype=torch.int32) for b in range(16)]
                     word_idx = torch.cat(runs + [torch.zeros(cap - m, dtype=torch.int32)]).to(dev)
 
+                    kn = [False]
+
                     def call():
-                        wt = wts[turn[0] % copies]
+                        wt = (ws if kn[0] else wts)[turn[0] % copies]
                         turn[0] += 1
                         if epi == "qkv":
                             ops.gemm_qkv_bias_split(a[:cap], wt, bias, heads, valid_rows=vr,
-                                                    rows_hint=m, a_row_index=word_idx,
+                                                    rows_hint=m, a_row_index=word_idx, w_kn=kn[0],
                                                     out=c[:3 * cap * k].view(3, heads, cap, 64))
                         elif epi == "gelu":
                             ops.gemm_bias_gelu(a[:cap], wt, bias, valid_rows=vr, rows_hint=m,
-                                               out=c[:cap * n].view(cap, n))
+                                               out=c[:cap * n].view(cap, n), w_kn=kn[0])
                         else:
                             ops.gemm(a[:cap], wt, valid_rows=vr, rows_hint=m,
-                                     out=c[:cap * n].view(cap, n))
+                                     out=c[:cap * n].view(cap, n), w_kn=kn[0])
 
                     ops.set_option("gemm_tile", 1)
                     _time_kernel(call, 8)      # warm the clocks for this shape
-                    us = {}
-                    for tile in TILES:
-                        if tile == 4 and m > SMALL_TILE_MAX_ROWS:
-                            continue
-                        ops.set_option("gemm_tile", tile)
-                        us[str(tile)] = round(_time_kernel(call, iters), 2)
-                    row = {"M": m, "N": n, "K": k, "epi": epi, "us": us}
-                    out.append(row)
-                    print(json.dumps(row), flush=True)
+                    for layout in (0, 1):
+                        kn[0] = bool(layout)
+                        us = {}
+                        for tile in TILES:
+                            if tile == 4 and m > SMALL_TILE_MAX_ROWS:
+                                continue
+                            ops.set_option("gemm_tile", tile)
+                            us[str(tile)] = round(_time_kernel(call, iters), 2)
+                        row = {"M": m, "N": n, "K": k, "epi": epi, "kn": layout, "us": us}
+                        out.append(row)
+                        print(json.dumps(row), flush=True)
     finally:
         ops.set_option("gemm_tile", -1)
     return out
 
 
+def merge_runs(rows):
+    """One row per (shape, layout, row count): the median of every tile's time over the runs
+    that measured it.  Boxes differ (one of four runs here had every loader-wave tile 20-30 %
+    slower than the others), and a table from one box alone inherits its quirks."""
+    import statistics
+    seen = {}
+    for r in rows:
+        key = (r["M"], r["N"], r["K"], r.get("epi", "plain"), r.get("kn", 0))
+        for tile, us in r["us"].items():
+            seen.setdefault(key, {}).setdefault(tile, []).append(us)
+    return [{"M": m, "N": n, "K": k, "epi": epi, "kn": kn,
+             "us": {t: round(statistics.median(v), 2) for t, v in by_tile.items()}}
+            for (m, n, k, epi, kn), by_tile in seen.items()]
+
+
 def write_inc(rows, path=INC):
     shapes = {}
-    for r in rows:
-        shapes.setdefault((r["N"], r["K"], EPI_CODE[r.get("epi", "plain")]), {})[r["M"]] = r["us"]
+    for r in merge_runs(rows):
+        shapes.setdefault((r["N"], r["K"], EPI_CODE[r.get("epi", "plain")], r.get("kn", 0)),
+                          {})[r["M"]] = r["us"]
     lines = ["// Generated by `python -m bytetransformer_amd.tune_gemm` from timings on one MI355X:",
              "// microseconds per launch of each tile shape (index = tile id; 0 = not measured)",
-             "// at kTunedRows live rows, per weight shape.  Do not edit by hand.",
+             "// at kTunedRows live rows, per weight shape and weight layout.  Do not edit by hand.",
              "constexpr int kTunedPoints = %d;" % len(M_GRID),
              "constexpr int kTunedTiles = %d;" % len(TILES),
              "constexpr int kTunedStep = %d;" % M_STEP,
              "static const int kTunedRows[kTunedPoints] = {%s};" % ", ".join(map(str, M_GRID)),
-             "struct TunedShape {", "  int n, k, epi;   // epi: the Epilogue the shape was timed with", "  float us[kTunedPoints][kTunedTiles];", "};",
+             "struct TunedShape {",
+             "  int n, k, epi, kn;   // epi: the Epilogue the shape was timed with; kn: 1 = [k, n] weight",
+             "  float us[kTunedPoints][kTunedTiles];", "};",
              "static const TunedShape kTunedShapes[] = {"]
-    for (n, k, epi), by_m in sorted(shapes.items()):
-        lines.append("    {%d, %d, %d, {" % (n, k, epi))
+    for (n, k, epi, kn), by_m in sorted(shapes.items()):
+        lines.append("    {%d, %d, %d, %d, {" % (n, k, epi, kn))
         for m in M_GRID:
             us = by_m.get(m, {})
             lines.append("        {%s},   // %d rows" % (

@@ -56,12 +56,8 @@ const char *bt_last_error_string(void);
  *   "attention_key_split"  -1 heuristic | 0 | 1: the 64-query streaming attention with four waves,
  *                   or with eight: two groups of four take alternate 64-key halves of every ring
  *                   slot and are merged at the end
- *   "prepack_check" 2 (default) | 1 | 0: how bt_layer_prologue checks reused weight copies:
- *                   the weights are fingerprinted whole | four rows of every 64 x 64 tile
- *                   (a write that touches every row is still seen, at a sixteenth of the
- *                   reads) | not at all (the caller's bookkeeping is trusted).  The one option
- *                   that can change results: below 2, a write to the weights that the caller's
- *                   bookkeeping misses can leave stale copies in use
+ *   "layer_prepack" -1 (default) | 0 | 1: answer of bt_gemm_prepack_pays: by the measured
+ *                   table | never | always
  *   "prefetch"      1 (default) | 0: honour / ignore the prefetch hint of the attention entries
  *   "prefetch_min_grid"  512 (default): attention launches of fewer workgroups ignore the hint
  *                   (there the warm-up costs more than it returns); 1 = every launch honours it
@@ -128,23 +124,17 @@ int bt_mask_is_prefix(const void *atten_mask, int mask_dtype, int batch_size, in
  *   - attention_work_list (nullable; needs head_num and padded_rows): the list of
  *     bt_attention_worklist for these offsets, when launches of this shape use one
  *     (bt_attention_worklist_bytes > 0; else nothing is written);
- *   - weight_count in [0, 4] matrices w[i] ([k[i], n[i]] as the caller stores them) whose
- *     pre-packed copies wt[i] ([n[i], k[i]], bt_transpose_weights) are being reused from an
- *     earlier call: 192 workgroups each fingerprint their fixed share of the w[i] (64 bits
- *     over every dword and its position) and compare with their record in prepack_state;
- *     a workgroup whose fingerprint moved - the weights were overwritten in a way the owner
- *     of the copies did not see - packs its share again inside this launch, so later
- *     launches of the stream never read copies of other weights.  prepack_state: device
- *     unsigned long long[BT_PREPACK_STATE_WORDS], all zero when the copies are made (the
- *     first prologue then records the fingerprints), owned by whoever owns the copies and
- *     used by one stream at a time.
+ *   - weight_count in [0, 4] matrices w[i] ([k[i], n[i]] as the caller stores them) to
+ *     pre-pack into wt[i] ([n[i], k[i]], as bt_transpose_weights does) for the products of
+ *     this call (see bt_gemm_prepack_pays): made afresh in every call from the weights as
+ *     they are at that moment - nothing is remembered between calls, so nothing can go
+ *     stale.
  */
-#define BT_PREPACK_STATE_WORDS 384
 int bt_layer_prologue(const void *atten_mask, int mask_dtype, int batch_size, int seq_len,
                       int *batch_idx, int *word_idx, int *seq_order, int *mask_prefix_slots,
                       void *attention_work_list, int head_num, int padded_rows, int weight_count,
                       const void *const *w, void *const *wt, const int *k, const int *n,
-                      unsigned long long *prepack_state, void *stream);
+                      void *stream);
 
 /*
  * Gather valid rows: to_tensor[t, :] = from_tensor[word_idx[t], :], t < M.
@@ -156,9 +146,10 @@ int bt_compress(const void *from_tensor, void *to_tensor, const int *batch_idx,
 
 /*
  * Weight pre-pack: wt[n, k] = w[k, n].  The reference hands cuBLAS the
- * [in, out] row-major weight directly (gemm.cu:27-39); the MFMA kernels here
- * want both operands contiguous along k, so the host transposes each weight
- * once per infer() into scratch.  k % 8 == 0, n % 8 == 0.
+ * [in, out] row-major weight directly (gemm.cu:27-39), and so do the per-layer entries
+ * here (weight_kn = 1 of the products below).  A caller that owns an immutable copy of
+ * its weights can pre-pack them once with this and pass weight_kn = 0: both operands
+ * are then contiguous along k.  k % 8 == 0, n % 8 == 0.
  */
 int bt_transpose_weight(const void *w, void *wt, int k, int n, void *stream);
 
@@ -171,11 +162,29 @@ int bt_transpose_weights(int count, const void *const *w, void *const *wt, const
  * c[rows, n] = a[rows, k] . w[k, n], fp16 in/out, fp32 accumulate on MFMA.
  * Replaces dense_layer_kernel_launcher (bytetransformer/src/gemm.cu:32-39) at
  * its attention-output-projection and FFN2 call sites
- * (bert_transformer.cu:102-104,115-117).  `wt` is the [n, k] pre-packed weight.
- * k % 64 == 0, n % 8 == 0.
+ * (bert_transformer.cu:102-104,115-117).  k % 64 == 0, n % 8 == 0.
+ * weight_kn (all fp16 products): 1 = `wt` is the row-major [k, n] weight itself, as the
+ * reference hands it to cuBLAS - nothing to prepare, nothing that could go stale;
+ * 0 = `wt` is the [n, k] copy made by bt_transpose_weights, for callers that own an
+ * immutable copy of the weights (the whole-encoder object): the 256 x 256 tile runs
+ * about 10 % faster on it.  Results are bit-identical either way.
  */
 int bt_gemm(const void *a, const void *wt, void *c, const int *valid_rows, int rows_cap,
-            int rows_hint, int n, int k, void *stream);
+            int rows_hint, int n, int k, int weight_kn, void *stream);
+
+/* Epilogue codes of the question below. */
+#define BT_EPILOGUE_PLAIN 0
+#define BT_EPILOGUE_BIAS_GELU 1
+#define BT_EPILOGUE_QKV_SPLIT 2
+/*
+ * 1 when, by the measured tile table, the product of about `rows` live rows with an
+ * [k, n] weight and this epilogue runs faster on a pre-packed copy even after paying for
+ * the copy (made per call inside bt_layer_prologue), else 0 - shapes outside the table
+ * included.  bt_set_option("layer_prepack", 0 | 1) overrides the table.  Only ever a
+ * matter of time: the products' results do not depend on the layout.  No counterpart in
+ * the reference.
+ */
+int bt_gemm_prepack_pays(long long rows, int n, int k, int epilogue);
 
 /*
  * c = gelu_tanh(a . w + bias).  Replaces gemm_bias_gelu
@@ -184,7 +193,7 @@ int bt_gemm(const void *a, const void *wt, void *c, const int *valid_rows, int r
  */
 int bt_gemm_bias_gelu(const void *a, const void *wt, const void *bias, void *c,
                       const int *valid_rows, int rows_cap, int rows_hint, int n, int k,
-                      void *stream);
+                      int weight_kn, void *stream);
 
 /*
  * QKV projection with the bias add and the head split fused into the store:
@@ -203,7 +212,7 @@ int bt_gemm_bias_gelu(const void *a, const void *wt, const void *bias, void *c,
 int bt_gemm_qkv_bias_split(const void *a, const int *a_row_index, const void *wt_qkv,
                            const void *bias_qkv, void *qkv_heads, const int *valid_rows,
                            int rows_cap, int rows_hint, int head_num, int size_per_head,
-                           void *stream);
+                           int weight_kn, void *stream);
 
 /*
  * Fused multi-head attention over the head-major Q/K/V written by
@@ -225,11 +234,12 @@ int bt_gemm_qkv_bias_split(const void *a, const int *a_row_index, const void *wt
  *                     term, as the reference's unfused softmax does (softmax.h:41-46,
  *                     attention_nofused.cu:78-95); positions are relative to the
  *                     start of the sequence in both row layouts.
- *   prefetch, prefetch_bytes (nullable / 0): a readable device range that LATER kernels
- *                     of the stream will read, typically the layer's remaining weight
- *                     matrices.  Workgroups that retire early touch it line by line so
- *                     that it sits in the memory-side cache by then; purely a hint, the
- *                     results do not depend on it.  No counterpart in the reference.
+ *   prefetch, prefetch_bytes, prefetch_count (nullable / 0): up to 4 readable device
+ *                     ranges (host arrays of pointers and sizes) that LATER kernels of the
+ *                     stream will read, typically the layer's remaining weight matrices.
+ *                     Workgroups that retire early touch them line by line so that they
+ *                     sit in the memory-side cache by then; purely a hint, the results do
+ *                     not depend on it.  No counterpart in the reference.
  *   seq_order (nullable): a permutation of the sequence indices from
  *                     bt_build_offsets; workgroups are issued in that order so the
  *                     longest sequences start first.  Results do not depend on it.
@@ -254,14 +264,16 @@ int bt_gemm_qkv_bias_split(const void *a, const int *a_row_index, const void *wt
 int bt_attention_short(const void *qkv_heads, void *attention_output, const int *batch_idx,
                        const int *seq_order, const void *atten_mask, const void *attention_bias,
                        int batch_size, int seq_len, int rows_cap, int head_num, int size_per_head,
-                       float scale, int padded_rows, const void *prefetch,
-                       unsigned long long prefetch_bytes, void *stream);
+                       float scale, int padded_rows, const void *const *prefetch,
+                       const unsigned long long *prefetch_bytes, int prefetch_count,
+                       void *stream);
 
 int bt_attention_grouped(const void *qkv_heads, void *attention_output, const int *batch_idx,
                          const int *seq_order, const void *atten_mask, const void *attention_bias,
                          int batch_size, int seq_len, int rows_cap, int head_num,
-                         int size_per_head, float scale, int padded_rows, const void *prefetch,
-                         unsigned long long prefetch_bytes, const int *mask_prefix_slots,
+                         int size_per_head, float scale, int padded_rows,
+                         const void *const *prefetch, const unsigned long long *prefetch_bytes,
+                         int prefetch_count, const int *mask_prefix_slots,
                          const void *work_list, void *stream);
 
 /*
@@ -326,7 +338,7 @@ int bt_add_bias_residual_layernorm_restore(const void *out, const void *residual
  * rows_cap that bt_gemm_splitk was given.
  */
 int bt_gemm_splitk(const void *a, const void *wt, void *partials, int splits,
-                   const int *valid_rows, int rows_cap, int n, int k, void *stream);
+                   const int *valid_rows, int rows_cap, int n, int k, int weight_kn, void *stream);
 
 int bt_splitk_layernorm(const void *partials, int splits, const void *residual,
                         const int *residual_row_index, const void *bias, const void *gamma,

@@ -41,8 +41,9 @@ struct AttentionInferParam {
   const int *seq_order = nullptr;
   // Extension: a device range later kernels of the stream will read (the layer's
   // remaining weights); the attention kernel warms the memory-side cache with it.
-  const void *prefetch = nullptr;
-  unsigned long long prefetch_bytes = 0;
+  const void *prefetch[4] = {nullptr, nullptr, nullptr, nullptr};
+  unsigned long long prefetch_bytes[4] = {0, 0, 0, 0};
+  int prefetch_count = 0;
   // Extension: what the caller knows about atten_mask: 1 = the plain prefix mask of
   // et_param's lengths (the padded rows then need no mask tensor: keys stop at each length,
   // the same result), 0 = something else, -1 = not checked.

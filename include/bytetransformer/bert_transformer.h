@@ -39,18 +39,12 @@ class BertTransformerParam {
 
   int cublas_Algo[3] = {Traits_::algo, Traits_::algo, Traits_::algo};  // unused, kept for callers
 
-  // Extension (no counterpart in the reference): the four weight matrices already
-  // pre-packed k-contiguous by bt_transpose_weights, in the order QKV [3H,H],
-  // attention output [H,H], FFN1 [F,H], FFN2 [H,F].  When all four are set,
-  // infer() uses them and skips its own pre-pack launch; the caller vouches that
-  // they match the *_kernel tensors above.
+  // Extension (no counterpart in the reference): k-contiguous copies of the four weight
+  // matrices as bt_transpose_weights makes them, in the order QKV [3H,H], attention
+  // output [H,H], FFN1 [F,H], FFN2 [H,F], for a caller that owns copies of immutable
+  // weights and vouches that they match the *_kernel tensors above.  Left null, infer()
+  // reads the *_kernel tensors as they are stored, in every call.
   const DataType_ *prepacked_kernels[4] = {nullptr, nullptr, nullptr, nullptr};
-  // ... and, optionally, the fingerprint record of those copies (device unsigned long
-  // long[BT_PREPACK_STATE_WORDS], all zero when the copies were made; see bt_layer_prologue).  When set, every
-  // infer() checks on the device that the *_kernel tensors still hold what the copies were
-  // made from and makes the copies again if not, so a caller that reuses copies across calls
-  // need not vouch for anything.  One stream at a time.
-  unsigned long long *prepack_state = nullptr;
 };
 
 template <typename T>

@@ -42,18 +42,27 @@ def test_host_library_exports_every_declared_symbol():
 def test_argument_validation_returns_codes_without_gpu():
     lib = bt.kernel_lib()
     err = lambda: lib.bt_last_error_string().decode()
-    assert lib.bt_gemm(None, None, None, None, 4, 0, 8, 64, None) == 1 and "null pointer" in err()
+    assert lib.bt_gemm(None, None, None, None, 4, 0, 8, 64, 0, None) == 1 and "null pointer" in err()
     p = ctypes.c_void_p(256)   # never dereferenced: validation fails first
-    assert lib.bt_gemm(p, p, p, None, 4, 0, 8, 100, None) == 2 and "multiple of 64" in err()
-    assert lib.bt_gemm(p, p, p, None, 4, 0, 12, 64, None) == 2 and "multiple of 8" in err()
-    assert lib.bt_gemm_qkv_bias_split(p, None, p, p, p, None, 4, 0, 1, 32, None) == 2
+    assert lib.bt_gemm(p, p, p, None, 4, 0, 8, 100, 0, None) == 2 and "multiple of 64" in err()
+    assert lib.bt_gemm(p, p, p, None, 4, 0, 12, 64, 1, None) == 2 and "multiple of 8" in err()
+    assert lib.bt_gemm(p, p, p, None, 4, 0, 8, 64, 2, None) == 1 and "weight_kn" in err()
+    assert lib.bt_gemm(p, p, p, None, 4, 0, 1 << 20, 1 << 11, 1, None) == 2 and "2 GiB" in err()
+    # the layout question: forced answers, and 0 for a shape outside the measured table
+    assert lib.bt_gemm_prepack_pays(5000, 520, 64, 0) == 0
+    for forced in (1, 0):
+        assert lib.bt_set_option(b"layer_prepack", forced) == 0
+        assert lib.bt_gemm_prepack_pays(5000, 3072, 768, 1) == forced
+    assert lib.bt_set_option(b"layer_prepack", -1) == 0
+    assert lib.bt_set_option(b"layer_prepack", 2) == 1
+    assert lib.bt_gemm_qkv_bias_split(p, None, p, p, p, None, 4, 0, 1, 32, 0, None) == 2
     assert "multiple of 64" in err()        # hidden = 1 * 32
-    assert lib.bt_gemm_qkv_bias_split(p, p, p, p, p, None, 4, 0, 12, 64, None) == 1
+    assert lib.bt_gemm_qkv_bias_split(p, p, p, p, p, None, 4, 0, 12, 64, 1, None) == 1
     assert "needs valid_rows" in err()
-    assert lib.bt_attention_short(p, p, p, None, None, None, 1, 1024, 1024, 12, 64, 0.125, 0, None, 0, None) == 2
+    assert lib.bt_attention_short(p, p, p, None, None, None, 1, 1024, 1024, 12, 64, 0.125, 0, None, None, 0, None) == 2
     assert "exceeds 512" in err()
-    assert lib.bt_attention_grouped(p, p, p, None, None, None, 1, 16, 16, 12, 48, 0.125, 0, None, 0, None, None, None) == 2
-    assert lib.bt_attention_grouped(p, p, p, None, p, None, 1, 16, 16, 12, 64, 0.125, 0, None, 0, None, None, None) == 1
+    assert lib.bt_attention_grouped(p, p, p, None, None, None, 1, 16, 16, 12, 48, 0.125, 0, None, None, 0, None, None, None) == 2
+    assert lib.bt_attention_grouped(p, p, p, None, p, None, 1, 16, 16, 12, 64, 0.125, 0, None, None, 0, None, None, None) == 1
     assert "only applied on padded rows" in err()
     assert lib.bt_compress(p, p, p, p, 2, 4, 12, None) == 2 and "multiple of 8" in err()
     assert lib.bt_build_offsets(p, 7, 2, 4, p, p, None, None, None) == 1 and "dtype" in err()
@@ -64,7 +73,7 @@ def test_argument_validation_returns_codes_without_gpu():
                                                       None) == 1
     assert lib.bt_transpose_weight(None, p, 8, 8, None) == 1
     odd = ctypes.c_void_p(264)   # 8-byte aligned only
-    assert lib.bt_gemm(odd, p, p, None, 4, 0, 8, 64, None) == 1 and "16-byte aligned" in err()
+    assert lib.bt_gemm(odd, p, p, None, 4, 0, 8, 64, 0, None) == 1 and "16-byte aligned" in err()
     assert lib.bt_add_bias_residual_layernorm(p, odd, None, p, p, p, 0, None, 4, 64, 1e-6, None) == 1
     assert "16-byte aligned" in err()
     # float entry points

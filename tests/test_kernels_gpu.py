@@ -46,6 +46,44 @@ def test_build_offsets_bit_exact(device, B, S, dtype):
     assert np.array_equal(g_wi.cpu().numpy()[:M], wi)
 
 
+# Every product test runs with the weight in both layouts: the [n, k] pre-pack and the
+# [k, n] matrix as the layer stores it.
+_KN = [False]
+
+
+@pytest.fixture(autouse=True)
+def weight_layout(request):
+    _KN[0] = getattr(request, "param", "nk") == "kn"
+    yield
+    _KN[0] = False
+
+
+def pytest_generate_tests(metafunc):
+    name = metafunc.function.__name__
+    if ("gemm" in name or "splitk" in name) and "weight_layout" in metafunc.fixturenames:
+        metafunc.parametrize("weight_layout", ["nk", "kn"], indirect=True)
+
+
+def _prep(w):
+    return w if _KN[0] else ops.transpose_weight(w)
+
+
+def _gemm(*a, **k):
+    return ops.gemm(*a, w_kn=_KN[0], **k)
+
+
+def _gemm_bias_gelu(*a, **k):
+    return ops.gemm_bias_gelu(*a, w_kn=_KN[0], **k)
+
+
+def _gemm_qkv_bias_split(*a, **k):
+    return ops.gemm_qkv_bias_split(*a, w_kn=_KN[0], **k)
+
+
+def _gemm_splitk(*a, **k):
+    return ops.gemm_splitk(*a, w_kn=_KN[0], **k)
+
+
 @pytest.mark.parametrize("B,S,dtype", [(1, 256, np.float16), (16, 512, np.float16),
                                        (3, 7, np.float32), (70, 33, np.float16),
                                        (130, 100, np.float16), (2, 1024, np.float16)])
@@ -80,79 +118,36 @@ def test_layer_prologue_offsets_and_prefix_verdict(device, B, S, dtype, kind):
     assert torch.equal(g_wi2[:M], g_wi[:M])
 
 
-def test_layer_prologue_repacks_weights_that_changed_behind_the_copies(device):
-    """The fingerprint check of reused weight copies: the first prologue records, an
-    unchanged weight set leaves the copies alone, ANY change of the weights - a whole
-    matrix or one element - is seen on the device and the copies are made again."""
-    _say("prologue fingerprint")
+def test_layer_prologue_packs_weights_afresh_in_every_call(device):
+    """The prologue's weight job: [n, k] copies of up to four [k, n] matrices, made in the
+    same launch as the offsets and from the weights as they are at that call - a weight
+    overwritten between two calls (with or without any host-side bookkeeping) is simply
+    packed again."""
+    _say("prologue pre-pack")
     rs = np.random.RandomState(5)
     shapes = [(128, 384), (128, 128), (128, 512), (512, 128)]
     ws = [_dev(rs.standard_normal(s).astype(np.float16), device) for s in shapes]
-    packed = ops.transpose_weights(ws)
-    state = torch.zeros(ops.PREPACK_STATE_WORDS, dtype=torch.int64, device=device)
-    mask = _dev(workload.make_mask([5, 9, 3], 9, np.float16), device)
-
-    def run():
-        ops.layer_prologue(mask, weights=ws, packed=packed, state=state)
-        torch.cuda.synchronize()
-        st = state.cpu().numpy().reshape(-1, 2)
-        assert (st[:, 1] == 1).all()                  # every share has a record
-        return st[:, 0].copy()
-
-    def copies_match():
-        return all(torch.equal(p, w.t().contiguous()) for p, w in zip(packed, ws))
-
-    fp0 = run()
-    assert (fp0 != 0).sum() >= 40                     # 48 tiles over 192 shares: most hold one
-    # poison one copy: unchanged fingerprints must NOT trigger a re-pack
-    keep = packed[1].clone()
-    packed[1].fill_(7)
-    assert np.array_equal(run(), fp0) and torch.equal(packed[1], torch.full_like(keep, 7))
-    packed[1].copy_(keep)
-    # a whole matrix rewritten without any host-side bookkeeping
+    packed = [torch.full((s[1], s[0]), 7, dtype=torch.float16, device=device) for s in shapes]
+    mask_np = workload.make_mask([5, 9, 3], 9, np.float16)
+    mask = _dev(mask_np, device)
+    bi, wi, order, _ = ops.layer_prologue(mask, weights=ws, packed=packed)
+    r_bi, r_wi, M = O.build_offsets(mask_np)
+    assert np.array_equal(bi.cpu().numpy(), r_bi) and np.array_equal(wi.cpu().numpy()[:M], r_wi[:M])
+    assert all(torch.equal(p, w.t().contiguous()) for p, w in zip(packed, ws))
     ws[2].data.copy_(_dev(rs.standard_normal(shapes[2]).astype(np.float16), device))
-    assert not copies_match()
-    fp1 = run()
-    assert (fp1 != fp0).sum() >= 8 and copies_match()  # FFN1's 16 tiles moved, nothing else
-    # one element of the last matrix: exactly one share notices
     ws[3].data[511, 127] += 1
-    fp2 = run()
-    assert (fp2 != fp1).sum() == 1 and copies_match()
-    # two elements of one tile swapped (the position is part of the fingerprint)
-    a, b = ws[0].data[0, 0].clone(), ws[0].data[5, 7].clone()
-    ws[0].data[0, 0], ws[0].data[5, 7] = b, a
-    fp3 = run()
-    assert ((fp3 != fp2).sum() == 1) == bool(a != b) and copies_match()
-    # option prepack_check: 1 = four rows of every tile are fingerprinted (a rewrite of a whole
-    # matrix is still seen), 0 = the copies are taken on trust (nothing is read or repaired)
-    ops.set_option("prepack_check", 1)
-    try:
-        sampled = torch.zeros(ops.PREPACK_STATE_WORDS, dtype=torch.int64, device=device)
-        ops.layer_prologue(mask, weights=ws, packed=packed, state=sampled)
-        ws[1].data.copy_(_dev(rs.standard_normal(shapes[1]).astype(np.float16), device))
-        ops.layer_prologue(mask, weights=ws, packed=packed, state=sampled)
-        torch.cuda.synchronize()
-        assert copies_match()
-        ops.set_option("prepack_check", 0)
-        before = [p.clone() for p in packed]
-        ws[1].data.copy_(_dev(rs.standard_normal(shapes[1]).astype(np.float16), device))
-        untouched = sampled.clone()
-        ops.layer_prologue(mask, weights=ws, packed=packed, state=sampled)
-        torch.cuda.synchronize()
-        assert torch.equal(sampled, untouched) and all(torch.equal(a, b) for a, b in zip(packed, before))
-    finally:
-        ops.set_option("prepack_check", 2)
-    assert ops.get_option("prepack_check") == 2
-    # shapes that do not fill their last tiles
+    ops.layer_prologue(mask, weights=ws, packed=packed)
+    assert all(torch.equal(p, w.t().contiguous()) for p, w in zip(packed, ws))
+    # a subset, and shapes that do not fill their last 64 x 64 tiles
     odd = [_dev(rs.standard_normal(sh).astype(np.float16), device) for sh in [(72, 200), (200, 72)]]
-    odd_packed = ops.transpose_weights(odd)
-    odd_state = torch.zeros(ops.PREPACK_STATE_WORDS, dtype=torch.int64, device=device)
-    ops.layer_prologue(mask, weights=odd, packed=odd_packed, state=odd_state)
-    odd[0].data[71, 199] += 1
-    odd[1].data.mul_(-1)
-    ops.layer_prologue(mask, weights=odd, packed=odd_packed, state=odd_state)
-    torch.cuda.synchronize()
+    guard = [torch.full((sh[1] * sh[0] + 64,), 3, dtype=torch.float16, device=device)
+             for sh in [(72, 200), (200, 72)]]
+    odd_packed = [g[:w.numel()].view(w.shape[1], w.shape[0]) for g, w in zip(guard, odd)]
+    ops.layer_prologue(mask, weights=odd, packed=odd_packed)
     assert all(torch.equal(p, w.t().contiguous()) for p, w in zip(odd_packed, odd))
+    assert all(bool((g[w.numel():] == 3).all()) for g, w in zip(guard, odd))
+    with pytest.raises(ValueError):
+        ops.layer_prologue(mask, weights=ws[:1], packed=[ws[0]])
 
 
 def test_build_offsets_threshold(device):
@@ -274,10 +269,10 @@ def test_gemm_plain(device, tile, rows, M, N, K):
     exp = O.gemm(a[:M], w)
     ops.set_option("gemm_tile", tile)
     try:
-        wt = ops.transpose_weight(_dev(w, device))
+        wt = _prep(_dev(w, device))
         vr = torch.tensor([M], dtype=torch.int32, device=device)
         out = torch.full((rows, N), 3.0, dtype=torch.float16, device=device)
-        g = ops.gemm(_dev(a, device), wt, valid_rows=vr, out=out).cpu().numpy()
+        g = _gemm(_dev(a, device), wt, valid_rows=vr, out=out).cpu().numpy()
     finally:
         ops.set_option("gemm_tile", -1)
     err = np.abs(g[:M].astype(np.float64) - exp)
@@ -301,13 +296,13 @@ def test_gemm_random_shapes_all_tiles_and_auto(device, seed):
     w = (rs.standard_normal((K, N)) * 0.05).astype(np.float16)
     exp = O.gemm(a[:M], w)
     tol = _gemm_tol(exp, K, np.abs(a[:M]).max() if M else 0.0, np.abs(w).max())
-    wt = ops.transpose_weight(_dev(w, device))
+    wt = _prep(_dev(w, device))
     vr = torch.tensor([M], dtype=torch.int32, device=device)
     try:
         for tile in (-1, 0, 1, 2, 3, 4, 5, 6, 7, 8):
             ops.set_option("gemm_tile", tile)
             out = torch.full((rows, N), 3.0, dtype=torch.float16, device=device)
-            g = ops.gemm(_dev(a, device), wt, valid_rows=vr, out=out, rows_hint=M).cpu().numpy()
+            g = _gemm(_dev(a, device), wt, valid_rows=vr, out=out, rows_hint=M).cpu().numpy()
             err = np.abs(g[:M].astype(np.float64) - exp)
             assert np.all(err <= tol), (tile, err.max())
             assert np.all(g[M:] == 3.0), tile
@@ -334,7 +329,7 @@ def test_gemm_row_hint_never_changes_the_result(device, seed):
     b1 = (rs.standard_normal(F) * 0.1).astype(np.float16)
     bq = (rs.standard_normal(3 * H) * 0.1).astype(np.float16)
     ad, vr = _dev(a, device), torch.tensor([M], dtype=torch.int32, device=device)
-    wt1, wtq = ops.transpose_weight(_dev(w1, device)), ops.transpose_weight(_dev(wq, device))
+    wt1, wtq = _prep(_dev(w1, device)), _prep(_dev(wq, device))
     b1d, bqd = _dev(b1, device), _dev(bq, device)
     exp = O.gemm(a[:M], w1)
     tol = _gemm_tol(exp, H, np.abs(a[:M]).max(), np.abs(w1).max())
@@ -343,9 +338,9 @@ def test_gemm_row_hint_never_changes_the_result(device, seed):
         o1 = torch.full((rows, F), 3.0, dtype=torch.float16, device=device)
         o2 = torch.full((rows, F), 3.0, dtype=torch.float16, device=device)
         o3 = torch.full((3, heads, rows, 64), 3.0, dtype=torch.float16, device=device)
-        ops.gemm(ad, wt1, valid_rows=vr, out=o1, rows_hint=hint)
-        ops.gemm_bias_gelu(ad, wt1, b1d, valid_rows=vr, out=o2, rows_hint=hint)
-        ops.gemm_qkv_bias_split(ad, wtq, bqd, heads, valid_rows=vr, out=o3, rows_hint=hint)
+        _gemm(ad, wt1, valid_rows=vr, out=o1, rows_hint=hint)
+        _gemm_bias_gelu(ad, wt1, b1d, valid_rows=vr, out=o2, rows_hint=hint)
+        _gemm_qkv_bias_split(ad, wtq, bqd, heads, valid_rows=vr, out=o3, rows_hint=hint)
         return o1, o2, o3
 
     try:
@@ -394,12 +389,12 @@ def test_splitk_gemm_and_layernorm(device, splits, restore, tight):
     exp = O.add_bias_residual_layernorm(prod, res[:M], bias, gamma, beta, 1e-6)
     g_bi, _, _ = ops.build_offsets(_dev(mask, device))
     vr = g_bi[B:]
-    wt = ops.transpose_weight(_dev(w, device))
+    wt = _prep(_dev(w, device))
     # tight: the launches are sized for exactly the live rows (the padded output of the
     # restore flavour still has batch * seq_len rows)
     cap = M if tight else rows
     a, res = a[:cap], res[:cap]
-    parts = ops.gemm_splitk(_dev(a, device), wt, splits, valid_rows=vr)
+    parts = _gemm_splitk(_dev(a, device), wt, splits, valid_rows=vr)
     assert tuple(parts.shape) == (splits, cap, H)
     # the partial sums add up to the product
     total = parts.sum(0).cpu().numpy()[:M]
@@ -422,7 +417,7 @@ def test_splitk_gemm_and_layernorm(device, splits, restore, tight):
         assert np.all(g[M:] == 5.0)
         # and the unsplit pair gives the same numbers except where the fp16 rounding of the
         # product flips on the last bit of the fp32 sum
-        plain = ops.gemm(_dev(a, device), wt, valid_rows=vr)
+        plain = _gemm(_dev(a, device), wt, valid_rows=vr)
         ref = ops.add_bias_residual_layernorm(plain, *args, valid_rows=vr).cpu().numpy()
         assert np.mean(ref[:M] == g[:M]) > 0.97
         assert np.abs(ref[:M].astype(np.float32) - g[:M].astype(np.float32)).max() <= 2e-2
@@ -440,7 +435,7 @@ def test_gemm_bias_gelu(device, tile):
     ops.set_option("gemm_tile", tile)
     try:
         vr = torch.tensor([M], dtype=torch.int32, device=device)
-        g = ops.gemm_bias_gelu(_dev(a, device), ops.transpose_weight(_dev(w, device)),
+        g = _gemm_bias_gelu(_dev(a, device), _prep(_dev(w, device)),
                                _dev(bias, device), valid_rows=vr).cpu().numpy()
     finally:
         ops.set_option("gemm_tile", -1)
@@ -464,7 +459,7 @@ def test_gemm_qkv_bias_split(device, tile, heads):
     ops.set_option("gemm_tile", tile)
     try:
         vr = torch.tensor([M], dtype=torch.int32, device=device)
-        g = ops.gemm_qkv_bias_split(_dev(a, device), ops.transpose_weight(_dev(w, device)),
+        g = _gemm_qkv_bias_split(_dev(a, device), _prep(_dev(w, device)),
                                     _dev(bias, device), heads, valid_rows=vr).cpu().numpy()
     finally:
         ops.set_option("gemm_tile", -1)
@@ -488,10 +483,10 @@ def test_gather_fused_into_qkv_gemm_and_layernorm(device):
     bias = (rs.standard_normal(3 * H) * 0.5).astype(np.float16)
     g_bi, g_wi, M = ops.build_offsets(_dev(mask, device), want_count=True)
     vr = g_bi[B:]
-    xd, wt = _dev(x, device), ops.transpose_weight(_dev(w, device))
+    xd, wt = _dev(x, device), _prep(_dev(w, device))
     packed = ops.compress(xd, g_bi, g_wi)
-    ref = ops.gemm_qkv_bias_split(packed, wt, _dev(bias, device), heads, valid_rows=vr)
-    got = ops.gemm_qkv_bias_split(xd.view(B * S, H), wt, _dev(bias, device), heads, valid_rows=vr,
+    ref = _gemm_qkv_bias_split(packed, wt, _dev(bias, device), heads, valid_rows=vr)
+    got = _gemm_qkv_bias_split(xd.view(B * S, H), wt, _dev(bias, device), heads, valid_rows=vr,
                                   a_row_index=g_wi)
     assert torch.equal(ref[:, :, :M], got[:, :, :M])
     exp = O.split_heads(O.gemm(O.compress(x, g_wi.cpu().numpy()[:M]), w, bias), heads, 64)
@@ -908,6 +903,19 @@ def test_attention_prefetch_hint_changes_nothing(device, kind, lens, S):
                 torch.cuda.synchronize()
                 assert torch.equal(got[:M], base[:M]), (nbytes, lead)
                 assert bool((whole == 7).all())
+        # several ranges (a layer's weights are separate tensors), empty ones among them
+        wholes = [torch.full((guard + n + guard,), 7, dtype=torch.uint8, device=device)
+                  for n in (131, 1, 70001, 4)]
+        for count in (2, 3, 4):
+            ranges = [w[guard:w.numel() - guard] for w in wholes[:count]]
+            got = fn(_dev(qkv, device), _dev(bi, device), len(lens), S, 0.125, False,
+                     prefetch=ranges)
+            torch.cuda.synchronize()
+            assert torch.equal(got[:M], base[:M]), count
+            assert all(bool((w == 7).all()) for w in wholes)
+        with pytest.raises(ops.BtError):
+            fn(_dev(qkv, device), _dev(bi, device), len(lens), S, 0.125, False,
+               prefetch=[w[guard:-guard] for w in wholes] + [wholes[0][guard:-guard]])
     finally:
         ops.set_option("prefetch_min_grid", 512)
 

@@ -674,11 +674,11 @@ def test_two_threads_two_streams_share_nothing(device):
         assert results[i] is not None and torch.equal(results[i], alone[i])
 
 
-def test_th_op_prepack_cache_tracks_weight_updates(device):
-    """The operator caches the k-contiguous weight copies per tensor object; an
-    in-place update of a weight (version counter bump) must be picked up, and a
-    new tensor at a recycled address must not hit a stale entry."""
-    _say("prepack cache")
+def test_th_op_tracks_weight_and_mask_updates(device):
+    """The operator reads weights and mask as they are at each call: an in-place update
+    of a weight or of the mask is picked up, and new tensors at recycled addresses are
+    simply other tensors."""
+    _say("weight and mask updates")
     bt.load_th_op()
     cfg = workload.EncoderConfig("pc", 4, 64, 2, layers=1, lens=(64, 20, 33, 50), seed=3)
     wl = workload.make_workload(cfg, bias_std=0.05, random_affine=True)
@@ -686,7 +686,7 @@ def test_th_op_prepack_cache_tracks_weight_updates(device):
     x, m = _dev(wl.x, device), _dev(wl.mask, device)
     op = torch.ops.ByteTransformer.BertTransformer
     a = op(2, 64, *w, x, m, True, True)
-    b = op(2, 64, *w, x, m, True, True)              # second call: cache hit
+    b = op(2, 64, *w, x, m, True, True)
     assert torch.equal(a, b)
     _check(a.cpu().numpy(), _oracle(wl), wl.lens, tag="cache/first")
     # in-place update of FFN2's weight
@@ -695,7 +695,7 @@ def test_th_op_prepack_cache_tracks_weight_updates(device):
     c = op(2, 64, *w, x, m, True, True)
     assert not torch.equal(a, c)
     _check(c.cpu().numpy(), _oracle(wl), wl.lens, tag="cache/after-inplace-update")
-    # in-place change of the mask: the cached offsets of that mask tensor must go
+    # in-place change of the mask: the token count kept for that mask tensor must go
     new_lens = np.array([30, 64, 10, 50])
     m.copy_(_dev(workload.make_mask(new_lens, 64, np.float16), device))
     wl_m = workload.Workload(wl.cfg, new_lens, wl.x, workload.make_mask(new_lens, 64, np.float16),
@@ -764,9 +764,35 @@ def test_th_op_caches_cannot_change_results(device):
     torch.ops.ByteTransformer.clear_caches()
 
 
+def test_layer_prepack_choice_never_changes_the_result(device):
+    """Which products run on a per-call k-contiguous copy of their weight is a matter of
+    time only: never, always and the measured table's choice give the same bits, on
+    packed and on padded rows."""
+    _say("layer_prepack")
+    from bytetransformer_amd import ops
+    bt.load_th_op()
+    op = torch.ops.ByteTransformer.BertTransformer
+    for cfg in (workload.EncoderConfig("pp", 6, 200, 12, layers=1, lens=(200, 20, 133, 50, 64, 7), seed=8),
+                workload.EncoderConfig("pp2", 2, 72, 2, layers=1, lens=(72, 31), seed=9)):
+        wl = workload.make_workload(cfg, bias_std=0.05, random_affine=True)
+        w = [_dev(wl.layers[0][n], device) for n in workload.WEIGHT_NAMES]
+        x, m = _dev(wl.x, device), _dev(wl.mask, device)
+        got = {}
+        try:
+            for choice in (0, 1, -1):
+                ops.set_option("layer_prepack", choice)
+                got[choice] = op(cfg.head_num, 64, *w, x, m, True, True)
+        finally:
+            ops.set_option("layer_prepack", -1)
+        assert torch.equal(got[0], got[1]) and torch.equal(got[0], got[-1])
+        out = got[1].cpu().numpy()
+        _check(out if cfg.batch > 2 else O.masked_output(out, wl.lens), _oracle(wl), wl.lens,
+               tag="layer_prepack " + cfg.name)
+
+
 def test_th_op_under_graph_capture(device):
-    """Two operator layers captured with torch.cuda.graph (the caches stay out of a
-    capture: the layer packs its weights and builds its offsets inside the graph), replayed
+    """Two operator layers captured with torch.cuda.graph (the host keeps out of a capture:
+    no token count is read back, the layer builds its offsets inside the graph), replayed
     with other lengths and inputs written into the same buffers, eager work in between."""
     _say("operator under capture")
     bt.load_th_op()
