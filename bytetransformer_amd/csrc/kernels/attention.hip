@@ -196,6 +196,17 @@ __device__ __forceinline__ half8_t load_vt_frag(const half_t *sV, int kk, int db
   return half8_t{l4[0], l4[1], l4[2], l4[3], h4[0], h4[1], h4[2], h4[3]};
 }
 
+// The same fragment from the address of its first read (a tile's first key pair-block plus
+// the lane's own offset): the second read lies 16 rows further on.
+__device__ __forceinline__ half8_t load_vt_frag_at(const half_t *p0) {
+  const fp16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4f16(
+      (__attribute__((address_space(3))) fp16x4_t *)p0);
+  const fp16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4f16(
+      (__attribute__((address_space(3))) fp16x4_t *)(p0 + 16 * kHeadDim));
+  const half4_t l4 = __builtin_bit_cast(half4_t, lo), h4 = __builtin_bit_cast(half4_t, hi);
+  return half8_t{l4[0], l4[1], l4[2], l4[3], h4[0], h4[1], h4[2], h4[3]};
+}
+
 __device__ __forceinline__ half8_t load_k_frag(const half_t *sK, int kb, int dh, int lq, int lg) {
   const int row = 16 * kb + lq;
   return *(const half8_t *)(sK + row * kHeadDim + (((4 * dh + lg) ^ swz_k(row)) << 3));
@@ -304,7 +315,7 @@ __global__ __launch_bounds__(kAttThreads * KS, KS == 1 ? 2 : 4) void attention_g
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave_all = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wave = wave_all & 3;        // which 16-query blocks
-  const int grp = wave_all >> 2;        // which 64-key half of a ring slot (KS = 2)
+  const int grp = KS > 1 ? wave_all >> 2 : 0;   // which 64-key half of a ring slot (KS = 2)
   const int lq = lane & 15, lg = lane >> 4;
 
   const size_t head_stride = (size_t)p.rows_cap * kHeadDim;
@@ -323,6 +334,22 @@ __global__ __launch_bounds__(kAttThreads * KS, KS == 1 ? 2 : 4) void attention_g
       if (q < nq) v = *(const uint4_t *)(Q + (size_t)q * kHeadDim + 32 * dh + 8 * lg);
       qf[qb][dh] = __builtin_bit_cast(half8_t, v);
     }
+  }
+
+  // Where this lane's operand fragments sit inside a K or V tile, in halfs: the swizzle
+  // term of a fragment's row does not depend on the key block (K: row = 16 kb + lq, V: row
+  // = 32 kk + 4 lg + (lq >> 2); the block index drops out of swz_k / swz_v), so the whole
+  // address is one of these six lane constants plus a compile-time offset - ring stage,
+  // key block - that fits the instruction's immediate field: no address arithmetic is
+  // left in the loop over the key tiles (it was a quarter of its vector instructions).
+  int koff[2], voff[4];
+#pragma unroll
+  for (int dh = 0; dh < 2; ++dh) koff[dh] = lq * kHeadDim + (((4 * dh + lg) ^ swz_k(lq)) << 3);
+#pragma unroll
+  for (int db = 0; db < 4; ++db) {
+    const int row0 = 4 * lg + (lq >> 2);
+    const int c = 2 * db + ((lq & 3) >> 1);
+    voff[db] = row0 * kHeadDim + ((c ^ swz_v(row0)) << 3) + 4 * (lq & 1);
   }
 
   // Slot copy: 16 load instructions per 64-key tile (8 rows each; 0-7 = K, 8-15 = V),
@@ -369,10 +396,12 @@ __global__ __launch_bounds__(kAttThreads * KS, KS == 1 ? 2 : 4) void attention_g
   // after the mask term is folded in, the logits already are in the exp2 domain
   const float cs = ADD ? 1.0f : c;
   const bool mask_vec = (p.S & 3) == 0;
-  int stage = 0;
 
-  auto process_tile = [&](int t, auto masked_tag) {
+  // ST: the ring stage of tile t, a compile-time constant (the loop below is unrolled over
+  // the stages)
+  auto process_tile = [&](int t, auto masked_tag, auto stage_tag) {
     constexpr bool MASKED = decltype(masked_tag)::value;
+    constexpr int ST = decltype(stage_tag)::value;
     // this wave's share of tile t has landed once only tile t+1's four loads are outstanding
     if (AHEAD > 1 && t + 1 < ntiles)
       att_wait_vmcnt<4>();
@@ -381,19 +410,12 @@ __global__ __launch_bounds__(kAttThreads * KS, KS == 1 ? 2 : 4) void attention_g
     asm volatile("" ::: "memory");
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
-    if (t + AHEAD < ntiles) {
-      int ps = stage + AHEAD;
-      if (ps >= STAGES) ps -= STAGES;
-      issue_tile(t + AHEAD, ps);
-    }
+    if (t + AHEAD < ntiles) issue_tile(t + AHEAD, (ST + AHEAD) % STAGES);
     // a wave whose queries all lie past the sequence, or whose half of the slot lies past
     // the last key, only copies and keeps the barriers
     const int k0 = t * kSlotKeys + grp * kKT;
-    if (!wave_live || (KS > 1 && k0 >= klen)) {
-      if (++stage == STAGES) stage = 0;
-      return;
-    }
-    const half_t *sK = ring + stage * kSlotHalfs + grp * 2 * kTileHalfs;
+    if (!wave_live || (KS > 1 && k0 >= klen)) return;
+    const half_t *sK = ring + ST * kSlotHalfs + grp * 2 * kTileHalfs;
     const half_t *sV = sK + kTileHalfs;
 
     // S^T = K . Q^T for this tile: 4 key blocks x QB query blocks
@@ -401,7 +423,8 @@ __global__ __launch_bounds__(kAttThreads * KS, KS == 1 ? 2 : 4) void attention_g
     const float4_t zero4 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int kb = 0; kb < 4; ++kb) {
-      const half8_t kf0 = load_k_frag(sK, kb, 0, lq, lg), kf1 = load_k_frag(sK, kb, 1, lq, lg);
+      const half8_t kf0 = *(const half8_t *)(sK + kb * 16 * kHeadDim + koff[0]);
+      const half8_t kf1 = *(const half8_t *)(sK + kb * 16 * kHeadDim + koff[1]);
 #pragma unroll
       for (int qb = 0; qb < QB; ++qb) {
         s[kb][qb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kf0, qf[qb][0], zero4, 0, 0, 0);
@@ -472,7 +495,7 @@ __global__ __launch_bounds__(kAttThreads * KS, KS == 1 ? 2 : 4) void attention_g
     for (int kk = 0; kk < 2; ++kk) {
 #pragma unroll
       for (int db = 0; db < 4; ++db) {
-        const half8_t vf = load_vt_frag(sV, kk, db, lq, lg);
+        const half8_t vf = load_vt_frag_at(sV + kk * 32 * kHeadDim + voff[db]);
 #pragma unroll
         for (int qb = 0; qb < QB; ++qb)
           o[db][qb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vf, pf[kk][qb], o[db][qb], 0, 0, 0);
@@ -481,16 +504,22 @@ __global__ __launch_bounds__(kAttThreads * KS, KS == 1 ? 2 : 4) void attention_g
       for (int qb = 0; qb < QB; ++qb)
         o[4][qb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ones, pf[kk][qb], o[4][qb], 0, 0, 0);
     }
-    if (++stage == STAGES) stage = 0;
   };
-
   // every tile but the last is full: no masking code on the steady-state path
-  for (int t = 0; t + 1 < ntiles; ++t) process_tile(t, std::false_type{});
-  if (ntiles > 0) {
-    if (klen % kSlotKeys == 0)
-      process_tile(ntiles - 1, std::false_type{});
+  const bool ragged_end = klen % kSlotKeys != 0;
+  auto step = [&](int t, auto stage_tag) {
+    if (ragged_end && t == ntiles - 1)
+      process_tile(t, std::true_type{}, stage_tag);
     else
-      process_tile(ntiles - 1, std::true_type{});
+      process_tile(t, std::false_type{}, stage_tag);
+  };
+  // one turn of the ring per iteration: tile t sits in stage t % STAGES
+  for (int t = 0; t < ntiles; t += STAGES) {
+    step(t, std::integral_constant<int, 0>{});
+    if (t + 1 < ntiles) step(t + 1, std::integral_constant<int, 1>{});
+    if constexpr (STAGES == 3) {
+      if (t + 2 < ntiles) step(t + 2, std::integral_constant<int, 2>{});
+    }
   }
 
   if (KS > 1) {

@@ -10,10 +10,17 @@
 
 namespace bt {
 
-constexpr int kLnRowsPerBlock = 4;
+constexpr int kLnRowsPerBlock = 4;   // 2, 8 and 16 rows per workgroup measured 0-20 % slower
 
 // SPLITS > 0: `src` holds SPLITS fp32 partial sums of the row ([SPLITS][split_rows][H], the
 // output of a split-k GEMM); their sum, rounded to fp16 once, takes the place of `out`.
+//
+// A launch of a few thousand rows is one round of waves, each living for the length of its
+// chain of dependent memory accesses, so the kernel is written to keep that chain short:
+// everything whose address does not depend on loaded data (bias, gamma, beta, the row
+// index or the sequence offsets, and on packed rows the row of `src` itself) is requested
+// at the top in one batch, a lane past the end of the row loads the last chunk again
+// instead of branching, and the only dependent step left is the row(s) behind an index.
 template <int NC, bool RESTORE, bool GB32, int SPLITS>
 __global__ __launch_bounds__(kLnRowsPerBlock *kWave) void layernorm_kernel(
     const half8_t *src, const half8_t *__restrict__ residual,
@@ -24,8 +31,41 @@ __global__ __launch_bounds__(kLnRowsPerBlock *kWave) void layernorm_kernel(
   const int r = blockIdx.x * kLnRowsPerBlock + (threadIdx.x >> 6);
   const int lane = threadIdx.x & 63;
   if (r >= rows_cap) return;
+  // fp32 gamma / beta of wide rows would not fit the registers next to the row: those
+  // instantiations fetch them after the statistics, as before
+  constexpr bool kAffineEarly = !GB32 || NC <= 2;
+
+  int cc[NC];        // this lane's chunks, clamped into the row
+  bool live[NC];
+#pragma unroll
+  for (int i = 0; i < NC; ++i) {
+    const int c = lane + i * kWave;
+    live[i] = c < chunks;
+    cc[i] = live[i] ? c : chunks - 1;
+  }
+
+  // ---- first batch: nothing here depends on loaded data ----
+  half8_t bias_v[NC];
+  half8_t gh[NC], bh[NC];
+  float4_t g32[kAffineEarly && GB32 ? NC : 1][2], b32[kAffineEarly && GB32 ? NC : 1][2];
+#pragma unroll
+  for (int i = 0; i < NC; ++i) {
+    bias_v[i] = bias[cc[i]];
+    if (kAffineEarly) {
+      if (GB32) {
+        g32[i][0] = ((const float4_t *)gamma)[2 * cc[i]];
+        g32[i][1] = ((const float4_t *)gamma)[2 * cc[i] + 1];
+        b32[i][0] = ((const float4_t *)beta)[2 * cc[i]];
+        b32[i][1] = ((const float4_t *)beta)[2 * cc[i] + 1];
+      } else {
+        gh[i] = ((const half8_t *)gamma)[cc[i]];
+        bh[i] = ((const half8_t *)beta)[cc[i]];
+      }
+    }
+  }
 
   size_t src_row, dst_row = r;
+  half8_t av[NC];
   if (RESTORE) {
     // r walks the padded [B, S] grid; idx = batch_idx
     const int b = r / S, s = r - b * S;
@@ -37,60 +77,67 @@ __global__ __launch_bounds__(kLnRowsPerBlock *kWave) void layernorm_kernel(
     }
     src_row = (size_t)start + s;
   } else {
-    // idx = pointer to the live-row count (or null: all rows live)
+    // idx = pointer to the live-row count (or null: all rows live).  Row r of `src` and
+    // entry r of the index lie inside their buffers whether or not the row is live, so they
+    // are requested before the count is known.
+    src_row = r;
+    if (SPLITS == 0) {
+#pragma unroll
+      for (int i = 0; i < NC; ++i) av[i] = src[src_row * chunks + cc[i]];
+    }
+    const int ridx = residual_row_index ? residual_row_index[src_row] : 0;
     const int M = idx ? *idx : rows_cap;
     if (r >= M) return;
-    src_row = r;
+    const size_t res_row = residual_row_index ? (size_t)ridx : src_row;
+    residual += res_row * chunks;
+  }
+  if (RESTORE) {
+    residual += src_row * chunks;
+    if (SPLITS == 0) {
+#pragma unroll
+      for (int i = 0; i < NC; ++i) av[i] = src[src_row * chunks + cc[i]];
+    }
+  }
+  half8_t rv[NC];
+#pragma unroll
+  for (int i = 0; i < NC; ++i) rv[i] = residual[cc[i]];
+  if (SPLITS > 0) {
+#pragma unroll
+    for (int i = 0; i < NC; ++i) {
+      const float4_t *pp = (const float4_t *)src + (src_row * chunks + cc[i]) * 2;
+      float4_t lo = pp[0], hi = pp[1];
+#pragma unroll
+      for (int sp = 1; sp < SPLITS; ++sp) {
+        lo += pp[(size_t)sp * split_rows * chunks * 2];
+        hi += pp[(size_t)sp * split_rows * chunks * 2 + 1];
+      }
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        av[i][j] = (half_t)lo[j];
+        av[i][4 + j] = (half_t)hi[j];
+      }
+    }
   }
 
-  const half8_t *a = src + src_row * chunks;
-  const size_t res_row = residual_row_index ? (size_t)residual_row_index[src_row] : src_row;
-  const half8_t *b = residual + res_row * chunks;
   float v[NC][8];
   float sum = 0.f;
 #pragma unroll
   for (int i = 0; i < NC; ++i) {
-    const int c = lane + i * kWave;
-    if (c < chunks) {
-      half8_t av;
-      if (SPLITS > 0) {
-        const float4_t *pp = (const float4_t *)src + (src_row * chunks + c) * 2;
-        float4_t lo = pp[0], hi = pp[1];
+    const half8_t x = (av[i] + rv[i]) + bias_v[i];  // two fp16-rounded adds
 #pragma unroll
-        for (int sp = 1; sp < SPLITS; ++sp) {
-          lo += pp[(size_t)sp * split_rows * chunks * 2];
-          hi += pp[(size_t)sp * split_rows * chunks * 2 + 1];
-        }
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          av[j] = (half_t)lo[j];
-          av[4 + j] = (half_t)hi[j];
-        }
-      } else {
-        av = a[c];
-      }
-      half8_t x = (av + b[c]) + bias[c];  // two fp16-rounded adds
-#pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        v[i][j] = (float)x[j];
-        sum += v[i][j];
-      }
-    } else {
-#pragma unroll
-      for (int j = 0; j < 8; ++j) v[i][j] = 0.f;
+    for (int j = 0; j < 8; ++j) {
+      v[i][j] = live[i] ? (float)x[j] : 0.f;
+      sum += v[i][j];
     }
   }
   const float mean = wave_sum(sum) * inv_n;
   float sq = 0.f;
 #pragma unroll
   for (int i = 0; i < NC; ++i) {
-    const int c = lane + i * kWave;
-    if (c < chunks) {
 #pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        v[i][j] -= mean;
-        sq += v[i][j] * v[i][j];
-      }
+    for (int j = 0; j < 8; ++j) {
+      v[i][j] = live[i] ? v[i][j] - mean : 0.f;
+      sq += v[i][j] * v[i][j];
     }
   }
   const float rstd = rsqrtf(wave_sum(sq) * inv_n + eps);
@@ -98,33 +145,34 @@ __global__ __launch_bounds__(kLnRowsPerBlock *kWave) void layernorm_kernel(
   half8_t *o = dst + dst_row * chunks;
 #pragma unroll
   for (int i = 0; i < NC; ++i) {
-    const int c = lane + i * kWave;
-    if (c < chunks) {
-      float g[8], bt_[8];
-      if (GB32) {
-        const float4_t *gp = (const float4_t *)gamma + 2 * c;
-        const float4_t *bp = (const float4_t *)beta + 2 * c;
-        float4_t g0 = gp[0], g1 = gp[1], b0 = bp[0], b1 = bp[1];
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          g[j] = g0[j];
-          g[4 + j] = g1[j];
-          bt_[j] = b0[j];
-          bt_[4 + j] = b1[j];
-        }
+    float g[8], bt_[8];
+    if (GB32) {
+      float4_t g0, g1, b0, b1;
+      if (kAffineEarly) {
+        g0 = g32[i][0], g1 = g32[i][1], b0 = b32[i][0], b1 = b32[i][1];
       } else {
-        half8_t gh = ((const half8_t *)gamma)[c], bh = ((const half8_t *)beta)[c];
-#pragma unroll
-        for (int j = 0; j < 8; ++j) {
-          g[j] = (float)gh[j];
-          bt_[j] = (float)bh[j];
-        }
+        const float4_t *gp = (const float4_t *)gamma + 2 * cc[i];
+        const float4_t *bp = (const float4_t *)beta + 2 * cc[i];
+        g0 = gp[0], g1 = gp[1], b0 = bp[0], b1 = bp[1];
       }
-      half8_t y;
 #pragma unroll
-      for (int j = 0; j < 8; ++j) y[j] = (half_t)(v[i][j] * rstd * g[j] + bt_[j]);
-      o[c] = y;
+      for (int j = 0; j < 4; ++j) {
+        g[j] = g0[j];
+        g[4 + j] = g1[j];
+        bt_[j] = b0[j];
+        bt_[4 + j] = b1[j];
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        g[j] = (float)gh[i][j];
+        bt_[j] = (float)bh[i][j];
+      }
     }
+    half8_t y;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) y[j] = (half_t)(v[i][j] * rstd * g[j] + bt_[j]);
+    if (live[i]) o[cc[i]] = y;
   }
 }
 
