@@ -39,7 +39,8 @@ KERNEL_ABI = {
     "bt_mask_is_prefix": (c_int, [_P, c_int, c_int, c_int, _IP, _IP, POINTER(c_int), _P]),
     "bt_layer_prologue": (c_int, [_P, c_int, c_int, c_int, _IP, _IP, _IP, _IP, _P, c_int, c_int,
                                   c_int, POINTER(c_void_p), POINTER(c_void_p), POINTER(c_int),
-                                  POINTER(c_int), _P]),
+                                  POINTER(c_int), c_int, POINTER(c_void_p), POINTER(c_ulonglong),
+                                  _P]),
     "bt_gemm_prepack_pays": (c_int, [c_longlong, c_int, c_int, c_int]),
     "bt_compress": (c_int, [_P, _P, _IP, _IP, c_int, c_int, c_int, _P]),
     "bt_transpose_weight": (c_int, [_P, _P, c_int, c_int, _P]),

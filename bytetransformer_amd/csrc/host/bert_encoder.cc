@@ -78,7 +78,7 @@ void BertEncoder<OpType>::infer(BertEncoderInferParam<DataType_> ip) {
                                    et_param.batch_idx, et_param.word_idx, seq_order,
                                    check_mask ? mask_slots : nullptr, work_list, head_num_,
                                    is_remove_padding_ ? 0 : 1, 0, nullptr, nullptr, nullptr,
-                                   nullptr, stream));
+                                   nullptr, 0, nullptr, nullptr, stream));
   const int *valid_rows = is_remove_padding_ ? et_param.batch_idx + batch_size : nullptr;
   const int rows_hint = ip.valid_rows_hint;
   const int L = (int)layers_.size();

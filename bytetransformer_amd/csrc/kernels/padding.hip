@@ -194,6 +194,12 @@ struct PrologueWeights {
   int tiles_n[4];            // 64 x 64 tiles along n
   int tile_end[4];           // tiles up to and including matrix i
   int count;                 // 0 = none
+  // ranges that the layer's products will read as they are (the weights that are not
+  // packed): range r holds the 128-byte lines [warm_end[r - 1], warm_end[r]) of their
+  // concatenation; the pack blocks touch one dword per line so that the lines sit in the
+  // memory-side cache when the products ask for them
+  const char *warm[4];
+  unsigned warm_end[4];
 };
 
 // The attention's balanced work list, built by blocks of their own beyond the others
@@ -326,6 +332,29 @@ __global__ __launch_bounds__(kPrologueThreads) void layer_prologue_kernel(
                         (tl % pw.tiles_n[j]) * 64, tile, tid & 255, t < tile_hi);
       __syncthreads();
     }
+  }
+
+  // ---- warm-up of the weights that are read as stored ----
+  const unsigned warm_lines = pw.warm_end[3];
+  if (warm_lines && (int)blockIdx.x >= kPackFirst && (int)blockIdx.x < kPackFirst + kPackBlocks) {
+    const unsigned pb = blockIdx.x - kPackFirst;
+    const unsigned per = (warm_lines + kPackBlocks - 1) / kPackBlocks;
+    const unsigned first = pb * per;
+    const unsigned last = first + per < warm_lines ? first + per : warm_lines;
+    for (unsigned l = first + tid; l < last; l += kPrologueThreads) {
+      const char *base = pw.warm[0];
+      unsigned begin = 0;
+#pragma unroll
+      for (int r = 1; r < 4; ++r)
+        if (l >= pw.warm_end[r - 1]) {
+          base = pw.warm[r];
+          begin = pw.warm_end[r - 1];
+        }
+      unsigned sink;
+      const char *addr = base + (unsigned long long)(l - begin) * 128;
+      asm volatile("global_load_dword %0, %1, off" : "=v"(sink) : "v"(addr) : "memory");
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   }
 }
 
@@ -463,7 +492,9 @@ extern "C" int bt_layer_prologue(const void *atten_mask, int mask_dtype, int bat
                                  int seq_len, int *batch_idx, int *word_idx, int *seq_order,
                                  int *mask_prefix_slots, void *attention_work_list, int head_num,
                                  int padded_rows, int weight_count, const void *const *w,
-                                 void *const *wt, const int *k, const int *n, void *stream) {
+                                 void *const *wt, const int *k, const int *n, int warm_count,
+                                 const void *const *warm, const unsigned long long *warm_bytes,
+                                 void *stream) {
   BT_REQUIRE(atten_mask && batch_idx && word_idx, BT_ERR_INVALID_ARGUMENT,
              "bt_layer_prologue: null pointer argument");
   BT_REQUIRE(batch_size > 0 && seq_len > 0, BT_ERR_INVALID_ARGUMENT,
@@ -503,6 +534,26 @@ extern "C" int bt_layer_prologue(const void *atten_mask, int mask_dtype, int bat
       pw.tile_end[i] = (int)tiles;
     }
   }
+  BT_REQUIRE(warm_count >= 0 && warm_count <= 4 && (warm_count == 0 || (warm && warm_bytes)),
+             BT_ERR_INVALID_ARGUMENT, "bt_layer_prologue: warm_count=%d outside [0, 4], or no ranges",
+             warm_count);
+  bool warming = false;
+  if (option_prefetch()) {
+    unsigned end = 0;
+    for (int r = 0; r < 4; ++r) {
+      if (r < warm_count && warm[r]) {
+        // one dword at the start of each 128-byte line; a last line of fewer than four bytes
+        // is left alone, so no byte outside the range is read
+        const unsigned long long lines = (warm_bytes[r] + 124) / 128;
+        BT_REQUIRE(lines < (1ull << 24), BT_ERR_UNSUPPORTED,
+                   "bt_layer_prologue: a range to warm beyond 2 GiB");
+        pw.warm[r] = (const char *)warm[r];
+        end += (unsigned)lines;
+      }
+      pw.warm_end[r] = end;
+    }
+    warming = end > 0;
+  }
   // the attention's balanced work list, when a launch of this shape uses one
   PrologueList pl;
   memset(&pl, 0, sizeof(pl));
@@ -531,7 +582,7 @@ extern "C" int bt_layer_prologue(const void *atten_mask, int mask_dtype, int bat
   // the verdict slots are an array of kPrefixBlocks entries, one per block; the
   // pre-pack blocks are the last kPackBlocks of the same grid
   static_assert(kPackFirst + kPackBlocks == kPrefixBlocks, "one grid for both jobs");
-  const int grid = ((mask_prefix_slots || weight_count > 0) ? kPrefixBlocks : offset_blocks) +
+  const int grid = ((mask_prefix_slots || weight_count > 0 || warming) ? kPrefixBlocks : offset_blocks) +
                    (pl.list ? kListBlocks : 0);
   if (mask_dtype == BT_F16)
     layer_prologue_kernel<half_t><<<grid, kPrologueThreads, smem, s>>>(

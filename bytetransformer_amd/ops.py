@@ -78,12 +78,13 @@ def mask_is_prefix(mask, batch_idx):
 
 
 def layer_prologue(mask, want_slots=False, weights=None, packed=None, out=None,
-                   work_list=None, head_num=0, padded_rows=False):
+                   work_list=None, head_num=0, padded_rows=False, warm=()):
     """bt_layer_prologue: offsets of `mask`, optionally the prefix-mask verdict slots and the
     [n, k] copies `packed` of the [k, n] `weights` (up to four).  Returns (batch_idx,
     word_idx, seq_order, slots or None); `out` = such a tuple to write into.  work_list
     (int32[entries, 4], with head_num and padded_rows): also filled with the attention's
-    balanced order, as attention_worklist would."""
+    balanced order, as attention_worklist would.  warm: up to four tensors that later launches
+    will read, touched line by line (a cache hint)."""
     B, S = mask.shape[0], mask.shape[1]
     dev = mask.device
     if out is not None:
@@ -104,10 +105,14 @@ def layer_prologue(mask, want_slots=False, weights=None, packed=None, out=None,
         ns = (ctypes.c_int * n)(*[w.shape[1] for w in weights])
     else:
         src = dst = ks = ns = None
+    warm = list(warm)
+    nw = len(warm)
+    wp = (ctypes.c_void_p * max(nw, 1))(*[_ptr(t).value for t in warm])
+    wb = (ctypes.c_ulonglong * max(nw, 1))(*[t.numel() * t.element_size() for t in warm])
     _check(kernel_lib().bt_layer_prologue(
         _ptr(mask), _dtype_code(mask), B, S, _ptr(batch_idx), _ptr(word_idx), _ptr(seq_order),
         _ptr(slots), _ptr(work_list), int(head_num), int(padded_rows), n, src, dst, ks, ns,
-        _stream()))
+        nw, wp, wb, _stream()))
     return batch_idx, word_idx, seq_order, slots
 
 

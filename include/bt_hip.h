@@ -128,13 +128,18 @@ int bt_mask_is_prefix(const void *atten_mask, int mask_dtype, int batch_size, in
  *     pre-pack into wt[i] ([n[i], k[i]], as bt_transpose_weights does) for the products of
  *     this call (see bt_gemm_prepack_pays): made afresh in every call from the weights as
  *     they are at that moment - nothing is remembered between calls, so nothing can go
- *     stale.
+ *     stale;
+ *   - warm_count in [0, 4] readable device ranges (host arrays of pointers and sizes) that
+ *     the layer's launches will read later - the weights that are used as stored: touched
+ *     line by line so that they sit in the memory-side cache by then.  Purely a hint
+ *     (bt_set_option("prefetch", 0) ignores it); the results do not depend on it.
  */
 int bt_layer_prologue(const void *atten_mask, int mask_dtype, int batch_size, int seq_len,
                       int *batch_idx, int *word_idx, int *seq_order, int *mask_prefix_slots,
                       void *attention_work_list, int head_num, int padded_rows, int weight_count,
                       const void *const *w, void *const *wt, const int *k, const int *n,
-                      void *stream);
+                      int warm_count, const void *const *warm,
+                      const unsigned long long *warm_bytes, void *stream);
 
 /*
  * Gather valid rows: to_tensor[t, :] = from_tensor[word_idx[t], :], t < M.

@@ -148,6 +148,21 @@ def test_layer_prologue_packs_weights_afresh_in_every_call(device):
     assert all(bool((g[w.numel():] == 3).all()) for g, w in zip(guard, odd))
     with pytest.raises(ValueError):
         ops.layer_prologue(mask, weights=ws[:1], packed=[ws[0]])
+    # ranges to warm are only read (guard bytes on both sides, odd sizes, up to four of them),
+    # alone and beside a pack job, and change nothing else
+    guard = 4096
+    wholes = [torch.full((guard + n + guard,), 7, dtype=torch.uint8, device=device)
+              for n in (131, 3, 1 << 20, 70001)]
+    for count in (1, 2, 4):
+        ranges = [w[guard:w.numel() - guard] for w in wholes[:count]]
+        for with_pack in (False, True):
+            bi2, wi2, _, _ = ops.layer_prologue(mask, weights=ws[:2] if with_pack else None,
+                                                packed=packed[:2] if with_pack else None, warm=ranges)
+            torch.cuda.synchronize()
+            assert torch.equal(bi2, bi) and torch.equal(wi2[:M], wi[:M])
+            assert all(bool((w == 7).all()) for w in wholes)
+    with pytest.raises(ops.BtError):
+        ops.layer_prologue(mask, warm=[w[guard:-guard] for w in wholes] + [wholes[0][guard:-guard]])
 
 
 def test_build_offsets_threshold(device):
