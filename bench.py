@@ -127,6 +127,7 @@ def kernel_table(wl, dev, iters):
     pro_out = (bo_bi, bo_wi, torch.empty_like(seq_order), None)
     pro_w = [w[n] for n, p in zip(names, pays) if p]
     pro_wt = [t_ for t_, p in zip((wt_qkv, wt_o, wt_1, wt_2), pays) if p]
+    pro_warm = [w[n] for n, p in zip(names, pays) if not p]      # read as stored: first touch
     pro_bytes = sum(2 * x_.numel() * 2 for x_ in pro_w)
 
     all_wt = [torch.empty(w[n].shape[1], w[n].shape[0], dtype=torch.float16, device=dev)
@@ -136,7 +137,7 @@ def kernel_table(wl, dev, iters):
         ("build_offsets", lambda: ops.build_offsets(mask, out=(bo_bi, bo_wi)), "hbm",
          2 * B * S + 4 * (B + 1) + 4 * M),
         ("layer_prologue", lambda: ops.layer_prologue(mask, weights=pro_w, packed=pro_wt,
-                                                      out=pro_out), "hbm",
+                                                      out=pro_out, warm=pro_warm), "hbm",
          2 * B * S + 4 * (B + 1) + 4 * M + pro_bytes),
         ("compress", lambda: ops.compress(x, batch_idx, word_idx, out=packed), "hbm",
          2 * M * H * 2 + 4 * M),

@@ -51,6 +51,21 @@ void BertTransformer<OpType>::bert_infer(BertTransformerInferParam infer_param) 
   et_param.valid_word_num = rows;
   int *seq_order = et_param.batch_idx + max_batch_size_ + 1;   // int[max_batch_size]
   off += align_up((max_rows * 2 + 2 * (unsigned long long)max_batch_size_ + 2) * sizeof(int), 256);
+  const bool have_offsets =
+      infer_param.offsets && infer_param.offsets->batch_idx && infer_param.offsets->word_idx;
+  const bool streaming_fp16 = OpType == OperationType::HALF && size_per_head_ == 64 &&
+                              !attention_layer_->uses_short_kernel(seq_len);
+  // Short sequences on padded rows: nothing but the attention would use the offsets there,
+  // and the attention can apply the mask tensor itself (all seq_len keys, masked ones
+  // shifted by -10000: the same probabilities) - so the layer goes without the prologue
+  // launch, which at a few dozen tokens is an eighth of its run time.
+  int direct_limit = 0;
+  bt_get_option("padded_mask_direct", &direct_limit);
+  // (only launches that take the plain workgroup order: the balanced one ranks the
+  // sequences by their lengths)
+  const bool mask_direct = streaming_fp16 && !is_remove_padding_ && !have_offsets &&
+                           seq_len <= direct_limit &&
+                           bt_attention_worklist_bytes(batch_size, seq_len, head_num_) == 0;
   // The four products read the [k, n] weights as the caller stores them, exactly as the
   // reference hands them to cuBLAS (gemm.cu:27-39): nothing is kept between calls and
   // nothing can go stale.  Where the measured tile table says that a product of this size
@@ -73,7 +88,7 @@ void BertTransformer<OpType>::bert_infer(BertTransformerInferParam infer_param) 
       w_use[i] = param_.prepacked_kernels[i];
       w_kn[i] = 0;
     }
-  } else if (OpType == OperationType::HALF) {
+  } else if (OpType == OperationType::HALF && !mask_direct) {   // (the copies are made by the prologue)
     const long long live = infer_param.valid_rows_hint > 0 ? infer_param.valid_rows_hint
                            : is_remove_padding_            ? (rows * 3LL + 4) / 5
                                                            : rows;
@@ -102,17 +117,14 @@ void BertTransformer<OpType>::bert_infer(BertTransformerInferParam infer_param) 
   // it finds the plain prefix mask of its lengths; the prologue leaves that verdict in the
   // attention's scratch and the kernel decides on the device.
   int *mask_slots = nullptr;
-  const bool have_offsets =
-      infer_param.offsets && infer_param.offsets->batch_idx && infer_param.offsets->word_idx;
-  if (OpType == OperationType::HALF && !is_remove_padding_ && size_per_head_ == 64 &&
-      !attention_layer_->uses_short_kernel(seq_len) && !(have_offsets && infer_param.mask_prefix >= 0))
+  if (streaming_fp16 && !is_remove_padding_ && !mask_direct &&
+      !(have_offsets && infer_param.mask_prefix >= 0))
     mask_slots = (int *)(base + inner_buf_size_);
 
   // The streaming attention's balanced work list, when a launch of this shape uses one: the
   // prologue builds it beside the offsets, the kernel then finds its work with one load.
   void *work_list = nullptr;
-  if (OpType == OperationType::HALF && size_per_head_ == 64 && !have_offsets &&
-      !attention_layer_->uses_short_kernel(seq_len) &&
+  if (streaming_fp16 && !have_offsets && !mask_direct &&
       bt_attention_worklist_bytes(batch_size, seq_len, head_num_) > 0)
     work_list = base + inner_buf_size_ + Attention<OpType>::work_list_offset();
 
@@ -133,7 +145,7 @@ void BertTransformer<OpType>::bert_infer(BertTransformerInferParam infer_param) 
         warm[warm_count] = w_use[i];
         warm_bytes[warm_count++] = (unsigned long long)w_k[i] * w_n[i] * sizeof(DataType_);
       }
-  if (!have_offsets || mask_slots || pack_count > 0)
+  if (!mask_direct && (!have_offsets || mask_slots || pack_count > 0))
     check_bt_error(bt_layer_prologue(atten_mask, Traits_::dtype, batch_size, seq_len,
                                      et_param.batch_idx, et_param.word_idx, seq_order,
                                      mask_slots, work_list, head_num_, is_remove_padding_ ? 0 : 1,
@@ -218,8 +230,9 @@ void BertTransformer<OpType>::bert_infer(BertTransformerInferParam infer_param) 
         infer_param.cublas_handle, stream, et_param
   };
   attention_infer_param.attention_bias = infer_param.attention_bias;
-  attention_infer_param.seq_order = seq_order;
-  attention_infer_param.mask_prefix = have_offsets ? infer_param.mask_prefix : -1;
+  attention_infer_param.seq_order = mask_direct ? nullptr : seq_order;   // (no offsets: none was written)
+  // (0 = "not known to be the prefix mask": the tensor is applied)
+  attention_infer_param.mask_prefix = have_offsets ? infer_param.mask_prefix : (mask_direct ? 0 : -1);
   attention_infer_param.mask_prefix_slots = mask_slots;
   attention_infer_param.work_list = work_list;
   // the three weight matrices the rest of the layer reads (as stored, or the copies of

@@ -33,6 +33,7 @@ static std::atomic<int> g_prefetch{1};
 static std::atomic<int> g_prefetch_min_grid{512};
 static std::atomic<int> g_attention_key_split{-1};
 static std::atomic<int> g_layer_prepack{-1};
+static std::atomic<int> g_padded_mask_direct{320};
 static std::atomic<int> g_f32_gemm_tile{-1};
 static std::atomic<int> g_attention_short_limit{0};
 static std::atomic<int> g_attention_xcd_map{2};
@@ -417,6 +418,10 @@ extern "C" int bt_set_option(const char *name, int value) {
     BT_REQUIRE(value >= -1 && value <= 1, BT_ERR_INVALID_ARGUMENT,
                "bt_set_option: layer_prepack=%d must be -1, 0 or 1", value);
     g_layer_prepack.store(value);
+  } else if (!strcmp(name, "padded_mask_direct")) {
+    BT_REQUIRE(value >= 0 && value <= (1 << 20), BT_ERR_INVALID_ARGUMENT,
+               "bt_set_option: padded_mask_direct=%d outside [0, 2^20]", value);
+    g_padded_mask_direct.store(value);
   } else if (!strcmp(name, "prefetch_min_grid")) {
     BT_REQUIRE(value >= 1 && value <= (1 << 20), BT_ERR_INVALID_ARGUMENT,
                "bt_set_option: prefetch_min_grid=%d outside [1, 2^20]", value);
@@ -442,6 +447,8 @@ extern "C" int bt_get_option(const char *name, int *value) {
     *value = g_attention_key_split.load();
   } else if (!strcmp(name, "layer_prepack")) {
     *value = g_layer_prepack.load();
+  } else if (!strcmp(name, "padded_mask_direct")) {
+    *value = g_padded_mask_direct.load();
   } else if (!strcmp(name, "f32_gemm_tile")) {
     *value = g_f32_gemm_tile.load();
   } else if (!strcmp(name, "attention_short_limit")) {

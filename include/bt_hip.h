@@ -58,6 +58,11 @@ const char *bt_last_error_string(void);
  *                   slot and are merged at the end
  *   "layer_prepack" -1 (default) | 0 | 1: answer of bt_gemm_prepack_pays: by the measured
  *                   table | never | always
+ *   "padded_mask_direct"  320 (default): on padded rows (batches of one and two) a layer of
+ *                   up to this many tokens per sequence goes without bt_layer_prologue: its
+ *                   attention applies the mask tensor itself, which needs no offsets, and a
+ *                   launch less is worth more there than the keys the lengths would skip;
+ *                   0 = every layer starts with the prologue.  Same results either way.
  *   "prefetch"      1 (default) | 0: honour / ignore the prefetch hint of the attention entries
  *   "prefetch_min_grid"  512 (default): attention launches of fewer workgroups ignore the hint
  *                   (there the warm-up costs more than it returns); 1 = every launch honours it

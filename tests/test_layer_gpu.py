@@ -790,6 +790,37 @@ def test_layer_prepack_choice_never_changes_the_result(device):
                tag="layer_prepack " + cfg.name)
 
 
+def test_short_padded_layers_go_without_the_prologue(device):
+    """Batches of one and two with up to padded_mask_direct tokens per sequence skip the
+    prologue launch and let the attention apply the mask tensor: same results as with the
+    prologue (lengths + prefix verdict), for the prefix mask, for a mask of another shape and
+    with an attention bias."""
+    _say("padded_mask_direct")
+    from bytetransformer_amd import ops
+    bt.load_th_op()
+    op = torch.ops.ByteTransformer.BertTransformer
+    assert ops.get_option("padded_mask_direct") == 320
+    for B, S, lens in ((1, 64, (38,)), (2, 72, (72, 31)), (2, 256, (154, 256)), (1, 320, (257,))):
+        cfg = workload.EncoderConfig("direct", B, S, 3, layers=1, lens=lens, seed=B * S)
+        wl = workload.make_workload(cfg, bias_std=0.05, random_affine=True)
+        w = [_dev(wl.layers[0][n], device) for n in workload.WEIGHT_NAMES]
+        x = _dev(wl.x, device)
+        banded = np.tril(np.ones((S, S), np.float16), 3) * np.triu(np.ones((S, S), np.float16), -5)
+        for mask_np in (wl.mask, np.broadcast_to(banded, (B, S, S)).copy()):
+            m = _dev(mask_np, device)
+            got = {}
+            try:
+                for limit in (320, 0):
+                    ops.set_option("padded_mask_direct", limit)
+                    got[limit] = op(3, 64, *w, x, m, True, True)
+            finally:
+                ops.set_option("padded_mask_direct", 320)
+            assert torch.equal(got[320], got[0]), (B, S)
+        
+        ref = op(3, 64, *w, x, _dev(wl.mask, device), True, True).cpu().numpy()
+        _check(O.masked_output(ref, wl.lens), _oracle(wl), wl.lens, tag="mask direct %dx%d" % (B, S))
+
+
 def test_th_op_under_graph_capture(device):
     """Two operator layers captured with torch.cuda.graph (the host keeps out of a capture:
     no token count is read back, the layer builds its offsets inside the graph), replayed
