@@ -233,6 +233,15 @@ def hipblaslt_calibration(wl, dev, iters):
         tf = 2.0 * m * n * k / (ms * 1e-3) / 1e12
         out[name] = {"m": m, "n": n, "k": k, "us": round(ms * 1e3, 2), "tflops": round(tf, 1),
                      "frac": round(tf / MFMA_F16_PEAK_TFLOPS, 4)}
+        if name == "square_8192":
+            # the in-tree product on the same large shape (plain epilogue, weight as stored and
+            # pre-packed): what its k loop sustains once fill, stores and tile quantisation are
+            # amortised, beside the vendor library's figure
+            from bytetransformer_amd import ops
+            bt_ = ops.transpose_weight(b)
+            for key, w_, kn in (("in_tree_tflops_as_stored", b, True), ("in_tree_tflops_prepacked", bt_, False)):
+                ms2 = time_kernel(lambda: ops.gemm(a, w_, out=c, w_kn=kn), max(5, iters // 5))
+                out[name][key] = round(2.0 * m * n * k / (ms2 * 1e-3) / 1e12, 1)
     return out
 
 
