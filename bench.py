@@ -160,7 +160,8 @@ def kernel_table(wl, dev, iters):
                                        w_kn=kn_2), "mfma",
          2 * M * F * H),
         ("layernorm_restore", lambda: ops.add_bias_residual_layernorm_restore(
-            ffn2, proj, w["output_bias"], g1, b1, batch_idx, B, S, out_padded=out_pad),
+            ffn2, proj, w["output_bias"], g1, b1, batch_idx, B, S, out_padded=out_pad,
+            word_idx=word_idx),
          "hbm", 2 * M * H * 2 + T * H * 2),
         ("transpose_weights", lambda: ops.transpose_weights([w[n] for n in names], out=all_wt),
          "hbm", 2 * (4 * H * H + 2 * H * F) * 2),

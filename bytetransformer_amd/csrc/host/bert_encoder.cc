@@ -205,7 +205,7 @@ void BertEncoder<OpType>::infer(BertEncoderInferParam<DataType_> ip) {
       check_bt_error(bt_add_bias_residual_layernorm_restore(
           ffn2_out, attr_matmul_buf, w.output_bias, w.output_layernorm_gamma,
           w.output_layernorm_beta, use_fp32_ ? 1 : 0, ip.transformer_output, et_param.batch_idx,
-          batch_size, seq_len, hidden, layernorm_eps, stream));
+          et_param.word_idx, batch_size, seq_len, hidden, layernorm_eps, stream));
     else
       check_bt_error(bt_add_bias_residual_layernorm(
           ffn2_out, attr_matmul_buf, nullptr, w.output_bias, w.output_layernorm_gamma,

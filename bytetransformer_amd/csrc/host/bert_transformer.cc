@@ -284,7 +284,10 @@ void BertTransformer<OpType>::bert_infer(BertTransformerInferParam infer_param) 
     check_bt_error(bt_add_bias_residual_layernorm_restore(
         transformer_out, attr_matmul_buf, param_.output_bias, param_.output_layernorm_gamma,
         param_.output_layernorm_beta, use_fp32_ ? 1 : 0, restore_target, et_param.batch_idx,
-        batch_size, seq_len, hidden, layernorm_eps, stream));
+        // the row map is this call's own word_idx (complete by construction); a caller's
+        // offsets keep the look-up through batch_idx
+        have_offsets ? nullptr : et_param.word_idx, batch_size, seq_len, hidden, layernorm_eps,
+        stream));
   else
     check_bt_error(bt_add_bias_residual_layernorm(
         transformer_out, attr_matmul_buf, nullptr, param_.output_bias, param_.output_layernorm_gamma,

@@ -12,6 +12,71 @@ namespace bt {
 
 constexpr int kLnRowsPerBlock = 4;   // 2, 8 and 16 rows per workgroup measured 0-20 % slower
 
+// Statistics and store of one row held in registers (x = (a + r) + bias, two fp16-rounded adds).
+template <int NC, bool GB32, bool kAffineEarly, int NG>
+__device__ __forceinline__ void ln_finish(const half8_t (&av)[NC], const half8_t (&rv)[NC],
+                                          const half8_t (&bias_v)[NC], const half8_t (&gh)[NC],
+                                          const half8_t (&bh)[NC], const float4_t (&g32)[NG][2],
+                                          const float4_t (&b32)[NG][2], const void *gamma,
+                                          const void *beta, const int (&cc)[NC],
+                                          const bool (&live)[NC], half8_t *o, float inv_n,
+                                          float eps) {
+  float v[NC][8];
+  float sum = 0.f;
+#pragma unroll
+  for (int i = 0; i < NC; ++i) {
+    const half8_t x = (av[i] + rv[i]) + bias_v[i];  // two fp16-rounded adds
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      v[i][j] = live[i] ? (float)x[j] : 0.f;
+      sum += v[i][j];
+    }
+  }
+  const float mean = wave_sum(sum) * inv_n;
+  float sq = 0.f;
+#pragma unroll
+  for (int i = 0; i < NC; ++i) {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      v[i][j] = live[i] ? v[i][j] - mean : 0.f;
+      sq += v[i][j] * v[i][j];
+    }
+  }
+  const float rstd = rsqrtf(wave_sum(sq) * inv_n + eps);
+
+#pragma unroll
+  for (int i = 0; i < NC; ++i) {
+    float g[8], bt_[8];
+    if (GB32) {
+      float4_t g0, g1, b0, b1;
+      if (kAffineEarly) {
+        g0 = g32[i][0], g1 = g32[i][1], b0 = b32[i][0], b1 = b32[i][1];
+      } else {
+        const float4_t *gp = (const float4_t *)gamma + 2 * cc[i];
+        const float4_t *bp = (const float4_t *)beta + 2 * cc[i];
+        g0 = gp[0], g1 = gp[1], b0 = bp[0], b1 = bp[1];
+      }
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        g[j] = g0[j];
+        g[4 + j] = g1[j];
+        bt_[j] = b0[j];
+        bt_[4 + j] = b1[j];
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        g[j] = (float)gh[i][j];
+        bt_[j] = (float)bh[i][j];
+      }
+    }
+    half8_t y;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) y[j] = (half_t)(v[i][j] * rstd * g[j] + bt_[j]);
+    if (live[i]) o[cc[i]] = y;
+  }
+}
+
 // SPLITS > 0: `src` holds SPLITS fp32 partial sums of the row ([SPLITS][split_rows][H], the
 // output of a split-k GEMM); their sum, rounded to fp16 once, takes the place of `out`.
 //
@@ -66,6 +131,28 @@ __global__ __launch_bounds__(kLnRowsPerBlock *kWave) void layernorm_kernel(
 
   size_t src_row, dst_row = r;
   half8_t av[NC];
+  if (RESTORE && residual_row_index && SPLITS == 0) {
+    // restore through the row map (word_idx of the offsets: entry r < M is the padded
+    // position of packed row r, the entries from M on are the padded positions that stay
+    // empty): only the store address depends on a loaded value, so the rows are requested
+    // together with it.  idx = batch_idx, M = idx[B].
+    src_row = r;
+#pragma unroll
+    for (int i = 0; i < NC; ++i) av[i] = src[src_row * chunks + cc[i]];
+    half8_t rv0[NC];
+#pragma unroll
+    for (int i = 0; i < NC; ++i) rv0[i] = residual[src_row * chunks + cc[i]];
+    dst_row = (size_t)residual_row_index[r];
+    const int M = idx[B];
+    if (r >= M) {
+      const half8_t z = {0, 0, 0, 0, 0, 0, 0, 0};
+      for (int c = lane; c < chunks; c += kWave) dst[dst_row * chunks + c] = z;
+      return;
+    }
+    ln_finish<NC, GB32, kAffineEarly>(av, rv0, bias_v, gh, bh, g32, b32, gamma, beta, cc, live,
+                                      dst + dst_row * chunks, inv_n, eps);
+    return;
+  }
   if (RESTORE) {
     // r walks the padded [B, S] grid; idx = batch_idx
     const int b = r / S, s = r - b * S;
@@ -119,61 +206,8 @@ __global__ __launch_bounds__(kLnRowsPerBlock *kWave) void layernorm_kernel(
     }
   }
 
-  float v[NC][8];
-  float sum = 0.f;
-#pragma unroll
-  for (int i = 0; i < NC; ++i) {
-    const half8_t x = (av[i] + rv[i]) + bias_v[i];  // two fp16-rounded adds
-#pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      v[i][j] = live[i] ? (float)x[j] : 0.f;
-      sum += v[i][j];
-    }
-  }
-  const float mean = wave_sum(sum) * inv_n;
-  float sq = 0.f;
-#pragma unroll
-  for (int i = 0; i < NC; ++i) {
-#pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      v[i][j] = live[i] ? v[i][j] - mean : 0.f;
-      sq += v[i][j] * v[i][j];
-    }
-  }
-  const float rstd = rsqrtf(wave_sum(sq) * inv_n + eps);
-
-  half8_t *o = dst + dst_row * chunks;
-#pragma unroll
-  for (int i = 0; i < NC; ++i) {
-    float g[8], bt_[8];
-    if (GB32) {
-      float4_t g0, g1, b0, b1;
-      if (kAffineEarly) {
-        g0 = g32[i][0], g1 = g32[i][1], b0 = b32[i][0], b1 = b32[i][1];
-      } else {
-        const float4_t *gp = (const float4_t *)gamma + 2 * cc[i];
-        const float4_t *bp = (const float4_t *)beta + 2 * cc[i];
-        g0 = gp[0], g1 = gp[1], b0 = bp[0], b1 = bp[1];
-      }
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        g[j] = g0[j];
-        g[4 + j] = g1[j];
-        bt_[j] = b0[j];
-        bt_[4 + j] = b1[j];
-      }
-    } else {
-#pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        g[j] = (float)gh[i][j];
-        bt_[j] = (float)bh[i][j];
-      }
-    }
-    half8_t y;
-#pragma unroll
-    for (int j = 0; j < 8; ++j) y[j] = (half_t)(v[i][j] * rstd * g[j] + bt_[j]);
-    if (live[i]) o[cc[i]] = y;
-  }
+  ln_finish<NC, GB32, kAffineEarly>(av, rv, bias_v, gh, bh, g32, b32, gamma, beta, cc, live,
+                                    dst + dst_row * chunks, inv_n, eps);
 }
 
 template <bool RESTORE, int SPLITS = 0>
@@ -240,8 +274,8 @@ extern "C" int bt_add_bias_residual_layernorm(void *out, const void *residual,
 
 extern "C" int bt_add_bias_residual_layernorm_restore(
     const void *out, const void *residual, const void *bias, const void *gamma, const void *beta,
-    int gamma_beta_fp32, void *out_padded, const int *batch_idx, int batch_size, int seq_len,
-    int hidden_dim, float eps, void *stream) {
+    int gamma_beta_fp32, void *out_padded, const int *batch_idx, const int *word_idx,
+    int batch_size, int seq_len, int hidden_dim, float eps, void *stream) {
   BT_REQUIRE(out && residual && bias && gamma && beta && out_padded && batch_idx,
              BT_ERR_INVALID_ARGUMENT,
              "bt_add_bias_residual_layernorm_restore: null pointer argument");
@@ -250,7 +284,7 @@ extern "C" int bt_add_bias_residual_layernorm_restore(
   BT_REQUIRE((long long)batch_size * seq_len < (1ll << 31), BT_ERR_UNSUPPORTED,
              "bt_add_bias_residual_layernorm_restore: too many rows");
   return launch_ln<true>(out, residual, bias, gamma, beta, gamma_beta_fp32, out_padded, batch_idx,
-                         nullptr, batch_size, seq_len, batch_size * seq_len, hidden_dim, eps,
+                         word_idx, batch_size, seq_len, batch_size * seq_len, hidden_dim, eps,
                          as_stream(stream), "bt_add_bias_residual_layernorm_restore");
 }
 

@@ -140,7 +140,11 @@ __global__ __launch_bounds__(kOffsetThreads) void build_offsets_kernel(
 
   for (int b = blockIdx.x; b < B; b += gridDim.x) {
     const int off = s_off[b], len = s_len[b];
-    for (int i = tid; i < len; i += kOffsetThreads) word_idx[off + i] = b * S + i;
+    // valid tokens first, in order; the padded positions fill the tail from M on (pad_at =
+    // number of padded positions of the sequences before b)
+    const int pad_at = s_off[B] + b * S - off;
+    for (int i = tid; i < S; i += kOffsetThreads)
+      word_idx[i < len ? off + i : pad_at + i - len] = b * S + i;
   }
 }
 
@@ -274,7 +278,9 @@ __global__ __launch_bounds__(kPrologueThreads) void layer_prologue_kernel(
     }
     for (int b = blockIdx.x; b < B; b += offset_blocks) {
       const int off = s_off[b], len = s_len[b];
-      for (int i = tid; i < len; i += kPrologueThreads) word_idx[off + i] = b * S + i;
+      const int pad_at = s_off[B] + b * S - off;   // the padded positions fill the tail from M on
+      for (int i = tid; i < S; i += kPrologueThreads)
+        word_idx[i < len ? off + i : pad_at + i - len] = b * S + i;
     }
   }
 

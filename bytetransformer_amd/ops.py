@@ -279,14 +279,21 @@ def add_bias_residual_layernorm(out, residual, bias, gamma, beta, eps=1e-6, vali
 
 
 def add_bias_residual_layernorm_restore(out, residual, bias, gamma, beta, batch_idx, batch_size,
-                                        seq_len, eps=1e-6, out_padded=None):
+                                        seq_len, eps=1e-6, out_padded=None, word_idx=None):
+    """word_idx: the complete word_idx of the same offsets (the row map); `out` and `residual`
+    must then hold batch_size * seq_len rows."""
     H = out.shape[-1]
+    if word_idx is not None:
+        rows = batch_size * seq_len
+        if word_idx.numel() < rows or out.numel() < rows * H or residual.numel() < rows * H:
+            raise ValueError("restore through word_idx needs batch_size * seq_len rows of out, "
+                             "residual and word_idx")
     if out_padded is None:
         out_padded = torch.empty(batch_size, seq_len, H, dtype=out.dtype, device=out.device)
     _check(kernel_lib().bt_add_bias_residual_layernorm_restore(
         _ptr(out), _ptr(residual), _ptr(bias), _ptr(gamma), _ptr(beta),
-        int(gamma.dtype == torch.float32), _ptr(out_padded), _ptr(batch_idx), batch_size, seq_len,
-        H, float(eps), _stream()))
+        int(gamma.dtype == torch.float32), _ptr(out_padded), _ptr(batch_idx), _ptr(word_idx),
+        batch_size, seq_len, H, float(eps), _stream()))
     return out_padded
 
 

@@ -88,7 +88,8 @@ int bt_get_option(const char *name, int *value);
  *   atten_mask  [batch_size, seq_len, seq_len], dtype mask_dtype (BT_F16/BT_F32);
  *               only row 0 of each batch is read; an element counts when >= 0.5
  *   batch_idx   int[batch_size + 1]  exclusive prefix sum of the lengths, total last
- *   word_idx    int[batch_size * seq_len]; first M entries = b*seq_len + i, i < len_b
+ *   word_idx    int[batch_size * seq_len]; first M entries = b*seq_len + i, i < len_b (the valid
+ *               positions in order), then the batch_size * seq_len - M padded positions
  *   seq_order   NULL, or int[batch_size]: the sequence indices by descending
  *               length (ties by index); the attention kernels use it to start the
  *               longest sequences first (no counterpart in the reference)
@@ -323,13 +324,18 @@ int bt_add_bias_residual_layernorm(void *out, const void *residual,
  * when s < len_b, else zeros.  Replaces
  * add_bias_input_layernorm_restore_output_kernel_launcher (layernorm.h:430-446,
  * kernels :334-373).
+ * word_idx (nullable): the word_idx that bt_build_offsets / bt_layer_prologue wrote beside
+ * this batch_idx, all batch_size * seq_len entries of it (valid positions first, the empty
+ * ones after them).  With it a wave knows its output row from one load that travels together
+ * with its input rows instead of ahead of them; `out` and `residual` must then hold
+ * batch_size * seq_len rows.  Same result.
  */
 int bt_add_bias_residual_layernorm_restore(const void *out, const void *residual,
                                            const void *bias, const void *gamma,
                                            const void *beta, int gamma_beta_fp32,
                                            void *out_padded, const int *batch_idx,
-                                           int batch_size, int seq_len, int hidden_dim,
-                                           float eps, void *stream);
+                                           const int *word_idx, int batch_size, int seq_len,
+                                           int hidden_dim, float eps, void *stream);
 
 /*
  * Split-k pair for launches with few rows and a long k (FFN2 at a few hundred tokens),

@@ -69,7 +69,7 @@ def test_argument_validation_returns_codes_without_gpu():
     assert lib.bt_build_offsets(p, 1, 0, 4, p, p, None, None, None) == 1
     assert lib.bt_add_bias_residual_layernorm(p, p, None, p, p, p, 0, None, 4, 12, 1e-6, None) == 2
     assert lib.bt_add_bias_residual_layernorm(p, p, None, p, p, p, 0, None, 4, 8192, 1e-6, None) == 2
-    assert lib.bt_add_bias_residual_layernorm_restore(p, p, p, p, p, 0, None, p, 2, 4, 64, 1e-6,
+    assert lib.bt_add_bias_residual_layernorm_restore(p, p, p, p, p, 0, None, p, None, 2, 4, 64, 1e-6,
                                                       None) == 1
     assert lib.bt_transpose_weight(None, p, 8, 8, None) == 1
     odd = ctypes.c_void_p(264)   # 8-byte aligned only

@@ -116,6 +116,10 @@ def test_layer_prologue_offsets_and_prefix_verdict(device, B, S, dtype, kind):
     g_bi2, g_wi2, order2, none = ops.layer_prologue(m)
     assert none is None and torch.equal(g_bi2, g_bi) and torch.equal(order2, order)
     assert torch.equal(g_wi2[:M], g_wi[:M])
+    # the tail of word_idx: the padded positions, as bt_build_offsets writes them
+    ref_wi = ops.build_offsets(m)[1]
+    assert torch.equal(g_wi, ref_wi) and torch.equal(g_wi2, ref_wi)
+    assert sorted(g_wi.cpu().tolist()) == list(range(g_wi.numel()))
 
 
 def test_layer_prologue_packs_weights_afresh_in_every_call(device):
@@ -237,15 +241,24 @@ def test_layernorm_restore_zero_fills_padding(device, B, S, H):
     beta = (0.3 * rs.standard_normal(H)).astype(np.float16)
     exp = O.restore(O.add_bias_residual_layernorm(out[:M], res[:M], bias, gamma, beta, 1e-6), bi,
                     B, S)
-    g_bi, _, _ = ops.build_offsets(_dev(mask, device))
-    target = torch.full((B, S, H), float("nan"), dtype=torch.float16, device=device)
-    g = ops.add_bias_residual_layernorm_restore(
-        _dev(out, device), _dev(res, device), _dev(bias, device), _dev(gamma, device),
-        _dev(beta, device), g_bi, B, S, 1e-6, out_padded=target).cpu().numpy()
-    for b in range(B):
-        assert np.all(g[b, lens[b]:].view(np.uint16) == 0)      # exact +0 fill
-    err = np.abs(g.astype(np.float64) - exp)
-    assert np.all(err <= 2.0 ** -10 * np.abs(exp) + 1e-4), err.max()
+    g_bi, g_wi, _ = ops.build_offsets(_dev(mask, device))
+    # word_idx lists the valid positions first and the padded ones after them: a permutation
+    wi_all = g_wi.cpu().numpy()
+    assert np.array_equal(wi_all[:M], wi[:M])
+    pads = np.concatenate([b * S + np.arange(lens[b], S) for b in range(B)]) if M < B * S else []
+    assert np.array_equal(np.sort(wi_all[M:]), np.sort(pads))
+    results = []
+    for row_map in (None, g_wi):        # look-up through batch_idx, and through the row map
+        target = torch.full((B, S, H), float("nan"), dtype=torch.float16, device=device)
+        g = ops.add_bias_residual_layernorm_restore(
+            _dev(out, device), _dev(res, device), _dev(bias, device), _dev(gamma, device),
+            _dev(beta, device), g_bi, B, S, 1e-6, out_padded=target, word_idx=row_map).cpu().numpy()
+        for b in range(B):
+            assert np.all(g[b, lens[b]:].view(np.uint16) == 0)      # exact +0 fill
+        err = np.abs(g.astype(np.float64) - exp)
+        assert np.all(err <= 2.0 ** -10 * np.abs(exp) + 1e-4), err.max()
+        results.append(g)
+    assert np.array_equal(results[0].view(np.uint16), results[1].view(np.uint16))
 
 
 # ---- weight pre-pack -----------------------------------------------------------
