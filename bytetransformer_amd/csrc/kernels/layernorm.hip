@@ -164,18 +164,18 @@ __global__ __launch_bounds__(kLnRowsPerBlock *kWave) void layernorm_kernel(
     }
     src_row = (size_t)start + s;
   } else {
-    // idx = pointer to the live-row count (or null: all rows live).  Row r of `src` and
-    // entry r of the index lie inside their buffers whether or not the row is live, so they
-    // are requested before the count is known.
+    // idx = pointer to the live-row count (or null: all rows live): one scalar load, the same
+    // address for every wave of the launch, and the one thing a wave waits for before it asks
+    // for its rows - the waves of the rows past the count (40 % of a launch sized for the
+    // padded batch) would otherwise read 1.5 KB each for nothing.
     src_row = r;
+    const int M = idx ? *idx : rows_cap;
+    if (r >= M) return;
     if (SPLITS == 0) {
 #pragma unroll
       for (int i = 0; i < NC; ++i) av[i] = src[src_row * chunks + cc[i]];
     }
-    const int ridx = residual_row_index ? residual_row_index[src_row] : 0;
-    const int M = idx ? *idx : rows_cap;
-    if (r >= M) return;
-    const size_t res_row = residual_row_index ? (size_t)ridx : src_row;
+    const size_t res_row = residual_row_index ? (size_t)residual_row_index[src_row] : src_row;
     residual += res_row * chunks;
   }
   if (RESTORE) {
