@@ -59,7 +59,6 @@ void BertEncoder<OpType>::infer(BertEncoderInferParam<DataType_> ip) {
   int *mask_slots = seq_order + max_batch_size_;       // int[256], padded path only
   off += align_up((max_rows * 2 + 2 * (unsigned long long)max_batch_size_ + 2 + 256) * sizeof(int),
                   256);
-  off += align_up(layer_weight_elems() * sizeof(DataType_), 256);
   float *splitk_buf = (float *)(base + off);
   off += align_up(splitk_scratch_bytes(max_rows, (unsigned long long)hidden), 256);
   // the streaming attention's balanced work list: built once per forward beside the offsets

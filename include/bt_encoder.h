@@ -103,8 +103,8 @@ int bt_encoder_layer_forward_static(const bt_encoder_config *cfg, const bt_layer
  *   bt_encoder_prepack_bytes    bytes of the pre-packed weight area of all layers
  *   bt_encoder_prepack          fills that area (one launch per layer); do it once per
  *                               weight set and pass it to every forward
- *   bt_encoder_forward          prepacked == NULL: each layer's weights are pre-packed
- *                               inside the call; attention_bias nullable, shared by
+ *   bt_encoder_forward          prepacked == NULL: the products read each layer's weights
+ *                               as they are stored; attention_bias nullable, shared by
  *                               all layers; valid_rows_hint = expected number of valid
  *                               tokens or 0 (steers tile shapes only)
  * cfg->max_batch_size <= 2 or is_remove_padding == 0 runs every layer on the padded rows.

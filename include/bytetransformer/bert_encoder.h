@@ -26,8 +26,8 @@ struct BertEncoderInferParam {
   int seq_len;
   hipStream_t stream;
   const T *attention_bias = nullptr;   // [head_num, seq_len, seq_len] or null, same for every layer
-  // all layers' pre-packed weights as written by BertEncoder::prepack, or null to
-  // pre-pack each layer's weights inside the call
+  // all layers' pre-packed weights as written by BertEncoder::prepack, or null: the
+  // products then read the weights as they are stored
   const void *prepacked = nullptr;
   int valid_rows_hint = 0;             // expected number of valid tokens (0 = unknown); tile choice only
 };
@@ -89,15 +89,13 @@ class BertEncoder {
   // Scratch (elements of DataType_, T = max_batch*max_seq*hidden): [0,3T) qkv heads |
   // [3T,4T) attention out | [4T,5T) projection / LN1 | [5T,6T) packed hidden state |
   // [6T,(6+mult)T) FFN1 | word_idx int[B*S] | batch_idx int[B+1] | seq order int[B] |
-  // one layer's pre-packed weights (used only when the caller passes none) | split-k partial
-  // sums | the streaming attention's work list
+  // split-k partial sums | the streaming attention's work list
   unsigned long long cal_bufsize() const {
     const unsigned long long rows = (unsigned long long)max_batch_size_ * max_seq_len_;
     const unsigned long long tensor = rows * head_num_ * size_per_head_;
     unsigned long long n = align_up((6 + intermediate_size_) * tensor * sizeof(DataType_), 256);
     // (+ 256 ints: the verdict slots of the prefix-mask check of the padded path)
     n += align_up((rows * 2 + 2 * (unsigned long long)max_batch_size_ + 2 + 256) * sizeof(int), 256);
-    n += align_up(layer_weight_elems() * sizeof(DataType_), 256);
     n += align_up(splitk_scratch_bytes(rows, (unsigned long long)head_num_ * size_per_head_), 256);
     n += align_up(attention_layer_->work_list_capacity(), 256);   // the attention's work list
     return n;
