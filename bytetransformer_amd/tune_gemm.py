@@ -112,7 +112,7 @@ def measure(iters=32):
 
 def merge_runs(rows):
     """One row per (shape, layout, row count): the median of every tile's time over the runs
-    that measured it.  Boxes differ (one of four runs here had every loader-wave tile 20-30 %
+    that measured it.  Boxes differ (one of five runs here had every loader-wave tile 20-30 %
     slower than the others), and a table from one box alone inherits its quirks."""
     import statistics
     seen = {}
