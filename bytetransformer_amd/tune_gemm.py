@@ -5,7 +5,7 @@ stored and the [n, k] pre-pack), and writes the table the launcher consults (csr
     python -m bytetransformer_amd.tune_gemm [--json timings.json] [--from-json run1.json run2.json ...]
 
 Needs a GPU unless --from-json replays earlier measurements; several runs (ideally from
-several machines) are merged by the median of each entry.  Shapes outside the table
+several machines) are merged by the upper quartile of each entry.  Shapes outside the table
 keep using the launcher's analytic cost model."""
 import argparse
 import json
@@ -111,17 +111,21 @@ def measure(iters=32):
 
 
 def merge_runs(rows):
-    """One row per (shape, layout, row count): the median of every tile's time over the runs
-    that measured it.  Boxes differ (one of five runs here had every loader-wave tile 20-30 %
-    slower than the others), and a table from one box alone inherits its quirks."""
-    import statistics
+    """One row per (shape, layout, row count): every tile's time at the upper quartile of the
+    runs that measured it (the second-largest of five).  Boxes differ - the tiles with
+    dedicated loader waves by up to +-15 % from box to box where the 256 x 256 tile moves
+    +-2 %, and one of five runs here had every loader-wave tile 20-30 % slower than the others
+    - so a tile that is fast on most boxes and slow on some is priced at its slow side, and a
+    table from one box alone would inherit that box's quirks."""
+    import math
     seen = {}
     for r in rows:
         key = (r["M"], r["N"], r["K"], r.get("epi", "plain"), r.get("kn", 0))
         for tile, us in r["us"].items():
             seen.setdefault(key, {}).setdefault(tile, []).append(us)
+    pick = lambda v: sorted(v)[math.ceil(0.75 * (len(v) - 1))]
     return [{"M": m, "N": n, "K": k, "epi": epi, "kn": kn,
-             "us": {t: round(statistics.median(v), 2) for t, v in by_tile.items()}}
+             "us": {t: round(pick(v), 2) for t, v in by_tile.items()}}
             for (m, n, k, epi, kn), by_tile in seen.items()]
 
 

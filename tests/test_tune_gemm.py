@@ -33,8 +33,10 @@ def test_committed_table_matches_the_tuner_grid():
     assert os.path.getsize(tune_gemm.INC) < 256 * 1024
 
 
-def test_runs_are_merged_by_the_median_of_each_entry():
+def test_runs_are_merged_by_the_upper_quartile_of_each_entry():
     mk = lambda us: {"M": 256, "N": 768, "K": 768, "epi": "plain", "kn": 0, "us": us}
-    merged = tune_gemm.merge_runs([mk({"0": 10.0, "1": 5.0}), mk({"0": 30.0, "1": 6.0}),
-                                   mk({"0": 11.0})])
-    assert len(merged) == 1 and merged[0]["us"] == {"0": 11.0, "1": 5.5}
+    five = [mk({"0": v, "1": 5.0}) for v in (10.0, 30.0, 11.0, 12.0, 9.0)] + [mk({"1": 7.0})]
+    merged = tune_gemm.merge_runs(five)
+    # tile 0: second-largest of five; tile 1: six values, index ceil(0.75 * 5) = 4
+    assert len(merged) == 1 and merged[0]["us"] == {"0": 12.0, "1": 5.0}
+    assert tune_gemm.merge_runs([mk({"0": 3.0})])[0]["us"] == {"0": 3.0}
