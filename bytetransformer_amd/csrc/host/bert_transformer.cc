@@ -5,6 +5,7 @@
 // stays in batch_idx[batch_size] and every kernel bounds itself with it.
 #include "bytetransformer/bert_transformer.h"
 
+
 namespace bytetransformer {
 
 template <OperationType OpType>
@@ -121,12 +122,10 @@ void BertTransformer<OpType>::bert_infer(BertTransformerInferParam infer_param) 
       !(have_offsets && infer_param.mask_prefix >= 0))
     mask_slots = (int *)(base + inner_buf_size_);
 
-  // The streaming attention's balanced work list, when a launch of this shape uses one: the
-  // prologue builds it beside the offsets, the kernel then finds its work with one load.
+  // No attention work list here: building it lengthens this layer's prologue by more than the
+  // attention saves with it (the kernel finds its balanced order by a look-up of its own).
+  // The whole-encoder entry, which builds one list for all its layers, does use it.
   void *work_list = nullptr;
-  if (streaming_fp16 && !have_offsets && !mask_direct &&
-      bt_attention_worklist_bytes(batch_size, seq_len, head_num_) > 0)
-    work_list = base + inner_buf_size_ + Attention<OpType>::work_list_offset();
 
   // One launch ahead of the layer: lengths and offsets from the mask (needed on both
   // paths: keys past len_b are excluded), the prefix-mask verdict, the weight copies.
