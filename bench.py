@@ -145,6 +145,15 @@ def kernel_table(wl, dev, iters):
             x2d, wt_qkv, w["qkv_bias"], heads, valid_rows=vr, out=qkv, a_row_index=word_idx,
             rows_hint=M, w_kn=kn_qkv),
          "mfma", 2 * M * H * 3 * H),
+    ]
+    if ops.gemm_qkv_mask_rows_supported(B, S, mask.dtype):
+        # the same product with the live rows counted from the mask inside the launch (what a
+        # layer starts with when no per-call weight copy pays; stand-alone entry otherwise)
+        mr_out = (torch.empty_like(batch_idx), torch.empty_like(word_idx), torch.empty_like(seq_order))
+        rows.append(("gemm_qkv_bias_split_mask_rows", lambda: ops.gemm_qkv_bias_split_mask_rows(
+            x, mask, w["qkv_kernel"], w["qkv_bias"], heads, out=qkv, offsets_out=mr_out,
+            rows_hint=M, w_kn=True), "mfma", 2 * M * H * 3 * H))
+    rows += [
         ("attention", lambda: att_fn(qkv, batch_idx, B, S, scale, out=att, seq_order=seq_order),
          "mfma", 4 * H * sq),
         ("gemm_proj", lambda: ops.gemm(att_m, wt_o, valid_rows=vr, out=proj_m, rows_hint=M,

@@ -67,6 +67,16 @@ void BertTransformer<OpType>::bert_infer(BertTransformerInferParam infer_param) 
   const bool mask_direct = streaming_fp16 && !is_remove_padding_ && !have_offsets &&
                            seq_len <= direct_limit &&
                            bt_attention_worklist_bytes(batch_size, seq_len, head_num_) == 0;
+  // Padding-free fp16 layers that have to build their offsets: the QKV product can count the
+  // mask rows itself and leave the offsets for the kernels after it, so that the layer goes
+  // without the launch ahead of it - and without the per-call weight copies that launch
+  // would make, which is why the choice follows the copy plan below.
+  int qkv_mask_rows_opt = -1;
+  bt_get_option("qkv_mask_rows", &qkv_mask_rows_opt);
+  const bool qkv_mask_rows_fits =
+      OpType == OperationType::HALF && is_remove_padding_ && !have_offsets &&
+      qkv_mask_rows_opt != 0 &&
+      bt_gemm_qkv_mask_rows_supported(batch_size, seq_len, Traits_::dtype);
   // The four products read the [k, n] weights as the caller stores them, exactly as the
   // reference hands them to cuBLAS (gemm.cu:27-39): nothing is kept between calls and
   // nothing can go stale.  Where the measured tile table says that a product of this size
@@ -89,7 +99,8 @@ void BertTransformer<OpType>::bert_infer(BertTransformerInferParam infer_param) 
       w_use[i] = param_.prepacked_kernels[i];
       w_kn[i] = 0;
     }
-  } else if (OpType == OperationType::HALF && !mask_direct) {   // (the copies are made by the prologue)
+  } else if (OpType == OperationType::HALF && !mask_direct &&
+             !(qkv_mask_rows_fits && qkv_mask_rows_opt == 1)) {   // (the copies are made by the prologue)
     const long long live = infer_param.valid_rows_hint > 0 ? infer_param.valid_rows_hint
                            : is_remove_padding_            ? (rows * 3LL + 4) / 5
                                                            : rows;
@@ -113,6 +124,7 @@ void BertTransformer<OpType>::bert_infer(BertTransformerInferParam infer_param) 
                       sizeof(DataType_),
                   256);
   float *splitk_buf = (float *)(base + off);
+  const bool qkv_mask_rows = qkv_mask_rows_fits && pack_count == 0;
 
   // Padded rows, fp16 streaming attention: the mask tensor is applied unless one pass over
   // it finds the plain prefix mask of its lengths; the prologue leaves that verdict in the
@@ -144,7 +156,7 @@ void BertTransformer<OpType>::bert_infer(BertTransformerInferParam infer_param) 
         warm[warm_count] = w_use[i];
         warm_bytes[warm_count++] = (unsigned long long)w_k[i] * w_n[i] * sizeof(DataType_);
       }
-  if (!mask_direct && (!have_offsets || mask_slots || pack_count > 0))
+  if (!mask_direct && !qkv_mask_rows && (!have_offsets || mask_slots || pack_count > 0))
     check_bt_error(bt_layer_prologue(atten_mask, Traits_::dtype, batch_size, seq_len,
                                      et_param.batch_idx, et_param.word_idx, seq_order,
                                      mask_slots, work_list, head_num_, is_remove_padding_ ? 0 : 1,
@@ -219,10 +231,16 @@ void BertTransformer<OpType>::bert_infer(BertTransformerInferParam infer_param) 
 
   const DataType_ *wt_qkv = w_use[0], *wt_proj = w_use[1], *wt_inter = w_use[2], *wt_out = w_use[3];
 
-  check_bt_error(bt_gemm_qkv_bias_split(from_tensor, gather, wt_qkv,
-                                        param_.attention_param.attr_bias_QKV, qkv_buf, valid_rows,
-                                        rows, rows_hint, head_num_, size_per_head_, w_kn[0],
-                                        stream));
+  if (qkv_mask_rows)
+    check_bt_error(bt_gemm_qkv_bias_split_mask_rows(
+        from_tensor, atten_mask, Traits_::dtype, batch_size, seq_len, wt_qkv,
+        param_.attention_param.attr_bias_QKV, qkv_buf, et_param.batch_idx, et_param.word_idx,
+        seq_order, rows_hint, head_num_, size_per_head_, w_kn[0], stream));
+  else
+    check_bt_error(bt_gemm_qkv_bias_split(from_tensor, gather, wt_qkv,
+                                          param_.attention_param.attr_bias_QKV, qkv_buf,
+                                          valid_rows, rows, rows_hint, head_num_, size_per_head_,
+                                          w_kn[0], stream));
 
   struct AttentionInferParam<DataType_> attention_infer_param {
     qkv_buf, atten_mask, attr_out_buf, base + inner_buf_size_, batch_size, seq_len,

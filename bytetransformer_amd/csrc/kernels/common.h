@@ -114,6 +114,84 @@ __device__ __forceinline__ int wave_inclusive_scan(int v, int lane) {
 }
 
 
+// Inclusive prefix sum over the 64 lanes with data-parallel-primitive adds only: four
+// shifts inside each row of 16, then lane 15 of rows 0 / 2 into rows 1 / 3 and lane 31
+// into the upper half.
+__device__ __forceinline__ int wave_inclusive_sum(int v) {
+  v += __builtin_amdgcn_update_dpp(0, v, 0x111, 0xf, 0xf, true);   // row_shr:1
+  v += __builtin_amdgcn_update_dpp(0, v, 0x112, 0xf, 0xf, true);   // row_shr:2
+  v += __builtin_amdgcn_update_dpp(0, v, 0x114, 0xf, 0xf, true);   // row_shr:4
+  v += __builtin_amdgcn_update_dpp(0, v, 0x118, 0xf, 0xf, true);   // row_shr:8
+  v += __builtin_amdgcn_update_dpp(0, v, 0x142, 0xa, 0xf, false);  // row_bcast:15 -> rows 1, 3
+  v += __builtin_amdgcn_update_dpp(0, v, 0x143, 0xc, 0xf, false);  // row_bcast:31 -> rows 2, 3
+  return v;
+}
+
+// Sum over the 64 lanes, as a wave-uniform value.
+__device__ __forceinline__ int wave_total(int v) {
+  return __builtin_amdgcn_readlane(wave_inclusive_sum(v), 63);
+}
+
+// Number of row elements >= 0.5 (the length rule of the offsets, remove_padding.h:36-86),
+// counted by one wave for R mask rows at a time (row r may be null: length 0).
+// A mask row that has not been touched since the last layer comes from HBM: the wave
+// fetches it with 16-byte loads, 4 per lane in flight over the R rows (R rows of up to
+// 2048 / R halfs are one round trip; element by element a 512-token row was eight
+// dependent ones).
+template <typename T, int R>
+__device__ __forceinline__ void wave_row_lengths(const T *const *row, int S, int lane,
+                                                 int (&count)[R]) {
+  constexpr int kVec = 16 / (int)sizeof(T);
+  constexpr int kUnroll = 4 / R;
+  static_assert(R == 1 || R == 2 || R == 4, "rows per call");
+  bool vec = S % kVec == 0;
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    count[r] = 0;
+    vec = vec && (reinterpret_cast<uintptr_t>(row[r]) & 15) == 0;
+  }
+  if (vec) {
+    for (int j0 = 0; j0 < S; j0 += kWave * kVec * kUnroll) {
+      uint4_t raw[R][kUnroll];
+#pragma unroll
+      for (int r = 0; r < R; ++r)
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) {
+          const int j = j0 + (u * kWave + lane) * kVec;
+          raw[r][u] = uint4_t{0u, 0u, 0u, 0u};
+          if (row[r] && j < S) raw[r][u] = *(const uint4_t *)(row[r] + j);
+        }
+#pragma unroll
+      for (int r = 0; r < R; ++r)
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) {
+          const T *e = (const T *)&raw[r][u];
+#pragma unroll
+          for (int i = 0; i < kVec; ++i) count[r] += (float)e[i] >= 0.5f;
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < R; ++r) count[r] = wave_total(count[r]);
+    return;
+  }
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    if (!row[r]) continue;
+    for (int i0 = 0; i0 < S; i0 += kWave) {
+      const int i = i0 + lane;
+      const bool on = (i < S) && ((float)row[r][i] >= 0.5f);
+      count[r] += __popcll(__ballot(on));
+    }
+  }
+}
+template <typename T>
+__device__ __forceinline__ int wave_row_length(const T *__restrict__ row, int S, int lane) {
+  const T *const rows[1] = {row};
+  int count[1];
+  wave_row_lengths<T, 1>(rows, S, lane, count);
+  return count[0];
+}
+
 // ---- 64 x 64 tile of the weight pre-pack: wt[n][k] = w[k][n] ---------------------------
 // 256 threads (t = 0..255) move one tile through `tile`; both sides are 16-byte accesses.
 // `live` = false keeps a thread group in step (it meets the barrier) without touching memory.
@@ -165,19 +243,6 @@ __device__ __forceinline__ void transpose_tile_64(const half_t *__restrict__ w,
 // sum invert j -> (rank, head, tile) with the two dependent loads a plain look-up needs
 // as well.  Args: a kernel argument struct with B, S, heads, nqb, padded_rows, batch_idx
 // and seq_order.
-
-// Inclusive prefix sum over the 64 lanes with data-parallel-primitive adds only: four
-// shifts inside each row of 16, then lane 15 of rows 0 / 2 into rows 1 / 3 and lane 31
-// into the upper half.
-__device__ __forceinline__ int wave_inclusive_sum(int v) {
-  v += __builtin_amdgcn_update_dpp(0, v, 0x111, 0xf, 0xf, true);   // row_shr:1
-  v += __builtin_amdgcn_update_dpp(0, v, 0x112, 0xf, 0xf, true);   // row_shr:2
-  v += __builtin_amdgcn_update_dpp(0, v, 0x114, 0xf, 0xf, true);   // row_shr:4
-  v += __builtin_amdgcn_update_dpp(0, v, 0x118, 0xf, 0xf, true);   // row_shr:8
-  v += __builtin_amdgcn_update_dpp(0, v, 0x142, 0xa, 0xf, false);  // row_bcast:15 -> rows 1, 3
-  v += __builtin_amdgcn_update_dpp(0, v, 0x143, 0xc, 0xf, false);  // row_bcast:31 -> rows 2, 3
-  return v;
-}
 
 struct AttWork {
   int b, head, qb, seq_start, len;

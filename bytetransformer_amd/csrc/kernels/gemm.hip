@@ -31,6 +31,8 @@
 // `valid_rows`; workgroups beyond the live tiles retire at once.
 #include "common.h"
 
+#include <type_traits>
+
 namespace bt {
 
 
@@ -50,7 +52,124 @@ struct GemmArgs {
   int rows_hint;        // host-side estimate of the live rows (0 = unknown); tile choice only
   float *c32;           // kEpiPartial only: [splits][rows_cap][N]
   int w_kn;             // 1: wt is the row-major [K, N] matrix itself
+  // Rows taken straight from the attention mask (the QKV projection of a padding-free
+  // layer): A is the padded [mask_B * mask_S, K] tensor, the live rows and their order are
+  // what the mask's row lengths say, counted by every workgroup for itself - no launch
+  // ahead of the product has to build a row index first.  Workgroup 0 leaves the offsets
+  // for the kernels that follow (each pointer may be null).
+  const void *mask;     // [mask_B, mask_S, mask_S] or null
+  int mask_f32;         // element type: 0 half, 1 float
+  int mask_B, mask_S;
+  int *out_batch_idx;   // [mask_B + 1]
+  int *out_word_idx;    // [mask_B * mask_S]: the complete row map (valid positions, then the padded ones)
+  int *out_seq_order;   // [mask_B]
 };
+
+// ---- rows from the mask ---------------------------------------------------------
+constexpr int kMaskRowsMaxBatch = 64;   // one wave scans the lengths
+
+// Per-lane view of the offsets, the same in every wave: lane l < B holds sequence l.
+struct MaskRows {
+  int len;     // its length
+  int excl;    // its first packed row (lanes >= B: M)
+  int delta;   // l * S - excl: padded row = packed row + delta
+  int M;       // live rows
+};
+
+// All `nwaves` waves of the workgroup take part (one barrier inside).  `s_len`: 64 ints of
+// LDS that nothing else writes until every wave has left this function.
+__device__ __forceinline__ MaskRows mask_rows_setup(const GemmArgs &p, int wave, int nwaves,
+                                                    int lane, int *s_len) {
+  const int B = p.mask_B, S = p.mask_S;
+  const size_t plane = (size_t)S * S;
+  // R rows per wave in flight at a time: two for up to 2 * nwaves sequences (their 16-byte
+  // loads cover rows of up to 1024 halfs in one round trip), four beyond
+  auto count_rows = [&](auto elem_tag, auto r_tag) {
+    using T = decltype(elem_tag);
+    constexpr int R = decltype(r_tag)::value;
+    const T *m = (const T *)p.mask;
+    for (int b0 = wave; b0 < B; b0 += R * nwaves) {
+      const T *rows[R];
+      int count[R];
+#pragma unroll
+      for (int r = 0; r < R; ++r)
+        rows[r] = b0 + r * nwaves < B ? m + (b0 + r * nwaves) * plane : nullptr;
+      wave_row_lengths<T, R>(rows, S, lane, count);
+      if (lane == 0) {
+#pragma unroll
+        for (int r = 0; r < R; ++r)
+          if (b0 + r * nwaves < B) s_len[b0 + r * nwaves] = count[r];
+      }
+    }
+  };
+  using two = std::integral_constant<int, 2>;
+  using four = std::integral_constant<int, 4>;
+  if (p.mask_f32) {
+    if (B <= 2 * nwaves) count_rows(float{}, two{}); else count_rows(float{}, four{});
+  } else {
+    if (B <= 2 * nwaves) count_rows(half_t{}, two{}); else count_rows(half_t{}, four{});
+  }
+  __syncthreads();
+  MaskRows mr;
+  mr.len = lane < B ? s_len[lane] : 0;
+  const int incl = wave_inclusive_sum(mr.len);
+  mr.excl = incl - mr.len;
+  mr.delta = lane * S - mr.excl;
+  mr.M = __builtin_amdgcn_readlane(incl, 63);
+  return mr;
+}
+
+// Which sequences the packed rows [r0, r1] (0 <= r0 <= r1 < M, wave-uniform) belong to: the
+// first one and how many more.  The first packed rows rise with the lane, so the lanes whose
+// sequence starts at or before a row form a prefix; the last of them holds the row (empty
+// sequences in between start at the same row and lose to it).
+struct MaskRowSpan {
+  int first, more;
+};
+__device__ __forceinline__ MaskRowSpan mask_rows_span(const MaskRows &mr, int B, int lane, int r0,
+                                                      int r1) {
+  const int lo = __popcll(__ballot(lane < B && mr.excl <= r0)) - 1;
+  const int hi = __popcll(__ballot(lane < B && mr.excl <= r1)) - 1;
+  return MaskRowSpan{lo, hi - lo};
+}
+
+// Padded row of packed row r inside such a span.  Every lane of the wave must call it (the
+// look-ups read the other lanes' registers).
+__device__ __forceinline__ int mask_rows_map(const MaskRows &mr, const MaskRowSpan &sp, int r) {
+  int b = sp.first;
+  for (int k = 1; k <= sp.more; ++k) b += r >= __builtin_amdgcn_readlane(mr.excl, sp.first + k);
+  return r + __shfl(mr.delta, b, 64);
+}
+
+// The offsets as the stand-alone launch writes them (padding.hip), by `nthreads` threads
+// (whole waves, t = thread index among them) of one workgroup.
+__device__ __forceinline__ void mask_rows_write(const GemmArgs &p, const MaskRows &mr, int t,
+                                                int nthreads, int lane) {
+  const int B = p.mask_B, S = p.mask_S;
+  if (t < 64) {   // the first of the writing waves
+    if (p.out_batch_idx) {
+      if (lane < B) p.out_batch_idx[lane] = mr.excl;
+      if (lane == 0) p.out_batch_idx[B] = mr.M;
+    }
+    if (p.out_seq_order) {
+      // sequences by descending length (ties by index): rank by counting
+      int rank = 0;
+      for (int o = 0; o < B; ++o) {
+        const int lo = __shfl(mr.len, o, 64);
+        rank += (lo > mr.len) || (lo == mr.len && o < lane);
+      }
+      if (lane < B) p.out_seq_order[rank] = lane;
+    }
+  }
+  if (p.out_word_idx) {
+    for (int b = 0; b < B; ++b) {
+      const int off = __shfl(mr.excl, b, 64), len = __shfl(mr.len, b, 64);
+      const int pad_at = mr.M + b * S - off;   // the padded positions fill the tail from M on
+      for (int i = t; i < S; i += nthreads)
+        p.out_word_idx[i < len ? off + i : pad_at + i - len] = b * S + i;
+    }
+  }
+}
 
 __device__ __forceinline__ float gelu_tanh_f32(float x) {
   // 0.5 x (1 + tanh(u)) == x / (1 + exp(-2u)),  u = 0.79788456 (x + 0.044715 x^3)
@@ -174,7 +293,17 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs &p) {
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int M = p.valid_rows ? min(*p.valid_rows, p.rows_cap) : p.rows_cap;
+  int M;
+  MaskRows mr{};
+  if (p.mask) {
+    // the last ring stage is first written after the first barrier of the k loop, which
+    // every wave reaches only after it has read the lengths
+    mr = mask_rows_setup(p, wave, NW + NP, lane, (int *)(smem + (STAGES - 1) * STAGE_HALFS));
+    M = min(mr.M, p.rows_cap);
+    if (blockIdx.x == 0 && blockIdx.y == 0 && wave < NW) mask_rows_write(p, mr, tid, NW * 64, lane);
+  } else {
+    M = p.valid_rows ? min(*p.valid_rows, p.rows_cap) : p.rows_cap;
+  }
 
   // XCD-aware tile order over the live tiles
   int tile_m, tile_n;
@@ -207,7 +336,7 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs &p) {
   // (load clocks ~ MFMA clocks) that serialisation costs half of the throughput.
   const bool loader = NP == 0 || wave >= NW;
   const int lw = NP == 0 ? wave : wave - NW;    // index among the loading waves
-  const bool gather = p.a_row_index != nullptr;
+  const bool gather = p.a_row_index != nullptr || p.mask != nullptr;
   const rsrc_t rs_a =
       gather ? make_rsrc(p.a + k_first, ((size_t)p.rows_cap * p.K - k_first) * sizeof(half_t))
              : make_rsrc(p.a + (size_t)m0 * p.K + k_first,
@@ -221,12 +350,17 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs &p) {
                       ((size_t)(p.N - n0) * p.K - k_first) * sizeof(half_t));
   int voff[NI];
   if (loader) {
+    MaskRowSpan span{};
+    if (p.mask) span = mask_rows_span(mr, p.mask_B, lane, m0, min(m0 + BM, M) - 1);
 #pragma unroll
     for (int i = 0; i < NI; ++i) {
       const int r = (i * NL + lw) * 8 + (lane >> 3);
       const int kc = (lane & 7) ^ swz(r);
       int row = i < NIA ? r : r - BM;
-      if (i < NIA && gather) row = p.a_row_index[min(m0 + r, M - 1)];   // live rows only hold valid indices
+      if (i < NIA && gather) {   // live rows only hold valid indices
+        const int live_row = min(m0 + r, M - 1);
+        row = p.mask ? mask_rows_map(mr, span, live_row) : p.a_row_index[live_row];
+      }
       voff[i] = (row * p.K + kc * 8) * (int)sizeof(half_t);
       if (WKN && i >= NIA) voff[i] = kn_load_offset<BN>((i - NIA) * NL + lw, lane, p.N, p.N - n0);
     }
@@ -432,7 +566,16 @@ __device__ __forceinline__ void gemm_tiles_flat(const GemmArgs &p) {
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int M = p.valid_rows ? min(*p.valid_rows, p.rows_cap) : p.rows_cap;
+  int M;
+  MaskRows mr{};
+  if (p.mask) {
+    // (the last ring stage: first written after the first barrier of the k loop)
+    mr = mask_rows_setup(p, wave, NW + NP, lane, (int *)(smem + (STAGES - 1) * STAGE_HALFS));
+    M = min(mr.M, p.rows_cap);
+    if (blockIdx.x == 0 && wave < NW) mask_rows_write(p, mr, tid, NW * 64, lane);
+  } else {
+    M = p.valid_rows ? min(*p.valid_rows, p.rows_cap) : p.rows_cap;
+  }
 
   // XCD x owns the contiguous range [x * per, (x + 1) * per) of the live tiles; its
   // workgroups take them round-robin
@@ -450,7 +593,7 @@ __device__ __forceinline__ void gemm_tiles_flat(const GemmArgs &p) {
   // ---- loading side: a cursor (tile, k-step) STAGES - 1 steps ahead of the products ----
   const bool loader = NP == 0 || wave >= NW;
   const int lw = NP == 0 ? wave : wave - NW;
-  const bool gather = p.a_row_index != nullptr;
+  const bool gather = p.a_row_index != nullptr || p.mask != nullptr;
   rsrc_t rs_a = make_rsrc(p.a, 0), rs_w = make_rsrc(p.wt, 0);
   constexpr bool kHasBias = EPI == kEpiBiasGelu || EPI == kEpiQkvSplit || EPI == kEpiBias;
   // The bias of a tile's columns reaches the computing waves through LDS, fetched by the
@@ -464,10 +607,13 @@ __device__ __forceinline__ void gemm_tiles_flat(const GemmArgs &p) {
   int ld_L = L0, ld_kt = 0, ld_left = loader ? total : 0;
   auto fetch_indices = [&](int Lt) {
     const int m0 = (Lt / p.tiles_n) * BM;
+    MaskRowSpan span{};
+    if (p.mask) span = mask_rows_span(mr, p.mask_B, lane, m0, min(m0 + BM, M) - 1);
 #pragma unroll
     for (int i = 0; i < NIA; ++i) {
       const int r = (i * NL + lw) * 8 + (lane >> 3);
-      idx_next[i] = p.a_row_index[min(m0 + r, M - 1)];   // live rows only hold valid indices
+      const int live_row = min(m0 + r, M - 1);   // live rows only hold valid indices
+      idx_next[i] = p.mask ? mask_rows_map(mr, span, live_row) : p.a_row_index[live_row];
     }
   };
   auto load_setup = [&](int Lt, bool more, bool bias_to_lds) {
@@ -788,7 +934,7 @@ static int cu_count() {
 // caller's hint when it has one, else 60 % of the capacity (the fill the padding-free
 // path is built for).
 static long long estimated_rows(const GemmArgs &p) {
-  if (!p.valid_rows) return p.rows_cap;
+  if (!p.valid_rows && !p.mask) return p.rows_cap;
   if (p.rows_hint > 0) return p.rows_hint < p.rows_cap ? p.rows_hint : p.rows_cap;
   return (p.rows_cap * 3LL + 4) / 5;
 }
@@ -1040,6 +1186,49 @@ extern "C" int bt_gemm_qkv_bias_split(const void *a, const int *a_row_index, con
   // the head-major split is the layout of the fp16 attention kernels, which are built for
   // 64-wide heads; any other head size keeps the projections token-major [rows_cap, 3H]
   // for bt_attention_generic_f16
+  if (size_per_head != 64) return launch_gemm<kEpiBias>(p, as_stream(stream));
+  return launch_gemm<kEpiQkvSplit>(p, as_stream(stream));
+}
+
+extern "C" int bt_gemm_qkv_mask_rows_supported(int batch_size, int seq_len, int mask_dtype) {
+  if (batch_size <= 0 || batch_size > kMaskRowsMaxBatch || seq_len <= 0) return 0;
+  if (mask_dtype != BT_F16 && mask_dtype != BT_F32) return 0;
+  // every workgroup reads row 0 of every sequence's mask: keep that to 64 KB
+  return (long long)batch_size * seq_len * (mask_dtype == BT_F32 ? 4 : 2) <= 64 * 1024;
+}
+
+extern "C" int bt_gemm_qkv_bias_split_mask_rows(const void *from_tensor, const void *atten_mask,
+                                                int mask_dtype, int batch_size, int seq_len,
+                                                const void *wt_qkv, const void *bias_qkv,
+                                                void *qkv_heads, int *batch_idx, int *word_idx,
+                                                int *seq_order, int rows_hint, int head_num,
+                                                int size_per_head, int weight_kn, void *stream) {
+  const char *who = "bt_gemm_qkv_bias_split_mask_rows";
+  BT_REQUIRE(head_num > 0 && size_per_head > 0, BT_ERR_INVALID_ARGUMENT,
+             "%s: head_num=%d size_per_head=%d", who, head_num, size_per_head);
+  BT_REQUIRE(batch_size > 0 && seq_len > 0, BT_ERR_INVALID_ARGUMENT,
+             "%s: batch_size=%d seq_len=%d must be positive", who, batch_size, seq_len);
+  BT_REQUIRE(bt_gemm_qkv_mask_rows_supported(batch_size, seq_len, mask_dtype), BT_ERR_UNSUPPORTED,
+             "%s: batch_size=%d seq_len=%d mask_dtype=%d is outside what "
+             "bt_gemm_qkv_mask_rows_supported allows", who, batch_size, seq_len, mask_dtype);
+  const int H = head_num * size_per_head;
+  const int rows_cap = batch_size * seq_len;
+  int rc = check_gemm_args(who, from_tensor, wt_qkv, qkv_heads, rows_cap, 3 * H, H, weight_kn);
+  if (rc) return rc;
+  BT_REQUIRE(bias_qkv && atten_mask && batch_idx, BT_ERR_INVALID_ARGUMENT,
+             "%s: null pointer argument", who);
+  BT_REQUIRE(aligned16({atten_mask}), BT_ERR_INVALID_ARGUMENT,
+             "%s: tensor pointers must be 16-byte aligned", who);
+  // gathered rows are addressed with 32-bit byte offsets from the start of the input
+  BT_REQUIRE((long long)rows_cap * H * 2 <= 0x7fffffffLL, BT_ERR_UNSUPPORTED,
+             "%s: a gathered input of %d x %d halfs is beyond 2 GiB", who, rows_cap, H);
+  GemmArgs p{(const half_t *)from_tensor, (const half_t *)wt_qkv, (const half_t *)bias_qkv,
+             (half_t *)qkv_heads, nullptr, nullptr, rows_cap, 3 * H, H, 0, rows_hint,
+             nullptr, weight_kn};
+  p.mask = atten_mask;
+  p.mask_f32 = mask_dtype == BT_F32;
+  p.mask_B = batch_size, p.mask_S = seq_len;
+  p.out_batch_idx = batch_idx, p.out_word_idx = word_idx, p.out_seq_order = seq_order;
   if (size_per_head != 64) return launch_gemm<kEpiBias>(p, as_stream(stream));
   return launch_gemm<kEpiQkvSplit>(p, as_stream(stream));
 }

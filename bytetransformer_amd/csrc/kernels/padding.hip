@@ -34,6 +34,7 @@ static std::atomic<int> g_prefetch_min_grid{512};
 static std::atomic<int> g_attention_key_split{-1};
 static std::atomic<int> g_layer_prepack{-1};
 static std::atomic<int> g_padded_mask_direct{320};
+static std::atomic<int> g_qkv_mask_rows{-1};
 static std::atomic<int> g_f32_gemm_tile{-1};
 static std::atomic<int> g_attention_short_limit{0};
 static std::atomic<int> g_attention_xcd_map{2};
@@ -49,43 +50,6 @@ int option_layer_prepack() { return g_layer_prepack.load(std::memory_order_relax
 // ---- offsets ----------------------------------------------------------------
 constexpr int kOffsetThreads = 1024;
 constexpr int kOffsetWaves = kOffsetThreads / kWave;
-
-// Number of row elements >= 0.5 (the length rule of the offsets), counted by one wave.
-// A mask row that has not been touched since the last layer comes from HBM: the wave
-// fetches it with 16-byte loads, four per lane in flight (a row of up to 2048 halfs is one
-// round trip; element by element a 512-token row was eight dependent ones).
-template <typename T>
-__device__ __forceinline__ int wave_row_length(const T *__restrict__ row, int S, int lane) {
-  constexpr int kVec = 16 / (int)sizeof(T);
-  int count = 0;
-  if (S % kVec == 0 && (reinterpret_cast<uintptr_t>(row) & 15) == 0) {
-    constexpr int kUnroll = 4;
-    for (int j0 = 0; j0 < S; j0 += kWave * kVec * kUnroll) {
-      uint4_t raw[kUnroll];
-#pragma unroll
-      for (int u = 0; u < kUnroll; ++u) {
-        const int j = j0 + (u * kWave + lane) * kVec;
-        raw[u] = uint4_t{0u, 0u, 0u, 0u};
-        if (j < S) raw[u] = *(const uint4_t *)(row + j);
-      }
-#pragma unroll
-      for (int u = 0; u < kUnroll; ++u) {
-        const T *e = (const T *)&raw[u];
-#pragma unroll
-        for (int i = 0; i < kVec; ++i) count += (float)e[i] >= 0.5f;
-      }
-    }
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) count += __shfl_xor(count, o, 64);
-    return count;
-  }
-  for (int i0 = 0; i0 < S; i0 += kWave) {
-    const int i = i0 + lane;
-    const bool on = (i < S) && ((float)row[i] >= 0.5f);
-    count += __popcll(__ballot(on));
-  }
-  return count;
-}
 
 // Every block recomputes all B lengths (B*S mask elements, a few KB) and the
 // exclusive scan, then writes word_idx for the sequences it owns; block 0 also
@@ -428,6 +392,10 @@ extern "C" int bt_set_option(const char *name, int value) {
     BT_REQUIRE(value >= 0 && value <= (1 << 20), BT_ERR_INVALID_ARGUMENT,
                "bt_set_option: padded_mask_direct=%d outside [0, 2^20]", value);
     g_padded_mask_direct.store(value);
+  } else if (!strcmp(name, "qkv_mask_rows")) {
+    BT_REQUIRE(value >= -1 && value <= 1, BT_ERR_INVALID_ARGUMENT,
+               "bt_set_option: qkv_mask_rows=%d must be -1, 0 or 1", value);
+    g_qkv_mask_rows.store(value);
   } else if (!strcmp(name, "prefetch_min_grid")) {
     BT_REQUIRE(value >= 1 && value <= (1 << 20), BT_ERR_INVALID_ARGUMENT,
                "bt_set_option: prefetch_min_grid=%d outside [1, 2^20]", value);
@@ -455,6 +423,8 @@ extern "C" int bt_get_option(const char *name, int *value) {
     *value = g_layer_prepack.load();
   } else if (!strcmp(name, "padded_mask_direct")) {
     *value = g_padded_mask_direct.load();
+  } else if (!strcmp(name, "qkv_mask_rows")) {
+    *value = g_qkv_mask_rows.load();
   } else if (!strcmp(name, "f32_gemm_tile")) {
     *value = g_f32_gemm_tile.load();
   } else if (!strcmp(name, "attention_short_limit")) {

@@ -210,6 +210,44 @@ def gemm_qkv_bias_split(a, wt_qkv, bias_qkv, head_num, size_per_head=64, valid_r
     return out
 
 
+def gemm_qkv_mask_rows_supported(batch_size, seq_len, mask_dtype=torch.float16):
+    code = BT_F16 if mask_dtype == torch.float16 else BT_F32 if mask_dtype == torch.float32 else -1
+    return bool(kernel_lib().bt_gemm_qkv_mask_rows_supported(batch_size, seq_len, code))
+
+
+def gemm_qkv_bias_split_mask_rows(x, mask, wt_qkv, bias_qkv, head_num, size_per_head=64, out=None,
+                                  offsets_out=None, rows_hint=0, w_kn=False):
+    """QKV projection of the padded x [B, S, H] whose live rows come from the mask inside the
+    launch; returns (qkv_heads, batch_idx, word_idx, seq_order)."""
+    B, S = mask.shape[0], mask.shape[1]
+    H = head_num * size_per_head
+    rows = B * S
+    want = (H, 3 * H) if w_kn else (3 * H, H)
+    if tuple(wt_qkv.shape) != want or x.numel() != rows * H or bias_qkv.numel() != 3 * H:
+        raise ValueError("gemm_qkv_bias_split_mask_rows: x [%d, %d, %d], weight %s and bias [%d] "
+                         "expected" % (B, S, H, list(want), 3 * H))
+    if tuple(mask.shape) != (B, S, S):
+        raise ValueError("gemm_qkv_bias_split_mask_rows: mask must be [B, S, S]")
+    if out is not None and out.numel() < rows * 3 * H:
+        raise ValueError("gemm_qkv_bias_split_mask_rows: out holds %d elements, the launch "
+                         "writes up to %d" % (out.numel(), rows * 3 * H))
+    if out is None:
+        out = torch.zeros(3, head_num, rows, size_per_head, dtype=x.dtype, device=x.device)
+    if offsets_out is None:
+        offsets_out = (torch.empty(B + 1, dtype=torch.int32, device=x.device),
+                       torch.empty(rows, dtype=torch.int32, device=x.device),
+                       torch.empty(B, dtype=torch.int32, device=x.device))
+    batch_idx, word_idx, seq_order = offsets_out
+    if batch_idx.numel() < B + 1 or (word_idx is not None and word_idx.numel() < rows) or \
+            (seq_order is not None and seq_order.numel() < B):
+        raise ValueError("gemm_qkv_bias_split_mask_rows: offset outputs too small")
+    _check(kernel_lib().bt_gemm_qkv_bias_split_mask_rows(
+        _ptr(x), _ptr(mask), _dtype_code(mask), B, S, _ptr(wt_qkv), _ptr(bias_qkv), _ptr(out),
+        _ptr(batch_idx), _ptr(word_idx), _ptr(seq_order), int(rows_hint), head_num, size_per_head,
+        int(w_kn), _stream()))
+    return out, batch_idx, word_idx, seq_order
+
+
 def _attention(fn, qkv_heads, batch_idx, batch_size, seq_len, scale, padded_rows, out,
                seq_order=None, mask=None, bias=None, prefetch=None, extra=()):
     _, head_num, rows_cap, d = qkv_heads.shape

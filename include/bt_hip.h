@@ -63,6 +63,11 @@ const char *bt_last_error_string(void);
  *                   attention applies the mask tensor itself, which needs no offsets, and a
  *                   launch less is worth more there than the keys the lengths would skip;
  *                   0 = every layer starts with the prologue.  Same results either way.
+ *   "qkv_mask_rows" -1 (default) | 0 | 1: a padding-free fp16 layer that has to build its
+ *                   offsets starts with bt_gemm_qkv_bias_split_mask_rows (one launch less,
+ *                   every weight read as stored) where that entry takes the shape and no
+ *                   per-call weight copy pays | always with bt_layer_prologue | with the
+ *                   fused entry wherever it takes the shape.  Same results either way.
  *   "prefetch"      1 (default) | 0: honour / ignore the prefetch hint of the attention entries
  *   "prefetch_min_grid"  512 (default): attention launches of fewer workgroups ignore the hint
  *                   (there the warm-up costs more than it returns); 1 = every launch honours it
@@ -224,6 +229,28 @@ int bt_gemm_qkv_bias_split(const void *a, const int *a_row_index, const void *wt
                            const void *bias_qkv, void *qkv_heads, const int *valid_rows,
                            int rows_cap, int rows_hint, int head_num, int size_per_head,
                            int weight_kn, void *stream);
+
+/*
+ * The same product for a padding-free layer that has not built its offsets yet: the live
+ * rows of the padded from_tensor [batch_size * seq_len, hidden] and their order are taken
+ * from the mask inside the launch (every workgroup counts row 0 of each sequence's mask
+ * itself, remove_padding.h:36-86's length rule), so no launch ahead of the product has
+ * to produce word_idx first.  Workgroup 0 also writes batch_idx [batch_size + 1], word_idx
+ * [batch_size * seq_len] and seq_order [batch_size] exactly as bt_build_offsets /
+ * bt_layer_prologue would (word_idx and seq_order may be null), for the kernels that follow
+ * on the stream.  rows_cap of qkv_heads is batch_size * seq_len.  Covers
+ * build_sequence_length_padding_offset_kernelLauncher + compressBertInput + the QKV GEMM +
+ * the bias add of one layer call (bert_transformer.cu:62-87) in one launch.
+ * bt_gemm_qkv_mask_rows_supported: 1 when the launch takes this shape (at most 64
+ * sequences whose mask rows fit 64 KB), else 0 - then build the offsets first.
+ */
+int bt_gemm_qkv_mask_rows_supported(int batch_size, int seq_len, int mask_dtype);
+int bt_gemm_qkv_bias_split_mask_rows(const void *from_tensor, const void *atten_mask,
+                                     int mask_dtype, int batch_size, int seq_len,
+                                     const void *wt_qkv, const void *bias_qkv, void *qkv_heads,
+                                     int *batch_idx, int *word_idx, int *seq_order,
+                                     int rows_hint, int head_num, int size_per_head,
+                                     int weight_kn, void *stream);
 
 /*
  * Fused multi-head attention over the head-major Q/K/V written by

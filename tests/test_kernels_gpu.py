@@ -497,6 +497,80 @@ def test_gemm_qkv_bias_split(device, tile, heads):
     assert np.all(g[:, :, M:] == 0)
 
 
+@pytest.mark.parametrize("tile", [-1, 0, 1, 2, 3, 4, 5, 6, 7, 8])
+@pytest.mark.parametrize("case", ["ragged", "cfg2", "full", "empty-ends", "one", "f32-mask", "wide"])
+def test_gemm_qkv_rows_from_the_mask(device, tile, case):
+    """The QKV product that counts the mask rows itself: offsets bit-exact with the
+    stand-alone launch (and the oracle), projections bit-identical to offsets -> gather."""
+    _say("gemm_qkv mask rows", tile, case)
+    rs = np.random.RandomState(len(case) + 3 * (tile + 1))
+    heads, mdt = 2, np.float16
+    if case == "ragged":
+        B, S, lens = 5, 70, np.array([70, 0, 33, 1, 64])
+    elif case == "cfg2":
+        B, S = 16, 512
+        lens = rs.randint(100, 513, B)
+    elif case == "full":
+        B, S, lens = 3, 128, np.array([128, 128, 128])
+    elif case == "empty-ends":
+        B, S, lens = 6, 48, np.array([0, 0, 17, 48, 0, 0])
+    elif case == "one":
+        B, S, lens = 1, 200, np.array([77])
+    elif case == "f32-mask":
+        B, S, mdt, lens = 7, 36, np.float32, np.array([36, 5, 5, 0, 20, 1, 36])
+    else:
+        B, S, lens = 64, 64, rs.randint(0, 65, 64)
+    H = heads * 64
+    x = rs.standard_normal((B, S, H)).astype(np.float16)
+    mask = workload.make_mask(lens, S, mdt)
+    w = (rs.standard_normal((H, 3 * H)) * 0.05).astype(np.float16)
+    bias = (rs.standard_normal(3 * H) * 0.5).astype(np.float16)
+    md, xd, wt, bd = _dev(mask, device), _dev(x, device), _prep(_dev(w, device)), _dev(bias, device)
+    assert ops.gemm_qkv_mask_rows_supported(B, S, md.dtype)
+    e_bi, e_wi, e_so, _ = ops.layer_prologue(md)
+    M = int(lens.sum())
+    ops.set_option("gemm_tile", tile)
+    try:
+        ref = _gemm_qkv_bias_split(xd.view(B * S, H), wt, bd, heads, valid_rows=e_bi[B:],
+                                   a_row_index=e_wi)
+        sentinel = lambda n: torch.full((n,), -7, dtype=torch.int32, device=device)
+        outs = (sentinel(B + 1), sentinel(B * S), sentinel(B))
+        got, g_bi, g_wi, g_so = ops.gemm_qkv_bias_split_mask_rows(
+            xd, md, wt, bd, heads, offsets_out=outs, rows_hint=M, w_kn=_KN[0])
+    finally:
+        ops.set_option("gemm_tile", -1)
+    o_bi, o_wi, _ = O.build_offsets(mask)
+    assert np.array_equal(g_bi.cpu().numpy(), o_bi)
+    assert np.array_equal(g_wi.cpu().numpy()[:M], o_wi[:M])
+    assert torch.equal(g_bi, e_bi) and torch.equal(g_wi, e_wi) and torch.equal(g_so, e_so)
+    assert torch.equal(ref[:, :, :M], got[:, :, :M])
+    assert torch.all(got[:, :, M:] == 0)
+    if M:
+        exp = O.split_heads(O.gemm(O.compress(x, o_wi[:M]), w, bias), heads, 64)
+        err = np.abs(got.cpu().numpy()[:, :, :M].astype(np.float64) - exp)
+        assert np.all(err <= 2.0 ** -10 * np.abs(exp) + 2e-4)
+    # without the optional outputs
+    got2, _, _, _ = ops.gemm_qkv_bias_split_mask_rows(
+        xd, md, wt, bd, heads, offsets_out=(sentinel(B + 1), None, None), w_kn=_KN[0])
+    assert torch.equal(got2[:, :, :M], got[:, :, :M])
+
+
+def test_gemm_qkv_rows_from_the_mask_limits(device):
+    assert ops.gemm_qkv_mask_rows_supported(16, 512) and ops.gemm_qkv_mask_rows_supported(32, 1024)
+    assert ops.gemm_qkv_mask_rows_supported(16, 1024, torch.float32)
+    assert not ops.gemm_qkv_mask_rows_supported(65, 16)
+    assert not ops.gemm_qkv_mask_rows_supported(64, 1024)
+    assert not ops.gemm_qkv_mask_rows_supported(16, 2048, torch.float32)
+    assert not ops.gemm_qkv_mask_rows_supported(4, 64, torch.float64)
+    B, S, H = 65, 16, 64
+    with pytest.raises(ops.BtError, match="bt_gemm_qkv_mask_rows_supported"):
+        ops.gemm_qkv_bias_split_mask_rows(
+            torch.zeros(B, S, H, dtype=torch.float16, device=device),
+            torch.ones(B, S, S, dtype=torch.float16, device=device),
+            torch.zeros(3 * H, H, dtype=torch.float16, device=device),
+            torch.zeros(3 * H, dtype=torch.float16, device=device), 1)
+
+
 def test_gather_fused_into_qkv_gemm_and_layernorm(device):
     """a_row_index / residual_row_index = word_idx reads the valid tokens straight from
     the padded input: bit-identical to compress followed by the plain call."""

@@ -790,6 +790,35 @@ def test_layer_prepack_choice_never_changes_the_result(device):
                tag="layer_prepack " + cfg.name)
 
 
+def test_qkv_rows_from_the_mask_never_change_the_result(device):
+    """A padding-free layer may start with the QKV product that counts the mask rows itself
+    instead of the prologue launch: never, wherever the entry takes the shape, and the
+    automatic choice give the same bits - ragged lengths with an empty sequence, the
+    headline shape, and a batch beyond the entry's 64 sequences (which falls back by
+    itself)."""
+    _say("qkv_mask_rows")
+    from bytetransformer_amd import ops
+    bt.load_th_op()
+    op = torch.ops.ByteTransformer.BertTransformer
+    assert ops.get_option("qkv_mask_rows") == -1
+    cases = (workload.EncoderConfig("mr", 6, 200, 12, layers=1, lens=(200, 0, 133, 50, 64, 7), seed=18),
+             workload.EncoderConfig("mr2", 16, 512, 4, layers=1, seed=19),
+             workload.EncoderConfig("mr3", 70, 16, 2, layers=1, seed=20))
+    for cfg in cases:
+        wl = workload.make_workload(cfg, bias_std=0.05, random_affine=True)
+        w = [_dev(wl.layers[0][n], device) for n in workload.WEIGHT_NAMES]
+        x, m = _dev(wl.x, device), _dev(wl.mask, device)
+        got = {}
+        try:
+            for choice in (0, 1, -1):
+                ops.set_option("qkv_mask_rows", choice)
+                got[choice] = op(cfg.head_num, 64, *w, x, m, True, True)
+        finally:
+            ops.set_option("qkv_mask_rows", -1)
+        assert torch.equal(got[0], got[1]) and torch.equal(got[0], got[-1])
+        _check(got[1].cpu().numpy(), _oracle(wl), wl.lens, tag="qkv_mask_rows " + cfg.name)
+
+
 def test_short_padded_layers_go_without_the_prologue(device):
     """Batches of one and two with up to padded_mask_direct tokens per sequence skip the
     prologue launch and let the attention apply the mask tensor: same results as with the
