@@ -248,6 +248,10 @@ __device__ __forceinline__ float4_t add_terms4(const half_t *mask_row, const hal
 // grouped / streaming kernel
 // ---------------------------------------------------------------------------
 constexpr int kKT = 64;                          // keys per streamed tile
+#ifndef BT_LAZY_MAX
+#define BT_LAZY_MAX 8.0f
+#endif
+constexpr float kLazyMax = BT_LAZY_MAX;          // see the running maximum in the tile loop
 constexpr int kTileHalfs = kKT * kHeadDim;       // one K or V tile
 
 // QB 16-query blocks per wave; workgroup covers 4*QB*16 queries.  ADD: a mask tensor and / or an
@@ -467,9 +471,14 @@ __global__ __launch_bounds__(kAttThreads * KS, KS == 1 ? 2 : 4) void attention_g
         mx = fmaxf(fmaxf(mx, s[kb][qb][2]), s[kb][qb][3]);
       }
       mx = rows_max(mx);
-      const float m_new = fmaxf(m_run[qb], mx);
+      // The reference point of a query's exponentials follows its maximum lazily: it moves
+      // only when the maximum has grown by more than kLazyMax binary orders (the first tile
+      // always does).  Probabilities then reach at most 2^kLazyMax - far inside fp16, the
+      // sums are fp32 - and the quotient O / l does not depend on the reference point, while
+      // the rescaling of the running output, a quarter of the vector work of a tile, is
+      // left to the few tiles where a maximum jumps.
+      const float m_new = (mx - m_run[qb]) * cs > kLazyMax ? mx : m_run[qb];
       const float mc = m_new * cs;
-      // rescale the running output only when some query's maximum moved
       if (__builtin_amdgcn_ballot_w64(m_new != m_run[qb]) != 0) {
         const float alpha = fast_exp2(m_run[qb] * cs - mc);
 #pragma unroll
