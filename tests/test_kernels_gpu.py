@@ -555,6 +555,37 @@ def test_gemm_qkv_rows_from_the_mask(device, tile, case):
     assert torch.equal(got2[:, :, :M], got[:, :, :M])
 
 
+@pytest.mark.parametrize("seed", range(12))
+def test_gemm_qkv_rows_from_the_mask_random_shapes(device, seed):
+    """Seeded random batch sizes, sequence lengths (odd ones too: the scalar mask-row path),
+    head counts and lengths with empty sequences: offsets and projections bit-identical to
+    the offsets launch followed by the gathered product."""
+    rs = np.random.RandomState(1000 + seed)
+    B = int(rs.randint(1, 65))
+    S = int(rs.randint(1, min(512, 32768 // B) + 1))
+    heads = int(rs.randint(1, 4))
+    lens = rs.randint(0, S + 1, B)
+    lens[rs.rand(B) < 0.15] = 0
+    _say("gemm_qkv mask rows random", seed, B, S, heads, int(lens.sum()))
+    H = heads * 64
+    mdt = np.float32 if seed % 4 == 3 and B * S * 4 <= 65536 else np.float16
+    x = rs.standard_normal((B, S, H)).astype(np.float16)
+    mask = workload.make_mask(lens, S, mdt)
+    w = (rs.standard_normal((H, 3 * H)) * 0.05).astype(np.float16)
+    bias = (rs.standard_normal(3 * H) * 0.5).astype(np.float16)
+    md, xd, wt, bd = _dev(mask, device), _dev(x, device), _prep(_dev(w, device)), _dev(bias, device)
+    assert ops.gemm_qkv_mask_rows_supported(B, S, md.dtype)
+    e_bi, e_wi, e_so, _ = ops.layer_prologue(md)
+    M = int(lens.sum())
+    ref = _gemm_qkv_bias_split(xd.view(B * S, H), wt, bd, heads, valid_rows=e_bi[B:],
+                               a_row_index=e_wi, rows_hint=M)
+    got, g_bi, g_wi, g_so = ops.gemm_qkv_bias_split_mask_rows(xd, md, wt, bd, heads, rows_hint=M,
+                                                              w_kn=_KN[0])
+    assert torch.equal(g_bi, e_bi) and torch.equal(g_wi, e_wi) and torch.equal(g_so, e_so)
+    assert torch.equal(ref[:, :, :M], got[:, :, :M])
+    assert torch.all(got[:, :, M:] == 0)
+
+
 def test_gemm_qkv_rows_from_the_mask_limits(device):
     assert ops.gemm_qkv_mask_rows_supported(16, 512) and ops.gemm_qkv_mask_rows_supported(32, 1024)
     assert ops.gemm_qkv_mask_rows_supported(16, 1024, torch.float32)
