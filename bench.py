@@ -45,6 +45,9 @@ def parse():
                     help="skip the child process that times the C++ API (profilers that "
                          "initialise the GPU before this program starts forbid spawning it)")
     ap.add_argument("--kernel-iters", type=int, default=50)
+    ap.add_argument("--vendor-compare", action="store_true",
+                    help="counter mode: only the FFN1 shape and 8192^3 through the vendor library "
+                         "and through the in-tree product (see vendor_compare)")
     return ap.parse_args()
 
 
@@ -119,9 +122,9 @@ def kernel_table(wl, dev, iters):
     g1, b1 = w["attr_output_layernorm_gamma"], w["attr_output_layernorm_beta"]
     bo_bi, bo_wi = torch.empty_like(batch_idx), torch.empty_like(word_idx)
     x2d = x.view(T, H)
-    # the operator knows the live row count and sizes the launches after the attention for
-    # it (the QKV product and the attention keep batch * seq_len): time them that way
-    att_m, proj_m, inter_m, ffn2_m, ln_m = att[:M], proj[:M], inter[:M], ffn2[:M], ln_buf[:M]
+    # every launch after the attention is sized for batch * seq_len rows, as the operator sizes
+    # it (the live row count is read on the device; `rows_hint` only steers the tile choice)
+    att_m, proj_m, inter_m, ffn2_m, ln_m = att, proj, inter, ffn2, ln_buf
 
     # the layer's first launch: offsets + the k-contiguous copies of the weights that pay
     pro_out = (bo_bi, bo_wi, torch.empty_like(seq_order), None)
@@ -252,7 +255,54 @@ def hipblaslt_calibration(wl, dev, iters):
             for key, w_, kn in (("in_tree_tflops_as_stored", b, True), ("in_tree_tflops_prepacked", bt_, False)):
                 ms2 = time_kernel(lambda: ops.gemm(a, w_, out=c, w_kn=kn), max(5, iters // 5))
                 out[name][key] = round(2.0 * m * n * k / (ms2 * 1e-3) / 1e12, 1)
+                out[name][key.replace("tflops", "us")] = round(ms2 * 1e3, 2)
     return out
+
+
+def in_tree_over_vendor(kernels, calib):
+    """Run time of each in-tree product (with its epilogue, launched as the operator launches
+    it) over the vendor library's plain product of the same shape, both timed in this run on
+    this box: a figure that separates a change of the kernels from the spread between boxes.
+    Below 1 the in-tree kernel is the faster one."""
+    out = {}
+    for shape, kern in (("qkv", "gemm_qkv_bias_split"), ("proj", "gemm_proj"),
+                        ("ffn1", "gemm_bias_gelu"), ("ffn2", "gemm_ffn2")):
+        out[shape] = round(kernels[kern]["us"] / calib[shape]["us"], 3)
+    sq = calib["square_8192"]
+    out["square_8192_as_stored"] = round(sq["in_tree_us_as_stored"] / sq["us"], 3)
+    out["square_8192_prepacked"] = round(sq["in_tree_us_prepacked"] / sq["us"], 3)
+    return out
+
+
+def vendor_compare(wl, dev, iters):
+    """Counter mode (`--vendor-compare`): nothing but the FFN1 shape of the workload and
+    8192^3, each through torch.matmul (the vendor library) and through the in-tree product
+    (plain epilogue, weight pre-packed and as stored; FFN1 also with its bias + GELU
+    epilogue), `iters` eager launches each, so that a rocprofv3 --pmc run of this command
+    lists the two libraries' kernels side by side.  Prints the launch order as JSON."""
+    import torch
+    from bytetransformer_amd import ops
+    cfg = wl.cfg
+    H, F, M = cfg.hidden, cfg.ffn_mult * cfg.hidden, wl.valid_tokens
+    order = []
+    for name, (m, n, k) in (("ffn1", (M, F, H)), ("square_8192", (8192, 8192, 8192))):
+        a = torch.empty(m, k, dtype=torch.float16, device=dev).normal_()
+        b = torch.empty(k, n, dtype=torch.float16, device=dev).normal_(std=0.02)
+        bias = torch.zeros(n, dtype=torch.float16, device=dev)
+        c = torch.empty(m, n, dtype=torch.float16, device=dev)
+        bt_ = ops.transpose_weight(b)
+        runs = [("vendor torch.matmul", lambda: torch.matmul(a, b, out=c)),
+                ("in-tree bt_gemm, weight [n,k]", lambda: ops.gemm(a, bt_, out=c, w_kn=False)),
+                ("in-tree bt_gemm, weight [k,n]", lambda: ops.gemm(a, b, out=c, w_kn=True))]
+        if name == "ffn1":
+            runs.append(("in-tree bt_gemm_bias_gelu, weight [n,k]",
+                         lambda: ops.gemm_bias_gelu(a, bt_, bias, out=c, w_kn=False)))
+        for label, fn in runs:
+            for _ in range(iters):
+                fn()
+            torch.cuda.synchronize()
+            order.append({"shape": name, "m": m, "n": n, "k": k, "what": label, "launches": iters})
+    print(json.dumps({"vendor_compare": order}))
 
 
 def cpp_api_layer_ms(wl, iters=50):
@@ -370,6 +420,9 @@ def main():
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     dev = torch.device("cuda:0")
     bt.load_th_op()
+    if args.vendor_compare:
+        vendor_compare(wl, dev, min(args.kernel_iters, 10))
+        return
     t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dev)
     layers = [[t(w[n]) for n in workload.WEIGHT_NAMES] for w in wl.layers]
     x, mask = t(wl.x), t(wl.mask)
@@ -411,6 +464,26 @@ def main():
             fn()
         torch.cuda.synchronize()
         return round((time.perf_counter() - t1) * 1e3 / args.steps, 4)
+
+    # A serving loop sees a new mask tensor with every batch: the same forward with a mask
+    # tensor the operator has not met before in each forward (fresh clones made outside the
+    # timed region), so that whatever the operator does once per mask tensor is inside the figure.
+    def fresh_mask_ms():
+        n_fwd = args.warmup + args.steps
+        masks = [mask.clone() for _ in range(n_fwd)]
+        torch.cuda.synchronize()
+        t1 = None
+        for i, mk in enumerate(masks):
+            if i == args.warmup:
+                torch.cuda.synchronize()
+                t1 = time.perf_counter()
+            h = x
+            for w in layers:
+                h = op(cfg.head_num, cfg.head_size, *w, h, mk, True, True)
+        torch.cuda.synchronize()
+        return round((time.perf_counter() - t1) * 1e3 / args.steps, 4)
+
+    fresh_ms = fresh_mask_ms()
 
     # the same forward through the other entry points (reported beside `value`, which
     # stays the reference's protocol: one operator call per layer)
@@ -458,6 +531,7 @@ def main():
                                   "runs of this command, not measured in this run)",
                 "launch_us": d["us"]}
     pub = PUBLISHED_A100_MS.get(args.workload)
+    calib = hipblaslt_calibration(wl, dev, args.kernel_iters)
     line = {
         "metric": "ms per %d-layer BERT fwd, bs%d, avg len 0.6*max (valid-token throughput alongside)"
                   % (cfg.layers, cfg.batch),
@@ -475,9 +549,11 @@ def main():
         "model_tflops": round(cfg.layers * (gemm_f + attn_f) / (ms * 1e-3) / 1e12, 2),
         "roofline": roofline,
         "parity": parity,
+        "fresh_mask_ms": fresh_ms,
         "other_entry_points": other,
         "cpp_api_layer_ms": cpp_layer_ms,
-        "hipblaslt_calibration": hipblaslt_calibration(wl, dev, args.kernel_iters),
+        "hipblaslt_calibration": calib,
+        "in_tree_over_vendor": in_tree_over_vendor(kernels, calib),
         "kernels": kernels,
     }
     if not args.no_cpu_baseline:

@@ -69,19 +69,24 @@ void BertTransformer<OpType>::bert_infer(BertTransformerInferParam infer_param) 
                            bt_attention_worklist_bytes(batch_size, seq_len, head_num_) == 0;
   // Padding-free fp16 layers that have to build their offsets: the QKV product can count the
   // mask rows itself and leave the offsets for the kernels after it, so that the layer goes
-  // without the launch ahead of it - and without the per-call weight copies that launch
-  // would make, which is why the choice follows the copy plan below.
+  // without the launch ahead of it.  By default only where that launch would have no
+  // per-call weight copy to make; with the option at 2 everywhere the entry takes the shape,
+  // and a few workgroups of the QKV launch which compute no tile then make the copies and
+  // the attention's work list (not the default: faster at batch 16 x 512, slower at
+  // 16 x 1024 and 32 x 384, where every workgroup of several rounds pays for counting the
+  // mask rows).
   int qkv_mask_rows_opt = -1;
   bt_get_option("qkv_mask_rows", &qkv_mask_rows_opt);
   const bool qkv_mask_rows_fits =
       OpType == OperationType::HALF && is_remove_padding_ && !have_offsets &&
       qkv_mask_rows_opt != 0 &&
       bt_gemm_qkv_mask_rows_supported(batch_size, seq_len, Traits_::dtype);
+  const bool side_jobs = qkv_mask_rows_fits && qkv_mask_rows_opt == 2;
   // The four products read the [k, n] weights as the caller stores them, exactly as the
   // reference hands them to cuBLAS (gemm.cu:27-39): nothing is kept between calls and
   // nothing can go stale.  Where the measured tile table says that a product of this size
-  // runs faster on a k-contiguous copy even after paying for the copy, the prologue launch
-  // makes that copy in the scratch, afresh in every call.  A caller that owns
+  // runs faster on a k-contiguous copy even after paying for the copy, the layer's first
+  // launch makes that copy in the scratch, afresh in every call.  A caller that owns
   // k-contiguous copies of immutable weights (prepacked_kernels) passes those instead.
   const bool have_prepack = OpType == OperationType::HALF && param_.prepacked_kernels[0] &&
                             param_.prepacked_kernels[1] && param_.prepacked_kernels[2] &&
@@ -100,7 +105,7 @@ void BertTransformer<OpType>::bert_infer(BertTransformerInferParam infer_param) 
       w_kn[i] = 0;
     }
   } else if (OpType == OperationType::HALF && !mask_direct &&
-             !(qkv_mask_rows_fits && qkv_mask_rows_opt == 1)) {   // (the copies are made by the prologue)
+             !(qkv_mask_rows_fits && qkv_mask_rows_opt == 1)) {   // (the copies are made by the first launch)
     const long long live = infer_param.valid_rows_hint > 0 ? infer_param.valid_rows_hint
                            : is_remove_padding_            ? (rows * 3LL + 4) / 5
                                                            : rows;
@@ -108,7 +113,9 @@ void BertTransformer<OpType>::bert_infer(BertTransformerInferParam infer_param) 
                              BT_EPILOGUE_PLAIN, BT_EPILOGUE_BIAS_GELU, BT_EPILOGUE_PLAIN};
     DataType_ *slot = (DataType_ *)(base + off);
     for (int i = 0; i < 4; ++i) {
-      if (epilogue[i] >= 0 && bt_gemm_prepack_pays(live, w_n[i], w_k[i], epilogue[i])) {
+      // (a QKV launch that makes the copies itself reads its own weight as stored)
+      if (epilogue[i] >= 0 && !(i == 0 && side_jobs) &&
+          bt_gemm_prepack_pays(live, w_n[i], w_k[i], epilogue[i])) {
         pack_src[pack_count] = w_use[i];
         pack_dst[pack_count] = slot;
         pack_k[pack_count] = w_k[i];
@@ -124,7 +131,7 @@ void BertTransformer<OpType>::bert_infer(BertTransformerInferParam infer_param) 
                       sizeof(DataType_),
                   256);
   float *splitk_buf = (float *)(base + off);
-  const bool qkv_mask_rows = qkv_mask_rows_fits && pack_count == 0;
+  const bool qkv_mask_rows = qkv_mask_rows_fits && (pack_count == 0 || side_jobs);
 
   // Padded rows, fp16 streaming attention: the mask tensor is applied unless one pass over
   // it finds the plain prefix mask of its lengths; the prologue leaves that verdict in the
@@ -134,10 +141,16 @@ void BertTransformer<OpType>::bert_infer(BertTransformerInferParam infer_param) 
       !(have_offsets && infer_param.mask_prefix >= 0))
     mask_slots = (int *)(base + inner_buf_size_);
 
-  // No attention work list here: building it lengthens this layer's prologue by more than the
-  // attention saves with it (the kernel finds its balanced order by a look-up of its own).
-  // The whole-encoder entry, which builds one list for all its layers, does use it.
+  // The attention's balanced work list: built by spare workgroups of the QKV launch where that
+  // launch carries jobs.  A prologue launch does not build it: there it lengthens the
+  // launch by more than the attention saves (the kernel then finds its balanced order by a
+  // look-up of its own).
   void *work_list = nullptr;
+  if (side_jobs && streaming_fp16) {
+    const unsigned long long need = bt_attention_worklist_bytes(batch_size, seq_len, head_num_);
+    if (need > 0 && need <= attention_layer_->work_list_capacity())
+      work_list = base + inner_buf_size_ + Attention<OpType>::work_list_offset();
+  }
 
   // One launch ahead of the layer: lengths and offsets from the mask (needed on both
   // paths: keys past len_b are excluded), the prefix-mask verdict, the weight copies.
@@ -150,8 +163,11 @@ void BertTransformer<OpType>::bert_infer(BertTransformerInferParam infer_param) 
   const void *warm[4];
   unsigned long long warm_bytes[4];
   int warm_count = 0;
-  if (OpType == OperationType::HALF && !have_prepack)
-    for (int i = 0; i < 4; ++i)
+  // (the QKV launch that carries the jobs is already reading its own weight, and touches the
+  // others only where it has workgroups for jobs anyway)
+  if (OpType == OperationType::HALF && !have_prepack &&
+      (!qkv_mask_rows || pack_count > 0 || work_list))
+    for (int i = qkv_mask_rows ? 1 : 0; i < 4; ++i)
       if (w_kn[i]) {
         warm[warm_count] = w_use[i];
         warm_bytes[warm_count++] = (unsigned long long)w_k[i] * w_n[i] * sizeof(DataType_);
@@ -159,7 +175,7 @@ void BertTransformer<OpType>::bert_infer(BertTransformerInferParam infer_param) 
   if (!mask_direct && !qkv_mask_rows && (!have_offsets || mask_slots || pack_count > 0))
     check_bt_error(bt_layer_prologue(atten_mask, Traits_::dtype, batch_size, seq_len,
                                      et_param.batch_idx, et_param.word_idx, seq_order,
-                                     mask_slots, work_list, head_num_, is_remove_padding_ ? 0 : 1,
+                                     mask_slots, nullptr, head_num_, is_remove_padding_ ? 0 : 1,
                                      pack_count, pack_src, pack_dst, pack_k, pack_n, warm_count,
                                      warm, warm_bytes, stream));
   if (have_offsets) {
@@ -235,7 +251,8 @@ void BertTransformer<OpType>::bert_infer(BertTransformerInferParam infer_param) 
     check_bt_error(bt_gemm_qkv_bias_split_mask_rows(
         from_tensor, atten_mask, Traits_::dtype, batch_size, seq_len, wt_qkv,
         param_.attention_param.attr_bias_QKV, qkv_buf, et_param.batch_idx, et_param.word_idx,
-        seq_order, rows_hint, head_num_, size_per_head_, w_kn[0], stream));
+        seq_order, rows_hint, head_num_, size_per_head_, w_kn[0], work_list, pack_count, pack_src,
+        pack_dst, pack_k, pack_n, warm_count, warm, warm_bytes, stream));
   else
     check_bt_error(bt_gemm_qkv_bias_split(from_tensor, gather, wt_qkv,
                                           param_.attention_param.attr_bias_QKV, qkv_buf,

@@ -228,6 +228,105 @@ __device__ __forceinline__ void transpose_tile_64(const half_t *__restrict__ w,
   }
 }
 
+// ---- jobs that ride along with a layer's first launch ----------------------------------
+// k-contiguous copies [N, K] of up to four [K, N] weight matrices, and ranges whose
+// 128-byte lines are touched once so that later launches find them in the memory-side cache.
+struct WeightJobs {
+  const half_t *w[4];        // [K, N] as the caller stores them
+  half_t *wt[4];             // [N, K] copies to make
+  int K[4], N[4];
+  int tiles_n[4];            // 64 x 64 tiles along n
+  int tile_end[4];           // tiles up to and including matrix i
+  int count;                 // 0 = none
+  // range r holds the 128-byte lines [warm_end[r - 1], warm_end[r]) of the concatenation
+  const char *warm[4];
+  unsigned warm_end[4];
+};
+// Fills `out` from the tail arguments of the C entries that take such jobs (checks them and
+// reports errors under the name `who`; returns a BT status).  With the `prefetch` option off
+// the ranges to warm are dropped.
+int make_weight_jobs(const char *who, WeightJobs *out, int weight_count, const void *const *w,
+                     void *const *wt, const int *k, const int *n, int warm_count,
+                     const void *const *warm, const unsigned long long *warm_bytes);
+
+// U tiles at a time per group of 256 threads (t = thread index in the group): tiles t0 .. t0 +
+// U - 1 of the concatenated tile list of the jobs (ids from pw.tile_end[pw.count - 1] on do not
+// exist).  All the loads of the U tiles are in flight together, so a group that has several
+// tiles to move pays one memory round trip for U of them.  `tiles` holds U consecutive LDS
+// tiles of this group.  The whole workgroup must call it together (two barriers inside).
+template <int U>
+__device__ __forceinline__ void transpose_tiles_64(const WeightJobs &pw, int t0,
+                                                   half_t (*tiles)[kTransposePitch], int t) {
+  const int r = t >> 3, c = (t & 7) * 8;
+  const int t_end = pw.tile_end[pw.count - 1];
+  uint4_t v[U][2];
+  const half_t *src[U];
+  half_t *dst[U];
+  int K[U], N[U], k0[U], n0[U];
+#pragma unroll
+  for (int u = 0; u < U; ++u) {
+    const int tile = t0 + u;
+    int j = 0, first = 0;
+#pragma unroll
+    for (int q = 1; q < 4; ++q)
+      if (q < pw.count && tile >= pw.tile_end[q - 1]) {
+        j = q;
+        first = pw.tile_end[q - 1];
+      }
+    const int tl = tile - first;
+    src[u] = pw.w[j], dst[u] = pw.wt[j], K[u] = tile < t_end ? pw.K[j] : 0, N[u] = pw.N[j];
+    k0[u] = (tl / pw.tiles_n[j]) * 64, n0[u] = (tl % pw.tiles_n[j]) * 64;
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const int k = k0[u] + r + 32 * i, n = n0[u] + c;
+      v[u][i] = uint4_t{0u, 0u, 0u, 0u};
+      if (k < K[u] && n < N[u]) v[u][i] = *(const uint4_t *)(src[u] + (size_t)k * N[u] + n);
+    }
+  }
+#pragma unroll
+  for (int u = 0; u < U; ++u)
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const half_t *h = (const half_t *)&v[u][i];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) tiles[u * 64 + r + 32 * i][c + e] = h[e];
+    }
+  __syncthreads();
+#pragma unroll
+  for (int u = 0; u < U; ++u) {
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const int n = n0[u] + r + 32 * i, k = k0[u] + c;
+      if (n < N[u] && k < K[u]) {
+        half8_t o;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) o[e] = tiles[u * 64 + c + e][r + 32 * i];
+        *(half8_t *)(dst[u] + (size_t)n * K[u] + k) = o;
+      }
+    }
+  }
+  __syncthreads();
+}
+
+// One dword per 128-byte line of the ranges, lines [first, last) in steps of `stride`.
+__device__ __forceinline__ void warm_lines(const WeightJobs &pw, unsigned first, unsigned last,
+                                           unsigned stride) {
+  for (unsigned l = first; l < last; l += stride) {
+    const char *base = pw.warm[0];
+    unsigned begin = 0;
+#pragma unroll
+    for (int r = 1; r < 4; ++r)
+      if (l >= pw.warm_end[r - 1]) {
+        base = pw.warm[r];
+        begin = pw.warm_end[r - 1];
+      }
+    unsigned sink;
+    const char *addr = base + (unsigned long long)(l - begin) * 128;
+    asm volatile("global_load_dword %0, %1, off" : "=v"(sink) : "v"(addr) : "memory");
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+}
+
 // ---- balanced work list of the streaming attention kernels -------------------------
 // Within an XCD the hardware deals consecutive workgroups to its 32 CUs round-robin
 // (slot s of the XCD lands on CU s % 32), and a launch of a few workgroups per CU is

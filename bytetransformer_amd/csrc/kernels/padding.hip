@@ -156,21 +156,6 @@ constexpr int kPackGroups = kPrologueThreads / 256;   // 64 x 64 tiles one block
 constexpr int kPackFirst = 64;     // blocks below build offsets (at most 64 of them)
 constexpr int kPackBlocks = 192;
 
-struct PrologueWeights {
-  const half_t *w[4];        // [K, N] as the caller stores them
-  half_t *wt[4];             // [N, K] copies to make
-  int K[4], N[4];
-  int tiles_n[4];            // 64 x 64 tiles along n
-  int tile_end[4];           // tiles up to and including matrix i
-  int count;                 // 0 = none
-  // ranges that the layer's products will read as they are (the weights that are not
-  // packed): range r holds the 128-byte lines [warm_end[r - 1], warm_end[r]) of their
-  // concatenation; the pack blocks touch one dword per line so that the lines sit in the
-  // memory-side cache when the products ask for them
-  const char *warm[4];
-  unsigned warm_end[4];
-};
-
 // The attention's balanced work list, built by blocks of their own beyond the others
 // (kListBlocks of them, each with its own copy of the lengths in LDS): one wave per entry.
 constexpr int kListBlocks = 48;
@@ -184,7 +169,7 @@ template <typename T>
 __global__ __launch_bounds__(kPrologueThreads) void layer_prologue_kernel(
     const T *__restrict__ mask, int *__restrict__ batch_idx, int *__restrict__ word_idx,
     int *__restrict__ seq_order, int *__restrict__ slots, int B, int S, int offset_blocks,
-    PrologueWeights pw, PrologueList pl) {
+    WeightJobs pw, PrologueList pl) {
   extern __shared__ __attribute__((aligned(16))) int smem[];
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -306,26 +291,13 @@ __global__ __launch_bounds__(kPrologueThreads) void layer_prologue_kernel(
   }
 
   // ---- warm-up of the weights that are read as stored ----
-  const unsigned warm_lines = pw.warm_end[3];
-  if (warm_lines && (int)blockIdx.x >= kPackFirst && (int)blockIdx.x < kPackFirst + kPackBlocks) {
+  const unsigned n_lines = pw.warm_end[3];
+  if (n_lines && (int)blockIdx.x >= kPackFirst && (int)blockIdx.x < kPackFirst + kPackBlocks) {
     const unsigned pb = blockIdx.x - kPackFirst;
-    const unsigned per = (warm_lines + kPackBlocks - 1) / kPackBlocks;
+    const unsigned per = (n_lines + kPackBlocks - 1) / kPackBlocks;
     const unsigned first = pb * per;
-    const unsigned last = first + per < warm_lines ? first + per : warm_lines;
-    for (unsigned l = first + tid; l < last; l += kPrologueThreads) {
-      const char *base = pw.warm[0];
-      unsigned begin = 0;
-#pragma unroll
-      for (int r = 1; r < 4; ++r)
-        if (l >= pw.warm_end[r - 1]) {
-          base = pw.warm[r];
-          begin = pw.warm_end[r - 1];
-        }
-      unsigned sink;
-      const char *addr = base + (unsigned long long)(l - begin) * 128;
-      asm volatile("global_load_dword %0, %1, off" : "=v"(sink) : "v"(addr) : "memory");
-    }
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    const unsigned last = first + per < n_lines ? first + per : n_lines;
+    warm_lines(pw, first + tid, last, kPrologueThreads);
   }
 }
 
@@ -344,6 +316,60 @@ __global__ __launch_bounds__(kRowsPerBlock *kWave) void compress_kernel(
   const size_t src = (size_t)word_idx[t] * chunks;
   const size_t dst = (size_t)t * chunks;
   for (int c = lane; c < chunks; c += kWave) to[dst + c] = from[src + c];
+}
+
+int make_weight_jobs(const char *who, WeightJobs *out, int weight_count, const void *const *w,
+                     void *const *wt, const int *k, const int *n, int warm_count,
+                     const void *const *warm, const unsigned long long *warm_bytes) {
+  WeightJobs &pw = *out;
+  memset(&pw, 0, sizeof(pw));
+  BT_REQUIRE(weight_count >= 0 && weight_count <= 4, BT_ERR_INVALID_ARGUMENT,
+             "%s: weight_count=%d outside [0, 4]", who, weight_count);
+  pw.count = weight_count;
+  if (weight_count > 0) {
+    BT_REQUIRE(w && wt && k && n, BT_ERR_INVALID_ARGUMENT,
+               "%s: weights to pre-pack need w, wt, k and n", who);
+    long long tiles = 0;
+    for (int i = 0; i < weight_count; ++i) {
+      BT_REQUIRE(w[i] && wt[i], BT_ERR_INVALID_ARGUMENT, "%s: null matrix pointer #%d", who, i);
+      BT_REQUIRE(aligned16({w[i], wt[i]}), BT_ERR_INVALID_ARGUMENT,
+                 "%s: matrix pointers must be 16-byte aligned", who);
+      BT_REQUIRE(k[i] > 0 && n[i] > 0 && k[i] % 8 == 0 && n[i] % 8 == 0, BT_ERR_UNSUPPORTED,
+                 "%s: k=%d n=%d must be positive multiples of 8", who, k[i], n[i]);
+      tiles += (long long)((k[i] + 63) / 64) * ((n[i] + 63) / 64);
+      BT_REQUIRE(tiles < (1ll << 21), BT_ERR_UNSUPPORTED,
+                 "%s: weight matrices beyond 2^21 tiles of 64 x 64", who);
+      pw.w[i] = (const half_t *)w[i];
+      pw.wt[i] = (half_t *)wt[i];
+      pw.K[i] = k[i];
+      pw.N[i] = n[i];
+      pw.tiles_n[i] = (n[i] + 63) / 64;
+      pw.tile_end[i] = (int)tiles;
+    }
+    for (int i = weight_count; i < 4; ++i) {
+      pw.tiles_n[i] = 1;
+      pw.tile_end[i] = (int)tiles;
+    }
+  }
+  BT_REQUIRE(warm_count >= 0 && warm_count <= 4 && (warm_count == 0 || (warm && warm_bytes)),
+             BT_ERR_INVALID_ARGUMENT, "%s: warm_count=%d outside [0, 4], or no ranges", who,
+             warm_count);
+  if (option_prefetch()) {
+    unsigned end = 0;
+    for (int r = 0; r < 4; ++r) {
+      if (r < warm_count && warm[r]) {
+        // one dword at the start of each 128-byte line; a last line of fewer than four bytes
+        // is left alone, so no byte outside the range is read
+        const unsigned long long lines = (warm_bytes[r] + 124) / 128;
+        BT_REQUIRE(lines < (1ull << 24), BT_ERR_UNSUPPORTED, "%s: a range to warm beyond 2 GiB",
+                   who);
+        pw.warm[r] = (const char *)warm[r];
+        end += (unsigned)lines;
+      }
+      pw.warm_end[r] = end;
+    }
+  }
+  return BT_OK;
 }
 
 }  // namespace bt
@@ -393,8 +419,8 @@ extern "C" int bt_set_option(const char *name, int value) {
                "bt_set_option: padded_mask_direct=%d outside [0, 2^20]", value);
     g_padded_mask_direct.store(value);
   } else if (!strcmp(name, "qkv_mask_rows")) {
-    BT_REQUIRE(value >= -1 && value <= 1, BT_ERR_INVALID_ARGUMENT,
-               "bt_set_option: qkv_mask_rows=%d must be -1, 0 or 1", value);
+    BT_REQUIRE(value >= -1 && value <= 2, BT_ERR_INVALID_ARGUMENT,
+               "bt_set_option: qkv_mask_rows=%d must be -1, 0, 1 or 2", value);
     g_qkv_mask_rows.store(value);
   } else if (!strcmp(name, "prefetch_min_grid")) {
     BT_REQUIRE(value >= 1 && value <= (1 << 20), BT_ERR_INVALID_ARGUMENT,
@@ -486,57 +512,11 @@ extern "C" int bt_layer_prologue(const void *atten_mask, int mask_dtype, int bat
              "bt_layer_prologue: unknown mask dtype %d", mask_dtype);
   BT_REQUIRE((long long)batch_size * seq_len < (1ll << 31), BT_ERR_UNSUPPORTED,
              "bt_layer_prologue: batch_size*seq_len overflows int32");
-  BT_REQUIRE(weight_count >= 0 && weight_count <= 4, BT_ERR_INVALID_ARGUMENT,
-             "bt_layer_prologue: weight_count=%d outside [0, 4]", weight_count);
-  PrologueWeights pw;
-  memset(&pw, 0, sizeof(pw));
-  pw.count = weight_count;
-  if (weight_count > 0) {
-    BT_REQUIRE(w && wt && k && n, BT_ERR_INVALID_ARGUMENT,
-               "bt_layer_prologue: weights to pre-pack need w, wt, k and n");
-    long long tiles = 0;
-    for (int i = 0; i < weight_count; ++i) {
-      BT_REQUIRE(w[i] && wt[i], BT_ERR_INVALID_ARGUMENT,
-                 "bt_layer_prologue: null matrix pointer #%d", i);
-      BT_REQUIRE(aligned16({w[i], wt[i]}), BT_ERR_INVALID_ARGUMENT,
-                 "bt_layer_prologue: matrix pointers must be 16-byte aligned");
-      BT_REQUIRE(k[i] > 0 && n[i] > 0 && k[i] % 8 == 0 && n[i] % 8 == 0, BT_ERR_UNSUPPORTED,
-                 "bt_layer_prologue: k=%d n=%d must be positive multiples of 8", k[i], n[i]);
-      tiles += (long long)((k[i] + 63) / 64) * ((n[i] + 63) / 64);
-      BT_REQUIRE(tiles < (1ll << 21), BT_ERR_UNSUPPORTED,
-                 "bt_layer_prologue: weight matrices beyond 2^21 tiles of 64 x 64");
-      pw.w[i] = (const half_t *)w[i];
-      pw.wt[i] = (half_t *)wt[i];
-      pw.K[i] = k[i];
-      pw.N[i] = n[i];
-      pw.tiles_n[i] = (n[i] + 63) / 64;
-      pw.tile_end[i] = (int)tiles;
-    }
-    for (int i = weight_count; i < 4; ++i) {
-      pw.tiles_n[i] = 1;
-      pw.tile_end[i] = (int)tiles;
-    }
-  }
-  BT_REQUIRE(warm_count >= 0 && warm_count <= 4 && (warm_count == 0 || (warm && warm_bytes)),
-             BT_ERR_INVALID_ARGUMENT, "bt_layer_prologue: warm_count=%d outside [0, 4], or no ranges",
-             warm_count);
-  bool warming = false;
-  if (option_prefetch()) {
-    unsigned end = 0;
-    for (int r = 0; r < 4; ++r) {
-      if (r < warm_count && warm[r]) {
-        // one dword at the start of each 128-byte line; a last line of fewer than four bytes
-        // is left alone, so no byte outside the range is read
-        const unsigned long long lines = (warm_bytes[r] + 124) / 128;
-        BT_REQUIRE(lines < (1ull << 24), BT_ERR_UNSUPPORTED,
-                   "bt_layer_prologue: a range to warm beyond 2 GiB");
-        pw.warm[r] = (const char *)warm[r];
-        end += (unsigned)lines;
-      }
-      pw.warm_end[r] = end;
-    }
-    warming = end > 0;
-  }
+  WeightJobs pw;
+  const int rc_jobs = make_weight_jobs("bt_layer_prologue", &pw, weight_count, w, wt, k, n,
+                                       warm_count, warm, warm_bytes);
+  if (rc_jobs != BT_OK) return rc_jobs;
+  const bool warming = pw.warm_end[3] > 0;
   // the attention's balanced work list, when a launch of this shape uses one
   PrologueList pl;
   memset(&pl, 0, sizeof(pl));

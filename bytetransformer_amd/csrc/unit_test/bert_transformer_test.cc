@@ -271,7 +271,7 @@ int main(int argc, char *argv[]) {
   if (argc < 5) {
     printf("./bert_transformer_test <batch_size> <seq_len> <head_num> <size_per_head> "
            "[--data DIR] [--iters N] [--tol MAX_ABS] [--no-rm] [--no-fused] [--fp32] "
-           "[--synthetic [--lens L0,L1,...]]\n");
+           "[--synthetic [--lens L0,L1,...]] [--option NAME=VALUE ...]\n");
     return 0;
   }
   Options o;
@@ -289,6 +289,16 @@ int main(int argc, char *argv[]) {
     else if (!strcmp(argv[i], "--no-fused")) o.use_fused_attention = false;
     else if (!strcmp(argv[i], "--fp32")) fp32 = true;
     else if (!strcmp(argv[i], "--synthetic")) o.synthetic = true;
+    else if (!strcmp(argv[i], "--option") && i + 1 < argc) {
+      // a tuning knob of the kernel library (bt_set_option), e.g. qkv_mask_rows=0
+      const std::string kv = argv[++i];
+      const size_t eq = kv.find('=');
+      if (eq == std::string::npos ||
+          bt_set_option(kv.substr(0, eq).c_str(), atoi(kv.c_str() + eq + 1)) != BT_OK) {
+        fprintf(stderr, "bad --option %s: %s\n", kv.c_str(), bt_last_error_string());
+        return 2;
+      }
+    }
     else if (!strcmp(argv[i], "--lens") && i + 1 < argc) {
       for (const char *p = argv[++i]; *p;) {
         o.lens.push_back(atoi(p));

@@ -77,6 +77,27 @@ def mask_is_prefix(mask, batch_idx):
     return bool(verdict.value)
 
 
+def _weight_jobs(weights, packed, warm):
+    """ctypes arguments (count, w, wt, k, n, warm_count, warm, warm_bytes) of the entries that
+    make k-contiguous weight copies and touch ranges on behalf of later launches."""
+    n = len(weights) if weights else 0
+    if n:
+        for w, t in zip(weights, packed):
+            if tuple(t.shape) != tuple(w.shape[::-1]) or t.dtype != w.dtype:
+                raise ValueError("packed copies must be the [n, k] counterparts of the weights")
+        src = (ctypes.c_void_p * n)(*[_ptr(w).value for w in weights])
+        dst = (ctypes.c_void_p * n)(*[_ptr(w).value for w in packed])
+        ks = (ctypes.c_int * n)(*[w.shape[0] for w in weights])
+        ns = (ctypes.c_int * n)(*[w.shape[1] for w in weights])
+    else:
+        src = dst = ks = ns = None
+    warm = list(warm)
+    nw = len(warm)
+    wp = (ctypes.c_void_p * max(nw, 1))(*[_ptr(t).value for t in warm])
+    wb = (ctypes.c_ulonglong * max(nw, 1))(*[t.numel() * t.element_size() for t in warm])
+    return n, src, dst, ks, ns, nw, wp, wb
+
+
 def layer_prologue(mask, want_slots=False, weights=None, packed=None, out=None,
                    work_list=None, head_num=0, padded_rows=False, warm=()):
     """bt_layer_prologue: offsets of `mask`, optionally the prefix-mask verdict slots and the
@@ -94,25 +115,10 @@ def layer_prologue(mask, want_slots=False, weights=None, packed=None, out=None,
         word_idx = torch.empty(B * S, dtype=torch.int32, device=dev)
         seq_order = torch.empty(B, dtype=torch.int32, device=dev)
         slots = torch.full((256,), -1, dtype=torch.int32, device=dev) if want_slots else None
-    n = len(weights) if weights else 0
-    if n:
-        for w, t in zip(weights, packed):
-            if tuple(t.shape) != tuple(w.shape[::-1]) or t.dtype != w.dtype:
-                raise ValueError("packed copies must be the [n, k] counterparts of the weights")
-        src = (ctypes.c_void_p * n)(*[_ptr(w).value for w in weights])
-        dst = (ctypes.c_void_p * n)(*[_ptr(w).value for w in packed])
-        ks = (ctypes.c_int * n)(*[w.shape[0] for w in weights])
-        ns = (ctypes.c_int * n)(*[w.shape[1] for w in weights])
-    else:
-        src = dst = ks = ns = None
-    warm = list(warm)
-    nw = len(warm)
-    wp = (ctypes.c_void_p * max(nw, 1))(*[_ptr(t).value for t in warm])
-    wb = (ctypes.c_ulonglong * max(nw, 1))(*[t.numel() * t.element_size() for t in warm])
+    jobs = _weight_jobs(weights, packed, warm)
     _check(kernel_lib().bt_layer_prologue(
         _ptr(mask), _dtype_code(mask), B, S, _ptr(batch_idx), _ptr(word_idx), _ptr(seq_order),
-        _ptr(slots), _ptr(work_list), int(head_num), int(padded_rows), n, src, dst, ks, ns,
-        nw, wp, wb, _stream()))
+        _ptr(slots), _ptr(work_list), int(head_num), int(padded_rows), *jobs, _stream()))
     return batch_idx, word_idx, seq_order, slots
 
 
@@ -216,9 +222,13 @@ def gemm_qkv_mask_rows_supported(batch_size, seq_len, mask_dtype=torch.float16):
 
 
 def gemm_qkv_bias_split_mask_rows(x, mask, wt_qkv, bias_qkv, head_num, size_per_head=64, out=None,
-                                  offsets_out=None, rows_hint=0, w_kn=False):
+                                  offsets_out=None, rows_hint=0, w_kn=False, work_list=None,
+                                  weights=None, packed=None, warm=()):
     """QKV projection of the padded x [B, S, H] whose live rows come from the mask inside the
-    launch; returns (qkv_heads, batch_idx, word_idx, seq_order)."""
+    launch; returns (qkv_heads, batch_idx, word_idx, seq_order).  Jobs that ride along with
+    the launch: work_list (int32[entries, 4]) is filled with the attention's balanced order as
+    attention_worklist would, `packed` with the [n, k] copies of the [k, n] `weights`, and the
+    tensors of `warm` are touched line by line (a cache hint)."""
     B, S = mask.shape[0], mask.shape[1]
     H = head_num * size_per_head
     rows = B * S
@@ -244,7 +254,7 @@ def gemm_qkv_bias_split_mask_rows(x, mask, wt_qkv, bias_qkv, head_num, size_per_
     _check(kernel_lib().bt_gemm_qkv_bias_split_mask_rows(
         _ptr(x), _ptr(mask), _dtype_code(mask), B, S, _ptr(wt_qkv), _ptr(bias_qkv), _ptr(out),
         _ptr(batch_idx), _ptr(word_idx), _ptr(seq_order), int(rows_hint), head_num, size_per_head,
-        int(w_kn), _stream()))
+        int(w_kn), _ptr(work_list), *_weight_jobs(weights, packed, warm), _stream()))
     return out, batch_idx, word_idx, seq_order
 
 

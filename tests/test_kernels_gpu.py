@@ -555,6 +555,66 @@ def test_gemm_qkv_rows_from_the_mask(device, tile, case):
     assert torch.equal(got2[:, :, :M], got[:, :, :M])
 
 
+@pytest.mark.parametrize("tile", [-1, 0, 3, 4, 7])
+@pytest.mark.parametrize("case", ["cfg2-like", "many-short", "f32-mask"])
+def test_gemm_qkv_rows_from_the_mask_side_jobs(device, case, tile):
+    """The jobs that ride along with the launch (the attention's work list, k-contiguous
+    weight copies, cache warm-up) are done by workgroups of their own: the list equals the
+    stand-alone builder's, the copies equal the transposed weights, and the projections and
+    offsets are what the launch gives without any job."""
+    rs = np.random.RandomState(len(case) + 10 * (tile + 1))
+    mdt = np.float16
+    if case == "cfg2-like":
+        B, S, heads = 16, 512, 2
+        lens = rs.randint(100, 513, B)
+    elif case == "many-short":
+        B, S, heads = 40, 96, 3
+        lens = rs.randint(0, 97, B)
+    else:
+        B, S, heads, mdt = 9, 160, 1, np.float32
+        lens = rs.randint(1, 161, B)
+    _say("gemm_qkv mask rows side jobs", case, tile, B, S, heads, int(lens.sum()))
+    H = heads * 64
+    x = rs.standard_normal((B, S, H)).astype(np.float16)
+    mask = workload.make_mask(lens, S, mdt)
+    w = (rs.standard_normal((H, 3 * H)) * 0.05).astype(np.float16)
+    bias = (rs.standard_normal(3 * H) * 0.5).astype(np.float16)
+    md, xd, wt, bd = _dev(mask, device), _dev(x, device), _prep(_dev(w, device)), _dev(bias, device)
+    M = int(lens.sum())
+    # weights to copy: shapes with partial 64 x 64 tiles too
+    ws = [_dev((rs.standard_normal(shape) * 0.1).astype(np.float16), device)
+          for shape in ((H, 4 * H), (4 * H, H), (72, 200))]
+    packed = [torch.full((v.shape[1], v.shape[0]), 7.0, dtype=torch.float16, device=device) for v in ws]
+    warm = [torch.zeros(1000, dtype=torch.float16, device=device), ws[0]]
+    ops.set_option("gemm_tile", tile)
+    ops.set_option("attention_xcd_map", 3)          # the balanced order at any size
+    try:
+        plain, p_bi, p_wi, p_so = ops.gemm_qkv_bias_split_mask_rows(xd, md, wt, bd, heads, rows_hint=M,
+                                                                    w_kn=_KN[0])
+        want_list = ops.attention_worklist(p_bi, B, S, heads, False, seq_order=p_so)
+        assert want_list is not None
+        got_list = torch.full_like(want_list, -7)
+        got, g_bi, g_wi, g_so = ops.gemm_qkv_bias_split_mask_rows(
+            xd, md, wt, bd, heads, rows_hint=M, w_kn=_KN[0], work_list=got_list, weights=ws,
+            packed=packed, warm=warm)
+        # the jobs one at a time
+        only_list = torch.full_like(want_list, -7)
+        ops.gemm_qkv_bias_split_mask_rows(xd, md, wt, bd, heads, w_kn=_KN[0], work_list=only_list)
+        only_packed = [torch.zeros_like(v) for v in packed[:1]]
+        ops.gemm_qkv_bias_split_mask_rows(xd, md, wt, bd, heads, w_kn=_KN[0], weights=ws[:1],
+                                          packed=only_packed, warm=warm[:1])
+    finally:
+        ops.set_option("gemm_tile", -1)
+        ops.set_option("attention_xcd_map", 2)
+    assert torch.equal(got_list, want_list) and torch.equal(only_list, want_list)
+    for v, t in zip(ws, packed):
+        assert torch.equal(t, v.t().contiguous())
+    assert torch.equal(only_packed[0], ws[0].t().contiguous())
+    assert torch.equal(g_bi, p_bi) and torch.equal(g_wi, p_wi) and torch.equal(g_so, p_so)
+    assert torch.equal(got[:, :, :M], plain[:, :, :M])
+    assert torch.all(got[:, :, M:] == 0)
+
+
 @pytest.mark.parametrize("seed", range(12))
 def test_gemm_qkv_rows_from_the_mask_random_shapes(device, seed):
     """Seeded random batch sizes, sequence lengths (odd ones too: the scalar mask-row path),

@@ -792,9 +792,11 @@ def test_layer_prepack_choice_never_changes_the_result(device):
 
 def test_qkv_rows_from_the_mask_never_change_the_result(device):
     """A padding-free layer may start with the QKV product that counts the mask rows itself
-    instead of the prologue launch: never, wherever the entry takes the shape, and the
-    automatic choice give the same bits - ragged lengths with an empty sequence, the
-    headline shape, and a batch beyond the entry's 64 sequences (which falls back by
+    instead of the prologue launch: never, wherever the entry takes the shape (without the
+    per-call weight copies, or with workgroups of that launch making them and the
+    attention's work list), and the automatic choice give the same bits - ragged lengths
+    with an empty sequence, the headline shape (12 heads: a copy pays and the attention takes
+    the balanced list), and a batch beyond the entry's 64 sequences (which falls back by
     itself)."""
     _say("qkv_mask_rows")
     from bytetransformer_amd import ops
@@ -803,6 +805,7 @@ def test_qkv_rows_from_the_mask_never_change_the_result(device):
     assert ops.get_option("qkv_mask_rows") == -1
     cases = (workload.EncoderConfig("mr", 6, 200, 12, layers=1, lens=(200, 0, 133, 50, 64, 7), seed=18),
              workload.EncoderConfig("mr2", 16, 512, 4, layers=1, seed=19),
+             workload.EncoderConfig("mr4", 16, 512, 12, layers=1, seed=21),
              workload.EncoderConfig("mr3", 70, 16, 2, layers=1, seed=20))
     for cfg in cases:
         wl = workload.make_workload(cfg, bias_std=0.05, random_affine=True)
@@ -810,12 +813,13 @@ def test_qkv_rows_from_the_mask_never_change_the_result(device):
         x, m = _dev(wl.x, device), _dev(wl.mask, device)
         got = {}
         try:
-            for choice in (0, 1, -1):
+            for choice in (0, 1, 2, -1):
                 ops.set_option("qkv_mask_rows", choice)
                 got[choice] = op(cfg.head_num, 64, *w, x, m, True, True)
         finally:
             ops.set_option("qkv_mask_rows", -1)
         assert torch.equal(got[0], got[1]) and torch.equal(got[0], got[-1])
+        assert torch.equal(got[0], got[2])
         _check(got[1].cpu().numpy(), _oracle(wl), wl.lens, tag="qkv_mask_rows " + cfg.name)
 
 
