@@ -10,8 +10,13 @@ namespace bytetransformer {
 
 template <OperationType OpType>
 void Attention<OpType>::infer(AttentionInferParam infer_param) {
-  if (infer_param.et_param.batch_idx == nullptr)
+  if (infer_param.et_param.batch_idx == nullptr && !infer_param.no_offsets)
     throw std::runtime_error("[BT][ERROR] Attention: et_param.batch_idx must be set");
+  if (infer_param.no_offsets &&
+      (OpType != OperationType::HALF || is_remove_padding_ || size_per_head_ != 64 ||
+       infer_param.mask_prefix != 0 || uses_short_kernel(infer_param.seq_len)))
+    throw std::runtime_error("[BT][ERROR] Attention: no_offsets is for the streaming fp16 kernel "
+                             "on padded rows with the mask tensor applied (mask_prefix == 0)");
   if (infer_param.batch_size > max_batch_size_ || infer_param.seq_len > max_seq_len_)
     throw std::runtime_error("[BT][ERROR] Attention: batch_size/seq_len exceed the constructed maximum");
 
@@ -70,7 +75,8 @@ void Attention<OpType>::infer(AttentionInferParam infer_param) {
       slots = verdict;
     }
     check_bt_error(bt_attention_grouped(
-        infer_param.qkv, infer_param.attention_output, infer_param.et_param.batch_idx,
+        infer_param.qkv, infer_param.attention_output,
+        infer_param.no_offsets ? nullptr : infer_param.et_param.batch_idx,
         infer_param.seq_order, mask, infer_param.attention_bias, infer_param.batch_size,
         infer_param.seq_len, rows_cap, head_num_, size_per_head_, scale, padded_rows,
         infer_param.prefetch, infer_param.prefetch_bytes, infer_param.prefetch_count, slots,

@@ -269,6 +269,7 @@ void BertTransformer<OpType>::bert_infer(BertTransformerInferParam infer_param) 
   attention_infer_param.mask_prefix = have_offsets ? infer_param.mask_prefix : (mask_direct ? 0 : -1);
   attention_infer_param.mask_prefix_slots = mask_slots;
   attention_infer_param.work_list = work_list;
+  attention_infer_param.no_offsets = mask_direct;   // (nothing has written them)
   // the three weight matrices the rest of the layer reads (as stored, or the copies of
   // this call): the attention kernel pulls them into the memory-side cache while it runs
   {

@@ -294,8 +294,13 @@ __global__ __launch_bounds__(kAttThreads * KS, KS == 1 ? 2 : 4) void attention_g
       return;
     }
     b = p.seq_order ? p.seq_order[item.rank] : item.rank, head = item.head;
-    seq_start = p.batch_idx[b];
-    seq_len = p.batch_idx[b + 1] - seq_start;
+    if (p.batch_idx) {
+      seq_start = p.batch_idx[b];
+      seq_len = p.batch_idx[b + 1] - seq_start;
+    } else {   // no offsets: padded rows under a mask tensor, which says everything
+      seq_start = b * p.S;
+      seq_len = p.S;
+    }
     qb_index = item.qb;
   }
   // A mask tensor that the device-side check found to be the plain prefix mask adds 0 to
@@ -931,12 +936,16 @@ extern "C" int bt_attention_grouped(const void *qkv_heads, void *attention_outpu
                                     const unsigned long long *prefetch_bytes, int prefetch_count,
                                     const int *mask_prefix_slots, const void *work_list,
                                     void *stream) {
-  int rc = check_att_args("bt_attention_grouped", qkv_heads, attention_output, batch_idx,
-                          atten_mask, padded_rows, batch_size, seq_len, rows_cap, head_num,
-                          size_per_head);
+  // without offsets: only where nothing would read them (padded rows, the mask tensor
+  // applied element by element, no verdict that could drop it, no balanced order)
+  const bool no_offsets = !batch_idx && padded_rows && atten_mask && !mask_prefix_slots;
+  int rc = check_att_args("bt_attention_grouped", qkv_heads, attention_output,
+                          no_offsets ? (const int *)qkv_heads : batch_idx, atten_mask,
+                          padded_rows, batch_size, seq_len, rows_cap, head_num, size_per_head);
   if (rc) return rc;
   BT_REQUIRE(aligned16({work_list}), BT_ERR_INVALID_ARGUMENT,
              "bt_attention_grouped: work_list must be 16-byte aligned");
+  if (no_offsets) seq_order = nullptr;
   AttArgs a{(const half_t *)qkv_heads, (half_t *)attention_output, batch_idx, seq_order,
             (const half_t *)atten_mask, (const half_t *)attention_bias,
             {}, {}, batch_size, seq_len,
@@ -945,7 +954,11 @@ extern "C" int bt_attention_grouped(const void *qkv_heads, void *attention_outpu
   a.work_list = (const int4 *)work_list;   // read only when the launch uses the balanced order
   hipStream_t s = as_stream(stream);
   const bool add = a.mask || a.bias;
-  const GroupedPlan plan = plan_grouped(a, batch_size, seq_len, head_num);
+  GroupedPlan plan = plan_grouped(a, batch_size, seq_len, head_num);
+  if (no_offsets && a.xcd_map == 2) {   // the balanced order ranks the sequences by length
+    a.xcd_map = 1;
+    plan.grid = ((unsigned)batch_size * head_num + 7) / 8 * 8 * a.nqb;
+  }
   const unsigned grid = plan.grid;
   rc = set_prefetch(a, grid, prefetch, prefetch_bytes, prefetch_count);
   if (rc) return rc;

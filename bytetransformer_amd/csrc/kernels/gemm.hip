@@ -687,11 +687,16 @@ __device__ __forceinline__ void gemm_tiles_flat(const GemmArgs &p) {
   // first loading wave together with the tile's first k-step: a global load in a computing
   // wave after its stores would wait for every one of them to complete - the very wait this
   // form of the kernel exists to avoid.  (Only the first tile's bias is loaded directly.)
-  half_t *s_bias = smem + STAGES * STAGE_HALFS;          // [BN]
+  // It is requested as soon as the cursor moves to the tile, one k-step ahead of the tile's
+  // first loads (so that the wait for those loads' predecessors covers it), and the cursor
+  // runs STAGES - 1 k-steps ahead of the products: with k = 64 (one k-step per tile) up to
+  // STAGES biases are waiting to be read, hence STAGES buffers, taken in turn.
+  half_t *s_bias = smem + STAGES * STAGE_HALFS;          // [STAGES][BN]
   const rsrc_t rs_bias = make_rsrc(kHasBias ? p.bias : p.wt, kHasBias ? (size_t)p.N * sizeof(half_t) : 0);
   int voff[NI];
   int idx_next[NIA];   // gathered A rows of the tile after the one being loaded
   int ld_L = L0, ld_kt = 0, ld_left = loader ? total : 0;
+  int ld_slot = 0;     // bias buffer of the tile being set up: its position in the sequence mod STAGES
   auto fetch_indices = [&](int Lt) {
     const int m0 = (Lt / p.tiles_n) * BM;
     MaskRowSpan span{};
@@ -711,7 +716,8 @@ __device__ __forceinline__ void gemm_tiles_flat(const GemmArgs &p) {
 #pragma unroll
       for (int i = 0; i < BN / 128; ++i)
         __builtin_amdgcn_raw_ptr_buffer_load_lds(
-            rs_bias, (__attribute__((address_space(3))) void *)(s_bias + i * 128), 4,
+            rs_bias,
+            (__attribute__((address_space(3))) void *)(s_bias + ld_slot * BN + i * 128), 4,
             (lane + i * 64) * 4, n0 * (int)sizeof(half_t), 0, 0);
     }
     rs_a = gather ? make_rsrc(p.a, (size_t)p.rows_cap * p.K * sizeof(half_t))
@@ -756,6 +762,7 @@ __device__ __forceinline__ void gemm_tiles_flat(const GemmArgs &p) {
     if (++ld_kt == nk) {
       ld_kt = 0;
       ld_L += wgx;
+      if (++ld_slot == STAGES) ld_slot = 0;
       if (ld_left) load_setup(ld_L, ld_left > nk, true);
     }
   };
@@ -809,7 +816,7 @@ __device__ __forceinline__ void gemm_tiles_flat(const GemmArgs &p) {
       for (int j = 0; j < TM; ++j) acc[i][j] = init;
     }
   };
-  int cL = L0;
+  int cL = L0, c_slot = 0;
   {
     const int n0 = (cL % p.tiles_n) * BN;
     init_acc(kHasBias ? p.bias + n0 : nullptr, p.N - 4 - n0);   // the first tile: straight from memory
@@ -905,7 +912,8 @@ __device__ __forceinline__ void gemm_tiles_flat(const GemmArgs &p) {
         }
       }
       cL += wgx;
-      if (g + 1 < total) init_acc(s_bias, BN - 4);   // from LDS, where the loading side has put it
+      if (++c_slot == STAGES) c_slot = 0;
+      if (g + 1 < total) init_acc(s_bias + c_slot * BN, BN - 4);   // from LDS, where the loading side has put it
     }
     if (++stage == STAGES) stage = 0;
   }
@@ -981,7 +989,7 @@ static int cu_count();
 // looping over its tiles on the device.
 template <int BM, int BN, int STAGES, int WM, int WN, int NP, int SCHED, int EPI, bool WKN>
 static int launch_gemm_flat_as(GemmArgs p, hipStream_t s) {
-  constexpr size_t smem = (size_t)STAGES * (BM + BN) * kBK * sizeof(half_t) + BN * sizeof(half_t);
+  constexpr size_t smem = (size_t)STAGES * (BM + BN) * kBK * sizeof(half_t) + STAGES * BN * sizeof(half_t);
   static_assert(smem <= 160 * 1024, "LDS budget");
   static std::atomic<bool> configured[kMaxDevices];
   const int rc = allow_dynamic_lds(gemm_flat_kernel<BM, BN, STAGES, WM, WN, NP, SCHED, EPI, WKN>,

@@ -304,6 +304,10 @@ int bt_gemm_qkv_bias_split_mask_rows(const void *from_tensor, const void *atten_
  *                     stream.  When all are 1 the kernel ignores the tensor and stops at
  *                     the lengths, which gives the same result; decided on the device,
  *                     so the call stays asynchronous.
+ *   batch_idx == NULL (bt_attention_grouped only): allowed on padded rows with an
+ *                     atten_mask and no mask_prefix_slots - every one of the seq_len keys
+ *                     takes part under the mask tensor, so no length is read (seq_order and
+ *                     work_list are then ignored).
  *
  * bt_attention_short keeps the whole logits row of a query tile in registers
  * (exact two-pass softmax, seq_len <= 512).  Replaces wmma_attention[_rm]_kernel

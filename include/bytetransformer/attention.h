@@ -56,6 +56,11 @@ struct AttentionInferParam {
   // (bt_attention_worklist for this shape and these offsets), or null: the kernel then
   // looks its work up itself.
   const void *work_list = nullptr;
+  // Extension: et_param's offsets have not been built (a short layer on padded rows that
+  // goes without the launch that builds them): the streaming fp16 kernel then applies the
+  // mask tensor to all seq_len keys and reads no offsets.  Needs padded rows and
+  // mask_prefix == 0.
+  bool no_offsets = false;
 };
 
 template <OperationType OpType>
