@@ -42,6 +42,7 @@ KERNEL_ABI = {
                                   POINTER(c_int), c_int, POINTER(c_void_p), POINTER(c_ulonglong),
                                   _P]),
     "bt_gemm_prepack_pays": (c_int, [c_longlong, c_int, c_int, c_int]),
+    "bt_gemm_prepack_gain_us": (c_float, [c_longlong, c_int, c_int, c_int]),
     "bt_compress": (c_int, [_P, _P, _IP, _IP, c_int, c_int, c_int, _P]),
     "bt_transpose_weight": (c_int, [_P, _P, c_int, c_int, _P]),
     "bt_transpose_weights": (c_int, [c_int, POINTER(c_void_p), POINTER(c_void_p), POINTER(c_int),

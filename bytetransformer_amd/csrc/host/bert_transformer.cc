@@ -112,10 +112,22 @@ void BertTransformer<OpType>::bert_infer(BertTransformerInferParam infer_param) 
     const int epilogue[4] = {size_per_head_ == 64 ? BT_EPILOGUE_QKV_SPLIT : -1,
                              BT_EPILOGUE_PLAIN, BT_EPILOGUE_BIAS_GELU, BT_EPILOGUE_PLAIN};
     DataType_ *slot = (DataType_ *)(base + off);
+    // A layer whose QKV product can count the mask rows itself goes without a launch ahead
+    // of it as long as it makes no copy - one round of tiles pays about 3 us for that launch
+    // beyond the copy itself (measured per forward up to 10 k padded rows: never copying
+    // wins 1.5-1.8 % there, with several rounds of tiles it loses as much) - so there the
+    // copies have to return that much more.
+    const bool launch_at_stake = qkv_mask_rows_fits && !side_jobs && rows <= 10240;
+    float gain[4] = {0.f, 0.f, 0.f, 0.f}, total = 0.f;
     for (int i = 0; i < 4; ++i) {
       // (a QKV launch that makes the copies itself reads its own weight as stored)
-      if (epilogue[i] >= 0 && !(i == 0 && side_jobs) &&
-          bt_gemm_prepack_pays(live, w_n[i], w_k[i], epilogue[i])) {
+      if (epilogue[i] < 0 || (i == 0 && side_jobs)) continue;
+      gain[i] = bt_gemm_prepack_gain_us(live, w_n[i], w_k[i], epilogue[i]);
+      if (gain[i] > 1.0f) total += gain[i];
+    }
+    const bool copy_any = !launch_at_stake || total > 1e8f || total >= 4.0f;
+    for (int i = 0; i < 4; ++i) {
+      if (copy_any && gain[i] > 1.0f) {
         pack_src[pack_count] = w_use[i];
         pack_dst[pack_count] = slot;
         pack_k[pack_count] = w_k[i];

@@ -244,12 +244,12 @@ __device__ __forceinline__ rsrc_t make_rsrc(const void *base, size_t bytes) {
 
 // One stage's loads of one wave: instruction i lands 8 tile rows (1 KB) at
 // lds + i * lds_step; the first NIA instructions read A, the rest W.
-template <int NI, int NIA>
+template <int NI, int NIA, int COUNT = NI>
 __device__ __forceinline__ void issue_stage_loads(rsrc_t rs_a, rsrc_t rs_w, const int (&voff)[NI],
                                                   half_t *lds, int lds_step, int k_bytes,
                                                   int k_bytes_w) {
 #pragma unroll
-  for (int i = 0; i < NI; ++i)
+  for (int i = 0; i < COUNT; ++i)
     __builtin_amdgcn_raw_ptr_buffer_load_lds(i < NIA ? rs_a : rs_w,
                                              (__attribute__((address_space(3))) void *)(lds + i * lds_step),
                                              16, voff[i], i < NIA ? k_bytes : k_bytes_w, 0, 0);
@@ -344,6 +344,80 @@ __device__ __forceinline__ void gemm_side_jobs(const GemmArgs &p, int sb, int nt
   }
 }
 
+// ---- the epilogue's wave-private staging tile -------------------------------------------
+// 32 rows of WTN halfs, written 8 bytes per lane straight from the accumulator layout (lane l
+// owns row l & 31, the 8-byte half l >> 5 of a 16-byte chunk) and read back 16 bytes per lane,
+// row-contiguous, for the global stores.  With 128-byte rows (WTN = 64) the tile is
+// swizzled instead of padded: chunk ^= (row >> 1) & 7 and half ^= row >> 4 put the 32 lanes
+// of one write pass on 32 distinct bank pairs (a padded pitch leaves rows r and r + 16 on the
+// same banks: every write two passes); a reader undoes the half swap in registers.
+template <int WTN>
+struct Staging {
+  static constexpr bool kSwizzled = WTN == 64;
+  static constexpr int kPitch = kSwizzled ? WTN : WTN + 8;   // halfs
+  // where lane (row, half hf of the chunk) writes the 4 halfs of 16-byte chunk `chunk`
+  __device__ static __forceinline__ int write_at(int row, int hf, int chunk) {
+    if (kSwizzled) return row * kPitch + ((chunk ^ ((row >> 1) & 7)) << 3) + (((hf ^ (row >> 4)) & 1) << 2);
+    return row * kPitch + (chunk << 3) + (hf << 2);
+  }
+  // the 8 halfs of chunk `chunk` of row `row`, in order
+  __device__ static __forceinline__ uint4_t read(const half_t *st, int row, int chunk) {
+    if (kSwizzled) {
+      const uint4_t v = *(const uint4_t *)(st + row * kPitch + ((chunk ^ ((row >> 1) & 7)) << 3));
+      return (row >> 4) & 1 ? uint4_t{v[2], v[3], v[0], v[1]} : v;
+    }
+    return *(const uint4_t *)(st + row * kPitch + (chunk << 3));
+  }
+};
+
+// ---- a [K, N] weight tile of 256 columns through registers ----------------------------
+// The LDS transpose read runs at half the rate of the 16-byte read, and the 256 x 256 tile
+// (eight waves that load and compute, LDS reads ~ 3/4 of its MFMA time) is the one shape
+// that cannot hide that.  There the 64 x 256 tile of a row-major [K, N] weight is fetched
+// into registers instead - each of the 512 lanes takes a block of 4 k-rows x 8 columns, four
+// 16-byte loads - transposed in the lane (16 byte permutes) and written k-contiguous with
+// eight 8-byte LDS writes into the very image the pre-packed [N, K] layout lands in, so the
+// k loop reads both layouts the same way.  Lane -> block: four consecutive lanes take four
+// consecutive column blocks (64 contiguous bytes per k-row), the next lanes the next k-rows.
+// Which lanes write odd rows first and which even ones, together with the image's swizzle,
+// puts the 32 lanes of one write pass on 32 distinct bank pairs.
+struct RegW {
+  uint4_t r[4];        // k-rows k_base .. k_base + 3, columns n_base .. n_base + 7
+  int voff[4];         // byte offsets of the four loads from the tile's first element
+  int woff[8];         // LDS offsets (halfs, from the W image of a stage) of the eight writes
+  unsigned sel[2];     // permute selectors of even / odd write instructions
+};
+__device__ __forceinline__ void regw_setup(RegW &w, int wave, int lane, int N, int cols, int BM) {
+  const int kq = lane >> 2, ngl = lane & 3, ng = wave * 4 + ngl;
+  const int k_base = 4 * kq, n_base = 8 * ng, bit = ngl >> 1;
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+    w.voff[i] = n_base < cols ? ((k_base + i) * N + n_base) * (int)sizeof(half_t) : 0x7ffffff0;
+  const int c = kq >> 1, h = kq & 1;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const int n = n_base + (i ^ bit);
+    w.woff[i] = n * kBK + ((c ^ swz(n + BM)) << 3) + h * 4;
+  }
+  // write i moves column n_base + (i ^ bit): its halfs are the low or the high halves of
+  // dword (i >> 1) of the four loads
+  w.sel[0] = bit ? 0x07060302u : 0x05040100u;
+  w.sel[1] = bit ? 0x05040100u : 0x07060302u;
+}
+__device__ __forceinline__ void regw_load(RegW &w, rsrc_t rs_w, int k_bytes_w) {
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+    w.r[i] = __builtin_amdgcn_raw_buffer_load_b128(rs_w, w.voff[i], k_bytes_w, 0);
+}
+__device__ __forceinline__ void regw_store(const RegW &w, half_t *sW) {
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const unsigned lo = __builtin_amdgcn_perm(w.r[1][i >> 1], w.r[0][i >> 1], w.sel[i & 1]);
+    const unsigned hi = __builtin_amdgcn_perm(w.r[3][i >> 1], w.r[2][i >> 1], w.sel[i & 1]);
+    *(uint2_t *)(sW + w.woff[i]) = uint2_t{lo, hi};
+  }
+}
+
 template <int BM, int BN, int STAGES, int WM, int WN, int NP, int SCHED, int EPI, bool WKN>
 __device__ __forceinline__ void gemm_tile(const GemmArgs &p) {
   constexpr int BK = kBK;
@@ -358,6 +432,8 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs &p) {
   static_assert(BM % (8 * NL) == 0 && BN % (8 * NL) == 0, "tile rows must split evenly over the loading waves");
   static_assert(STAGES >= 2 && STAGES <= 5 && (STAGES - 2) * NI < 64, "pipeline depth");
   constexpr int YOUNG = STAGES - 2;   // stages that may still be in flight at a barrier
+  // a [K, N] weight tile goes through registers (see RegW) where every wave loads and computes
+  constexpr bool kRegW = WKN && NP == 0 && BN == 256 && NW == 8 && STAGES == 2;
 
   extern __shared__ __attribute__((aligned(1024))) half_t gemm_smem[];
   half_t *smem = gemm_smem;
@@ -445,14 +521,30 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs &p) {
     }
   }
   const int w_step_bytes = (WKN ? BK * p.N : BK) * (int)sizeof(half_t);   // one k-step further
-#define BT_ISSUE_LOADS(kt, stage)                                                        \
-  issue_stage_loads<NI, NIA>(rs_a, rs_w, voff, smem + (stage)*STAGE_HALFS + lw * 8 * BK, \
-                             NL * 8 * BK, (kt)*BK * (int)sizeof(half_t), (kt)*w_step_bytes)
+  RegW rw;
+  if (kRegW) regw_setup(rw, wave, lane, p.N, p.N - n0, BM);
+#define BT_ISSUE_LOADS(kt, stage)                                                              \
+  issue_stage_loads<NI, NIA, kRegW ? NIA : NI>(                                                \
+      rs_a, rs_w, voff, smem + (stage)*STAGE_HALFS + lw * 8 * BK, NL * 8 * BK,                 \
+      (kt)*BK * (int)sizeof(half_t), (kt)*w_step_bytes)
+  // Register-staged weight tile: the loads of k-step s + 1 go out at the top of step s, ahead
+  // of the A tile's direct-to-LDS loads (waiting until only those are outstanding then means
+  // the registers have arrived), and the tile is written to LDS behind the step's MFMAs.
+  // (Measured alternatives: writing it earlier in the step stalls on the loads; loads two
+  // steps ahead need a second register set, which no longer fits the register file.)
+#define BT_LOAD_W(kt) regw_load(rw, rs_w, (kt)*w_step_bytes)
+#define BT_STORE_W(stage)                                              \
+  do {                                                                 \
+    wait_vmcnt<NIA>();                                                 \
+    regw_store(rw, smem + (stage)*STAGE_HALFS + BM * BK);              \
+  } while (0)
 
   if (loader) {
+    if (kRegW) BT_LOAD_W(0);
 #pragma unroll
     for (int s = 0; s < STAGES - 1; ++s)
       if (s < nk) BT_ISSUE_LOADS(s, s);
+    if (kRegW) BT_STORE_W(0);
   }
 
   if (NP > 0 && wave >= NW) {
@@ -506,7 +598,7 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs &p) {
 #pragma unroll
     for (int i = 0; i < TN; ++i) {
       const int r = wn * WTN + i * 32 + fr_row;
-      if (WKN)
+      if (WKN && !kRegW)
         fw[b][i] = load_kn_frag<BN>(sB, wn * WTN + i * 32, 16 * ks, lane);
       else
         fw[b][i] = *(const half8_t *)(sB + r * BK + (((2 * ks + fr_kc) ^ swz(r + BM)) * 8));
@@ -520,10 +612,14 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs &p) {
   int stage = 0;
   for (int kt = 0; kt < nk; ++kt) {
     // tile kt has landed for this wave once only the younger stages' loads are outstanding
-    if (NP == 0) wait_stages<NI, YOUNG>(nk - 1 - kt);
+    if (kRegW)
+      __builtin_amdgcn_s_waitcnt(0x0070);   // vmcnt(0) lgkmcnt(0): also this wave's LDS writes of the W tile
+    else if (NP == 0)
+      wait_stages<NI, YOUNG>(nk - 1 - kt);
     asm volatile("" ::: "memory");
     __builtin_amdgcn_s_barrier();   // everyone's tile is in LDS; stage (kt-1) is free again
     asm volatile("" ::: "memory");
+    if (kRegW && kt + 1 < nk) BT_LOAD_W(kt + 1);
     if (NP == 0 && kt + STAGES - 1 < nk) {
       int ps = stage + STAGES - 1;
       if (ps >= STAGES) ps -= STAGES;
@@ -543,14 +639,17 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs &p) {
           acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fw[ks & 1][i], fa[ks & 1][j],
                                                             acc[i][j], 0, 0, 0);
     }
+    if (kRegW && kt + 1 < nk) BT_STORE_W(stage ^ 1);   // the W tile of step kt + 1
     if (++stage == STAGES) stage = 0;
   }
 
 #undef BT_ISSUE_LOADS
+#undef BT_LOAD_W
+#undef BT_STORE_W
   // ---- epilogue -------------------------------------------------------------
   // accumulator block (i, j), quad q: columns n..n+3 of row m with
   //   n = n0 + wn*WTN + i*32 + q*8 + (lane>>5)*4,  m = m0 + wm*WTM + j*32 + (lane&31)
-  constexpr int EP = WTN + 8;   // pitch (halfs) of the wave-private staging tile
+  constexpr int EP = Staging<WTN>::kPitch;   // pitch (halfs) of the wave-private staging tile
   static_assert((size_t)NW * 32 * EP <= (size_t)STAGES * STAGE_HALFS, "staging fits the ring");
   __builtin_amdgcn_s_barrier();   // all waves are done with the last stage
   half_t *st = smem + wave * 32 * EP;
@@ -591,7 +690,7 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs &p) {
           v2 = gelu_tanh_f32(v2);
           v3 = gelu_tanh_f32(v3);
         }
-        *(half4_t *)(st + row_in * EP + i * 32 + q * 8 + col_in) =
+        *(half4_t *)(st + Staging<WTN>::write_at(row_in, lane >> 5, i * 4 + q)) =
             half4_t{(half_t)v0, (half_t)v1, (half_t)v2, (half_t)v3};
       }
     }
@@ -600,7 +699,7 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs &p) {
       const int r = r0 + sr;
       if (sr >= RPS || r >= 32) continue;   // lanes left over when 64 % CPRW != 0
       const int m = m0 + wm * WTM + j * 32 + r, n = n0 + wn * WTN + sc;
-      const uint4_t v = *(const uint4_t *)(st + r * EP + sc);
+      const uint4_t v = Staging<WTN>::read(st, r, sc >> 3);
       if (m < M && n < p.N) {
         if (EPI == kEpiQkvSplit) {
           // column n = which*H + g*64 + dd  ->  [which*heads + g][m][dd]
@@ -637,7 +736,7 @@ __device__ __forceinline__ void gemm_tiles_flat(const GemmArgs &p) {
   static_assert(STAGES >= 2 && STAGES <= 5 && (STAGES - 2) * NI < 64, "pipeline depth");
   static_assert(EPI != kEpiPartial, "split-k launches keep one tile per workgroup");
   constexpr int YOUNG = STAGES - 2;
-  constexpr int EP = WTN + 8;   // pitch (halfs) of the wave-private staging tile
+  constexpr int EP = Staging<WTN>::kPitch;   // pitch (halfs) of the wave-private staging tile
   static_assert((size_t)NW * 32 * EP <= (size_t)STAGE_HALFS, "staging fits one stage of the ring");
 
   extern __shared__ __attribute__((aligned(1024))) half_t gemm_smem[];
@@ -891,7 +990,7 @@ __device__ __forceinline__ void gemm_tiles_flat(const GemmArgs &p) {
               v2 = gelu_tanh_f32(v2);
               v3 = gelu_tanh_f32(v3);
             }
-            *(half4_t *)(st + row_in * EP + i * 32 + q * 8 + col_in) =
+            *(half4_t *)(st + Staging<WTN>::write_at(row_in, lane >> 5, i * 4 + q)) =
                 half4_t{(half_t)v0, (half_t)v1, (half_t)v2, (half_t)v3};
           }
         }
@@ -900,7 +999,7 @@ __device__ __forceinline__ void gemm_tiles_flat(const GemmArgs &p) {
           const int r = r0 + sr;
           if (sr >= RPS || r >= 32) continue;   // lanes left over when 64 % CPRW != 0
           const int m = m0 + wm * WTM + j * 32 + r, n = n0 + wn * WTN + sc;
-          const uint4_t v = *(const uint4_t *)(st + r * EP + sc);
+          const uint4_t v = Staging<WTN>::read(st, r, sc >> 3);
           if (m < M && n < p.N) {
             if (EPI == kEpiQkvSplit) {
               // column n = which*H + g*64 + dd  ->  [which*heads + g][m][dd]
@@ -1044,13 +1143,13 @@ static long long estimated_rows(const GemmArgs &p) {
 // tile, so the row used has the same number of row tiles as m or one more: run time moves
 // in steps with the number of rounds of workgroups, and interpolating between two row
 // counts on either side of such a step would describe neither.
-static const float *tuned_times(long long m, int n, int k, int epi, int kn) {
+static const float *tuned_times(long long m, int n, int k, int epi, int kn, int full) {
   if (cu_count() != 256) return nullptr;     // the table was measured on a 256-CU part
   // below about a thousand rows a launch is latency bound and a loop of identical
   // launches says little about the layer sequence
   if (m < 1024 || m > kTunedRows[kTunedPoints - 1]) return nullptr;
   for (const TunedShape &ts : kTunedShapes) {
-    if (ts.n != n || ts.k != k || ts.epi != epi || ts.kn != kn) continue;
+    if (ts.n != n || ts.k != k || ts.epi != epi || ts.kn != kn || ts.full != full) continue;
     int at = 0;
     while (at < kTunedPoints - 1 && kTunedRows[at] < m) ++at;
     return ts.us[at];
@@ -1115,7 +1214,10 @@ static int launch_gemm(GemmArgs p, hipStream_t s) {
     // the table overrides the model only for a clear win: the timings come from a loop
     // of identical launches, and differences of a few per cent do not carry over to the
     // layer sequence
-    if (const float *us = tuned_times(estimated_rows(p), p.N, p.K, EPI, p.w_kn)) {
+    // (a launch whose estimated live rows fill its capacity to within one tile row is looked
+    // up among the all-live measurements)
+    const long long m_est = estimated_rows(p);
+    if (const float *us = tuned_times(m_est, p.N, p.K, EPI, p.w_kn, m_est + kTunedStep > p.rows_cap)) {
       int tuned = -1;
       for (int t = 0; t < kTunedTiles; ++t)
         if (us[t] > 0.f && (tuned < 0 || us[t] < us[tuned])) tuned = t;
@@ -1199,22 +1301,27 @@ extern "C" int bt_transpose_weight(const void *w, void *wt, int k, int n, void *
   return bt_transpose_weights(1, ws, wts, &k, &n, stream);
 }
 
-extern "C" int bt_gemm_prepack_pays(long long rows, int n, int k, int epilogue) {
+extern "C" float bt_gemm_prepack_gain_us(long long rows, int n, int k, int epilogue) {
   const int forced = option_layer_prepack();
-  if (forced >= 0) return forced;
-  const float *nk = tuned_times(rows, n, k, epilogue, 0), *kn = tuned_times(rows, n, k, epilogue, 1);
-  if (!nk || !kn) return 0;
+  if (forced >= 0) return forced ? 1e9f : -1e9f;
+  // (asked for the padded batch: the layer's launches are sized for batch x seq_len rows)
+  const float *nk = tuned_times(rows, n, k, epilogue, 0, 0), *kn = tuned_times(rows, n, k, epilogue, 1, 0);
+  if (!nk || !kn) return 0.f;
   float best_nk = 0.f, best_kn = 0.f;
   for (int t = 0; t < kTunedTiles; ++t) {
     if (nk[t] > 0.f && (best_nk == 0.f || nk[t] < best_nk)) best_nk = nk[t];
     if (kn[t] > 0.f && (best_kn == 0.f || kn[t] < best_kn)) best_kn = kn[t];
   }
-  if (best_nk == 0.f || best_kn == 0.f) return 0;
-  // the copy is made inside the layer's prologue launch, beside the offsets: measured in
-  // the layer sequence it adds about 0.5 us per megabyte of weight to that launch (2.4 us
-  // for FFN1 of BERT-base, 7.4 us for all four matrices); asked to return a microsecond more
+  if (best_nk == 0.f || best_kn == 0.f) return 0.f;
+  // the copy is made inside the layer's first launch, beside the offsets: measured in the
+  // layer sequence it adds about 0.5 us per megabyte of weight to that launch (2.4 us for
+  // FFN1 of BERT-base, 7.4 us for all four matrices)
   const float pack_us = 0.5e-6f * (float)n * (float)k * sizeof(half_t);
-  return best_nk + pack_us + 1.0f < best_kn ? 1 : 0;
+  return best_kn - best_nk - pack_us;
+}
+
+extern "C" int bt_gemm_prepack_pays(long long rows, int n, int k, int epilogue) {
+  return bt_gemm_prepack_gain_us(rows, n, k, epilogue) > 1.0f ? 1 : 0;   // asked to return a microsecond more
 }
 
 extern "C" int bt_gemm(const void *a, const void *wt, void *c, const int *valid_rows,

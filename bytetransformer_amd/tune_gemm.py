@@ -1,6 +1,7 @@
 """Measures every fp16 GEMM tile shape of libbt_hip.so over a grid of row counts for
 the four weight shapes of BERT-base and BERT-large, in both weight layouts ([k, n] as
-stored and the [n, k] pre-pack), and writes the table the launcher consults (csrc/kernels/gemm_tuned.inc; rebuild the kernels afterwards).
+stored and the [n, k] pre-pack) and both launch shapes (a padded batch of which 60 % of the
+rows are live, and a launch whose rows are all live), and writes the table the launcher consults (csrc/kernels/gemm_tuned.inc; rebuild the kernels afterwards).
 
     python -m bytetransformer_amd.tune_gemm [--json timings.json] [--from-json run1.json run2.json ...]
 
@@ -45,7 +46,9 @@ def _time_kernel(fn, iters):
 def measure(iters=32):
     """Each weight shape as the layer launches it: with its epilogue (QKV: bias + head
     split, FFN1: bias + GELU, the two others plain), with a row capacity of m / 0.6 (the
-    padded batch: launches are sized for batch x seq_len rows, of which m are live), the
+    padded batch: launches are sized for batch x seq_len rows, of which m are live) and with
+    a row capacity of m (every row live: the padded path, or a caller that sizes its launches
+    for the live rows), the
     QKV product gathering its rows from the padded input through a word_idx of 16 runs, and
     with the weights cold: the launches of one timing loop walk through enough copies of
     the weight matrix to exceed the memory-side cache, as the layers of a model do.  Every
@@ -67,10 +70,10 @@ def measure(iters=32):
                 wts = [ops.transpose_weight(w) for w in ws]
                 bias = torch.zeros(n, device=dev, dtype=torch.float16)
                 c = torch.empty(rows_cap * n, device=dev, dtype=torch.float16)
-                for m in M_GRID:
+                for m, full in [(m, f) for m in M_GRID for f in (0, 1)]:
                     vr = torch.tensor([m], dtype=torch.int32, device=dev)
                     turn = [0]
-                    cap = cap_of(m)
+                    cap = m if full else cap_of(m)
                     # 16 sequences of cap / 16 padded rows each, m / 16 of them valid
                     runs = [torch.arange(b * (cap // 16), b * (cap // 16) + (m * (b + 1)) // 16
                                          - (m * b) // 16, dtype=torch.int32) for b in range(16)]
@@ -102,7 +105,8 @@ def measure(iters=32):
                                 continue
                             ops.set_option("gemm_tile", tile)
                             us[str(tile)] = round(_time_kernel(call, iters), 2)
-                        row = {"M": m, "N": n, "K": k, "epi": epi, "kn": layout, "us": us}
+                        row = {"M": m, "N": n, "K": k, "epi": epi, "kn": layout, "full": full,
+                               "us": us}
                         out.append(row)
                         print(json.dumps(row), flush=True)
     finally:
@@ -120,33 +124,34 @@ def merge_runs(rows):
     import math
     seen = {}
     for r in rows:
-        key = (r["M"], r["N"], r["K"], r.get("epi", "plain"), r.get("kn", 0))
+        key = (r["M"], r["N"], r["K"], r.get("epi", "plain"), r.get("kn", 0), r.get("full", 0))
         for tile, us in r["us"].items():
             seen.setdefault(key, {}).setdefault(tile, []).append(us)
     pick = lambda v: sorted(v)[math.ceil(0.75 * (len(v) - 1))]
-    return [{"M": m, "N": n, "K": k, "epi": epi, "kn": kn,
+    return [{"M": m, "N": n, "K": k, "epi": epi, "kn": kn, "full": full,
              "us": {t: round(pick(v), 2) for t, v in by_tile.items()}}
-            for (m, n, k, epi, kn), by_tile in seen.items()]
+            for (m, n, k, epi, kn, full), by_tile in seen.items()]
 
 
 def write_inc(rows, path=INC):
     shapes = {}
     for r in merge_runs(rows):
-        shapes.setdefault((r["N"], r["K"], EPI_CODE[r.get("epi", "plain")], r.get("kn", 0)),
-                          {})[r["M"]] = r["us"]
+        shapes.setdefault((r["N"], r["K"], EPI_CODE[r.get("epi", "plain")], r.get("kn", 0),
+                           r.get("full", 0)), {})[r["M"]] = r["us"]
     lines = ["// Generated by `python -m bytetransformer_amd.tune_gemm` from timings on one MI355X:",
              "// microseconds per launch of each tile shape (index = tile id; 0 = not measured)",
-             "// at kTunedRows live rows, per weight shape and weight layout.  Do not edit by hand.",
+             "// at kTunedRows live rows, per weight shape, weight layout and launch shape (full = 1:",
+             "// every row of the launch live; 0: a padded batch with 60 % live rows).  Do not edit by hand.",
              "constexpr int kTunedPoints = %d;" % len(M_GRID),
              "constexpr int kTunedTiles = %d;" % len(TILES),
              "constexpr int kTunedStep = %d;" % M_STEP,
              "static const int kTunedRows[kTunedPoints] = {%s};" % ", ".join(map(str, M_GRID)),
              "struct TunedShape {",
-             "  int n, k, epi, kn;   // epi: the Epilogue the shape was timed with; kn: 1 = [k, n] weight",
+             "  int n, k, epi, kn, full;   // epi: the Epilogue the shape was timed with; kn: 1 = [k, n] weight",
              "  float us[kTunedPoints][kTunedTiles];", "};",
              "static const TunedShape kTunedShapes[] = {"]
-    for (n, k, epi, kn), by_m in sorted(shapes.items()):
-        lines.append("    {%d, %d, %d, %d, {" % (n, k, epi, kn))
+    for (n, k, epi, kn, full), by_m in sorted(shapes.items()):
+        lines.append("    {%d, %d, %d, %d, %d, {" % (n, k, epi, kn, full))
         for m in M_GRID:
             us = by_m.get(m, {})
             lines.append("        {%s},   // %d rows" % (

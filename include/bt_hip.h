@@ -203,6 +203,14 @@ int bt_gemm(const void *a, const void *wt, void *c, const int *valid_rows, int r
  * the reference.
  */
 int bt_gemm_prepack_pays(long long rows, int n, int k, int epilogue);
+/*
+ * The same answer as a quantity: the microseconds per launch that the product saves on a
+ * pre-packed copy after paying for the copy (bt_gemm_prepack_pays = more than one); 0 for
+ * shapes outside the table, +-1e9 under bt_set_option("layer_prepack", 1 | 0).  A layer
+ * that could go without its prologue launch altogether if it made no copy asks for more
+ * than that launch costs.
+ */
+float bt_gemm_prepack_gain_us(long long rows, int n, int k, int epilogue);
 
 /*
  * c = gelu_tanh(a . w + bias).  Replaces gemm_bias_gelu

@@ -6,7 +6,7 @@ from bytetransformer_amd import tune_gemm
 
 
 def test_table_writer_lays_rows_out_by_row_count_and_tile(tmp_path):
-    rows = [{"M": m, "N": 2304, "K": 768, "epi": "qkv", "kn": 1,
+    rows = [{"M": m, "N": 2304, "K": 768, "epi": "qkv", "kn": 1, "full": 0,
              "us": {str(t): float(m + t) for t in tune_gemm.TILES if t != 4}}
             for m in tune_gemm.M_GRID[:3]]
     path = tune_gemm.write_inc(rows, str(tmp_path / "t.inc"))
@@ -14,7 +14,7 @@ def test_table_writer_lays_rows_out_by_row_count_and_tile(tmp_path):
     assert "kTunedPoints = %d;" % len(tune_gemm.M_GRID) in text
     assert "kTunedTiles = %d;" % len(tune_gemm.TILES) in text
     assert "kTunedStep = %d;" % tune_gemm.M_STEP in text
-    assert "{2304, 768, %d, 1, {" % tune_gemm.EPI_CODE["qkv"] in text
+    assert "{2304, 768, %d, 1, 0, {" % tune_gemm.EPI_CODE["qkv"] in text
     body = [l for l in text.splitlines() if l.strip().startswith("{") and "rows" in l]
     assert len(body) == len(tune_gemm.M_GRID)
     first = [float(v) for v in re.findall(r"([0-9.]+)f", body[0])]
