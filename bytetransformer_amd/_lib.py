@@ -43,6 +43,7 @@ KERNEL_ABI = {
                                   _P]),
     "bt_gemm_prepack_pays": (c_int, [c_longlong, c_int, c_int, c_int]),
     "bt_gemm_prepack_gain_us": (c_float, [c_longlong, c_int, c_int, c_int]),
+    "bt_publish_int": (c_int, [_IP, _IP, _P]),
     "bt_compress": (c_int, [_P, _P, _IP, _IP, c_int, c_int, c_int, _P]),
     "bt_transpose_weight": (c_int, [_P, _P, c_int, c_int, _P]),
     "bt_transpose_weights": (c_int, [c_int, POINTER(c_void_p), POINTER(c_void_p), POINTER(c_int),
@@ -103,6 +104,7 @@ class EncoderConfig(ctypes.Structure):
 
 HOST_ABI = {
     "bt_encoder_bufsize": (c_ulonglong, [POINTER(EncoderConfig)]),
+    "bt_encoder_layer_plan": (c_int, [POINTER(EncoderConfig), c_int, c_int, c_int, POINTER(c_int)]),
     "bt_encoder_layer_forward": (c_int, [POINTER(EncoderConfig), POINTER(LayerWeights), _P, _P,
                                          _P, _P, c_int, c_int, _P]),
     "bt_encoder_layer_forward_bias": (c_int, [POINTER(EncoderConfig), POINTER(LayerWeights), _P,

@@ -9,6 +9,55 @@
 namespace bytetransformer {
 
 template <OperationType OpType>
+LayerPlan BertTransformer<OpType>::plan(int batch_size, int seq_len, bool have_offsets,
+                                        int valid_rows_hint) const {
+  LayerPlan lp;
+  const int hidden = head_num_ * size_per_head_;
+  const int inter = hidden * param_.intermediate_size;
+  const long long rows = (long long)batch_size * seq_len;
+  const bool streaming_fp16 = OpType == OperationType::HALF && size_per_head_ == 64 &&
+                              !attention_layer_->uses_short_kernel(seq_len);
+  // Short sequences on padded rows: nothing but the attention would use the offsets there,
+  // and the attention can apply the mask tensor itself (all seq_len keys, masked ones
+  // shifted by -10000: the same probabilities) - so the layer goes without the prologue
+  // launch, which at a few dozen tokens is an eighth of its run time.
+  int direct_limit = 0;
+  bt_get_option("padded_mask_direct", &direct_limit);
+  // (only launches that take the plain workgroup order: the balanced one ranks the
+  // sequences by their lengths)
+  lp.mask_direct = streaming_fp16 && !is_remove_padding_ && !have_offsets &&
+                   seq_len <= direct_limit &&
+                   bt_attention_worklist_bytes(batch_size, seq_len, head_num_) == 0;
+  // Padding-free fp16 layers that have to build their offsets: the QKV product can count the
+  // mask rows itself and leave the offsets for the kernels after it, so that the layer goes
+  // without the launch ahead of it.  By default only where that launch would have no
+  // per-call weight copy to make; with the option at 2 everywhere the entry takes the shape,
+  // and a few workgroups of the QKV launch which compute no tile then make the copies and
+  // the attention's work list (not the default: faster at batch 16 x 512, slower at
+  // 16 x 1024 and 32 x 384, where every workgroup of several rounds pays for counting the
+  // mask rows).
+  int qkv_mask_rows_opt = -1;
+  bt_get_option("qkv_mask_rows", &qkv_mask_rows_opt);
+  const bool fits = OpType == OperationType::HALF && is_remove_padding_ && !have_offsets &&
+                    qkv_mask_rows_opt != 0 &&
+                    bt_gemm_qkv_mask_rows_supported(batch_size, seq_len, Traits_::dtype);
+  lp.side_jobs = fits && qkv_mask_rows_opt == 2;
+  const bool have_prepack = OpType == OperationType::HALF && param_.prepacked_kernels[0] &&
+                            param_.prepacked_kernels[1] && param_.prepacked_kernels[2] &&
+                            param_.prepacked_kernels[3];
+  if (!have_prepack && OpType == OperationType::HALF && !lp.mask_direct &&
+      !(fits && qkv_mask_rows_opt == 1)) {
+    const long long live = valid_rows_hint > 0  ? valid_rows_hint
+                           : is_remove_padding_ ? (rows * 3LL + 4) / 5
+                                                : rows;
+    lp.copies = plan_weight_copies(live, rows, hidden, inter, size_per_head_ == 64,
+                                   fits && !lp.side_jobs, lp.side_jobs, lp.copy);
+  }
+  lp.starts_with_qkv = fits && (lp.copies == 0 || lp.side_jobs);
+  return lp;
+}
+
+template <OperationType OpType>
 void BertTransformer<OpType>::bert_infer(BertTransformerInferParam infer_param) {
   if (inner_buf_size_ == 0) cal_bufsize();
 
@@ -56,32 +105,9 @@ void BertTransformer<OpType>::bert_infer(BertTransformerInferParam infer_param) 
       infer_param.offsets && infer_param.offsets->batch_idx && infer_param.offsets->word_idx;
   const bool streaming_fp16 = OpType == OperationType::HALF && size_per_head_ == 64 &&
                               !attention_layer_->uses_short_kernel(seq_len);
-  // Short sequences on padded rows: nothing but the attention would use the offsets there,
-  // and the attention can apply the mask tensor itself (all seq_len keys, masked ones
-  // shifted by -10000: the same probabilities) - so the layer goes without the prologue
-  // launch, which at a few dozen tokens is an eighth of its run time.
-  int direct_limit = 0;
-  bt_get_option("padded_mask_direct", &direct_limit);
-  // (only launches that take the plain workgroup order: the balanced one ranks the
-  // sequences by their lengths)
-  const bool mask_direct = streaming_fp16 && !is_remove_padding_ && !have_offsets &&
-                           seq_len <= direct_limit &&
-                           bt_attention_worklist_bytes(batch_size, seq_len, head_num_) == 0;
-  // Padding-free fp16 layers that have to build their offsets: the QKV product can count the
-  // mask rows itself and leave the offsets for the kernels after it, so that the layer goes
-  // without the launch ahead of it.  By default only where that launch would have no
-  // per-call weight copy to make; with the option at 2 everywhere the entry takes the shape,
-  // and a few workgroups of the QKV launch which compute no tile then make the copies and
-  // the attention's work list (not the default: faster at batch 16 x 512, slower at
-  // 16 x 1024 and 32 x 384, where every workgroup of several rounds pays for counting the
-  // mask rows).
-  int qkv_mask_rows_opt = -1;
-  bt_get_option("qkv_mask_rows", &qkv_mask_rows_opt);
-  const bool qkv_mask_rows_fits =
-      OpType == OperationType::HALF && is_remove_padding_ && !have_offsets &&
-      qkv_mask_rows_opt != 0 &&
-      bt_gemm_qkv_mask_rows_supported(batch_size, seq_len, Traits_::dtype);
-  const bool side_jobs = qkv_mask_rows_fits && qkv_mask_rows_opt == 2;
+  const LayerPlan lp = plan(batch_size, seq_len, have_offsets, infer_param.valid_rows_hint);
+  const bool mask_direct = lp.mask_direct, side_jobs = lp.side_jobs;
+  const bool qkv_mask_rows = lp.starts_with_qkv;
   // The four products read the [k, n] weights as the caller stores them, exactly as the
   // reference hands them to cuBLAS (gemm.cu:27-39): nothing is kept between calls and
   // nothing can go stale.  Where the measured tile table says that a product of this size
@@ -104,30 +130,11 @@ void BertTransformer<OpType>::bert_infer(BertTransformerInferParam infer_param) 
       w_use[i] = param_.prepacked_kernels[i];
       w_kn[i] = 0;
     }
-  } else if (OpType == OperationType::HALF && !mask_direct &&
-             !(qkv_mask_rows_fits && qkv_mask_rows_opt == 1)) {   // (the copies are made by the first launch)
-    const long long live = infer_param.valid_rows_hint > 0 ? infer_param.valid_rows_hint
-                           : is_remove_padding_            ? (rows * 3LL + 4) / 5
-                                                           : rows;
-    const int epilogue[4] = {size_per_head_ == 64 ? BT_EPILOGUE_QKV_SPLIT : -1,
-                             BT_EPILOGUE_PLAIN, BT_EPILOGUE_BIAS_GELU, BT_EPILOGUE_PLAIN};
+  } else if (lp.copies > 0) {   // (the copies are made by the first launch)
+    const bool *copy = lp.copy;
     DataType_ *slot = (DataType_ *)(base + off);
-    // A layer whose QKV product can count the mask rows itself goes without a launch ahead
-    // of it as long as it makes no copy - one round of tiles pays about 3 us for that launch
-    // beyond the copy itself (measured per forward up to 10 k padded rows: never copying
-    // wins 1.5-1.8 % there, with several rounds of tiles it loses as much) - so there the
-    // copies have to return that much more.
-    const bool launch_at_stake = qkv_mask_rows_fits && !side_jobs && rows <= 10240;
-    float gain[4] = {0.f, 0.f, 0.f, 0.f}, total = 0.f;
     for (int i = 0; i < 4; ++i) {
-      // (a QKV launch that makes the copies itself reads its own weight as stored)
-      if (epilogue[i] < 0 || (i == 0 && side_jobs)) continue;
-      gain[i] = bt_gemm_prepack_gain_us(live, w_n[i], w_k[i], epilogue[i]);
-      if (gain[i] > 1.0f) total += gain[i];
-    }
-    const bool copy_any = !launch_at_stake || total > 1e8f || total >= 4.0f;
-    for (int i = 0; i < 4; ++i) {
-      if (copy_any && gain[i] > 1.0f) {
+      if (copy[i]) {
         pack_src[pack_count] = w_use[i];
         pack_dst[pack_count] = slot;
         pack_k[pack_count] = w_k[i];
@@ -143,7 +150,6 @@ void BertTransformer<OpType>::bert_infer(BertTransformerInferParam infer_param) 
                       sizeof(DataType_),
                   256);
   float *splitk_buf = (float *)(base + off);
-  const bool qkv_mask_rows = qkv_mask_rows_fits && (pack_count == 0 || side_jobs);
 
   // Padded rows, fp16 streaming attention: the mask tensor is applied unless one pass over
   // it finds the plain prefix mask of its lengths; the prologue leaves that verdict in the
@@ -223,6 +229,9 @@ void BertTransformer<OpType>::bert_infer(BertTransformerInferParam infer_param) 
     check_bt_error(bt_gemm_f32(from_tensor, gather, param_.attr_kernel_QKV,
                                param_.attention_param.attr_bias_QKV, qkv_buf, 0, valid_rows, rows, rows_hint,
                                3 * hidden, hidden, stream));
+    if (infer_param.valid_word_num_out && is_remove_padding_ && !have_offsets)
+      check_bt_error(bt_publish_int(et_param.batch_idx + batch_size,
+                                    infer_param.valid_word_num_out, stream));
     struct AttentionInferParam<DataType_> attention_infer_param {
       qkv_buf, atten_mask, attr_out_buf, base + inner_buf_size_, batch_size, seq_len,
           infer_param.cublas_handle, stream, et_param
@@ -270,6 +279,12 @@ void BertTransformer<OpType>::bert_infer(BertTransformerInferParam infer_param) 
                                           param_.attention_param.attr_bias_QKV, qkv_buf,
                                           valid_rows, rows, rows_hint, head_num_, size_per_head_,
                                           w_kn[0], stream));
+
+  // the count that this call's first launch has left in batch_idx[batch_size], for a host that
+  // wants it without waiting (one more launch of one wave, only when asked for)
+  if (infer_param.valid_word_num_out && is_remove_padding_ && !have_offsets)
+    check_bt_error(bt_publish_int(et_param.batch_idx + batch_size, infer_param.valid_word_num_out,
+                                  stream));
 
   struct AttentionInferParam<DataType_> attention_infer_param {
     qkv_buf, atten_mask, attr_out_buf, base + inner_buf_size_, batch_size, seq_len,

@@ -85,6 +85,38 @@ void layer_forward(const bt_encoder_config *cfg, const bt_layer_weights *weights
 }
 }  // namespace
 
+namespace {
+template <OperationType Op>
+void layer_plan(const bt_encoder_config *cfg, int batch_size, int seq_len, int rows_hint,
+                int *plan) {
+  BertTransformer<Op> enc(cfg->max_batch_size, cfg->head_num, cfg->size_per_head,
+                          cfg->max_seq_len, cfg->use_fused_attention != 0,
+                          cfg->is_remove_padding != 0, cfg->gamma_beta_fp32 != 0);
+  BertTransformerParam<Op> p;
+  p.intermediate_size = cfg->intermediate_size;
+  enc.initialize(p);
+  const bytetransformer::LayerPlan lp = enc.plan(batch_size, seq_len, false, rows_hint);
+  for (int i = 0; i < 4; ++i) plan[i] = lp.copy[i];
+  plan[4] = lp.starts_with_qkv;
+  plan[5] = lp.mask_direct;
+}
+}  // namespace
+
+extern "C" int bt_encoder_layer_plan(const bt_encoder_config *cfg, int batch_size, int seq_len,
+                                     int rows_hint, int *plan) {
+  int rc = validate(cfg);
+  if (rc != BT_OK) return rc;
+  if (!plan || batch_size <= 0 || seq_len <= 0) {
+    g_error = "[BT][ERROR] bt_encoder_layer_plan: null plan or non-positive size";
+    return BT_ERR_INVALID_ARGUMENT;
+  }
+  if (cfg->dtype == BT_F32)
+    layer_plan<OperationType::FP32>(cfg, batch_size, seq_len, rows_hint, plan);
+  else
+    layer_plan<OperationType::HALF>(cfg, batch_size, seq_len, rows_hint, plan);
+  return BT_OK;
+}
+
 extern "C" unsigned long long bt_encoder_bufsize(const bt_encoder_config *cfg) {
   if (validate(cfg) != BT_OK) return 0;
   return cfg->dtype == BT_F32 ? layer_bufsize<OperationType::FP32>(cfg)

@@ -388,8 +388,11 @@ struct RegW {
   unsigned sel[2];     // permute selectors of even / odd write instructions
 };
 __device__ __forceinline__ void regw_setup(RegW &w, int wave, int lane, int N, int cols, int BM) {
+  // (eight consecutive lanes on whole 128-byte lines measured slower: their writes then
+  // collide two ways, and the memory side does not mind the 64-byte pieces)
   const int kq = lane >> 2, ngl = lane & 3, ng = wave * 4 + ngl;
-  const int k_base = 4 * kq, n_base = 8 * ng, bit = ngl >> 1;
+  const int bit = ngl >> 1;
+  const int k_base = 4 * kq, n_base = 8 * ng;
 #pragma unroll
   for (int i = 0; i < 4; ++i)
     w.voff[i] = n_base < cols ? ((k_base + i) * N + n_base) * (int)sizeof(half_t) : 0x7ffffff0;
@@ -527,24 +530,27 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs &p) {
   issue_stage_loads<NI, NIA, kRegW ? NIA : NI>(                                                \
       rs_a, rs_w, voff, smem + (stage)*STAGE_HALFS + lw * 8 * BK, NL * 8 * BK,                 \
       (kt)*BK * (int)sizeof(half_t), (kt)*w_step_bytes)
-  // Register-staged weight tile: the loads of k-step s + 1 go out at the top of step s, ahead
-  // of the A tile's direct-to-LDS loads (waiting until only those are outstanding then means
-  // the registers have arrived), and the tile is written to LDS behind the step's MFMAs.
-  // (Measured alternatives: writing it earlier in the step stalls on the loads; loads two
-  // steps ahead need a second register set, which no longer fits the register file.)
+  // Register-staged weight tile: one register set.  The loads of k-step s + 1 go out early in
+  // step s - 1 (right after the registers have been emptied into LDS), have the rest of that
+  // step and the start of step s to arrive, and are written to LDS early in step s, behind
+  // the first quarter of its MFMAs: neither the loads nor the writes are waited for where
+  // they were issued.  In vmcnt terms every wait is "at most the NIA youngest outstanding":
+  // at the top of a step those are the weight loads (the A tile's direct-to-LDS loads are
+  // older), at the write they are the A tile's loads of the next step.
 #define BT_LOAD_W(kt) regw_load(rw, rs_w, (kt)*w_step_bytes)
-#define BT_STORE_W(stage)                                              \
-  do {                                                                 \
-    wait_vmcnt<NIA>();                                                 \
-    regw_store(rw, smem + (stage)*STAGE_HALFS + BM * BK);              \
-  } while (0)
+#define BT_STORE_W(stage) regw_store(rw, smem + (stage)*STAGE_HALFS + BM * BK)
+  static_assert(!kRegW || NIA == 4, "the weight tile's four loads per lane pair with four A loads");
 
   if (loader) {
-    if (kRegW) BT_LOAD_W(0);
 #pragma unroll
     for (int s = 0; s < STAGES - 1; ++s)
       if (s < nk) BT_ISSUE_LOADS(s, s);
-    if (kRegW) BT_STORE_W(0);
+    if (kRegW) {
+      BT_LOAD_W(0);
+      wait_vmcnt<0>();
+      BT_STORE_W(0);
+      if (nk > 1) BT_LOAD_W(1);
+    }
   }
 
   if (NP > 0 && wave >= NW) {
@@ -612,14 +618,18 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs &p) {
   int stage = 0;
   for (int kt = 0; kt < nk; ++kt) {
     // tile kt has landed for this wave once only the younger stages' loads are outstanding
-    if (kRegW)
-      __builtin_amdgcn_s_waitcnt(0x0070);   // vmcnt(0) lgkmcnt(0): also this wave's LDS writes of the W tile
-    else if (NP == 0)
+    if (kRegW) {
+      // this wave's A loads of tile kt and its LDS writes of the W tile; the weight loads of
+      // tile kt + 1 stay in flight
+      if (kt + 1 < nk)
+        __builtin_amdgcn_s_waitcnt(0x0074);   // vmcnt(4) lgkmcnt(0)
+      else
+        __builtin_amdgcn_s_waitcnt(0x0070);   // vmcnt(0) lgkmcnt(0)
+    } else if (NP == 0)
       wait_stages<NI, YOUNG>(nk - 1 - kt);
     asm volatile("" ::: "memory");
     __builtin_amdgcn_s_barrier();   // everyone's tile is in LDS; stage (kt-1) is free again
     asm volatile("" ::: "memory");
-    if (kRegW && kt + 1 < nk) BT_LOAD_W(kt + 1);
     if (NP == 0 && kt + STAGES - 1 < nk) {
       int ps = stage + STAGES - 1;
       if (ps >= STAGES) ps -= STAGES;
@@ -632,6 +642,11 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs &p) {
 #pragma unroll
     for (int ks = 0; ks < BK / 16; ++ks) {
       if (ks + 1 < BK / 16) load_frags(stage, ks + 1, (ks + 1) & 1);
+      if (kRegW && ks == 1 && kt + 1 < nk) {
+        wait_vmcnt<NIA>();            // the weight registers of step kt + 1 (older than its A loads)
+        BT_STORE_W(stage ^ 1);
+        if (kt + 2 < nk) BT_LOAD_W(kt + 2);
+      }
 #pragma unroll
       for (int i = 0; i < TN; ++i)
 #pragma unroll
@@ -639,7 +654,6 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs &p) {
           acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fw[ks & 1][i], fa[ks & 1][j],
                                                             acc[i][j], 0, 0, 0);
     }
-    if (kRegW && kt + 1 < nk) BT_STORE_W(stage ^ 1);   // the W tile of step kt + 1
     if (++stage == STAGES) stage = 0;
   }
 

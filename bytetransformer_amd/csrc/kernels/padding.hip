@@ -301,6 +301,13 @@ __global__ __launch_bounds__(kPrologueThreads) void layer_prologue_kernel(
   }
 }
 
+// ---- one int from device memory to wherever the caller reads it -----------------
+// (pinned host memory that the device can write: the host then learns a count without ever
+// waiting for the stream)
+__global__ void publish_int_kernel(const int *__restrict__ src, int *__restrict__ dst) {
+  if (threadIdx.x == 0) *dst = *src;
+}
+
 // ---- compress ---------------------------------------------------------------
 // One wave per packed row, 16-byte lanes.  M is read from batch_idx[B]; rows
 // past it retire immediately, so the grid is sized for B*S without a host sync.
@@ -494,6 +501,13 @@ extern "C" int bt_build_offsets(const void *atten_mask, int mask_dtype, int batc
     e = hipStreamSynchronize(s);
     if (e != hipSuccess) return hip_fail(e, "stream synchronize for valid_word_num");
   }
+  return BT_OK;
+}
+
+extern "C" int bt_publish_int(const int *src, int *dst, void *stream) {
+  BT_REQUIRE(src && dst, BT_ERR_INVALID_ARGUMENT, "bt_publish_int: null pointer argument");
+  publish_int_kernel<<<1, kWave, 0, as_stream(stream)>>>(src, dst);
+  BT_CHECK_LAUNCH("publish_int_kernel");
   return BT_OK;
 }
 

@@ -98,31 +98,19 @@ class BTEncoder : public IBTEncoder {
     // The layer reads the weights as they are and rebuilds the offsets from the mask on the
     // device, in every call; all the host keeps between calls is the valid-token count per
     // mask tensor, as a hint for tile shapes (the packed rows only: on the padded rows
-    // every row is live).
-    if (!capturing && encoder.is_remove_padding())
-      infer_param.valid_rows_hint = valid_rows_hint(attr_mask, batch_size, seq_len, stream);
+    // every row is live).  It never waits for that count: the first call that meets a mask
+    // asks the layer to publish it into pinned memory, later calls use it once it is there.
+    if (!capturing && encoder.is_remove_padding()) {
+      // (what is published is the count of THIS device: the slot is per mask and stream)
+      int count = 0;
+      infer_param.valid_word_num_out =
+          MaskHintCache::instance().lookup_or_reserve(attr_mask, stream, &count);
+      infer_param.valid_rows_hint = count;
+    }
     encoder.infer(infer_param);
   }
 
  private:
-  // The number of valid tokens of this mask, read back once per mask tensor (the one host
-  // synchronisation; the reference has one in every call, remove_padding.h:99-100).
-  // 0 = unknown.
-  int valid_rows_hint(const Tensor &mask, int batch_size, int seq_len, hipStream_t stream) {
-    if (!caches_enabled().load(std::memory_order_relaxed) || mask.is_inference()) return 0;
-    auto &cache = MaskHintCache::instance();
-    int count = 0;
-    if (cache.lookup(mask, stream, &count)) return count;
-    auto opts = torch::dtype(torch::kInt32).device(mask.device());
-    auto batch_idx = torch::empty({(int64_t)batch_size + 1}, opts);
-    auto word_idx = torch::empty({(int64_t)batch_size * seq_len}, opts);
-    check_bt_error(bt_build_offsets(mask.data_ptr(), Traits<kOp>::dtype, batch_size, seq_len,
-                                    batch_idx.data_ptr<int>(), word_idx.data_ptr<int>(), nullptr,
-                                    &count, stream));
-    cache.store(mask, stream, count);
-    return count;
-  }
-
   const int head_num_, head_size_;
   bool use_fp32_ = false;
   std::vector<Tensor> weights_;

@@ -127,6 +127,11 @@ def gemm_prepack_pays(rows, n, k, epilogue):
     return bool(kernel_lib().bt_gemm_prepack_pays(int(rows), int(n), int(k), int(epilogue)))
 
 
+def gemm_prepack_gain_us(rows, n, k, epilogue):
+    """bt_gemm_prepack_gain_us: microseconds per launch that a per-call [n, k] copy returns."""
+    return float(kernel_lib().bt_gemm_prepack_gain_us(int(rows), int(n), int(k), int(epilogue)))
+
+
 def compress(x, batch_idx, word_idx, out=None):
     B, S, H = x.shape
     if out is None:

@@ -58,6 +58,19 @@ int bt_encoder_layer_forward(const bt_encoder_config *cfg, const bt_layer_weight
                              const void *input, const void *atten_mask, void *output, void *buf,
                              int batch_size, int seq_len, void *stream);
 
+/*
+ * What a call of bt_encoder_layer_forward with these sizes will launch around its QKV
+ * product, for benchmarks that time the kernels one by one (host decisions only - sizes,
+ * options, the measured tile table -, never a matter of results; no counterpart in the
+ * reference).  rows_hint: the expected number of valid tokens, 0 = unknown.  plan[0..3]:
+ * 1 where the QKV / projection / FFN1 / FFN2 product runs on a k-contiguous copy of its
+ * weight made in the call's first launch; plan[4]: 1 when the layer starts with the QKV
+ * product that counts the mask rows itself (bt_gemm_qkv_bias_split_mask_rows) instead of
+ * bt_layer_prologue; plan[5]: 1 when a layer on padded rows goes without offsets altogether.
+ */
+int bt_encoder_layer_plan(const bt_encoder_config *cfg, int batch_size, int seq_len,
+                          int rows_hint, int *plan);
+
 /* The same with the optional attention bias of the reference's infer parameters
  * (bert_transformer.h:93, attention.h:56): [head_num, seq_len, seq_len] of cfg->dtype,
  * added to the scaled logits before the mask term (softmax.h:41-46).  NULL = none. */

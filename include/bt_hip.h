@@ -108,6 +108,15 @@ int bt_build_offsets(const void *atten_mask, int mask_dtype, int batch_size, int
                      void *stream);
 
 /*
+ * *dst = *src by one lane of a one-wave launch on `stream`.  `dst` may be host memory that
+ * the device can write (hipHostMalloc): a host that polls it learns the valid-token count
+ * (src = batch_idx + batch_size) some time after the launch without ever waiting for the
+ * stream - the asynchronous form of the reference's blocking copy of valid_word_num
+ * (remove_padding.h:99-100).
+ */
+int bt_publish_int(const int *src, int *dst, void *stream);
+
+/*
  * Is atten_mask exactly the prefix mask of the lengths in batch_idx, i.e. for every
  * batch b and EVERY row i: mask[b, i, j] == 1 for j < len_b and == 0 from there on, with
  * no empty sequence?  Then the padded-row attention may ignore the tensor and stop at

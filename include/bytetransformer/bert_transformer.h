@@ -78,6 +78,22 @@ struct BertTransformerInferParam {
   // no offsets.  A hint: it picks tile shapes and the split-k FFN2, never a launch size, so
   // a wrong value costs time and nothing else.
   int valid_rows_hint = 0;
+  // Extension: where the layer leaves the number of valid tokens it counted (padding-free
+  // layers that build their own offsets), or NULL.  Memory the device can write and the host
+  // can read (hipHostMalloc): written by a one-wave launch behind the layer's first launch,
+  // so a host that polls it learns the count without waiting for the stream - and can pass
+  // it as valid_rows_hint from then on.
+  int *valid_word_num_out = NULL;
+};
+
+// What one call of a layer will launch ahead of and around its QKV product (decided on the
+// host from sizes, options and the measured tile table; never changes a result).
+struct LayerPlan {
+  bool mask_direct = false;      // padded rows, short sequences: no offsets at all
+  bool starts_with_qkv = false;  // the QKV product counts the mask rows itself: no launch ahead of it
+  bool side_jobs = false;        // ... and carries the copies and the attention's work list
+  bool copy[4] = {false, false, false, false};   // QKV, projection, FFN1, FFN2 run on a per-call copy
+  int copies = 0;
 };
 
 template <OperationType OpType>
@@ -158,6 +174,9 @@ class BertTransformer {
   }
 
   void infer(BertTransformerInferParam infer_param) { bert_infer(infer_param); }
+
+  // The plan of a call with these sizes (have_offsets: the caller passes offsets of its own).
+  LayerPlan plan(int batch_size, int seq_len, bool have_offsets, int valid_rows_hint) const;
 
   void bert_infer(BertTransformerInferParam infer_param);
 

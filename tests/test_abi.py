@@ -175,3 +175,25 @@ def test_package_does_not_import_the_oracle():
             if f.endswith((".py", ".cc", ".hip", ".h")):
                 text = open(os.path.join(dirpath, f)).read()
                 assert "oracle" not in text, os.path.join(dirpath, f)
+
+
+def test_layer_plan_is_a_host_side_decision():
+    """bt_encoder_layer_plan answers without a GPU: at the headline shape the layer makes no
+    weight copy and starts with the QKV product that counts the mask rows; with several rounds
+    of tiles FFN1's copy pays again and the layer starts with its prologue; a short batch of
+    one goes without offsets."""
+    import ctypes
+    from bytetransformer_amd._lib import EncoderConfig, host_lib
+    lib = host_lib()
+
+    def plan(batch, seq, hint, rm=1):
+        cfg = EncoderConfig(1, batch, seq, 12, 64, 4, 1, rm, 0, 1.0, 1e-6)
+        out = (ctypes.c_int * 6)()
+        assert lib.bt_encoder_layer_plan(ctypes.byref(cfg), batch, seq, hint, out) == 0
+        return list(out)
+
+    assert plan(16, 512, 4809) == [0, 0, 0, 0, 1, 0]
+    big = plan(16, 1024, 9800)
+    assert big[4] == 0 and big[5] == 0 and sum(big[:4]) >= 1
+    assert plan(1, 64, 0) == [0, 0, 0, 0, 0, 1]
+    assert lib.bt_encoder_layer_plan(None, 1, 1, 0, (ctypes.c_int * 6)()) != 0
