@@ -426,7 +426,7 @@ def main():
     wl = workload.make_workload(args.workload)
     cfg = wl.cfg
     # the torch-free C++ loop runs as a child process, before this process touches the GPU
-    cpp_layer_ms = None if args.no_cpp_driver else cpp_api_layer_ms(wl)
+    cpp_layer_ms = None if (args.no_cpp_driver or args.vendor_compare) else cpp_api_layer_ms(wl)
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     dev = torch.device("cuda:0")
     bt.load_th_op()
