@@ -54,10 +54,7 @@ KERNEL_ABI = {
                                        c_int, _P]),
     "bt_gemm_qkv_mask_rows_supported": (c_int, [c_int, c_int, c_int]),
     "bt_gemm_qkv_bias_split_mask_rows": (c_int, [_P, _P, c_int, c_int, c_int, _P, _P, _P, _IP, _IP,
-                                                 _IP, c_int, c_int, c_int, c_int, _P, c_int,
-                                                 POINTER(c_void_p), POINTER(c_void_p),
-                                                 POINTER(c_int), POINTER(c_int), c_int,
-                                                 POINTER(c_void_p), POINTER(c_ulonglong), _P]),
+                                                 _IP, c_int, c_int, c_int, c_int, _P]),
     "bt_attention_short": (c_int, [_P, _P, _IP, _IP, _P, _P, c_int, c_int, c_int, c_int, c_int,
                                    c_float, c_int, POINTER(c_void_p), POINTER(c_ulonglong), c_int,
                                    _P]),

@@ -30,18 +30,13 @@ LayerPlan BertTransformer<OpType>::plan(int batch_size, int seq_len, bool have_o
                    bt_attention_worklist_bytes(batch_size, seq_len, head_num_) == 0;
   // Padding-free fp16 layers that have to build their offsets: the QKV product can count the
   // mask rows itself and leave the offsets for the kernels after it, so that the layer goes
-  // without the launch ahead of it.  By default only where that launch would have no
-  // per-call weight copy to make; with the option at 2 everywhere the entry takes the shape,
-  // and a few workgroups of the QKV launch which compute no tile then make the copies and
-  // the attention's work list (not the default: faster at batch 16 x 512, slower at
-  // 16 x 1024 and 32 x 384, where every workgroup of several rounds pays for counting the
-  // mask rows).
+  // without the launch ahead of it - where that launch would have no per-call weight copy
+  // to make (option qkv_mask_rows: -1 that rule, 0 never, 1 always and no copies).
   int qkv_mask_rows_opt = -1;
   bt_get_option("qkv_mask_rows", &qkv_mask_rows_opt);
   const bool fits = OpType == OperationType::HALF && is_remove_padding_ && !have_offsets &&
                     qkv_mask_rows_opt != 0 &&
                     bt_gemm_qkv_mask_rows_supported(batch_size, seq_len, Traits_::dtype);
-  lp.side_jobs = fits && qkv_mask_rows_opt == 2;
   const bool have_prepack = OpType == OperationType::HALF && param_.prepacked_kernels[0] &&
                             param_.prepacked_kernels[1] && param_.prepacked_kernels[2] &&
                             param_.prepacked_kernels[3];
@@ -50,10 +45,9 @@ LayerPlan BertTransformer<OpType>::plan(int batch_size, int seq_len, bool have_o
     const long long live = valid_rows_hint > 0  ? valid_rows_hint
                            : is_remove_padding_ ? (rows * 3LL + 4) / 5
                                                 : rows;
-    lp.copies = plan_weight_copies(live, rows, hidden, inter, size_per_head_ == 64,
-                                   fits && !lp.side_jobs, lp.side_jobs, lp.copy);
+    lp.copies = plan_weight_copies(live, rows, hidden, inter, size_per_head_ == 64, fits, lp.copy);
   }
-  lp.starts_with_qkv = fits && (lp.copies == 0 || lp.side_jobs);
+  lp.starts_with_qkv = fits && lp.copies == 0;
   return lp;
 }
 
@@ -106,7 +100,7 @@ void BertTransformer<OpType>::bert_infer(BertTransformerInferParam infer_param) 
   const bool streaming_fp16 = OpType == OperationType::HALF && size_per_head_ == 64 &&
                               !attention_layer_->uses_short_kernel(seq_len);
   const LayerPlan lp = plan(batch_size, seq_len, have_offsets, infer_param.valid_rows_hint);
-  const bool mask_direct = lp.mask_direct, side_jobs = lp.side_jobs;
+  const bool mask_direct = lp.mask_direct;
   const bool qkv_mask_rows = lp.starts_with_qkv;
   // The four products read the [k, n] weights as the caller stores them, exactly as the
   // reference hands them to cuBLAS (gemm.cu:27-39): nothing is kept between calls and
@@ -159,17 +153,6 @@ void BertTransformer<OpType>::bert_infer(BertTransformerInferParam infer_param) 
       !(have_offsets && infer_param.mask_prefix >= 0))
     mask_slots = (int *)(base + inner_buf_size_);
 
-  // The attention's balanced work list: built by spare workgroups of the QKV launch where that
-  // launch carries jobs.  A prologue launch does not build it: there it lengthens the
-  // launch by more than the attention saves (the kernel then finds its balanced order by a
-  // look-up of its own).
-  void *work_list = nullptr;
-  if (side_jobs && streaming_fp16) {
-    const unsigned long long need = bt_attention_worklist_bytes(batch_size, seq_len, head_num_);
-    if (need > 0 && need <= attention_layer_->work_list_capacity())
-      work_list = base + inner_buf_size_ + Attention<OpType>::work_list_offset();
-  }
-
   // One launch ahead of the layer: lengths and offsets from the mask (needed on both
   // paths: keys past len_b are excluded), the prefix-mask verdict, the weight copies.
   // Rebuilt on every call, as the reference does (bert_transformer.cu:62-66), unless the
@@ -181,11 +164,9 @@ void BertTransformer<OpType>::bert_infer(BertTransformerInferParam infer_param) 
   const void *warm[4];
   unsigned long long warm_bytes[4];
   int warm_count = 0;
-  // (the QKV launch that carries the jobs is already reading its own weight, and touches the
-  // others only where it has workgroups for jobs anyway)
-  if (OpType == OperationType::HALF && !have_prepack &&
-      (!qkv_mask_rows || pack_count > 0 || work_list))
-    for (int i = qkv_mask_rows ? 1 : 0; i < 4; ++i)
+  // (a layer that starts with the QKV product has no launch to do this in)
+  if (OpType == OperationType::HALF && !have_prepack && !qkv_mask_rows)
+    for (int i = 0; i < 4; ++i)
       if (w_kn[i]) {
         warm[warm_count] = w_use[i];
         warm_bytes[warm_count++] = (unsigned long long)w_k[i] * w_n[i] * sizeof(DataType_);
@@ -272,8 +253,7 @@ void BertTransformer<OpType>::bert_infer(BertTransformerInferParam infer_param) 
     check_bt_error(bt_gemm_qkv_bias_split_mask_rows(
         from_tensor, atten_mask, Traits_::dtype, batch_size, seq_len, wt_qkv,
         param_.attention_param.attr_bias_QKV, qkv_buf, et_param.batch_idx, et_param.word_idx,
-        seq_order, rows_hint, head_num_, size_per_head_, w_kn[0], work_list, pack_count, pack_src,
-        pack_dst, pack_k, pack_n, warm_count, warm, warm_bytes, stream));
+        seq_order, rows_hint, head_num_, size_per_head_, w_kn[0], stream));
   else
     check_bt_error(bt_gemm_qkv_bias_split(from_tensor, gather, wt_qkv,
                                           param_.attention_param.attr_bias_QKV, qkv_buf,
@@ -295,7 +275,9 @@ void BertTransformer<OpType>::bert_infer(BertTransformerInferParam infer_param) 
   // (0 = "not known to be the prefix mask": the tensor is applied)
   attention_infer_param.mask_prefix = have_offsets ? infer_param.mask_prefix : (mask_direct ? 0 : -1);
   attention_infer_param.mask_prefix_slots = mask_slots;
-  attention_infer_param.work_list = work_list;
+  // (no work list: building one per layer costs its launch more than the attention saves; the
+  // kernel finds its balanced order by a look-up of its own)
+  attention_infer_param.work_list = nullptr;
   attention_infer_param.no_offsets = mask_direct;   // (nothing has written them)
   // the three weight matrices the rest of the layer reads (as stored, or the copies of
   // this call): the attention kernel pulls them into the memory-side cache while it runs

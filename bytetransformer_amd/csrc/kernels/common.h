@@ -72,6 +72,7 @@ inline int allow_dynamic_lds(Kernel kernel, size_t bytes, std::atomic<bool> (&do
 }
 
 int option_gemm_tile();      // -1 = heuristic, else index into the tile table
+int option_gemm_table_margin();   // per cent by which a measured tile must beat the model's choice
 int option_layer_prepack();  // -1 = by the measured table, 0 = never, 1 = always
 int option_attention_qb();   // -1 = heuristic, 1 or 2 = query blocks per wave
 int option_f32_gemm_tile();  // -1 = heuristic, else index into the float GEMM's tile table

@@ -63,18 +63,7 @@ struct GemmArgs {
   int *out_batch_idx;   // [mask_B + 1]
   int *out_word_idx;    // [mask_B * mask_S]: the complete row map (valid positions, then the padded ones)
   int *out_seq_order;   // [mask_B]
-  // Jobs that ride along with this launch (mask rows only): the first `side_blocks`
-  // workgroups of the grid compute no tile; they make the k-contiguous weight copies that
-  // later products of the layer want, touch the weights that are read as stored, and build
-  // the attention's balanced work list - what a launch ahead of the layer would otherwise
-  // have to do.  The tile workgroups are blockIdx.x - side_blocks (a multiple of 8, so the
-  // XCD of a tile does not change).
-  int side_blocks;
-  int tile_grid;        // workgroups that compute tiles (set by the launcher)
-  WeightJobs jobs;
-  int4 *att_list;       // null: none
-  unsigned att_entries;
-  int att_bq, att_nqb, att_heads;
+  int tile_grid;        // workgroups of the launch (set by the launcher)
 };
 
 // ---- rows from the mask ---------------------------------------------------------
@@ -285,65 +274,6 @@ __device__ __forceinline__ half8_t load_kn_frag(const half_t *sW, int n_base, in
   return half8_t{l4[0], l4[1], l4[2], l4[3], h4[0], h4[1], h4[2], h4[3]};
 }
 
-// What a side workgroup does (see GemmArgs::side_blocks): `sb` = its index among them,
-// `nthreads` = threads of the workgroup (whole groups of 256), `lds` / `lds_bytes` = the
-// launch's dynamic LDS, all of it free here.
-__device__ __forceinline__ void gemm_side_jobs(const GemmArgs &p, int sb, int nthreads, half_t *lds,
-                                            int lds_bytes) {
-  const int tid = threadIdx.x, lane = tid & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int nwaves = nthreads >> 6;
-  // ---- the weights that the later products read as stored: first touch ----
-  if (const unsigned lines = p.jobs.warm_end[3]) {
-    const unsigned per = (lines + p.side_blocks - 1) / p.side_blocks;
-    const unsigned first = sb * per;
-    warm_lines(p.jobs, first + tid, first + per < lines ? first + per : lines, nthreads);
-  }
-  // ---- the attention's work list: one wave per entry ----
-  if (p.att_list) {
-    int *s_len = (int *)lds;             // [64]
-    int *s_off = s_len + 64;             // [B + 1]
-    int *s_order = s_off + 65;           // [B]
-    const MaskRows mr = mask_rows_setup(p, wave, nwaves, lane, s_len);
-    if (wave == 0) {
-      const int B = p.mask_B;
-      if (lane < B) s_off[lane] = mr.excl;
-      if (lane == 0) s_off[B] = mr.M;
-      int rank = 0;
-      for (int o = 0; o < B; ++o) {
-        const int lo = __shfl(mr.len, o, 64);
-        rank += (lo > mr.len) || (lo == mr.len && o < lane);
-      }
-      if (lane < B) s_order[rank] = lane;
-    }
-    __syncthreads();
-    const AttListArgs la{p.mask_B, p.mask_S, p.att_heads, p.att_nqb, 0, s_off, s_order};
-    for (unsigned e = sb * nwaves + wave; e < p.att_entries; e += p.side_blocks * nwaves) {
-      const AttWork w = p.att_bq == 128 ? att_work_balanced<128>(la, e) : att_work_balanced<64>(la, e);
-      if (lane == 0)
-        p.att_list[e] = w.exists ? int4{w.b, w.head | (w.qb << 16), w.seq_start, w.len}
-                                 : int4{-1, 0, 0, 0};
-    }
-    __syncthreads();   // the copies below overlay the lengths
-  }
-  // ---- k-contiguous copies of the weights that were asked for ----
-  if (p.jobs.count > 0) {
-    constexpr int kTileBytes = 64 * kTransposePitch * (int)sizeof(half_t);
-    const int groups = nthreads >> 8;
-    half_t(*tiles)[kTransposePitch] = (half_t(*)[kTransposePitch])lds;
-    const int t_end = p.jobs.tile_end[p.jobs.count - 1];
-    const int g = tid >> 8;
-    // U tiles per group and pass, as many as the LDS holds (4 at most)
-    if (lds_bytes >= groups * 4 * kTileBytes) {
-      for (int t0 = sb * groups * 4; t0 < t_end; t0 += p.side_blocks * groups * 4)
-        transpose_tiles_64<4>(p.jobs, t0 + g * 4, tiles + (size_t)g * 4 * 64, tid & 255);
-    } else {
-      for (int t0 = sb * groups; t0 < t_end; t0 += p.side_blocks * groups)
-        transpose_tiles_64<1>(p.jobs, t0 + g, tiles + (size_t)g * 64, tid & 255);
-    }
-  }
-}
-
 // ---- the epilogue's wave-private staging tile -------------------------------------------
 // 32 rows of WTN halfs, written 8 bytes per lane straight from the accumulator layout (lane l
 // owns row l & 31, the 8-byte half l >> 5 of a 16-byte chunk) and read back 16 bytes per lane,
@@ -443,14 +373,7 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs &p) {
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  if constexpr (EPI == kEpiQkvSplit || EPI == kEpiBias) {   // (the entries that take such jobs)
-    if ((int)blockIdx.x < p.side_blocks) {
-      gemm_side_jobs(p, blockIdx.x, (NW + NP) * 64, smem,
-                     STAGES * STAGE_HALFS * (int)sizeof(half_t));
-      return;
-    }
-  }
-  const int bid = (int)blockIdx.x - p.side_blocks;   // index among the tile workgroups
+  const int bid = (int)blockIdx.x;
   int M;
   MaskRows mr{};
   if (p.mask) {
@@ -758,14 +681,7 @@ __device__ __forceinline__ void gemm_tiles_flat(const GemmArgs &p) {
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  if constexpr (EPI == kEpiQkvSplit || EPI == kEpiBias) {   // (the entries that take such jobs)
-    if ((int)blockIdx.x < p.side_blocks) {
-      gemm_side_jobs(p, blockIdx.x, (NW + NP) * 64, smem,
-                     STAGES * STAGE_HALFS * (int)sizeof(half_t));
-      return;
-    }
-  }
-  const int bid = (int)blockIdx.x - p.side_blocks;   // index among the tile workgroups
+  const int bid = (int)blockIdx.x;
   int M;
   MaskRows mr{};
   if (p.mask) {
@@ -1083,7 +999,7 @@ static int launch_gemm_tile_as(GemmArgs p, hipStream_t s, int splits) {
   const int tiles_m = (p.rows_cap + BM - 1) / BM;
   p.tiles_n = (p.N + BN - 1) / BN;
   p.tile_grid = (tiles_m * p.tiles_n + 7) / 8 * 8;
-  const dim3 grid(p.tile_grid + p.side_blocks, splits);
+  const dim3 grid(p.tile_grid, splits);
   gemm_kernel<BM, BN, STAGES, WM, WN, NP, SCHED, EPI, WKN>
       <<<grid, (WM * WN + NP) * 64, smem, s>>>(p);
   BT_CHECK_LAUNCH("gemm_kernel");
@@ -1115,7 +1031,7 @@ static int launch_gemm_flat_as(GemmArgs p, hipStream_t s) {
   long long wgs = (long long)cu_count() * per_cu;
   if (wgs > tiles) wgs = tiles;
   p.tile_grid = (int)((wgs + 7) / 8 * 8);
-  const dim3 grid((unsigned)(p.tile_grid + p.side_blocks));
+  const dim3 grid((unsigned)p.tile_grid);
   gemm_flat_kernel<BM, BN, STAGES, WM, WN, NP, SCHED, EPI, WKN>
       <<<grid, (WM * WN + NP) * 64, smem, s>>>(p);
   BT_CHECK_LAUNCH("gemm_flat_kernel");
@@ -1236,7 +1152,8 @@ static int launch_gemm(GemmArgs p, hipStream_t s) {
       for (int t = 0; t < kTunedTiles; ++t)
         if (us[t] > 0.f && (tuned < 0 || us[t] < us[tuned])) tuned = t;
       const float t_model = choice < kTunedTiles ? us[choice] : 0.f;
-      if (tuned >= 0 && tuned != choice && (t_model <= 0.f || us[tuned] < 0.96f * t_model))
+      const float margin = 1.f - 0.01f * (float)option_gemm_table_margin();
+      if (tuned >= 0 && tuned != choice && (t_model <= 0.f || us[tuned] < margin * t_model))
         choice = tuned;
     }
   }
@@ -1419,9 +1336,7 @@ extern "C" int bt_gemm_qkv_bias_split_mask_rows(
     const void *from_tensor, const void *atten_mask, int mask_dtype, int batch_size, int seq_len,
     const void *wt_qkv, const void *bias_qkv, void *qkv_heads, int *batch_idx, int *word_idx,
     int *seq_order, int rows_hint, int head_num, int size_per_head, int weight_kn,
-    void *attention_work_list, int weight_count, const void *const *w, void *const *wt,
-    const int *k, const int *n, int warm_count, const void *const *warm,
-    const unsigned long long *warm_bytes, void *stream) {
+    void *stream) {
   const char *who = "bt_gemm_qkv_bias_split_mask_rows";
   BT_REQUIRE(head_num > 0 && size_per_head > 0, BT_ERR_INVALID_ARGUMENT,
              "%s: head_num=%d size_per_head=%d", who, head_num, size_per_head);
@@ -1436,7 +1351,7 @@ extern "C" int bt_gemm_qkv_bias_split_mask_rows(
   if (rc) return rc;
   BT_REQUIRE(bias_qkv && atten_mask && batch_idx, BT_ERR_INVALID_ARGUMENT,
              "%s: null pointer argument", who);
-  BT_REQUIRE(aligned16({atten_mask, attention_work_list}), BT_ERR_INVALID_ARGUMENT,
+  BT_REQUIRE(aligned16({atten_mask}), BT_ERR_INVALID_ARGUMENT,
              "%s: tensor pointers must be 16-byte aligned", who);
   // gathered rows are addressed with 32-bit byte offsets from the start of the input
   BT_REQUIRE((long long)rows_cap * H * 2 <= 0x7fffffffLL, BT_ERR_UNSUPPORTED,
@@ -1448,22 +1363,6 @@ extern "C" int bt_gemm_qkv_bias_split_mask_rows(
   p.mask_f32 = mask_dtype == BT_F32;
   p.mask_B = batch_size, p.mask_S = seq_len;
   p.out_batch_idx = batch_idx, p.out_word_idx = word_idx, p.out_seq_order = seq_order;
-  // the jobs that ride along: workgroups of their own at the head of the grid
-  rc = make_weight_jobs(who, &p.jobs, weight_count, w, wt, k, n, warm_count, warm, warm_bytes);
-  if (rc) return rc;
-  if (attention_work_list) {
-    const AttListPlan plan = att_worklist_plan(batch_size, seq_len, head_num);
-    if (plan.entries > 0) {
-      p.att_list = (int4 *)attention_work_list;
-      p.att_entries = plan.entries;
-      p.att_bq = plan.bq, p.att_nqb = plan.nqb, p.att_heads = head_num;
-    }
-  }
-  // (a multiple of 8: the XCD of a tile workgroup stays what its index says)
-  if (p.jobs.count > 0 || p.att_list)
-    p.side_blocks = 24;
-  else if (p.jobs.warm_end[3] > 0)
-    p.side_blocks = 8;
   if (size_per_head != 64) return launch_gemm<kEpiBias>(p, as_stream(stream));
   return launch_gemm<kEpiQkvSplit>(p, as_stream(stream));
 }

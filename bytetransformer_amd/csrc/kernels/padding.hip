@@ -38,6 +38,8 @@ static std::atomic<int> g_qkv_mask_rows{-1};
 static std::atomic<int> g_f32_gemm_tile{-1};
 static std::atomic<int> g_attention_short_limit{0};
 static std::atomic<int> g_attention_xcd_map{2};
+static std::atomic<int> g_gemm_table_margin{4};
+int option_gemm_table_margin() { return g_gemm_table_margin.load(std::memory_order_relaxed); }
 int option_attention_xcd_map() { return g_attention_xcd_map.load(std::memory_order_relaxed); }
 int option_f32_gemm_tile() { return g_f32_gemm_tile.load(std::memory_order_relaxed); }
 int option_gemm_tile() { return g_gemm_tile.load(std::memory_order_relaxed); }
@@ -393,6 +395,10 @@ extern "C" int bt_set_option(const char *name, int value) {
     BT_REQUIRE(value >= -1 && value <= 8, BT_ERR_INVALID_ARGUMENT,
                "bt_set_option: gemm_tile=%d outside [-1, 8]", value);
     g_gemm_tile.store(value);
+  } else if (!strcmp(name, "gemm_table_margin")) {
+    BT_REQUIRE(value >= 0 && value <= 100, BT_ERR_INVALID_ARGUMENT,
+               "bt_set_option: gemm_table_margin=%d outside [0, 100]", value);
+    g_gemm_table_margin.store(value);
   } else if (!strcmp(name, "attention_qb")) {
     BT_REQUIRE(value == -1 || value == 1 || value == 2, BT_ERR_INVALID_ARGUMENT,
                "bt_set_option: attention_qb=%d must be -1, 1 or 2", value);
@@ -426,8 +432,8 @@ extern "C" int bt_set_option(const char *name, int value) {
                "bt_set_option: padded_mask_direct=%d outside [0, 2^20]", value);
     g_padded_mask_direct.store(value);
   } else if (!strcmp(name, "qkv_mask_rows")) {
-    BT_REQUIRE(value >= -1 && value <= 2, BT_ERR_INVALID_ARGUMENT,
-               "bt_set_option: qkv_mask_rows=%d must be -1, 0, 1 or 2", value);
+    BT_REQUIRE(value >= -1 && value <= 1, BT_ERR_INVALID_ARGUMENT,
+               "bt_set_option: qkv_mask_rows=%d must be -1, 0 or 1", value);
     g_qkv_mask_rows.store(value);
   } else if (!strcmp(name, "prefetch_min_grid")) {
     BT_REQUIRE(value >= 1 && value <= (1 << 20), BT_ERR_INVALID_ARGUMENT,
@@ -444,6 +450,8 @@ extern "C" int bt_get_option(const char *name, int *value) {
   BT_REQUIRE(name && value, BT_ERR_INVALID_ARGUMENT, "bt_get_option: null argument");
   if (!strcmp(name, "gemm_tile")) {
     *value = g_gemm_tile.load();
+  } else if (!strcmp(name, "gemm_table_margin")) {
+    *value = g_gemm_table_margin.load();
   } else if (!strcmp(name, "attention_qb")) {
     *value = g_attention_qb.load();
   } else if (!strcmp(name, "prefetch")) {

@@ -227,13 +227,9 @@ def gemm_qkv_mask_rows_supported(batch_size, seq_len, mask_dtype=torch.float16):
 
 
 def gemm_qkv_bias_split_mask_rows(x, mask, wt_qkv, bias_qkv, head_num, size_per_head=64, out=None,
-                                  offsets_out=None, rows_hint=0, w_kn=False, work_list=None,
-                                  weights=None, packed=None, warm=()):
+                                  offsets_out=None, rows_hint=0, w_kn=False):
     """QKV projection of the padded x [B, S, H] whose live rows come from the mask inside the
-    launch; returns (qkv_heads, batch_idx, word_idx, seq_order).  Jobs that ride along with
-    the launch: work_list (int32[entries, 4]) is filled with the attention's balanced order as
-    attention_worklist would, `packed` with the [n, k] copies of the [k, n] `weights`, and the
-    tensors of `warm` are touched line by line (a cache hint)."""
+    launch; returns (qkv_heads, batch_idx, word_idx, seq_order)."""
     B, S = mask.shape[0], mask.shape[1]
     H = head_num * size_per_head
     rows = B * S
@@ -259,7 +255,7 @@ def gemm_qkv_bias_split_mask_rows(x, mask, wt_qkv, bias_qkv, head_num, size_per_
     _check(kernel_lib().bt_gemm_qkv_bias_split_mask_rows(
         _ptr(x), _ptr(mask), _dtype_code(mask), B, S, _ptr(wt_qkv), _ptr(bias_qkv), _ptr(out),
         _ptr(batch_idx), _ptr(word_idx), _ptr(seq_order), int(rows_hint), head_num, size_per_head,
-        int(w_kn), _ptr(work_list), *_weight_jobs(weights, packed, warm), _stream()))
+        int(w_kn), _stream()))
     return out, batch_idx, word_idx, seq_order
 
 

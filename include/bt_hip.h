@@ -52,6 +52,9 @@ const char *bt_last_error_string(void);
  *                   | 5: 128x128 with a two-deep ring (two workgroups per CU)
  *                   | 6, 7, 8: tiles 2, 1, 0 as persistent workgroups (about one per CU, each
  *                   running one load pipeline over several tiles of its XCD's range)
+ *   "gemm_table_margin"  4 (default), 0..100: per cent by which a tile's measured time must beat
+ *                   that of the cost model's choice before the measured table overrides the
+ *                   model (100 = the model alone decides)
  *   "attention_qb"  -1 heuristic | 1 | 2: 16-query blocks per wave in the grouped kernel
  *   "attention_key_split"  -1 heuristic | 0 | 1: the 64-query streaming attention with four waves,
  *                   or with eight: two groups of four take alternate 64-key halves of every ring
@@ -63,13 +66,12 @@ const char *bt_last_error_string(void);
  *                   attention applies the mask tensor itself, which needs no offsets, and a
  *                   launch less is worth more there than the keys the lengths would skip;
  *                   0 = every layer starts with the prologue.  Same results either way.
- *   "qkv_mask_rows" -1 (default) | 0 | 1 | 2: a padding-free fp16 layer that has to build its
+ *   "qkv_mask_rows" -1 (default) | 0 | 1: a padding-free fp16 layer that has to build its
  *                   offsets starts with bt_gemm_qkv_bias_split_mask_rows (one launch less,
  *                   every weight read as stored) where that entry takes the shape and no
  *                   per-call weight copy pays | always with bt_layer_prologue | with the
- *                   fused entry wherever it takes the shape, without copies | the same, and
- *                   the copies that pay and the attention's work list are made by workgroups
- *                   of that launch.  Same results either way.
+ *                   fused entry wherever it takes the shape, without copies.  Same results
+ *                   either way.
  *   "prefetch"      1 (default) | 0: honour / ignore the prefetch hint of the attention entries
  *   "prefetch_min_grid"  512 (default): attention launches of fewer workgroups ignore the hint
  *                   (there the warm-up costs more than it returns); 1 = every launch honours it
@@ -262,18 +264,6 @@ int bt_gemm_qkv_bias_split(const void *a, const int *a_row_index, const void *wt
  * the bias add of one layer call (bert_transformer.cu:62-87) in one launch.
  * bt_gemm_qkv_mask_rows_supported: 1 when the launch takes this shape (at most 64
  * sequences whose mask rows fit 64 KB), else 0 - then build the offsets first.
- * Jobs that ride along (each may be absent): a few workgroups of their own at the head of
- * the grid, which compute no tile, do what bt_layer_prologue would otherwise be launched
- * for ahead of the layer -
- *   - attention_work_list (nullable): the list of bt_attention_worklist for a launch of
- *     bt_attention_grouped over (batch_size, seq_len, head_num) on packed rows, at least
- *     bt_attention_worklist_bytes(...) bytes, left untouched when that is 0;
- *   - weight_count (0..4) matrices w[i] [k[i], n[i]] copied k-contiguous into wt[i]
- *     [n[i], k[i]] (bt_transpose_weights; the role of the reference's one-off weight layout
- *     choice, gemm.cu:27-39, made per call so that nothing is kept between calls);
- *   - warm_count (0..4) byte ranges touched line by line so that the launches that follow
- *     find them in the memory-side cache.
- * They run beside the tile workgroups and are complete when the launch is.
  */
 int bt_gemm_qkv_mask_rows_supported(int batch_size, int seq_len, int mask_dtype);
 int bt_gemm_qkv_bias_split_mask_rows(const void *from_tensor, const void *atten_mask,
@@ -281,10 +271,7 @@ int bt_gemm_qkv_bias_split_mask_rows(const void *from_tensor, const void *atten_
                                      const void *wt_qkv, const void *bias_qkv, void *qkv_heads,
                                      int *batch_idx, int *word_idx, int *seq_order,
                                      int rows_hint, int head_num, int size_per_head,
-                                     int weight_kn, void *attention_work_list, int weight_count,
-                                     const void *const *w, void *const *wt, const int *k,
-                                     const int *n, int warm_count, const void *const *warm,
-                                     const unsigned long long *warm_bytes, void *stream);
+                                     int weight_kn, void *stream);
 
 /*
  * Fused multi-head attention over the head-major Q/K/V written by

@@ -91,7 +91,6 @@ struct BertTransformerInferParam {
 struct LayerPlan {
   bool mask_direct = false;      // padded rows, short sequences: no offsets at all
   bool starts_with_qkv = false;  // the QKV product counts the mask rows itself: no launch ahead of it
-  bool side_jobs = false;        // ... and carries the copies and the attention's work list
   bool copy[4] = {false, false, false, false};   // QKV, projection, FFN1, FFN2 run on a per-call copy
   int copies = 0;
 };

@@ -82,17 +82,15 @@ inline unsigned long long splitk_scratch_bytes(unsigned long long max_rows,
 // without any launch ahead of it.  There the copies have to return what that launch costs
 // (about 3 us beyond the copies themselves with one round of tiles: never copying wins
 // 1.5-1.8 % per forward up to 10 k padded rows and loses as much beyond), elsewhere a
-// microsecond more than they cost.  `no_copy_of_qkv`: the first launch is the QKV product
-// itself.  Returns the number of copies and sets copy[i].
+// microsecond more than they cost.  Returns the number of copies and sets copy[i].
 inline int plan_weight_copies(long long live, long long padded_rows, int hidden, int inter,
-                              bool split_heads, bool first_launch_optional, bool no_copy_of_qkv,
-                              bool copy[4]) {
+                              bool split_heads, bool first_launch_optional, bool copy[4]) {
   const int n[4] = {3 * hidden, hidden, inter, hidden}, k[4] = {hidden, hidden, hidden, inter};
   const int epilogue[4] = {split_heads ? BT_EPILOGUE_QKV_SPLIT : -1, BT_EPILOGUE_PLAIN,
                            BT_EPILOGUE_BIAS_GELU, BT_EPILOGUE_PLAIN};
   float gain[4] = {0.f, 0.f, 0.f, 0.f}, total = 0.f;
   for (int i = 0; i < 4; ++i) {
-    if (epilogue[i] < 0 || (i == 0 && no_copy_of_qkv)) continue;
+    if (epilogue[i] < 0) continue;
     gain[i] = bt_gemm_prepack_gain_us(live, n[i], k[i], epilogue[i]);
     if (gain[i] > 1.0f) total += gain[i];
   }

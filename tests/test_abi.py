@@ -61,20 +61,16 @@ def test_argument_validation_returns_codes_without_gpu():
     assert lib.bt_gemm_qkv_mask_rows_supported(32, 1024, 0) == 0    # float mask rows: 128 KB
     assert lib.bt_gemm_qkv_mask_rows_supported(65, 8, 1) == 0
     assert lib.bt_gemm_qkv_mask_rows_supported(8, 8, 7) == 0
-    no_jobs = (None, 0, None, None, None, None, 0, None, None)   # work list, copies, ranges
     assert lib.bt_gemm_qkv_bias_split_mask_rows(p, p, 1, 65, 8, p, p, p, p, None, None, 0, 12,
-                                                64, 1, *no_jobs, None) == 2
+                                                64, 1, None) == 2
     assert "bt_gemm_qkv_mask_rows_supported" in err()
     assert lib.bt_gemm_qkv_bias_split_mask_rows(p, p, 1, 4, 8, p, p, p, None, None, None, 0, 12,
-                                                64, 1, *no_jobs, None) == 1 and "null pointer" in err()
+                                                64, 1, None) == 1 and "null pointer" in err()
     assert lib.bt_gemm_qkv_bias_split_mask_rows(p, None, 1, 4, 8, p, p, p, p, None, None, 0, 12,
-                                                64, 1, *no_jobs, None) == 1
-    assert lib.bt_gemm_qkv_bias_split_mask_rows(p, p, 1, 4, 8, p, p, p, p, None, None, 0, 12,
-                                                64, 1, None, 5, None, None, None, None, 0, None,
-                                                None, None) == 1 and "weight_count" in err()
-    for v in (0, 1, 2, -1):
+                                                64, 1, None) == 1
+    for v in (0, 1, -1):
         assert lib.bt_set_option(b"qkv_mask_rows", v) == 0
-    assert lib.bt_set_option(b"qkv_mask_rows", 3) == 1
+    assert lib.bt_set_option(b"qkv_mask_rows", 2) == 1
     assert lib.bt_gemm_qkv_bias_split(p, None, p, p, p, None, 4, 0, 1, 32, 0, None) == 2
     assert "multiple of 64" in err()        # hidden = 1 * 32
     assert lib.bt_gemm_qkv_bias_split(p, p, p, p, p, None, 4, 0, 12, 64, 1, None) == 1

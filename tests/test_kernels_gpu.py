@@ -592,6 +592,10 @@ def test_gemm_qkv_rows_from_the_mask(device, tile, case):
     assert torch.equal(got2[:, :, :M], got[:, :, :M])
 
 
+@pytest.mark.skip(reason="the side workgroups of the QKV launch were taken out of the library: a "
+                         "layer that used them by default left the GPU faulted once under the "
+                         "stand-alone C++ driver (batch 16 x 512) and no cause was found; the "
+                         "entry no longer takes work_list / weights / packed / warm")
 @pytest.mark.parametrize("tile", [-1, 0, 3, 4, 7])
 @pytest.mark.parametrize("case", ["cfg2-like", "many-short", "f32-mask"])
 def test_gemm_qkv_rows_from_the_mask_side_jobs(device, case, tile):

@@ -793,11 +793,11 @@ def test_layer_prepack_choice_never_changes_the_result(device):
 def test_qkv_rows_from_the_mask_never_change_the_result(device):
     """A padding-free layer may start with the QKV product that counts the mask rows itself
     instead of the prologue launch: never, wherever the entry takes the shape (without the
-    per-call weight copies, or with workgroups of that launch making them and the
-    attention's work list), and the automatic choice give the same bits - ragged lengths
-    with an empty sequence, the headline shape (12 heads: a copy pays and the attention takes
-    the balanced list), and a batch beyond the entry's 64 sequences (which falls back by
-    itself)."""
+    per-call weight copies), and the automatic choice give the same bits - ragged lengths
+    with an empty sequence, the headline shape with 4 and with 12 heads, and a batch beyond
+    the entry's 64 sequences (which falls back by itself).  (A fourth choice, workgroups of
+    that launch making the copies and the attention's work list, was taken out of the
+    library after one unexplained GPU fault under the C++ driver.)"""
     _say("qkv_mask_rows")
     from bytetransformer_amd import ops
     bt.load_th_op()
@@ -813,13 +813,12 @@ def test_qkv_rows_from_the_mask_never_change_the_result(device):
         x, m = _dev(wl.x, device), _dev(wl.mask, device)
         got = {}
         try:
-            for choice in (0, 1, 2, -1):
+            for choice in (0, 1, -1):
                 ops.set_option("qkv_mask_rows", choice)
                 got[choice] = op(cfg.head_num, 64, *w, x, m, True, True)
         finally:
             ops.set_option("qkv_mask_rows", -1)
         assert torch.equal(got[0], got[1]) and torch.equal(got[0], got[-1])
-        assert torch.equal(got[0], got[2])
         _check(got[1].cpu().numpy(), _oracle(wl), wl.lens, tag="qkv_mask_rows " + cfg.name)
 
 
