@@ -171,6 +171,15 @@ def kernel_table(wl, dev, iters):
         ("gemm_ffn2", lambda: ops.gemm(inter_m, wt_2, valid_rows=vr, out=ffn2_m, rows_hint=M,
                                        w_kn=kn_2), "mfma",
          2 * M * F * H),
+    ]
+    if kn_1:
+        # the same FFN1 launch on a k-contiguous copy of its weight: what the whole-encoder
+        # entry, which owns pre-packed copies, runs - and what the as-stored layout costs
+        wt_1_packed = ops.transpose_weight(w["inter_kernel"])
+        rows.append(("gemm_bias_gelu_prepacked", lambda: ops.gemm_bias_gelu(
+            proj_m, wt_1_packed, w["inter_bias"], valid_rows=vr, out=inter_m, rows_hint=M,
+            w_kn=False), "mfma", 2 * M * H * F))
+    rows += [
         ("layernorm_restore", lambda: ops.add_bias_residual_layernorm_restore(
             ffn2, proj, w["output_bias"], g1, b1, batch_idx, B, S, out_padded=out_pad,
             word_idx=word_idx),
@@ -278,6 +287,8 @@ def in_tree_over_vendor(kernels, calib):
     for shape, kern in (("qkv", qkv), ("proj", "gemm_proj"), ("ffn1", "gemm_bias_gelu"),
                         ("ffn2", "gemm_ffn2")):
         out[shape] = round(kernels[kern]["us"] / calib[shape]["us"], 3)
+    if "gemm_bias_gelu_prepacked" in kernels:
+        out["ffn1_prepacked"] = round(kernels["gemm_bias_gelu_prepacked"]["us"] / calib["ffn1"]["us"], 3)
     sq = calib["square_8192"]
     out["square_8192_as_stored"] = round(sq["in_tree_us_as_stored"] / sq["us"], 3)
     out["square_8192_prepacked"] = round(sq["in_tree_us_prepacked"] / sq["us"], 3)
