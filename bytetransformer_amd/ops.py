@@ -67,6 +67,14 @@ def build_offsets(mask, want_count=False, out=None, seq_order=None):
     return batch_idx, word_idx, (cnt.value if want_count else None)
 
 
+def publish_int(src, dst):
+    """*dst = *src on the current stream without any host wait: src is a device int32 (a view of
+    one element, e.g. batch_idx[B:]), dst a pinned host int32 tensor the device can write."""
+    if src.dtype != torch.int32 or dst.dtype != torch.int32 or not dst.is_pinned():
+        raise ValueError("publish_int: int32 device source and pinned int32 host destination expected")
+    _check(kernel_lib().bt_publish_int(_ptr(src), ctypes.c_void_p(dst.data_ptr()), _stream()))
+
+
 def mask_is_prefix(mask, batch_idx):
     """True when mask [B,S,S] is exactly (j < len_b) in every row and no sequence is empty."""
     B, S = mask.shape[0], mask.shape[1]

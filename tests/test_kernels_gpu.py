@@ -46,6 +46,24 @@ def test_build_offsets_bit_exact(device, B, S, dtype):
     assert np.array_equal(g_wi.cpu().numpy()[:M], wi)
 
 
+def test_valid_token_count_published_into_pinned_memory(device):
+    """The count the reference reads back with a blocking copy (remove_padding.h:99-100) is
+    stored into pinned host memory by a one-wave launch behind the offsets: after the stream
+    has drained the host finds the exact count there, for two masks in a row in the same slot."""
+    slot = torch.full((4,), -1, dtype=torch.int32, pin_memory=True)
+    for B, S, seed in ((16, 512, 1), (5, 33, 2)):
+        _say("publish count", B, S)
+        rs = np.random.RandomState(seed)
+        lens = rs.randint(0, S + 1, size=B)
+        mask = workload.make_mask(lens, S, np.float16)
+        bi, _, _ = ops.build_offsets(_dev(mask, device))
+        ops.publish_int(bi[B:], slot[1:2])
+        torch.cuda.synchronize()
+        assert slot.tolist() == [-1, int(lens.sum()), -1, -1]
+    with pytest.raises(ValueError):
+        ops.publish_int(bi[B:], torch.zeros(1, dtype=torch.int32))      # not pinned
+
+
 # Every product test runs with the weight in both layouts: the [n, k] pre-pack and the
 # [k, n] matrix as the layer stores it.
 _KN = [False]

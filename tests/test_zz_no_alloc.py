@@ -1,8 +1,9 @@
 """bt_encoder_layer_forward_static (the entry point that brings its own scratch and
 allocates nothing) against bt_encoder_layer_forward_bias with a caller-owned buffer:
-same kernels, same launches, so the outputs must agree bit for bit.  Two calls in a row
-share the library's device array, the second with a smaller input, so stale contents of
-the first call would show."""
+same kernels, same launches, so the outputs must agree bit for bit - and against the CPU
+oracle on the same inputs within the fp16 tolerance (max-abs 2e-2, mean-abs 2e-3 over the valid
+rows).  Two calls in a row share the library's device array, the second with a smaller input,
+so stale contents of the first call would show."""
 import ctypes
 
 import numpy as np
@@ -11,6 +12,7 @@ import torch
 
 from bytetransformer_amd import workload
 from bytetransformer_amd._lib import EncoderConfig, LayerWeights, host_lib
+from oracle import bert_oracle as O
 
 pytestmark = pytest.mark.gpu
 
@@ -66,6 +68,15 @@ def _both(device, batch, seq_len, lens, seed, with_bias=False):
     assert np.isfinite(ref.astype(np.float32)).all()
     assert np.array_equal(ref.view(np.uint16), got.view(np.uint16)), \
         "static-scratch layer differs from the caller-buffer layer"
+    # ... and the oracle's layer on the same inputs (valid rows; fp16 tolerance of the path)
+    w32 = {k: np.asarray(v, np.float32) for k, v in wl.layers[0].items()}
+    kw = {"attention_bias": bias.float().cpu().numpy()} if with_bias else {}
+    exp = O.encoder_layer(wl.x.astype(np.float32), wl.mask.astype(np.float32), w32,
+                          wl.cfg.head_num, **kw).numpy()
+    mx, mean, _ = O.parity_metrics(O.masked_output(got, wl.lens), O.masked_output(exp, wl.lens),
+                                   wl.lens)
+    print("static scratch against the oracle: max-abs %.3e mean-abs %.3e" % (mx, mean), flush=True)
+    assert mx <= 2e-2 and mean <= 2e-3, (mx, mean)
     return got
 
 
