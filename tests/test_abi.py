@@ -71,6 +71,13 @@ def test_argument_validation_returns_codes_without_gpu():
     for v in (0, 1, -1):
         assert lib.bt_set_option(b"qkv_mask_rows", v) == 0
     assert lib.bt_set_option(b"qkv_mask_rows", 2) == 1
+    assert lib.bt_set_option(b"qkv_mask_rows", -1) == 0
+    # the margin by which the measured tile table has to beat the cost model's choice
+    got = ctypes.c_int(-1)
+    assert lib.bt_get_option(b"gemm_table_margin", ctypes.byref(got)) == 0 and got.value == 4
+    assert lib.bt_set_option(b"gemm_table_margin", 100) == 0
+    assert lib.bt_set_option(b"gemm_table_margin", 101) == 1 and "gemm_table_margin" in err()
+    assert lib.bt_set_option(b"gemm_table_margin", 4) == 0
     assert lib.bt_gemm_qkv_bias_split(p, None, p, p, p, None, 4, 0, 1, 32, 0, None) == 2
     assert "multiple of 64" in err()        # hidden = 1 * 32
     assert lib.bt_gemm_qkv_bias_split(p, p, p, p, p, None, 4, 0, 12, 64, 1, None) == 1
