@@ -65,6 +65,10 @@ KERNEL_ABI = {
     "bt_attention_worklist": (c_int, [_IP, _IP, c_int, c_int, c_int, c_int, _P, _P]),
     "bt_add_bias_residual_layernorm": (c_int, [_P, _P, _IP, _P, _P, _P, c_int, _IP, c_int, c_int,
                                                c_float, _P]),
+    "bt_add_bias_residual_layernorm_copy": (c_int, [_P, _P, _IP, _P, _P, _P, c_int, _IP, c_int,
+                                                    c_int, c_float, c_int, POINTER(c_void_p),
+                                                    POINTER(c_void_p), POINTER(c_int),
+                                                    POINTER(c_int), _P]),
     "bt_add_bias_residual_layernorm_restore": (c_int, [_P, _P, _P, _P, _P, c_int, _P, _IP, _IP,
                                                        c_int, c_int, c_int, c_float, _P]),
     "bt_gemm_splitk": (c_int, [_P, _P, _P, c_int, _IP, c_int, c_int, c_int, c_int, _P]),

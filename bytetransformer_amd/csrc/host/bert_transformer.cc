@@ -31,7 +31,10 @@ LayerPlan BertTransformer<OpType>::plan(int batch_size, int seq_len, bool have_o
   // Padding-free fp16 layers that have to build their offsets: the QKV product can count the
   // mask rows itself and leave the offsets for the kernels after it, so that the layer goes
   // without the launch ahead of it - where that launch would have no per-call weight copy
-  // to make (option qkv_mask_rows: -1 that rule, 0 never, 1 always and no copies).
+  // to make (option qkv_mask_rows: -1 that rule, 0 never, 1 always and no copies).  Copies for
+  // FFN1 and FFN2 need no such launch: the first LayerNorm's can carry them (ln_weight_copy) -
+  // up to 32 sequences; beyond, counting the mask rows in every workgroup of several rounds
+  // costs more than the launch it saves (batch 64 x 256: +1.4 % per forward).
   int qkv_mask_rows_opt = -1;
   bt_get_option("qkv_mask_rows", &qkv_mask_rows_opt);
   const bool fits = OpType == OperationType::HALF && is_remove_padding_ && !have_offsets &&
@@ -40,12 +43,16 @@ LayerPlan BertTransformer<OpType>::plan(int batch_size, int seq_len, bool have_o
   const bool have_prepack = OpType == OperationType::HALF && param_.prepacked_kernels[0] &&
                             param_.prepacked_kernels[1] && param_.prepacked_kernels[2] &&
                             param_.prepacked_kernels[3];
-  if (!have_prepack && OpType == OperationType::HALF && !lp.mask_direct &&
-      !(fits && qkv_mask_rows_opt == 1)) {
+  if (!have_prepack && OpType == OperationType::HALF && !lp.mask_direct) {
     const long long live = valid_rows_hint > 0  ? valid_rows_hint
                            : is_remove_padding_ ? (rows * 3LL + 4) / 5
                                                 : rows;
-    lp.copies = plan_weight_copies(live, rows, hidden, inter, size_per_head_ == 64, fits, lp.copy);
+    int ln_weight_copy = 1;
+    bt_get_option("ln_weight_copy", &ln_weight_copy);
+    lp.copies = plan_weight_copies(live, rows, hidden, inter, size_per_head_ == 64,
+                                   !fits ? 0 : (qkv_mask_rows_opt == 1 ? 2 : 1),
+                                   fits && ln_weight_copy != 0 && batch_size <= 32, lp.copy,
+                                   lp.ln_copy);
   }
   lp.starts_with_qkv = fits && lp.copies == 0;
   return lp;
@@ -116,24 +123,35 @@ void BertTransformer<OpType>::bert_infer(BertTransformerInferParam infer_param) 
   int w_kn[4] = {1, 1, 1, 1};
   const int w_k[4] = {hidden, hidden, hidden, inter};
   const int w_n[4] = {3 * hidden, hidden, inter, hidden};
-  const void *pack_src[4];
-  void *pack_dst[4];
-  int pack_k[4], pack_n[4], pack_count = 0;
+  const void *pack_src[4], *ln_src[4];
+  void *pack_dst[4], *ln_dst[4];
+  int pack_k[4], pack_n[4], pack_count = 0, ln_k[4], ln_n[4], ln_count = 0;
+  // what the attention's cache warm-up touches: the matrices as the caller stores them where a
+  // later launch of the layer makes the copy (it does not exist yet when the attention runs)
+  const DataType_ *w_touch[4] = {w_use[0], w_use[1], w_use[2], w_use[3]};
   if (have_prepack) {
     for (int i = 0; i < 4; ++i) {
       w_use[i] = param_.prepacked_kernels[i];
       w_kn[i] = 0;
     }
-  } else if (lp.copies > 0) {   // (the copies are made by the first launch)
-    const bool *copy = lp.copy;
+  } else {
+    // (copies made by the launch ahead of the layer, or by the first LayerNorm's launch)
     DataType_ *slot = (DataType_ *)(base + off);
     for (int i = 0; i < 4; ++i) {
-      if (copy[i]) {
+      if (lp.copy[i]) {
         pack_src[pack_count] = w_use[i];
         pack_dst[pack_count] = slot;
         pack_k[pack_count] = w_k[i];
         pack_n[pack_count] = w_n[i];
         ++pack_count;
+        w_use[i] = slot;
+        w_kn[i] = 0;
+      } else if (lp.ln_copy[i]) {
+        ln_src[ln_count] = w_use[i];
+        ln_dst[ln_count] = slot;
+        ln_k[ln_count] = w_k[i];
+        ln_n[ln_count] = w_n[i];
+        ++ln_count;
         w_use[i] = slot;
         w_kn[i] = 0;
       }
@@ -284,7 +302,7 @@ void BertTransformer<OpType>::bert_infer(BertTransformerInferParam infer_param) 
   {
     const size_t elems[3] = {(size_t)hidden * hidden, (size_t)hidden * inter, (size_t)hidden * inter};
     for (int i = 0; i < 3; ++i) {
-      attention_infer_param.prefetch[i] = w_use[i + 1];
+      attention_infer_param.prefetch[i] = lp.ln_copy[i + 1] ? w_touch[i + 1] : w_use[i + 1];
       attention_infer_param.prefetch_bytes[i] = elems[i] * sizeof(DataType_);
     }
     attention_infer_param.prefetch_count = 3;
@@ -295,10 +313,16 @@ void BertTransformer<OpType>::bert_infer(BertTransformerInferParam infer_param) 
       bt_gemm(attr_out_buf, wt_proj, attr_matmul_buf, valid_rows, packed_cap, rows_hint, hidden,
               hidden, w_kn[1], stream));
 
-  check_bt_error(bt_add_bias_residual_layernorm(
-      attr_matmul_buf, from_tensor, gather, param_.attr_output_bias, param_.attr_output_layernorm_gamma,
-      param_.attr_output_layernorm_beta, use_fp32_ ? 1 : 0, valid_rows, packed_cap, hidden,
-      layernorm_eps, stream));
+  if (ln_count > 0)
+    check_bt_error(bt_add_bias_residual_layernorm_copy(
+        attr_matmul_buf, from_tensor, gather, param_.attr_output_bias,
+        param_.attr_output_layernorm_gamma, param_.attr_output_layernorm_beta, use_fp32_ ? 1 : 0,
+        valid_rows, packed_cap, hidden, layernorm_eps, ln_count, ln_src, ln_dst, ln_k, ln_n, stream));
+  else
+    check_bt_error(bt_add_bias_residual_layernorm(
+        attr_matmul_buf, from_tensor, gather, param_.attr_output_bias,
+        param_.attr_output_layernorm_gamma, param_.attr_output_layernorm_beta, use_fp32_ ? 1 : 0,
+        valid_rows, packed_cap, hidden, layernorm_eps, stream));
 
   check_bt_error(bt_gemm_bias_gelu(attr_matmul_buf, wt_inter, param_.inter_bias, inter_matmul_buf,
                                    valid_rows, packed_cap, rows_hint, inter, hidden, w_kn[2],

@@ -96,7 +96,7 @@ void layer_plan(const bt_encoder_config *cfg, int batch_size, int seq_len, int r
   p.intermediate_size = cfg->intermediate_size;
   enc.initialize(p);
   const bytetransformer::LayerPlan lp = enc.plan(batch_size, seq_len, false, rows_hint);
-  for (int i = 0; i < 4; ++i) plan[i] = lp.copy[i];
+  for (int i = 0; i < 4; ++i) plan[i] = lp.copy[i] ? 1 : (lp.ln_copy[i] ? 2 : 0);
   plan[4] = lp.starts_with_qkv;
   plan[5] = lp.mask_direct;
 }

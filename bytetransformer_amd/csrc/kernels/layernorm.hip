@@ -87,13 +87,13 @@ __device__ __forceinline__ void ln_finish(const half8_t (&av)[NC], const half8_t
 // at the top in one batch, a lane past the end of the row loads the last chunk again
 // instead of branching, and the only dependent step left is the row(s) behind an index.
 template <int NC, bool RESTORE, bool GB32, int SPLITS>
-__global__ __launch_bounds__(kLnRowsPerBlock *kWave) void layernorm_kernel(
-    const half8_t *src, const half8_t *__restrict__ residual,
+__device__ __forceinline__ void layernorm_block(
+    int block, const half8_t *src, const half8_t *__restrict__ residual,
     const half8_t *__restrict__ bias, const void *__restrict__ gamma,
     const void *__restrict__ beta, half8_t *dst, const int *__restrict__ idx,
     const int *__restrict__ residual_row_index, int B, int S, int rows_cap, int split_rows,
     int chunks, float inv_n, float eps) {
-  const int r = blockIdx.x * kLnRowsPerBlock + (threadIdx.x >> 6);
+  const int r = block * kLnRowsPerBlock + (threadIdx.x >> 6);
   const int lane = threadIdx.x & 63;
   if (r >= rows_cap) return;
   // fp32 gamma / beta of wide rows would not fit the registers next to the row: those
@@ -210,6 +210,44 @@ __global__ __launch_bounds__(kLnRowsPerBlock *kWave) void layernorm_kernel(
                                     dst + dst_row * chunks, inv_n, eps);
 }
 
+template <int NC, bool RESTORE, bool GB32, int SPLITS>
+__global__ __launch_bounds__(kLnRowsPerBlock *kWave) void layernorm_kernel(
+    const half8_t *src, const half8_t *__restrict__ residual,
+    const half8_t *__restrict__ bias, const void *__restrict__ gamma,
+    const void *__restrict__ beta, half8_t *dst, const int *__restrict__ idx,
+    const int *__restrict__ residual_row_index, int B, int S, int rows_cap, int split_rows,
+    int chunks, float inv_n, float eps) {
+  layernorm_block<NC, RESTORE, GB32, SPLITS>(blockIdx.x, src, residual, bias, gamma, beta, dst, idx,
+                                             residual_row_index, B, S, rows_cap, split_rows, chunks,
+                                             inv_n, eps);
+}
+
+// The packed LayerNorm with k-contiguous weight copies riding along: the first `copy_blocks`
+// workgroups of the grid move 64 x 64 tiles of the [K, N] matrices of `jobs` into their [N, K]
+// copies (through LDS, as the layer's prologue launch does), the others are the LayerNorm's.
+// A launch of a few thousand rows moves its 20 MB at half of what the memory system
+// sustains, so the copy of a few MB costs this launch less than a launch of its own would,
+// and the product behind it (FFN1) reads its weight k-contiguous.
+template <int NC, bool GB32>
+__global__ __launch_bounds__(kLnRowsPerBlock *kWave) void layernorm_copy_kernel(
+    const half8_t *src, const half8_t *__restrict__ residual,
+    const half8_t *__restrict__ bias, const void *__restrict__ gamma,
+    const void *__restrict__ beta, half8_t *dst, const int *__restrict__ idx,
+    const int *__restrict__ residual_row_index, int rows_cap, int chunks, float inv_n, float eps,
+    WeightJobs jobs, int copy_blocks) {
+  static_assert(kLnRowsPerBlock * kWave == 256, "a tile is moved by 256 threads");
+  if ((int)blockIdx.x < copy_blocks) {
+    __shared__ half_t tiles[64][kTransposePitch];
+    const int t_end = jobs.tile_end[jobs.count - 1];
+    for (int t0 = blockIdx.x; t0 < t_end; t0 += copy_blocks)
+      transpose_tiles_64<1>(jobs, t0, tiles, threadIdx.x);
+    return;
+  }
+  layernorm_block<NC, false, GB32, 0>((int)blockIdx.x - copy_blocks, src, residual, bias, gamma,
+                                      beta, dst, idx, residual_row_index, 0, 1, rows_cap, rows_cap,
+                                      chunks, inv_n, eps);
+}
+
 template <bool RESTORE, int SPLITS = 0>
 static int launch_ln(const void *src, const void *residual, const void *bias, const void *gamma,
                      const void *beta, int gb32, void *dst, const int *idx,
@@ -270,6 +308,64 @@ extern "C" int bt_add_bias_residual_layernorm(void *out, const void *residual,
   return launch_ln<false>(out, residual, bias, gamma, beta, gamma_beta_fp32, out, valid_rows,
                           residual_row_index, 0, 1, rows_cap, hidden_dim, eps, as_stream(stream),
                           "bt_add_bias_residual_layernorm");
+}
+
+extern "C" int bt_add_bias_residual_layernorm_copy(
+    void *out, const void *residual, const int *residual_row_index, const void *bias,
+    const void *gamma, const void *beta, int gamma_beta_fp32, const int *valid_rows, int rows_cap,
+    int hidden_dim, float eps, int weight_count, const void *const *w, void *const *wt,
+    const int *k, const int *n, void *stream) {
+  const char *who = "bt_add_bias_residual_layernorm_copy";
+  BT_REQUIRE(out && residual && bias && gamma && beta, BT_ERR_INVALID_ARGUMENT,
+             "%s: null pointer argument", who);
+  BT_REQUIRE(rows_cap >= 0, BT_ERR_INVALID_ARGUMENT, "%s: negative rows_cap", who);
+  BT_REQUIRE(!residual_row_index || valid_rows, BT_ERR_INVALID_ARGUMENT,
+             "%s: residual_row_index needs valid_rows", who);
+  WeightJobs jobs;
+  const int rc = make_weight_jobs(who, &jobs, weight_count, w, wt, k, n, 0, nullptr, nullptr);
+  if (rc != BT_OK) return rc;
+  if (jobs.count == 0)
+    return launch_ln<false>(out, residual, bias, gamma, beta, gamma_beta_fp32, out, valid_rows,
+                            residual_row_index, 0, 1, rows_cap, hidden_dim, eps, as_stream(stream),
+                            who);
+  const int H = hidden_dim;
+  BT_REQUIRE(H > 0 && H % 8 == 0, BT_ERR_UNSUPPORTED, "%s: hidden_dim %d must be a multiple of 8",
+             who, H);
+  BT_REQUIRE(aligned16({out, residual, bias, gamma, beta}), BT_ERR_INVALID_ARGUMENT,
+             "%s: tensor pointers must be 16-byte aligned", who);
+  const int chunks = H / 8;
+  const int nc = (chunks + kWave - 1) / kWave;
+  BT_REQUIRE(nc <= 8, BT_ERR_UNSUPPORTED, "%s: hidden_dim %d exceeds 4096", who, H);
+  // one tile per copying workgroup up to 1024 of them (a BERT-large FFN weight has 1024 tiles)
+  const int tiles = jobs.tile_end[jobs.count - 1];
+  const int copy_blocks = tiles < 1024 ? tiles : 1024;
+  const int grid = copy_blocks + (rows_cap + kLnRowsPerBlock - 1) / kLnRowsPerBlock;
+  const float inv_n = 1.0f / (float)H;
+  hipStream_t s = as_stream(stream);
+#define BT_LN_LAUNCH(NC_, GB_)                                                                  \
+  layernorm_copy_kernel<NC_, GB_><<<grid, kLnRowsPerBlock * kWave, 0, s>>>(                     \
+      (const half8_t *)out, (const half8_t *)residual, (const half8_t *)bias, gamma, beta,      \
+      (half8_t *)out, valid_rows, residual_row_index, rows_cap, chunks, inv_n, eps, jobs,       \
+      copy_blocks)
+#define BT_LN_NC(NC_)              \
+  do {                             \
+    if (gamma_beta_fp32)           \
+      BT_LN_LAUNCH(NC_, true);     \
+    else                           \
+      BT_LN_LAUNCH(NC_, false);    \
+  } while (0)
+  if (nc <= 1)
+    BT_LN_NC(1);
+  else if (nc <= 2)
+    BT_LN_NC(2);
+  else if (nc <= 4)
+    BT_LN_NC(4);
+  else
+    BT_LN_NC(8);
+#undef BT_LN_NC
+#undef BT_LN_LAUNCH
+  BT_CHECK_LAUNCH(who);
+  return BT_OK;
 }
 
 extern "C" int bt_add_bias_residual_layernorm_restore(

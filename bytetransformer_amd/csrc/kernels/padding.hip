@@ -39,6 +39,7 @@ static std::atomic<int> g_f32_gemm_tile{-1};
 static std::atomic<int> g_attention_short_limit{0};
 static std::atomic<int> g_attention_xcd_map{2};
 static std::atomic<int> g_gemm_table_margin{4};
+static std::atomic<int> g_ln_weight_copy{1};
 int option_gemm_table_margin() { return g_gemm_table_margin.load(std::memory_order_relaxed); }
 int option_attention_xcd_map() { return g_attention_xcd_map.load(std::memory_order_relaxed); }
 int option_f32_gemm_tile() { return g_f32_gemm_tile.load(std::memory_order_relaxed); }
@@ -395,6 +396,10 @@ extern "C" int bt_set_option(const char *name, int value) {
     BT_REQUIRE(value >= -1 && value <= 8, BT_ERR_INVALID_ARGUMENT,
                "bt_set_option: gemm_tile=%d outside [-1, 8]", value);
     g_gemm_tile.store(value);
+  } else if (!strcmp(name, "ln_weight_copy")) {
+    BT_REQUIRE(value == 0 || value == 1, BT_ERR_INVALID_ARGUMENT,
+               "bt_set_option: ln_weight_copy=%d must be 0 or 1", value);
+    g_ln_weight_copy.store(value);
   } else if (!strcmp(name, "gemm_table_margin")) {
     BT_REQUIRE(value >= 0 && value <= 100, BT_ERR_INVALID_ARGUMENT,
                "bt_set_option: gemm_table_margin=%d outside [0, 100]", value);
@@ -450,6 +455,8 @@ extern "C" int bt_get_option(const char *name, int *value) {
   BT_REQUIRE(name && value, BT_ERR_INVALID_ARGUMENT, "bt_get_option: null argument");
   if (!strcmp(name, "gemm_tile")) {
     *value = g_gemm_tile.load();
+  } else if (!strcmp(name, "ln_weight_copy")) {
+    *value = g_ln_weight_copy.load();
   } else if (!strcmp(name, "gemm_table_margin")) {
     *value = g_gemm_table_margin.load();
   } else if (!strcmp(name, "attention_qb")) {

@@ -65,14 +65,15 @@ class BertEncoderLayer:
 
     def plan(self, batch_size, seq_len, rows_hint=0):
         """bt_encoder_layer_plan for a call of this size: ([copy] * 4 for the QKV, projection,
-        FFN1 and FFN2 weights, starts_with_qkv, mask_direct) - what the layer will launch,
-        for benchmarks that time the kernels one by one."""
+        FFN1 and FFN2 weights - 0 read as stored, 1 copied by the launch ahead of the layer, 2 by
+        the first LayerNorm's launch -, starts_with_qkv, mask_direct): what the layer will
+        launch, for benchmarks that time the kernels one by one."""
         lib = host_lib()
         cfg = self._config(batch_size, seq_len)
         out = (ctypes.c_int * 6)()
         if lib.bt_encoder_layer_plan(ctypes.byref(cfg), batch_size, seq_len, int(rows_hint), out) != 0:
             raise RuntimeError(lib.bt_encoder_last_error().decode())
-        return [bool(v) for v in out[:4]], bool(out[4]), bool(out[5])
+        return [int(v) for v in out[:4]], bool(out[4]), bool(out[5])
 
     def __call__(self, x, mask, out=None, attention_bias=None):
         lib = host_lib()

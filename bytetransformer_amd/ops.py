@@ -335,6 +335,19 @@ def add_bias_residual_layernorm(out, residual, bias, gamma, beta, eps=1e-6, vali
     return out
 
 
+def add_bias_residual_layernorm_copy(out, residual, bias, gamma, beta, weights, packed, eps=1e-6,
+                                     valid_rows=None, residual_row_index=None):
+    """add_bias_residual_layernorm whose launch also fills `packed` with the [n, k] copies of the
+    [k, n] `weights` (up to four)."""
+    rows, H = out.shape
+    n, src, dst, ks, ns = _weight_jobs(weights, packed, ())[:5]
+    _check(kernel_lib().bt_add_bias_residual_layernorm_copy(
+        _ptr(out), _ptr(residual), _ptr(residual_row_index), _ptr(bias), _ptr(gamma), _ptr(beta),
+        int(gamma.dtype == torch.float32), _ptr(valid_rows), rows, H, float(eps), n, src, dst, ks,
+        ns, _stream()))
+    return out
+
+
 def add_bias_residual_layernorm_restore(out, residual, bias, gamma, beta, batch_idx, batch_size,
                                         seq_len, eps=1e-6, out_padded=None, word_idx=None):
     """word_idx: the complete word_idx of the same offsets (the row map); `out` and `residual`

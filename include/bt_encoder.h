@@ -63,8 +63,9 @@ int bt_encoder_layer_forward(const bt_encoder_config *cfg, const bt_layer_weight
  * product, for benchmarks that time the kernels one by one (host decisions only - sizes,
  * options, the measured tile table -, never a matter of results; no counterpart in the
  * reference).  rows_hint: the expected number of valid tokens, 0 = unknown.  plan[0..3]:
- * 1 where the QKV / projection / FFN1 / FFN2 product runs on a k-contiguous copy of its
- * weight made in the call's first launch; plan[4]: 1 when the layer starts with the QKV
+ * where the QKV / projection / FFN1 / FFN2 product runs on a k-contiguous copy of its
+ * weight made during the call, 1 = by the call's first launch (bt_layer_prologue), 2 = by the
+ * launch of the first LayerNorm (FFN1, FFN2), 0 = read as stored; plan[4]: 1 when the layer starts with the QKV
  * product that counts the mask rows itself (bt_gemm_qkv_bias_split_mask_rows) instead of
  * bt_layer_prologue; plan[5]: 1 when a layer on padded rows goes without offsets altogether.
  */

@@ -72,6 +72,10 @@ const char *bt_last_error_string(void);
  *                   per-call weight copy pays | always with bt_layer_prologue | with the
  *                   fused entry wherever it takes the shape, without copies.  Same results
  *                   either way.
+ *   "ln_weight_copy"  1 (default) | 0: a padding-free fp16 layer that goes without
+ *                   bt_layer_prologue lets the launch of its first LayerNorm make the k-contiguous
+ *                   copies that pay for FFN1 and FFN2 (bt_add_bias_residual_layernorm_copy) | such
+ *                   a layer makes no copies (or keeps the prologue for them).  Same results.
  *   "prefetch"      1 (default) | 0: honour / ignore the prefetch hint of the attention entries
  *   "prefetch_min_grid"  512 (default): attention launches of fewer workgroups ignore the hint
  *                   (there the warm-up costs more than it returns); 1 = every launch honours it
@@ -369,6 +373,24 @@ int bt_add_bias_residual_layernorm(void *out, const void *residual,
                                    const void *gamma, const void *beta, int gamma_beta_fp32,
                                    const int *valid_rows, int rows_cap, int hidden_dim,
                                    float eps, void *stream);
+
+/*
+ * The same launch with k-contiguous weight copies riding along: weight_count (0..4) matrices
+ * w[i] [k[i], n[i]] are copied into wt[i] [n[i], k[i]] (bt_transpose_weights) by workgroups of
+ * their own at the head of the grid, complete when the launch is.  A LayerNorm over a few
+ * thousand rows leaves most of the memory system idle, so the copies cost this launch less than
+ * a launch of their own would - the layer uses it for the weight of the product that follows
+ * (FFN1; the role of the reference's one-off weight layout choice, gemm.cu:27-39, made per
+ * call so that nothing is kept between calls).  With weight_count == 0 it is
+ * bt_add_bias_residual_layernorm.
+ */
+int bt_add_bias_residual_layernorm_copy(void *out, const void *residual,
+                                        const int *residual_row_index, const void *bias,
+                                        const void *gamma, const void *beta, int gamma_beta_fp32,
+                                        const int *valid_rows, int rows_cap, int hidden_dim,
+                                        float eps, int weight_count, const void *const *w,
+                                        void *const *wt, const int *k, const int *n,
+                                        void *stream);
 
 /*
  * Same LayerNorm, but reading packed rows and writing the padded layout:

@@ -92,7 +92,8 @@ struct LayerPlan {
   bool mask_direct = false;      // padded rows, short sequences: no offsets at all
   bool starts_with_qkv = false;  // the QKV product counts the mask rows itself: no launch ahead of it
   bool copy[4] = {false, false, false, false};   // QKV, projection, FFN1, FFN2 run on a per-call copy
-  int copies = 0;
+  int copies = 0;                                // ... made by the launch ahead of the layer
+  bool ln_copy[4] = {false, false, false, false};   // FFN1, FFN2: ... made by the first LayerNorm's launch
 };
 
 template <OperationType OpType>

@@ -76,28 +76,46 @@ inline unsigned long long splitk_scratch_bytes(unsigned long long max_rows,
 }
 
 // Which of a padding-free fp16 layer's four products (QKV, projection, FFN1, FFN2; weights
-// [k, n] as stored) run on a k-contiguous copy made afresh in the call's first launch.
-// `live` = expected valid tokens, `padded_rows` = batch x seq_len, `first_launch_optional` =
-// the QKV product could count the mask rows itself, so that a layer without copies goes
-// without any launch ahead of it.  There the copies have to return what that launch costs
-// (about 3 us beyond the copies themselves with one round of tiles: never copying wins
-// 1.5-1.8 % per forward up to 10 k padded rows and loses as much beyond), elsewhere a
-// microsecond more than they cost.  Returns the number of copies and sets copy[i].
+// [k, n] as stored) run on a k-contiguous copy made afresh in the call, and by which launch:
+// copy[i] - by the launch ahead of the layer (bt_layer_prologue), ln_copy[i] - by the first
+// LayerNorm's launch (FFN1 and FFN2 only: the products behind it).  A product gets a copy
+// when the measured tile table says it gains more than a microsecond beyond the cost of the
+// copy.  `live` = expected valid tokens, `padded_rows` = batch x seq_len,
+// `first_launch` = 0: the layer has a launch ahead of it in any case, 1: the QKV product could
+// count the mask rows itself, so that a layer with nothing for a prologue to do goes without
+// it, 2: it does so in any case; `ln_can_copy` = the LayerNorm's launch may carry copies.  Where the prologue is optional it is kept only if the copies that nothing
+// else can make (QKV, projection) return what it costs (about 4 us with one round of tiles) -
+// it then makes the others as well; without it the FFN copies ride in the LayerNorm's launch
+// (or, if they may not, are dropped unless they pay for a prologue: up to 10 k padded rows
+// never copying then wins 1.5-1.8 % per forward and loses as much beyond).
+// Returns the number of prologue copies.
 inline int plan_weight_copies(long long live, long long padded_rows, int hidden, int inter,
-                              bool split_heads, bool first_launch_optional, bool copy[4]) {
+                              bool split_heads, int first_launch, bool ln_can_copy, bool copy[4],
+                              bool ln_copy[4]) {
   const int n[4] = {3 * hidden, hidden, inter, hidden}, k[4] = {hidden, hidden, hidden, inter};
   const int epilogue[4] = {split_heads ? BT_EPILOGUE_QKV_SPLIT : -1, BT_EPILOGUE_PLAIN,
                            BT_EPILOGUE_BIAS_GELU, BT_EPILOGUE_PLAIN};
-  float gain[4] = {0.f, 0.f, 0.f, 0.f}, total = 0.f;
+  float gain[4] = {0.f, 0.f, 0.f, 0.f}, early = 0.f, total = 0.f;
+  bool want[4];
   for (int i = 0; i < 4; ++i) {
-    if (epilogue[i] < 0) continue;
-    gain[i] = bt_gemm_prepack_gain_us(live, n[i], k[i], epilogue[i]);
-    if (gain[i] > 1.0f) total += gain[i];
+    if (epilogue[i] >= 0) gain[i] = bt_gemm_prepack_gain_us(live, n[i], k[i], epilogue[i]);
+    want[i] = gain[i] > 1.0f;
+    if (want[i]) total += gain[i];
+    if (want[i] && i < 2) early += gain[i];
   }
-  const bool launch_at_stake = first_launch_optional && padded_rows <= 10240;
-  const bool copy_any = !launch_at_stake || total > 1e8f || total >= 4.0f;
+  bool prologue = true;
+  if (first_launch == 1)
+    prologue = ln_can_copy ? early >= 4.0f : (padded_rows > 10240 ? total > 0.f : total >= 4.0f);
+  if (first_launch == 2) prologue = false;
   int count = 0;
-  for (int i = 0; i < 4; ++i) count += (copy[i] = copy_any && gain[i] > 1.0f);
+  for (int i = 0; i < 4; ++i) {
+    copy[i] = prologue && want[i];
+    // (in the LayerNorm's launch a copy has to return more: that launch grows by 1-4 us and the
+    // product then reads a copy that was written a moment ago - measured: 1.5 us of table gain
+    // lose 0.6 % per forward at batch 16 x 512, 4.5 us win 1.8 % at 16 x 1024)
+    ln_copy[i] = !prologue && ln_can_copy && i >= 2 && gain[i] >= 3.0f;
+    count += copy[i];
+  }
   return count;
 }
 

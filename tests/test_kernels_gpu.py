@@ -244,6 +244,45 @@ def test_add_bias_residual_layernorm(device, H, gb32):
     assert np.all(err <= 2.0 ** -10 * np.abs(exp) + 1e-4)
 
 
+@pytest.mark.parametrize("H,gb32,rows,M", [(768, False, 300, 211), (1024, True, 37, 37),
+                                           (64, False, 5, 0), (2048, False, 130, 129)])
+def test_layernorm_with_weight_copies_riding_along(device, H, gb32, rows, M):
+    """The LayerNorm launch that also makes k-contiguous weight copies: the rows are the bits of
+    the plain launch (gathered residual, live-row count), the copies are the transposed
+    matrices - tiles that are partial in either direction, four matrices, guard bytes on both
+    sides of every copy, none at all."""
+    _say("layernorm + copies", H, gb32, rows, M)
+    rs = np.random.RandomState(H + rows)
+    out = rs.standard_normal((rows, H)).astype(np.float16)
+    res = (rs.standard_normal((rows + 9, H)) * 2).astype(np.float16)
+    ridx = rs.permutation(rows + 9)[:rows].astype(np.int32)
+    bias = (rs.standard_normal(H) * 0.5).astype(np.float16)
+    gdt = np.float32 if gb32 else np.float16
+    gamma = (1 + 0.2 * rs.standard_normal(H)).astype(gdt)
+    beta = (0.3 * rs.standard_normal(H)).astype(gdt)
+    vr = torch.tensor([M], dtype=torch.int32, device=device)
+    args = [_dev(a, device) for a in (res, bias, gamma, beta)]
+    ri = _dev(ridx, device)
+    plain = ops.add_bias_residual_layernorm(_dev(out, device), *args, 1e-6, valid_rows=vr,
+                                            residual_row_index=ri)
+    for shapes in (((H, 4 * H),), ((H, 4 * H), (4 * H, H), (72, 200), (8, 8)), ()):
+        ws = [_dev((rs.standard_normal(sh) * 0.1).astype(np.float16), device) for sh in shapes]
+        # each copy sits inside a larger buffer of sevens: nothing beside it may change
+        bufs = [torch.full((w.numel() + 256,), 7.0, dtype=torch.float16, device=device) for w in ws]
+        packed = [b[128:128 + w.numel()].view(w.shape[1], w.shape[0]) for b, w in zip(bufs, ws)]
+        got = ops.add_bias_residual_layernorm_copy(_dev(out, device), *args, ws, packed, 1e-6,
+                                                   valid_rows=vr, residual_row_index=ri)
+        assert torch.equal(got, plain), shapes
+        for w, t, b in zip(ws, packed, bufs):
+            assert torch.equal(t, w.t().contiguous()), tuple(w.shape)
+            assert bool((b[:128] == 7).all()) and bool((b[128 + w.numel():] == 7).all())
+    if M:
+        exp = O.add_bias_residual_layernorm(out[:M], res[ridx[:M]], bias, gamma, beta, 1e-6)
+        err = np.abs(plain.cpu().numpy()[:M].astype(np.float64) - exp)
+        assert np.all(err <= 2.0 ** -10 * np.abs(exp) + 1e-4), err.max()
+    assert np.array_equal(plain.cpu().numpy()[M:], out[M:])
+
+
 @pytest.mark.parametrize("B,S,H", [(4, 33, 768), (16, 128, 1024)])
 def test_layernorm_restore_zero_fills_padding(device, B, S, H):
     _say("layernorm_restore", B, S, H)

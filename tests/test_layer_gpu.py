@@ -822,6 +822,41 @@ def test_qkv_rows_from_the_mask_never_change_the_result(device):
         _check(got[1].cpu().numpy(), _oracle(wl), wl.lens, tag="qkv_mask_rows " + cfg.name)
 
 
+def test_weight_copies_in_the_layernorm_launch_never_change_the_result(device):
+    """FFN1's (and FFN2's) k-contiguous copy may be made by the first LayerNorm's launch instead
+    of a prologue, or not at all: the same bits with the option on and off, on the headline
+    shape, with several rounds of tiles, on BERT-large shapes, with the fused start forced and
+    with the prologue forced - and within tolerance of the oracle."""
+    _say("ln_weight_copy")
+    from bytetransformer_amd import ops
+    bt.load_th_op()
+    op = torch.ops.ByteTransformer.BertTransformer
+    assert ops.get_option("ln_weight_copy") == 1
+    cases = (workload.EncoderConfig("lc", 16, 512, 12, layers=1, seed=31),
+             workload.EncoderConfig("lc2", 16, 1024, 12, layers=1, seed=32),
+             workload.EncoderConfig("lc3", 32, 384, 16, layers=1, seed=33),
+             workload.EncoderConfig("lc4", 6, 200, 12, layers=1, lens=(200, 0, 133, 50, 64, 7), seed=34))
+    for cfg in cases:
+        wl = workload.make_workload(cfg, bias_std=0.05, random_affine=True)
+        w = [_dev(wl.layers[0][n], device) for n in workload.WEIGHT_NAMES]
+        x, m = _dev(wl.x, device), _dev(wl.mask, device)
+        got = {}
+        try:
+            for ln_copy, start, prepack in ((1, -1, -1), (0, -1, -1), (1, 1, -1), (1, 0, -1), (1, 1, 1), (0, 1, 1)):
+                ops.set_option("ln_weight_copy", ln_copy)
+                ops.set_option("qkv_mask_rows", start)
+                ops.set_option("layer_prepack", prepack)
+                got[(ln_copy, start, prepack)] = op(cfg.head_num, 64, *w, x, m, True, True)
+        finally:
+            ops.set_option("ln_weight_copy", 1)
+            ops.set_option("qkv_mask_rows", -1)
+            ops.set_option("layer_prepack", -1)
+        ref = got[(0, -1, -1)]
+        for key, val in got.items():
+            assert torch.equal(val, ref), (cfg.name, key)
+        _check(ref.cpu().numpy(), _oracle(wl), wl.lens, tag="ln_weight_copy " + cfg.name)
+
+
 def test_short_padded_layers_go_without_the_prologue(device):
     """Batches of one and two with up to padded_mask_direct tokens per sequence skip the
     prologue launch and let the attention apply the mask tensor: same results as with the
