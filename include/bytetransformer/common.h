@@ -110,10 +110,10 @@ inline int plan_weight_copies(long long live, long long padded_rows, int hidden,
   int count = 0;
   for (int i = 0; i < 4; ++i) {
     copy[i] = prologue && want[i];
-    // (in the LayerNorm's launch a copy has to return more: that launch grows by 1-4 us and the
-    // product then reads a copy that was written a moment ago - measured: 1.5 us of table gain
-    // lose 0.6 % per forward at batch 16 x 512, 4.5 us win 1.8 % at 16 x 1024)
-    ln_copy[i] = !prologue && ln_can_copy && i >= 2 && gain[i] >= 3.0f;
+    // (measured where the table's gain is smallest, 1.5 us for FFN1 at batch 16 x 512: kernel time
+    // -1 % per forward, wall time -0.5 % on one box and +0.6 % on another; with 4.5 us at
+    // 16 x 1024, where the copy also replaces the prologue, -2 %)
+    ln_copy[i] = !prologue && ln_can_copy && i >= 2 && want[i];
     count += copy[i];
   }
   return count;

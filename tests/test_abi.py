@@ -181,12 +181,12 @@ def test_package_does_not_import_the_oracle():
 
 
 def test_layer_plan_is_a_host_side_decision():
-    """bt_encoder_layer_plan answers without a GPU: at the headline shape the layer makes no
-    weight copy and starts with the QKV product that counts the mask rows; with several rounds
-    of tiles it still starts that way and lets its first LayerNorm's launch make FFN1's copy
-    (2) - without that option the prologue and its copy (1) again, as for a layer that may not
-    start with the QKV product; beyond 32 sequences the prologue makes the copies; a short
-    batch of one goes without offsets."""
+    """bt_encoder_layer_plan answers without a GPU: at the headline shape and with several
+    rounds of tiles the layer starts with the QKV product that counts the mask rows and lets
+    its first LayerNorm's launch make FFN1's copy (2) - without that option no copy at the
+    headline shape and the prologue with its copy (1) at the larger one, as for a layer that
+    may not start with the QKV product; beyond 32 sequences the prologue makes the copies; a
+    short batch of one goes without offsets."""
     import ctypes
     from bytetransformer_amd._lib import EncoderConfig, host_lib, kernel_lib
     lib = host_lib()
@@ -197,7 +197,7 @@ def test_layer_plan_is_a_host_side_decision():
         assert lib.bt_encoder_layer_plan(ctypes.byref(cfg), batch, seq, hint, out) == 0
         return list(out)
 
-    assert plan(16, 512, 4809) == [0, 0, 0, 0, 1, 0]
+    assert plan(16, 512, 4809) == [0, 0, 2, 0, 1, 0]
     assert plan(16, 1024, 9800) == [0, 0, 2, 0, 1, 0]
     big = plan(64, 256, 9800)
     assert big[4] == 0 and big[2] == 1
@@ -205,6 +205,7 @@ def test_layer_plan_is_a_host_side_decision():
     kl = kernel_lib()
     try:
         assert kl.bt_set_option(b"ln_weight_copy", 0) == 0
+        assert plan(16, 512, 4809) == [0, 0, 0, 0, 1, 0]
         big = plan(16, 1024, 9800)
         assert big[4] == 0 and big[5] == 0 and big[2] == 1
         assert kl.bt_set_option(b"ln_weight_copy", 2) == 1
