@@ -126,9 +126,6 @@ void BertTransformer<OpType>::bert_infer(BertTransformerInferParam infer_param) 
   const void *pack_src[4], *ln_src[4];
   void *pack_dst[4], *ln_dst[4];
   int pack_k[4], pack_n[4], pack_count = 0, ln_k[4], ln_n[4], ln_count = 0;
-  // what the attention's cache warm-up touches: the matrices as the caller stores them where a
-  // later launch of the layer makes the copy (it does not exist yet when the attention runs)
-  const DataType_ *w_touch[4] = {w_use[0], w_use[1], w_use[2], w_use[3]};
   if (have_prepack) {
     for (int i = 0; i < 4; ++i) {
       w_use[i] = param_.prepacked_kernels[i];
@@ -297,15 +294,21 @@ void BertTransformer<OpType>::bert_infer(BertTransformerInferParam infer_param) 
   // kernel finds its balanced order by a look-up of its own)
   attention_infer_param.work_list = nullptr;
   attention_infer_param.no_offsets = mask_direct;   // (nothing has written them)
-  // the three weight matrices the rest of the layer reads (as stored, or the copies of
-  // this call): the attention kernel pulls them into the memory-side cache while it runs
+  // the weight matrices the rest of the layer reads (as stored, or the copies that the first
+  // launch has made): the attention kernel pulls them into the memory-side cache while it
+  // runs.  A matrix that the first LayerNorm's launch copies is left alone: the copy reads
+  // its source once either way, and the product reads the copy (same box, with / without
+  // touching it: batch 16 x 512 1.519 / 1.514 ms, 16 x 1024 2.586 / 2.574, BERT-large 6.610 / 6.589).
   {
     const size_t elems[3] = {(size_t)hidden * hidden, (size_t)hidden * inter, (size_t)hidden * inter};
+    int pc = 0;
     for (int i = 0; i < 3; ++i) {
-      attention_infer_param.prefetch[i] = lp.ln_copy[i + 1] ? w_touch[i + 1] : w_use[i + 1];
-      attention_infer_param.prefetch_bytes[i] = elems[i] * sizeof(DataType_);
+      if (lp.ln_copy[i + 1]) continue;
+      attention_infer_param.prefetch[pc] = w_use[i + 1];
+      attention_infer_param.prefetch_bytes[pc] = elems[i] * sizeof(DataType_);
+      ++pc;
     }
-    attention_infer_param.prefetch_count = 3;
+    attention_infer_param.prefetch_count = pc;
   }
   attention_layer_->infer(attention_infer_param);
 
